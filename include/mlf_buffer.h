@@ -1,0 +1,79 @@
+/*
+ * C-ABI of the file-backed shared-memory buffer object and of the host-side bulk copy helpers.
+ *
+ * A buffer object is a regular file (normally on tmpfs) mapped MAP_SHARED into the process.  It is the
+ * destination of a checkpoint save and the source of a restore.  The entry points below are what a
+ * language binding binds in place of the reference's pybind11 class `BufferObject`
+ * (reference: src/ml_flashpoint/checkpoint_object_manager/buffer_object/bindings.cpp:27-100,
+ * buffer_object.h:24-85).
+ *
+ * Conventions: every function that can fail returns an mlf_status (0 = ok).  On failure a
+ * human-readable message is kept per thread and can be fetched with mlf_buffer_last_error(); the
+ * text follows the shape "<CODE_NAME>: <message>" that the reference's status strings have, so callers
+ * that match on substrings of those messages keep working.  No function throws across the boundary.
+ */
+#ifndef MLF_BUFFER_H_
+#define MLF_BUFFER_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum mlf_status {
+  MLF_OK = 0,
+  MLF_INVALID_ARGUMENT = 3, /* bad size, directory instead of file, empty file, closed handle */
+  MLF_ALREADY_EXISTS = 6,   /* create without overwrite on an existing path */
+  MLF_FAILED_PRECONDITION = 9,
+  MLF_INTERNAL = 13         /* a system call failed; message carries strerror text */
+} mlf_status;
+
+typedef struct mlf_buffer mlf_buffer; /* opaque */
+
+/* Creates (or, with overwrite != 0, truncates and re-creates) the file `object_id`, sizes it to
+ * `capacity` bytes and maps it read-write.  Parent directories are created.  Without overwrite an
+ * existing path fails with MLF_ALREADY_EXISTS.
+ * Replaces BufferObject(object_id, capacity, overwrite): buffer_object.cpp:25-49,
+ * buffer_helper.cpp:43-120. */
+int mlf_buffer_create(const char* object_id, size_t capacity, int overwrite, mlf_buffer** out);
+
+/* Maps an existing, non-empty regular file read-only; capacity is the file size.
+ * Replaces BufferObject(object_id): buffer_object.cpp:52-73, buffer_helper.cpp:122-185. */
+int mlf_buffer_open_readonly(const char* object_id, mlf_buffer** out);
+
+/* Unmaps, optionally truncates the file to `truncate_size` bytes (has_truncate != 0), closes the
+ * descriptor.  Idempotent; the handle stays valid (in the closed state) until mlf_buffer_destroy.
+ * A truncate request on a read-only mapping is ignored.  Every step is attempted even if an earlier
+ * one failed; the failures are joined in the error text.
+ * Replaces BufferObject::close: buffer_object.cpp:140-176, buffer_helper.cpp:187-271. */
+int mlf_buffer_close(mlf_buffer* b, int has_truncate, size_t truncate_size);
+
+/* Closes (without truncation) if still open and frees the handle. Replaces ~BufferObject. */
+void mlf_buffer_destroy(mlf_buffer* b);
+
+/* munmap + ftruncate + mmap to a new capacity; the data pointer changes.  Fails on closed or read-only
+ * handles and on new_capacity == 0.
+ * Replaces BufferObject::resize: buffer_object.cpp:178-197, buffer_helper.cpp:273-314. */
+int mlf_buffer_resize(mlf_buffer* b, size_t new_capacity);
+
+/* Accessors (bindings.cpp:43-76).  data_ptr is NULL and capacity 0 once closed. */
+void* mlf_buffer_data_ptr(const mlf_buffer* b);
+size_t mlf_buffer_capacity(const mlf_buffer* b);
+int mlf_buffer_is_closed(const mlf_buffer* b);
+int mlf_buffer_is_readonly(const mlf_buffer* b);
+const char* mlf_buffer_id(const mlf_buffer* b);
+
+/* Message of the last failure on the calling thread ("" if none). */
+const char* mlf_buffer_last_error(void);
+
+/* Copies n bytes with up to `threads` worker threads (page-aligned split).  Used for host-resident
+ * checkpoint items and for restore staging; stands where the reference relies on torch's intra-op
+ * threaded copy_ (src/ml_flashpoint/core/checkpoint_saver.py:443-450,797-800). */
+int mlf_host_parallel_memcpy(void* dst, const void* src, size_t n, int threads);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MLF_BUFFER_H_ */

@@ -1,0 +1,234 @@
+// File-backed MAP_SHARED buffer object and host bulk-copy helpers behind the C-ABI in
+// include/mlf_buffer.h.  Plain POSIX, no third-party dependencies.
+//
+// Behaviour follows the reference's native buffer object
+// (src/ml_flashpoint/checkpoint_object_manager/buffer_object/buffer_helper.cpp:43-314 and
+// buffer_object.cpp:25-197): same system-call sequence, same failure conditions, same message
+// fragments; the structure (one POD handle + free functions + thread-local error text) is this
+// library's own.
+#include "mlf_buffer.h"
+
+#include <errno.h>
+#include <fcntl.h>
+#include <string.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <algorithm>
+#include <string>
+#include <thread>
+#include <vector>
+
+struct mlf_buffer {
+  std::string id;
+  void* ptr = nullptr;
+  size_t cap = 0;
+  int fd = -1;
+  bool writable = false;
+  bool closed = true;
+};
+
+namespace {
+
+thread_local std::string g_err;
+
+const char* code_name(int code) {
+  switch (code) {
+    case MLF_INVALID_ARGUMENT: return "INVALID_ARGUMENT";
+    case MLF_ALREADY_EXISTS: return "ALREADY_EXISTS";
+    case MLF_FAILED_PRECONDITION: return "FAILED_PRECONDITION";
+    case MLF_INTERNAL: return "INTERNAL";
+    default: return "UNKNOWN";
+  }
+}
+
+int fail(int code, const std::string& msg) {
+  g_err = std::string(code_name(code)) + ": " + msg;
+  return code;
+}
+
+int fail_errno(const std::string& msg, int err) {
+  return fail(MLF_INTERNAL, msg + ": " + strerror(err));
+}
+
+// mkdir -p for the directory part of `path`.
+int make_parent_dirs(const std::string& path) {
+  size_t slash = path.find_last_of('/');
+  if (slash == std::string::npos || slash == 0) return 0;
+  std::string dir = path.substr(0, slash);
+  for (size_t i = 1; i <= dir.size(); ++i) {
+    if (i != dir.size() && dir[i] != '/') continue;
+    std::string sub = dir.substr(0, i);
+    if (mkdir(sub.c_str(), 0777) != 0 && errno != EEXIST) return errno;
+  }
+  struct stat st;
+  if (stat(dir.c_str(), &st) != 0) return errno;
+  return S_ISDIR(st.st_mode) ? 0 : ENOTDIR;
+}
+
+bool is_open(const mlf_buffer* b) {
+  return b && !b->closed && b->ptr != nullptr && b->ptr != MAP_FAILED && b->fd != -1;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* mlf_buffer_last_error(void) { return g_err.c_str(); }
+
+int mlf_buffer_create(const char* object_id, size_t capacity, int overwrite, mlf_buffer** out) {
+  if (!object_id || !out) return fail(MLF_INVALID_ARGUMENT, "null argument");
+  *out = nullptr;
+  std::string id(object_id);
+  if (capacity == 0)
+    return fail(MLF_INVALID_ARGUMENT, "create_file_and_mmap requires a size greater than 0 for file: " + id);
+  if (int e = make_parent_dirs(id))
+    return fail(MLF_INTERNAL, "Failed to create directories for: " + id + ": " + strerror(e));
+
+  int flags = O_CREAT | O_RDWR | (overwrite ? O_TRUNC : O_EXCL);
+  int fd = open(object_id, flags, 0666);
+  if (fd == -1) {
+    int e = errno;
+    if (e == EEXIST && !overwrite)
+      return fail(MLF_ALREADY_EXISTS,
+                  "open() failed for file: " + id + ". File already exists and overwrite is set to false.");
+    return fail_errno("open() failed for file: " + id, e);
+  }
+  if (ftruncate(fd, (off_t)capacity) == -1) {
+    int e = errno;
+    close(fd);
+    return fail_errno("ftruncate() failed for file: " + id, e);
+  }
+  void* p = mmap(nullptr, capacity, PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
+  if (p == MAP_FAILED) {
+    int e = errno;
+    close(fd);
+    return fail_errno("mmap() failed for file: " + id, e);
+  }
+  mlf_buffer* b = new mlf_buffer();
+  b->id = id;
+  b->ptr = p;
+  b->cap = capacity;
+  b->fd = fd;
+  b->writable = true;
+  b->closed = false;
+  *out = b;
+  return MLF_OK;
+}
+
+int mlf_buffer_open_readonly(const char* object_id, mlf_buffer** out) {
+  if (!object_id || !out) return fail(MLF_INVALID_ARGUMENT, "null argument");
+  *out = nullptr;
+  std::string id(object_id);
+  struct stat st;
+  if (stat(object_id, &st) == 0 && S_ISDIR(st.st_mode))
+    return fail(MLF_INVALID_ARGUMENT, "Path is a directory, not a file: " + id);
+  int fd = open(object_id, O_RDONLY);
+  if (fd == -1) return fail_errno("open() failed for file: " + id, errno);
+  if (fstat(fd, &st) == -1) {
+    int e = errno;
+    close(fd);
+    return fail_errno("fstat() failed for file: " + id, e);
+  }
+  if (st.st_size == 0) {
+    close(fd);
+    return fail(MLF_INVALID_ARGUMENT,
+                "File cannot be empty, open_file_and_mmap cannot handle zero-sized file: " + id);
+  }
+  void* p = mmap(nullptr, (size_t)st.st_size, PROT_READ, MAP_SHARED, fd, 0);
+  if (p == MAP_FAILED) {
+    int e = errno;
+    close(fd);
+    return fail_errno("mmap() failed for file: " + id, e);
+  }
+  mlf_buffer* b = new mlf_buffer();
+  b->id = id;
+  b->ptr = p;
+  b->cap = (size_t)st.st_size;
+  b->fd = fd;
+  b->writable = false;
+  b->closed = false;
+  *out = b;
+  return MLF_OK;
+}
+
+int mlf_buffer_close(mlf_buffer* b, int has_truncate, size_t truncate_size) {
+  if (!is_open(b)) return MLF_OK;
+  if (!b->writable) has_truncate = 0;  // read-only mappings are never truncated
+  std::string errs;
+  auto add = [&errs](const std::string& m) {
+    if (!errs.empty()) errs += "; ";
+    errs += m;
+  };
+  if (munmap(b->ptr, b->cap) == -1) add(std::string("munmap() failed: ") + strerror(errno));
+  if (has_truncate && ftruncate(b->fd, (off_t)truncate_size) == -1)
+    add(std::string("ftruncate() failed: ") + strerror(errno));
+  if (close(b->fd) == -1) add(std::string("close() failed: ") + strerror(errno));
+  b->closed = true;
+  b->fd = -1;
+  b->ptr = nullptr;
+  b->cap = 0;
+  if (!errs.empty()) return fail(MLF_INTERNAL, "Errors during unmap_and_close: " + errs);
+  return MLF_OK;
+}
+
+void mlf_buffer_destroy(mlf_buffer* b) {
+  if (!b) return;
+  mlf_buffer_close(b, 0, 0);
+  delete b;
+}
+
+int mlf_buffer_resize(mlf_buffer* b, size_t new_capacity) {
+  if (!is_open(b)) return fail(MLF_FAILED_PRECONDITION, "Cannot resize a closed buffer.");
+  if (!b->writable) return fail(MLF_FAILED_PRECONDITION, "Cannot resize a read-only buffer.");
+  if (new_capacity == 0) return fail(MLF_INVALID_ARGUMENT, "Cannot resize buffer to 0.");
+  if (new_capacity == b->cap) return MLF_OK;
+  if (munmap(b->ptr, b->cap) == -1) return fail_errno("munmap() failed during resize", errno);
+  b->ptr = nullptr;
+  if (ftruncate(b->fd, (off_t)new_capacity) == -1) {
+    int e = errno;
+    b->closed = true;  // mapping is gone; the handle cannot be used any more
+    return fail_errno("ftruncate() failed during resize", e);
+  }
+  void* p = mmap(nullptr, new_capacity, PROT_READ | PROT_WRITE, MAP_SHARED, b->fd, 0);
+  if (p == MAP_FAILED) {
+    int e = errno;
+    b->closed = true;
+    return fail_errno("mmap() failed during resize", e);
+  }
+  b->ptr = p;
+  b->cap = new_capacity;
+  return MLF_OK;
+}
+
+void* mlf_buffer_data_ptr(const mlf_buffer* b) { return is_open(b) ? b->ptr : nullptr; }
+size_t mlf_buffer_capacity(const mlf_buffer* b) { return is_open(b) ? b->cap : 0; }
+int mlf_buffer_is_closed(const mlf_buffer* b) { return is_open(b) ? 0 : 1; }
+int mlf_buffer_is_readonly(const mlf_buffer* b) { return (b && b->writable) ? 0 : 1; }
+const char* mlf_buffer_id(const mlf_buffer* b) { return b ? b->id.c_str() : ""; }
+
+int mlf_host_parallel_memcpy(void* dst, const void* src, size_t n, int threads) {
+  if (n == 0) return MLF_OK;
+  if (!dst || !src) return fail(MLF_INVALID_ARGUMENT, "null pointer passed to mlf_host_parallel_memcpy");
+  const size_t kMinPerThread = (size_t)4 << 20;
+  size_t want = std::max<size_t>(1, std::min<size_t>((size_t)std::max(threads, 1), n / kMinPerThread));
+  if (want <= 1) {
+    memcpy(dst, src, n);
+    return MLF_OK;
+  }
+  size_t per = (n + want - 1) / want;
+  per = (per + 4095) & ~(size_t)4095;
+  std::vector<std::thread> pool;
+  char* d = static_cast<char*>(dst);
+  const char* s = static_cast<const char*>(src);
+  for (size_t off = per; off < n; off += per) {
+    size_t len = std::min(per, n - off);
+    pool.emplace_back([d, s, off, len] { memcpy(d + off, s + off, len); });
+  }
+  memcpy(d, s, std::min(per, n));
+  for (auto& t : pool) t.join();
+  return MLF_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,65 @@
+"""Small helpers shared by the save/restore path (reference: src/ml_flashpoint/core/utils.py:27-159)."""
+
+import contextlib
+import logging
+import os
+import time
+
+import torch
+
+_ENV_PREFIX = "MLFLASHPOINT_"
+
+
+def get_env_var_prefix() -> str:
+    return _ENV_PREFIX
+
+
+def get_env_val_str(env_var_name: str, default_val: str) -> str:
+    return os.environ.get(_ENV_PREFIX + env_var_name, default_val)
+
+
+def get_env_val_int(env_var_name: str, default_val: int) -> int:
+    raw = os.environ.get(_ENV_PREFIX + env_var_name)
+    if raw is None:
+        return default_val
+    try:
+        return int(raw)
+    except ValueError:
+        return default_val
+
+
+def get_env_val_bool(env_var_name: str, default_val: bool) -> bool:
+    raw = os.environ.get(_ENV_PREFIX + env_var_name)
+    if raw is None:
+        return default_val
+    return raw.strip().lower() in ("1", "true", "yes", "on")
+
+
+def get_accelerator_count() -> int:
+    """Accelerators visible to this process (0 without a GPU)."""
+    try:
+        return torch.cuda.device_count()
+    except Exception:
+        return 0
+
+
+def get_num_of_nodes() -> int:
+    for var in ("NNODES", "SLURM_NNODES"):
+        raw = os.environ.get(var)
+        if raw:
+            try:
+                return max(int(raw), 1)
+            except ValueError:
+                pass
+    return 1
+
+
+@contextlib.contextmanager
+def log_execution_time(logger: logging.Logger, name: str, level: int = logging.DEBUG):
+    """Context manager *and* decorator that logs ``"<name> took <sec>s"`` (format kept: log parsers rely on it)."""
+    start = time.perf_counter()
+    try:
+        yield
+    finally:
+        if logger.isEnabledFor(level):
+            logger.log(level, "%s took %.4fs", name, time.perf_counter() - start)
