@@ -1,0 +1,154 @@
+/*
+ * C-ABI of the MI355X (gfx950) save/restore data path.
+ *
+ * The reference moves a checkpoint shard with three PyTorch calls per tensor and has no FFI for it:
+ *   save    - Tensor.to("cpu") per tensor + one device synchronize
+ *             (src/ml_flashpoint/core/checkpoint_saver.py:347-360,
+ *              src/ml_flashpoint/adapter/pytorch/memory_storage_writer.py:213-233), then
+ *             header + torch.frombuffer(mmap_slice).copy_(tensor) per tensor
+ *             (src/ml_flashpoint/core/checkpoint_saver.py:764-800);
+ *   restore - read() copy of each record, torch.frombuffer, narrow, target.copy_()
+ *             (src/ml_flashpoint/core/checkpoint_loader.py:177-219,300-336).
+ * The entry points below are what a binding binds instead.  They work on an "image": the byte-exact data
+ * section of one checkpoint object (records `<u32 len><pickled header><payload>` back to back), held in
+ * device memory.  Save = pack live tensors into the image, stream the image to the mapped buffer file;
+ * restore = stream the file into an image, unpack into live tensors.
+ *
+ * Conventions: plain pointers and sizes only; every function returns 0 on success or a non-zero code and
+ * keeps a message for mlf_hip_last_error() (per thread).  Device pointers are raw HIP device addresses.
+ * `stream` arguments are hipStream_t passed as void* (NULL = the default stream).  Handles are opaque.
+ * All calls act on the calling thread's current HIP device.
+ */
+#ifndef MLF_HIP_H_
+#define MLF_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MLF_MAX_DIMS 8
+
+/* What an item's bytes are copied from (pack) or to (unpack). */
+enum mlf_item_kind {
+  MLF_ITEM_DEVICE = 0, /* tensor in device memory described by shape/stride (contiguous or not)              */
+  MLF_ITEM_BLOB = 1    /* bytes that live in the plan's host blob: record headers, host-resident tensors,     */
+                       /* pickled non-tensor objects.  Pack only; ignored by unpack.                          */
+};
+
+/* One entry of the descriptor table handed to mlf_plan_create.  The plan keeps a device-resident form of it.
+ * `image_off` is where the item's first byte lies in the image.  For MLF_ITEM_DEVICE the logical index space
+ * is `shape[0..ndim)`; element (i0..ik) lives at ptr + esz * sum(i_d * stride[d]) on the tensor side and at
+ * image_off + esz * sum(i_d * image_stride[d]) on the image side.  On save the image side is the C-contiguous
+ * payload the reference writes (checkpoint_saver.py:797-800); on restore it is the requested sub-box of the
+ * stored tensor (checkpoint_loader.py:219 narrow_tensor_by_index) and the tensor side is the caller's target,
+ * which may itself be a strided view.  ndim == 0 means one element. */
+typedef struct mlf_item {
+  uint64_t ptr;       /* DEVICE: device address of element 0.  BLOB: byte offset into the host blob.          */
+  uint64_t image_off; /* byte offset in the image                                                              */
+  uint64_t nbytes;    /* total bytes of the item (numel * elem_size, or blob length)                           */
+  uint32_t kind;      /* enum mlf_item_kind                                                                    */
+  uint32_t elem_size; /* bytes per element: 1, 2, 4, 8 or 16 (DEVICE only)                                     */
+  uint32_t ndim;      /* 0..MLF_MAX_DIMS (DEVICE only)                                                         */
+  uint32_t reserved;
+  int64_t shape[MLF_MAX_DIMS];
+  int64_t stride[MLF_MAX_DIMS];       /* tensor side, in elements                                               */
+  int64_t image_stride[MLF_MAX_DIMS]; /* image side, in elements                                                */
+} mlf_item;
+
+typedef struct mlf_plan_opts {
+  uint32_t tile_bytes;       /* bytes one wavefront copies per work item (multiple of 1024; 0 = default)       */
+  uint32_t block_threads;    /* threads per workgroup for the copy kernels (multiple of 64; 0 = default)       */
+  uint32_t align_to_tensor;  /* 0: cut tiles at 16-byte boundaries of the image (pack); 1: of the tensor (unpack) */
+  uint32_t reserved;
+} mlf_plan_opts;
+
+typedef struct mlf_plan_info {
+  uint64_t n_items;
+  uint64_t n_flat_tiles;      /* wavefront work items of the flat (byte-segment) kernel                        */
+  uint64_t n_strided_items;   /* items that go through the generic strided kernel                              */
+  uint64_t n_strided_work;
+  uint64_t n_transposed_items;/* items that go through the LDS-tiled transpose kernel                          */
+  uint64_t n_transposed_work;
+  uint64_t device_bytes;      /* payload bytes that live in device tensors (P in the roofline figures)         */
+  uint64_t blob_bytes;        /* bytes that come from the host blob                                            */
+  uint64_t image_bytes;
+  uint64_t table_bytes;       /* device memory held by the plan's tables + blob                                */
+} mlf_plan_info;
+
+typedef struct mlf_plan mlf_plan;
+
+/* Message of the last failure on the calling thread ("" if none). */
+const char* mlf_hip_last_error(void);
+
+/* Number of visible devices / select the calling thread's device (HIP's current device is per thread). */
+int mlf_hip_device_count(int* out);
+int mlf_hip_set_device(int device);
+/* Free and total device memory in bytes. */
+int mlf_hip_mem_info(uint64_t* free_bytes, uint64_t* total_bytes);
+
+/* Builds the device-resident descriptor/work tables for `n_items` items and uploads `host_blob`.
+ * Validates that every item lies inside [0, image_bytes) and every blob item inside the blob.
+ * The plan stays valid while the tensors' addresses, shapes and strides stay the same; it can be launched
+ * any number of times.  Stands where the reference walks its Python list of (WriteItem, tensor) pairs
+ * (checkpoint_saver.py:668-682) or ReadItems (checkpoint_loader.py:322-336). */
+int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_blob, uint64_t blob_bytes,
+                    uint64_t image_bytes, const mlf_plan_opts* opts, mlf_plan** out);
+int mlf_plan_destroy(mlf_plan* plan);
+int mlf_plan_get_info(const mlf_plan* plan, mlf_plan_info* out);
+
+/* Save direction: tensors (+ blob) -> image.  Asynchronous on `stream`; the image is complete when the
+ * stream reaches the point after this call.  Replaces the per-tensor .to("cpu") staging
+ * (checkpoint_saver.py:347-360; memory_storage_writer.py:213-233) and the per-tensor
+ * frombuffer().copy_() (checkpoint_saver.py:797-800): afterwards the training stream may go on. */
+int mlf_pack_launch(const mlf_plan* plan, void* image_dev, void* stream);
+
+/* Restore direction: image -> tensors.  Asynchronous on `stream`.  Replaces frombuffer + narrow + copy_
+ * (checkpoint_loader.py:206-219,331-336). */
+int mlf_unpack_launch(const mlf_plan* plan, const void* image_dev, void* stream);
+
+/* CRC-32C (Castagnoli, reflected, init/xorout 0xFFFFFFFF as in RFC 3720) of consecutive `chunk_bytes`
+ * pieces of a device buffer; the last chunk may be short.  Writes ceil(nbytes/chunk_bytes) values to
+ * `out_host` and returns after they are valid.  The reference has no checksum; this is the integrity check
+ * of the copy pipeline (values are kept beside the object, never inside it). */
+int mlf_crc32c_device(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint32_t* out_host,
+                      uint64_t n_out, void* stream);
+/* Same function on host memory (SSE4.2), and the combine law crc(A||B) from crc(A), crc(B), len(B). */
+uint32_t mlf_crc32c_host(const void* data, uint64_t nbytes);
+uint32_t mlf_crc32c_combine(uint32_t crc_a, uint32_t crc_b, uint64_t len_b);
+
+/* Copy engine: a ring of pinned host slots, two copy streams and a pool of host threads that move data
+ * between device memory and pageable host memory (the MAP_SHARED buffer file) at link speed. */
+typedef struct mlf_engine mlf_engine;
+
+typedef struct mlf_xfer_stats {
+  double seconds;        /* wall time of the call                                                             */
+  double wait_seconds;   /* of which the calling thread spent waiting for the producer stream (d2h only)      */
+  uint64_t bytes;
+  uint64_t chunks;
+} mlf_xfer_stats;
+
+int mlf_engine_create(uint64_t slot_bytes, uint32_t n_slots, uint32_t n_threads, mlf_engine** out);
+int mlf_engine_destroy(mlf_engine* engine);
+
+/* Device -> host.  Waits (on the copy streams, not on the host) for everything enqueued so far on
+ * `producer_stream`, then copies `nbytes` from `src_dev` to `dst_host` and returns when the bytes are in
+ * place.  `dst_host` is typically BufferObject.get_data_ptr() + 4096 + position
+ * (bindings.cpp:59-72; buffer_io.py:342-343).  Replaces the D2H half of Tensor.to("cpu") and the CPU
+ * copy_ into the mapping.  Safe to call from a thread other than the one that launched the pack. */
+int mlf_engine_d2h(mlf_engine* engine, const void* src_dev, void* dst_host, uint64_t nbytes,
+                   void* producer_stream, mlf_xfer_stats* stats);
+
+/* Host -> device.  Copies `nbytes` from `src_host` (pageable, e.g. the read-only mapping) to `dst_dev`
+ * and makes `consumer_stream` wait for the last chunk, so an unpack launched on it afterwards sees the data.
+ * Returns once all chunks are enqueued and the host source is no longer needed.  Replaces BufferIO.read()'s
+ * copy plus the pageable H2D inside target.copy_() (buffer_io.py:206; checkpoint_loader.py:335). */
+int mlf_engine_h2d(mlf_engine* engine, const void* src_host, void* dst_dev, uint64_t nbytes,
+                   void* consumer_stream, mlf_xfer_stats* stats);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MLF_HIP_H_ */

@@ -1,0 +1,887 @@
+// MI355X (gfx950) save/restore data path behind the C-ABI in include/mlf_hip.h.
+//
+//   pack    live tensors (+ host blob of headers)  -> byte-exact image of a checkpoint object, in HBM
+//   unpack  image in HBM                           -> live tensors
+//   crc     CRC-32C per chunk of an image
+//   engine  image <-> pageable host memory through a ring of pinned slots and a host thread pool
+//
+// Everything on this path is integer byte movement, so the bound is HBM bandwidth (pack/unpack/crc) or the
+// host link (engine).  Kernels are written for 64-wide wavefronts and 16-byte accesses:
+//   * flat kernel: one wavefront per work item ("tile": <= tile_bytes of one contiguous item).  The
+//     destination is peeled to a 16-byte boundary, the body is non-temporal dwordx4 stores fed by dwordx4
+//     loads from a possibly misaligned source (gfx950 runs in unaligned-access mode), the tail is bytes.
+//     No LDS, no barriers; tiles of one item are consecutive so neighbouring waves stream neighbouring lines.
+//   * strided kernel: generic N-d index walk for non-contiguous sources/targets and sub-box restores.
+//   * crc kernel: per wavefront a 64 KiB segment is read as coalesced 1 KiB rows; every lane keeps four
+//     Horner accumulators advanced by x^8192 through LDS tables, then lanes are folded with GF(2) multiplies.
+#include "mlf_hip.h"
+
+#include <hip/hip_runtime.h>
+#include <nmmintrin.h>
+#include <string.h>
+
+#include <algorithm>
+#include <atomic>
+#include <chrono>
+#include <condition_variable>
+#include <functional>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <thread>
+#include <vector>
+
+// ---------------------------------------------------------------------------------------------------------
+// errors
+// ---------------------------------------------------------------------------------------------------------
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const std::string& msg) {
+  g_err = msg;
+  return code;
+}
+
+enum { MLF_HIP_OK = 0, MLF_HIP_BAD_ARG = 1, MLF_HIP_RUNTIME = 2 };
+
+#define HIP_TRY(expr)                                                                                   \
+  do {                                                                                                  \
+    hipError_t e__ = (expr);                                                                            \
+    if (e__ != hipSuccess)                                                                              \
+      return fail(MLF_HIP_RUNTIME, std::string(#expr) + " failed: " + hipGetErrorString(e__));          \
+  } while (0)
+
+double now_s() {
+  return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// device-side tables
+// ---------------------------------------------------------------------------------------------------------
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef u32x4 u32x4_u __attribute__((aligned(1)));  // dwordx4 access at any byte address
+
+struct FlatTile {   // one wavefront's work: copy n bytes between a tensor address and an image offset
+  uint64_t tensor;  // absolute device address on the tensor (or blob) side
+  uint64_t image;   // byte offset in the image
+  uint32_t n;
+  uint32_t pad;
+};
+
+struct StridedDesc {
+  uint64_t tensor;  // device address of element 0
+  uint64_t image;   // byte offset of element 0 in the image
+  uint32_t esz;
+  uint32_t ndim;
+  int64_t shape[MLF_MAX_DIMS];
+  int64_t tstride[MLF_MAX_DIMS];  // bytes
+  int64_t istride[MLF_MAX_DIMS];  // bytes
+};
+
+struct StridedWork {  // one workgroup's work: elements [start, start+count) of descriptor `desc`
+  uint64_t start;
+  uint32_t count;
+  uint32_t desc;
+};
+
+constexpr int kWave = 64;
+constexpr int kUnroll = 4;  // dwordx4 per lane in flight: 4 KiB per wavefront per loop trip
+
+// ---------------------------------------------------------------------------------------------------------
+// flat kernel
+// ---------------------------------------------------------------------------------------------------------
+template <bool PACK>
+__global__ void __launch_bounds__(1024) mlf_flat_kernel(const FlatTile* __restrict__ tiles, uint32_t n_tiles,
+                                                        char* __restrict__ image) {
+  const uint32_t waves_per_block = blockDim.x >> 6;
+  const uint32_t wave = blockIdx.x * waves_per_block + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  if (wave >= n_tiles) return;
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const FlatTile t = tiles[wave];
+  const char* src = PACK ? reinterpret_cast<const char*>(t.tensor) : image + t.image;
+  char* dst = PACK ? image + t.image : reinterpret_cast<char*>(t.tensor);
+  uint32_t n = t.n;
+
+  // bytes up to the first 16-byte boundary of the destination
+  uint32_t head = (16u - (uint32_t)(reinterpret_cast<uintptr_t>(dst) & 15u)) & 15u;
+  head = head < n ? head : n;
+  if (lane < head) dst[lane] = src[lane];
+  src += head;
+  dst += head;
+  n -= head;
+
+  const uint32_t nvec = n >> 4;
+  u32x4* __restrict__ d = reinterpret_cast<u32x4*>(dst);
+  uint32_t i = lane;
+  for (; i + (kUnroll - 1) * kWave < nvec; i += kUnroll * kWave) {
+    u32x4 v[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_u*>(src + (size_t)(i + u * kWave) * 16));
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) __builtin_nontemporal_store(v[u], &d[i + u * kWave]);
+  }
+  for (; i < nvec; i += kWave) {
+    u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_u*>(src + (size_t)i * 16));
+    __builtin_nontemporal_store(v, &d[i]);
+  }
+  const uint32_t tail = n & 15u;
+  if (lane < tail) {
+    const uint32_t o = (nvec << 4) + lane;
+    dst[o] = src[o];
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// strided kernel (generic)
+// ---------------------------------------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ void copy_elem(char* dst, const char* src) {
+  typedef T unaligned_t __attribute__((aligned(1)));
+  *reinterpret_cast<unaligned_t*>(dst) = *reinterpret_cast<const unaligned_t*>(src);
+}
+
+template <bool PACK>
+__global__ void __launch_bounds__(256) mlf_strided_kernel(const StridedDesc* __restrict__ descs,
+                                                          const StridedWork* __restrict__ work,
+                                                          char* __restrict__ image) {
+  const StridedWork w = work[blockIdx.x];
+  const StridedDesc* __restrict__ d = descs + w.desc;
+  const uint32_t esz = d->esz;
+  const int ndim = (int)d->ndim;
+  char* tbase = reinterpret_cast<char*>(d->tensor);
+  char* ibase = image + d->image;
+  for (uint32_t k = threadIdx.x; k < w.count; k += blockDim.x) {
+    uint64_t e = w.start + k;
+    int64_t toff = 0, ioff = 0;
+    for (int dim = ndim - 1; dim >= 0; --dim) {
+      const uint64_t extent = (uint64_t)d->shape[dim];
+      const uint64_t q = e / extent;
+      const int64_t idx = (int64_t)(e - q * extent);
+      e = q;
+      toff += idx * d->tstride[dim];
+      ioff += idx * d->istride[dim];
+    }
+    const char* s = PACK ? tbase + toff : ibase + ioff;
+    char* o = PACK ? ibase + ioff : tbase + toff;
+    switch (esz) {
+      case 1: *o = *s; break;
+      case 2: copy_elem<uint16_t>(o, s); break;
+      case 4: copy_elem<uint32_t>(o, s); break;
+      case 8: copy_elem<uint64_t>(o, s); break;
+      default: copy_elem<u32x4>(o, s); break;  // 16
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// CRC-32C
+// ---------------------------------------------------------------------------------------------------------
+constexpr uint32_t kPolyReflected = 0x82F63B78u;
+constexpr uint32_t kCrcSegBytes = 64 * 1024;  // bytes per wavefront
+constexpr uint32_t kCrcRowBytes = 1024;       // one coalesced wavefront row: 64 lanes x 16 bytes
+
+// a(x) * b(x) mod P in the reflected representation (bit 31 is x^0).
+__host__ __device__ inline uint32_t gf_mul(uint32_t a, uint32_t b) {
+  uint32_t p = 0;
+  for (int i = 31; i >= 0; --i) {
+    p ^= ((a >> i) & 1u) ? b : 0u;
+    b = (b >> 1) ^ ((b & 1u) ? kPolyReflected : 0u);
+  }
+  return p;
+}
+
+// x^(8*nbytes) mod P.
+uint32_t x_pow_bytes(uint64_t nbytes) {
+  uint32_t result = 0x80000000u;      // x^0
+  uint32_t sq = gf_mul(0x40000000u, 0x40000000u);  // x^2
+  sq = gf_mul(sq, sq);                // x^4
+  sq = gf_mul(sq, sq);                // x^8 : one byte
+  while (nbytes) {
+    if (nbytes & 1) result = gf_mul(result, sq);
+    sq = gf_mul(sq, sq);
+    nbytes >>= 1;
+  }
+  return result;
+}
+
+struct CrcConsts {
+  uint32_t row_tab[4][256];  // state advanced by one 1 KiB row, sliced by state byte
+  uint32_t x4, x16, x32, x64, x128, x256, x512;  // x^(8*n) for the fold steps
+  uint32_t xseg;             // x^(8*kCrcSegBytes)
+};
+
+__device__ __forceinline__ uint32_t crc_byte_step(uint32_t s, uint8_t b) {
+  s ^= b;
+  for (int k = 0; k < 8; ++k) s = (s >> 1) ^ ((s & 1u) ? kPolyReflected : 0u);
+  return s;
+}
+
+// One wavefront per segment: raw remainder (zero initial state, no final xor) of the segment's bytes.
+__global__ void __launch_bounds__(256) mlf_crc_segments_kernel(const char* __restrict__ data, uint64_t nbytes,
+                                                               const CrcConsts* __restrict__ consts,
+                                                               uint32_t* __restrict__ seg_crc, uint32_t n_segs) {
+  __shared__ uint32_t tab[4][256];
+  for (uint32_t i = threadIdx.x; i < 1024; i += blockDim.x) tab[i >> 8][i & 255] = consts->row_tab[i >> 8][i & 255];
+  __syncthreads();
+  const uint32_t seg = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (seg >= n_segs) return;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint64_t seg_off = (uint64_t)seg * kCrcSegBytes;
+  const uint64_t remaining = nbytes - seg_off;
+  const uint32_t seg_len = remaining < kCrcSegBytes ? (uint32_t)remaining : kCrcSegBytes;
+  const uint32_t rows = seg_len / kCrcRowBytes;
+  const u32x4* p = reinterpret_cast<const u32x4*>(data + seg_off) + lane;
+  uint32_t a0 = 0, a1 = 0, a2 = 0, a3 = 0;
+#define MLF_ROW_ADV(a) (tab[0][(a) & 255] ^ tab[1][((a) >> 8) & 255] ^ tab[2][((a) >> 16) & 255] ^ tab[3][(a) >> 24])
+  for (uint32_t r = 0; r < rows; ++r) {
+    const u32x4 v = __builtin_nontemporal_load(p + (size_t)r * 64);
+    a0 = MLF_ROW_ADV(a0) ^ v.x;
+    a1 = MLF_ROW_ADV(a1) ^ v.y;
+    a2 = MLF_ROW_ADV(a2) ^ v.z;
+    a3 = MLF_ROW_ADV(a3) ^ v.w;
+  }
+#undef MLF_ROW_ADV
+  // fold the four columns of this lane: x^128*a0 + x^96*a1 + x^64*a2 + x^32*a3
+  const uint32_t x4 = consts->x4;
+  uint32_t acc = gf_mul(x4, a0) ^ a1;
+  acc = gf_mul(x4, acc) ^ a2;
+  acc = gf_mul(x4, acc) ^ a3;
+  acc = gf_mul(x4, acc);
+  // fold lanes pairwise: lower lane is earlier in the message, so it is the one that gets shifted
+  const uint32_t xs[6] = {consts->x16, consts->x32, consts->x64, consts->x128, consts->x256, consts->x512};
+#pragma unroll
+  for (int s = 0; s < 6; ++s) {
+    const uint32_t other = __shfl_down(acc, 1u << s, 64);
+    acc = gf_mul(xs[s], acc) ^ other;
+  }
+  if (lane == 0) {
+    // bytes of a short last segment that do not fill a row
+    uint32_t state = rows ? acc : 0u;
+    const char* tailp = data + seg_off + (uint64_t)rows * kCrcRowBytes;
+    for (uint32_t i = 0, n = seg_len - rows * kCrcRowBytes; i < n; ++i) state = crc_byte_step(state, (uint8_t)tailp[i]);
+    seg_crc[seg] = state;
+  }
+}
+
+// One thread per chunk: chain the segment remainders, apply init and final xor.
+__global__ void mlf_crc_chunks_kernel(const uint32_t* __restrict__ seg_crc, uint32_t segs_per_chunk, uint32_t n_segs,
+                                      uint32_t xseg, uint32_t x_last_seg, uint32_t* __restrict__ out,
+                                      uint32_t n_chunks) {
+  const uint32_t c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= n_chunks) return;
+  uint32_t s = 0xFFFFFFFFu;
+  const uint32_t first = c * segs_per_chunk;
+  const uint32_t last = first + segs_per_chunk < n_segs ? first + segs_per_chunk : n_segs;
+  for (uint32_t i = first; i < last; ++i) s = gf_mul(i == n_segs - 1 ? x_last_seg : xseg, s) ^ seg_crc[i];
+  out[c] = s ^ 0xFFFFFFFFu;
+}
+
+std::once_flag g_crc_once;
+CrcConsts g_crc_host;
+
+void crc_init_host() {
+  const uint32_t xrow = x_pow_bytes(kCrcRowBytes);
+  for (int b = 0; b < 4; ++b)
+    for (uint32_t v = 0; v < 256; ++v) g_crc_host.row_tab[b][v] = gf_mul(xrow, v << (8 * b));
+  g_crc_host.x4 = x_pow_bytes(4);
+  g_crc_host.x16 = x_pow_bytes(16);
+  g_crc_host.x32 = x_pow_bytes(32);
+  g_crc_host.x64 = x_pow_bytes(64);
+  g_crc_host.x128 = x_pow_bytes(128);
+  g_crc_host.x256 = x_pow_bytes(256);
+  g_crc_host.x512 = x_pow_bytes(512);
+  g_crc_host.xseg = x_pow_bytes(kCrcSegBytes);
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// host thread pool: run(n, fn) executes fn(0..n-1) on the pool's threads plus the caller
+// ---------------------------------------------------------------------------------------------------------
+class WorkerPool {
+ public:
+  explicit WorkerPool(unsigned extra_threads) {
+    for (unsigned i = 0; i < extra_threads; ++i) threads_.emplace_back([this] { loop(); });
+  }
+  ~WorkerPool() {
+    {
+      std::lock_guard<std::mutex> g(m_);
+      stop_ = true;
+    }
+    cv_.notify_all();
+    for (auto& t : threads_) t.join();
+  }
+  unsigned width() const { return (unsigned)threads_.size() + 1; }
+
+  void run(unsigned n, const std::function<void(unsigned)>& fn) {
+    if (n == 0) return;
+    {
+      std::lock_guard<std::mutex> g(m_);
+      fn_ = &fn;
+      total_ = n;
+      next_ = 0;
+      pending_ = n;
+      ++generation_;
+    }
+    cv_.notify_all();
+    drain();
+    std::unique_lock<std::mutex> l(m_);
+    done_cv_.wait(l, [this] { return pending_ == 0; });
+    fn_ = nullptr;
+  }
+
+ private:
+  void drain() {
+    for (;;) {
+      unsigned idx;
+      const std::function<void(unsigned)>* fn;
+      {
+        std::lock_guard<std::mutex> g(m_);
+        if (!fn_ || next_ >= total_) return;
+        idx = next_++;
+        fn = fn_;
+      }
+      (*fn)(idx);
+      {
+        std::lock_guard<std::mutex> g(m_);
+        if (--pending_ == 0) done_cv_.notify_all();
+      }
+    }
+  }
+  void loop() {
+    uint64_t seen = 0;
+    for (;;) {
+      {
+        std::unique_lock<std::mutex> l(m_);
+        cv_.wait(l, [&] { return stop_ || generation_ != seen; });
+        if (stop_) return;
+        seen = generation_;
+      }
+      drain();
+    }
+  }
+  std::vector<std::thread> threads_;
+  std::mutex m_;
+  std::condition_variable cv_, done_cv_;
+  const std::function<void(unsigned)>* fn_ = nullptr;
+  unsigned total_ = 0, next_ = 0, pending_ = 0;
+  uint64_t generation_ = 0;
+  bool stop_ = false;
+};
+
+void pool_memcpy(WorkerPool& pool, char* dst, const char* src, size_t n) {
+  const unsigned parts = std::max<unsigned>(1, std::min<size_t>(pool.width(), n / ((size_t)1 << 20)));
+  size_t per = (n + parts - 1) / parts;
+  per = (per + 4095) & ~(size_t)4095;
+  pool.run(parts, [&](unsigned i) {
+    const size_t off = (size_t)i * per;
+    if (off < n) memcpy(dst + off, src + off, std::min(per, n - off));
+  });
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------------------
+// plan
+// ---------------------------------------------------------------------------------------------------------
+struct mlf_plan {
+  int device = 0;
+  FlatTile* d_tiles = nullptr;
+  StridedDesc* d_descs = nullptr;
+  StridedWork* d_work = nullptr;
+  char* d_blob = nullptr;
+  uint32_t block_threads = 256;
+  mlf_plan_info info{};
+};
+
+namespace {
+
+constexpr uint32_t kDefaultTileBytes = 64 * 1024;
+constexpr uint32_t kStridedElemsPerBlock = 32 * 1024;
+
+// Cuts [0, n) of one contiguous item into tiles whose destination starts are 16-byte aligned (except the first).
+void cut_tiles(std::vector<FlatTile>& out, uint64_t tensor_addr, uint64_t image_off, uint64_t n, uint32_t tile,
+               bool align_to_tensor) {
+  const uint64_t dst_addr = align_to_tensor ? tensor_addr : image_off;  // image base is 256-byte aligned
+  const uint64_t head = (16 - (dst_addr & 15)) & 15;
+  uint64_t done = 0;
+  while (done < n) {
+    uint64_t len = std::min<uint64_t>(n - done, done == 0 ? tile + head : tile);
+    out.push_back(FlatTile{tensor_addr + done, image_off + done, (uint32_t)len, 0});
+    done += len;
+  }
+}
+
+struct Collapsed {
+  int ndim;
+  int64_t shape[MLF_MAX_DIMS], ts[MLF_MAX_DIMS], is[MLF_MAX_DIMS];
+};
+
+// Drops size-1 dims and merges neighbours that are jointly contiguous on both sides (strides in elements).
+Collapsed collapse_dims(const mlf_item& it) {
+  Collapsed c{};
+  int n = 0;
+  for (uint32_t d = 0; d < it.ndim; ++d) {
+    if (it.shape[d] == 1) continue;
+    if (n > 0 && c.ts[n - 1] == it.stride[d] * it.shape[d] && c.is[n - 1] == it.image_stride[d] * it.shape[d]) {
+      c.shape[n - 1] *= it.shape[d];
+      c.ts[n - 1] = it.stride[d];
+      c.is[n - 1] = it.image_stride[d];
+    } else {
+      c.shape[n] = it.shape[d];
+      c.ts[n] = it.stride[d];
+      c.is[n] = it.image_stride[d];
+      ++n;
+    }
+  }
+  c.ndim = n;
+  return c;
+}
+
+template <typename T>
+int upload(const std::vector<T>& host, T** dev) {
+  *dev = nullptr;
+  if (host.empty()) return MLF_HIP_OK;
+  HIP_TRY(hipMalloc(reinterpret_cast<void**>(dev), host.size() * sizeof(T)));
+  HIP_TRY(hipMemcpy(*dev, host.data(), host.size() * sizeof(T), hipMemcpyHostToDevice));
+  return MLF_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* mlf_hip_last_error(void) { return g_err.c_str(); }
+
+int mlf_hip_device_count(int* out) {
+  if (!out) return fail(MLF_HIP_BAD_ARG, "null out");
+  HIP_TRY(hipGetDeviceCount(out));
+  return MLF_HIP_OK;
+}
+
+int mlf_hip_set_device(int device) {
+  HIP_TRY(hipSetDevice(device));
+  return MLF_HIP_OK;
+}
+
+int mlf_hip_mem_info(uint64_t* free_bytes, uint64_t* total_bytes) {
+  size_t f = 0, t = 0;
+  HIP_TRY(hipMemGetInfo(&f, &t));
+  if (free_bytes) *free_bytes = f;
+  if (total_bytes) *total_bytes = t;
+  return MLF_HIP_OK;
+}
+
+int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_blob, uint64_t blob_bytes,
+                    uint64_t image_bytes, const mlf_plan_opts* opts, mlf_plan** out) {
+  if (!out) return fail(MLF_HIP_BAD_ARG, "null out");
+  *out = nullptr;
+  if (n_items && !items) return fail(MLF_HIP_BAD_ARG, "null items");
+  if (blob_bytes && !host_blob) return fail(MLF_HIP_BAD_ARG, "null host_blob with blob_bytes > 0");
+  uint32_t tile = opts && opts->tile_bytes ? opts->tile_bytes : kDefaultTileBytes;
+  uint32_t threads = opts && opts->block_threads ? opts->block_threads : 256;
+  const bool align_to_tensor = opts && opts->align_to_tensor;
+  if (tile % 1024 || tile > (64u << 20)) return fail(MLF_HIP_BAD_ARG, "tile_bytes must be a multiple of 1024, at most 64 MiB");
+  if (threads % 64 || threads > 1024) return fail(MLF_HIP_BAD_ARG, "block_threads must be a multiple of 64, at most 1024");
+
+  std::unique_ptr<mlf_plan> plan(new mlf_plan());
+  HIP_TRY(hipGetDevice(&plan->device));
+  plan->block_threads = threads;
+  if (blob_bytes) {
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&plan->d_blob), blob_bytes));
+    HIP_TRY(hipMemcpy(plan->d_blob, host_blob, blob_bytes, hipMemcpyHostToDevice));
+  }
+  const uint64_t blob_base = reinterpret_cast<uint64_t>(plan->d_blob);
+
+  std::vector<FlatTile> tiles;
+  std::vector<StridedDesc> descs;
+  std::vector<StridedWork> work;
+  mlf_plan_info& info = plan->info;
+  info.n_items = n_items;
+  info.image_bytes = image_bytes;
+  int rc = MLF_HIP_OK;
+  for (uint64_t k = 0; k < n_items && rc == MLF_HIP_OK; ++k) {
+    const mlf_item& it = items[k];
+    if (it.nbytes == 0) continue;
+    if (it.image_off > image_bytes || it.nbytes > image_bytes - it.image_off) {
+      rc = fail(MLF_HIP_BAD_ARG, "item " + std::to_string(k) + " does not fit in the image");
+      break;
+    }
+    if (it.kind == MLF_ITEM_BLOB) {
+      if (it.ptr > blob_bytes || it.nbytes > blob_bytes - it.ptr) {
+        rc = fail(MLF_HIP_BAD_ARG, "blob item " + std::to_string(k) + " lies outside the host blob");
+        break;
+      }
+      cut_tiles(tiles, blob_base + it.ptr, it.image_off, it.nbytes, tile, false);
+      info.blob_bytes += it.nbytes;
+      continue;
+    }
+    if (it.kind != MLF_ITEM_DEVICE) {
+      rc = fail(MLF_HIP_BAD_ARG, "item " + std::to_string(k) + " has an unknown kind");
+      break;
+    }
+    const uint32_t esz = it.elem_size;
+    if (!(esz == 1 || esz == 2 || esz == 4 || esz == 8 || esz == 16) || it.ndim > MLF_MAX_DIMS || it.ptr == 0) {
+      rc = fail(MLF_HIP_BAD_ARG, "item " + std::to_string(k) + " has a bad element size, rank or null pointer");
+      break;
+    }
+    uint64_t numel = 1;
+    bool bad = false;
+    for (uint32_t d = 0; d < it.ndim; ++d) {
+      if (it.shape[d] <= 0) bad = true;
+      numel *= (uint64_t)it.shape[d];
+    }
+    if (bad || numel * esz != it.nbytes) {
+      rc = fail(MLF_HIP_BAD_ARG, "item " + std::to_string(k) + ": shape does not match nbytes");
+      break;
+    }
+    // the image side must stay inside the item's declared span of the image
+    {
+      int64_t lo = 0, hi = 0;
+      for (uint32_t d = 0; d < it.ndim; ++d) {
+        const int64_t reach = (it.shape[d] - 1) * it.image_stride[d];
+        (reach < 0 ? lo : hi) += reach;
+      }
+      const int64_t first = (int64_t)it.image_off + lo * (int64_t)esz;
+      const uint64_t last = it.image_off + (uint64_t)hi * esz + esz;
+      if (first < 0 || last > image_bytes) {
+        rc = fail(MLF_HIP_BAD_ARG, "item " + std::to_string(k) + ": image-side strides reach outside the image");
+        break;
+      }
+    }
+    info.device_bytes += it.nbytes;
+    const Collapsed c = collapse_dims(it);
+    if (c.ndim == 0 || (c.ndim == 1 && c.ts[0] == 1 && c.is[0] == 1)) {
+      cut_tiles(tiles, it.ptr, it.image_off, it.nbytes, tile, align_to_tensor);
+      continue;
+    }
+    // rows that are contiguous on both sides and long enough go through the flat kernel, one row at a time
+    const int last = c.ndim - 1;
+    const uint64_t row_bytes = (uint64_t)c.shape[last] * esz;
+    const uint64_t n_rows = numel / (uint64_t)c.shape[last];
+    if (c.ts[last] == 1 && c.is[last] == 1 && row_bytes >= 2048 && n_rows <= (1u << 22)) {
+      int64_t idx[MLF_MAX_DIMS] = {0};
+      for (uint64_t r = 0; r < n_rows; ++r) {
+        int64_t toff = 0, ioff = 0;
+        for (int d = 0; d < last; ++d) {
+          toff += idx[d] * c.ts[d];
+          ioff += idx[d] * c.is[d];
+        }
+        cut_tiles(tiles, it.ptr + (uint64_t)(toff * (int64_t)esz), it.image_off + (uint64_t)(ioff * (int64_t)esz),
+                  row_bytes, tile, align_to_tensor);
+        for (int d = last - 1; d >= 0; --d) {
+          if (++idx[d] < c.shape[d]) break;
+          idx[d] = 0;
+        }
+      }
+      continue;
+    }
+    StridedDesc sd{};
+    sd.tensor = it.ptr;
+    sd.image = it.image_off;
+    sd.esz = esz;
+    sd.ndim = (uint32_t)c.ndim;
+    for (int d = 0; d < c.ndim; ++d) {
+      sd.shape[d] = c.shape[d];
+      sd.tstride[d] = c.ts[d] * (int64_t)esz;
+      sd.istride[d] = c.is[d] * (int64_t)esz;
+    }
+    const uint32_t desc_idx = (uint32_t)descs.size();
+    descs.push_back(sd);
+    for (uint64_t s = 0; s < numel; s += kStridedElemsPerBlock)
+      work.push_back(StridedWork{s, (uint32_t)std::min<uint64_t>(kStridedElemsPerBlock, numel - s), desc_idx});
+    ++info.n_strided_items;
+  }
+  if (rc == MLF_HIP_OK && tiles.size() > 0xFFFFFFF0ull) rc = fail(MLF_HIP_BAD_ARG, "too many tiles: raise tile_bytes");
+  if (rc == MLF_HIP_OK) rc = upload(tiles, &plan->d_tiles);
+  if (rc == MLF_HIP_OK) rc = upload(descs, &plan->d_descs);
+  if (rc == MLF_HIP_OK) rc = upload(work, &plan->d_work);
+  if (rc != MLF_HIP_OK) {
+    std::string keep = g_err;
+    mlf_plan_destroy(plan.release());
+    g_err = keep;
+    return rc;
+  }
+  info.n_flat_tiles = tiles.size();
+  info.n_strided_work = work.size();
+  info.table_bytes = tiles.size() * sizeof(FlatTile) + descs.size() * sizeof(StridedDesc) +
+                     work.size() * sizeof(StridedWork) + blob_bytes;
+  *out = plan.release();
+  return MLF_HIP_OK;
+}
+
+int mlf_plan_destroy(mlf_plan* plan) {
+  if (!plan) return MLF_HIP_OK;
+  (void)hipFree(plan->d_tiles);
+  (void)hipFree(plan->d_descs);
+  (void)hipFree(plan->d_work);
+  (void)hipFree(plan->d_blob);
+  delete plan;
+  return MLF_HIP_OK;
+}
+
+int mlf_plan_get_info(const mlf_plan* plan, mlf_plan_info* out) {
+  if (!plan || !out) return fail(MLF_HIP_BAD_ARG, "null argument");
+  *out = plan->info;
+  return MLF_HIP_OK;
+}
+
+}  // extern "C"
+
+namespace {
+
+template <bool PACK>
+int launch_plan(const mlf_plan* plan, char* image, hipStream_t stream) {
+  if (!plan) return fail(MLF_HIP_BAD_ARG, "null plan");
+  if (!image && plan->info.image_bytes) return fail(MLF_HIP_BAD_ARG, "null image");
+  if (reinterpret_cast<uintptr_t>(image) & 255) return fail(MLF_HIP_BAD_ARG, "image must be 256-byte aligned");
+  const uint32_t n_tiles = (uint32_t)plan->info.n_flat_tiles;
+  if (n_tiles) {
+    const uint32_t waves = plan->block_threads / 64;
+    const uint32_t grid = (n_tiles + waves - 1) / waves;
+    hipLaunchKernelGGL((mlf_flat_kernel<PACK>), dim3(grid), dim3(plan->block_threads), 0, stream, plan->d_tiles,
+                       n_tiles, image);
+    HIP_TRY(hipGetLastError());
+  }
+  if (plan->info.n_strided_work) {
+    hipLaunchKernelGGL((mlf_strided_kernel<PACK>), dim3((uint32_t)plan->info.n_strided_work), dim3(256), 0, stream,
+                       plan->d_descs, plan->d_work, image);
+    HIP_TRY(hipGetLastError());
+  }
+  return MLF_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mlf_pack_launch(const mlf_plan* plan, void* image_dev, void* stream) {
+  return launch_plan<true>(plan, static_cast<char*>(image_dev), static_cast<hipStream_t>(stream));
+}
+
+int mlf_unpack_launch(const mlf_plan* plan, const void* image_dev, void* stream) {
+  return launch_plan<false>(plan, const_cast<char*>(static_cast<const char*>(image_dev)),
+                            static_cast<hipStream_t>(stream));
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// CRC entry points
+// ---------------------------------------------------------------------------------------------------------
+uint32_t mlf_crc32c_host(const void* data, uint64_t nbytes) {
+  const unsigned char* p = static_cast<const unsigned char*>(data);
+  uint64_t s = 0xFFFFFFFFu;
+  while (nbytes && (reinterpret_cast<uintptr_t>(p) & 7)) {
+    s = _mm_crc32_u8((uint32_t)s, *p++);
+    --nbytes;
+  }
+  for (; nbytes >= 8; nbytes -= 8, p += 8) {
+    uint64_t w;
+    memcpy(&w, p, 8);
+    s = _mm_crc32_u64(s, w);
+  }
+  while (nbytes--) s = _mm_crc32_u8((uint32_t)s, *p++);
+  return (uint32_t)s ^ 0xFFFFFFFFu;
+}
+
+uint32_t mlf_crc32c_combine(uint32_t crc_a, uint32_t crc_b, uint64_t len_b) {
+  return gf_mul(x_pow_bytes(len_b), crc_a) ^ crc_b;
+}
+
+int mlf_crc32c_device(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint32_t* out_host,
+                      uint64_t n_out, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (nbytes == 0) return MLF_HIP_OK;
+  if (!dev_ptr || !out_host) return fail(MLF_HIP_BAD_ARG, "null pointer");
+  if (reinterpret_cast<uintptr_t>(dev_ptr) & 15) return fail(MLF_HIP_BAD_ARG, "device buffer must be 16-byte aligned");
+  if (chunk_bytes == 0 || chunk_bytes % kCrcSegBytes)
+    return fail(MLF_HIP_BAD_ARG, "chunk_bytes must be a positive multiple of 65536");
+  const uint64_t n_chunks = (nbytes + chunk_bytes - 1) / chunk_bytes;
+  const uint64_t n_segs = (nbytes + kCrcSegBytes - 1) / kCrcSegBytes;
+  if (n_out < n_chunks) return fail(MLF_HIP_BAD_ARG, "output array too small");
+  if (n_segs > 0xFFFFFFF0ull) return fail(MLF_HIP_BAD_ARG, "buffer too large for one CRC call");
+  std::call_once(g_crc_once, crc_init_host);
+
+  CrcConsts* d_consts = nullptr;
+  uint32_t* d_seg = nullptr;
+  uint32_t* d_out = nullptr;
+  auto cleanup = [&] {
+    (void)hipFree(d_consts);
+    (void)hipFree(d_seg);
+    (void)hipFree(d_out);
+  };
+#define CRC_TRY(expr)                                                                             \
+  do {                                                                                            \
+    hipError_t e__ = (expr);                                                                      \
+    if (e__ != hipSuccess) {                                                                      \
+      cleanup();                                                                                  \
+      return fail(MLF_HIP_RUNTIME, std::string(#expr) + " failed: " + hipGetErrorString(e__));    \
+    }                                                                                             \
+  } while (0)
+  CRC_TRY(hipMalloc(reinterpret_cast<void**>(&d_consts), sizeof(CrcConsts)));
+  CRC_TRY(hipMalloc(reinterpret_cast<void**>(&d_seg), n_segs * sizeof(uint32_t)));
+  CRC_TRY(hipMalloc(reinterpret_cast<void**>(&d_out), n_chunks * sizeof(uint32_t)));
+  CRC_TRY(hipMemcpyAsync(d_consts, &g_crc_host, sizeof(CrcConsts), hipMemcpyHostToDevice, stream));
+  const uint32_t grid = (uint32_t)((n_segs + 3) / 4);
+  hipLaunchKernelGGL(mlf_crc_segments_kernel, dim3(grid), dim3(256), 0, stream, static_cast<const char*>(dev_ptr),
+                     nbytes, d_consts, d_seg, (uint32_t)n_segs);
+  CRC_TRY(hipGetLastError());
+  const uint64_t last_seg_len = nbytes - (n_segs - 1) * kCrcSegBytes;
+  hipLaunchKernelGGL(mlf_crc_chunks_kernel, dim3((uint32_t)((n_chunks + 63) / 64)), dim3(64), 0, stream, d_seg,
+                     (uint32_t)(chunk_bytes / kCrcSegBytes), (uint32_t)n_segs, g_crc_host.xseg,
+                     x_pow_bytes(last_seg_len), d_out, (uint32_t)n_chunks);
+  CRC_TRY(hipGetLastError());
+  CRC_TRY(hipMemcpyAsync(out_host, d_out, n_chunks * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+  CRC_TRY(hipStreamSynchronize(stream));
+#undef CRC_TRY
+  cleanup();
+  return MLF_HIP_OK;
+}
+
+}  // extern "C"
+
+// ---------------------------------------------------------------------------------------------------------
+// copy engine
+// ---------------------------------------------------------------------------------------------------------
+struct mlf_engine {
+  int device = 0;
+  uint64_t slot_bytes = 0;
+  std::vector<char*> slots;
+  std::vector<hipEvent_t> slot_done;
+  hipStream_t streams[2] = {nullptr, nullptr};
+  hipEvent_t gate = nullptr;
+  std::unique_ptr<WorkerPool> pool;
+  std::mutex busy;  // one transfer at a time per engine
+};
+
+extern "C" {
+
+int mlf_engine_destroy(mlf_engine* e) {
+  if (!e) return MLF_HIP_OK;
+  for (char* s : e->slots) (void)hipHostFree(s);
+  for (hipEvent_t ev : e->slot_done) (void)hipEventDestroy(ev);
+  if (e->gate) (void)hipEventDestroy(e->gate);
+  for (hipStream_t s : e->streams)
+    if (s) (void)hipStreamDestroy(s);
+  delete e;
+  return MLF_HIP_OK;
+}
+
+int mlf_engine_create(uint64_t slot_bytes, uint32_t n_slots, uint32_t n_threads, mlf_engine** out) {
+  if (!out) return fail(MLF_HIP_BAD_ARG, "null out");
+  *out = nullptr;
+  if (slot_bytes < (1u << 20) || slot_bytes % 4096) return fail(MLF_HIP_BAD_ARG, "slot_bytes must be a multiple of 4096, at least 1 MiB");
+  if (n_slots < 2 || n_slots > 64) return fail(MLF_HIP_BAD_ARG, "n_slots must be in [2, 64]");
+  if (n_threads < 1 || n_threads > 256) return fail(MLF_HIP_BAD_ARG, "n_threads must be in [1, 256]");
+  std::unique_ptr<mlf_engine> e(new mlf_engine());
+  e->slot_bytes = slot_bytes;
+  int rc = MLF_HIP_OK;
+  auto check = [&](hipError_t err, const char* what) {
+    if (err != hipSuccess && rc == MLF_HIP_OK) rc = fail(MLF_HIP_RUNTIME, std::string(what) + " failed: " + hipGetErrorString(err));
+  };
+  check(hipGetDevice(&e->device), "hipGetDevice");
+  for (int i = 0; i < 2 && rc == MLF_HIP_OK; ++i)
+    check(hipStreamCreateWithFlags(&e->streams[i], hipStreamNonBlocking), "hipStreamCreateWithFlags");
+  if (rc == MLF_HIP_OK) check(hipEventCreateWithFlags(&e->gate, hipEventDisableTiming), "hipEventCreateWithFlags");
+  for (uint32_t i = 0; i < n_slots && rc == MLF_HIP_OK; ++i) {
+    char* p = nullptr;
+    check(hipHostMalloc(reinterpret_cast<void**>(&p), slot_bytes, hipHostMallocDefault), "hipHostMalloc");
+    if (rc != MLF_HIP_OK) break;
+    memset(p, 0, slot_bytes);  // touch the pages once, outside any timed transfer
+    e->slots.push_back(p);
+    hipEvent_t ev = nullptr;
+    check(hipEventCreateWithFlags(&ev, hipEventDisableTiming), "hipEventCreateWithFlags");
+    if (rc == MLF_HIP_OK) e->slot_done.push_back(ev);
+  }
+  if (rc != MLF_HIP_OK) {
+    std::string keep = g_err;
+    mlf_engine_destroy(e.release());
+    g_err = keep;
+    return rc;
+  }
+  e->pool.reset(new WorkerPool(n_threads - 1));
+  *out = e.release();
+  return MLF_HIP_OK;
+}
+
+int mlf_engine_d2h(mlf_engine* e, const void* src_dev, void* dst_host, uint64_t nbytes, void* producer_stream,
+                   mlf_xfer_stats* stats) {
+  if (!e) return fail(MLF_HIP_BAD_ARG, "null engine");
+  if (nbytes && (!src_dev || !dst_host)) return fail(MLF_HIP_BAD_ARG, "null pointer");
+  std::lock_guard<std::mutex> g(e->busy);
+  HIP_TRY(hipSetDevice(e->device));
+  const double t0 = now_s();
+  // the copy streams start after whatever the producer has enqueued so far (the pack)
+  HIP_TRY(hipEventRecord(e->gate, static_cast<hipStream_t>(producer_stream)));
+  for (hipStream_t s : e->streams) HIP_TRY(hipStreamWaitEvent(s, e->gate, 0));
+  const char* src = static_cast<const char*>(src_dev);
+  char* dst = static_cast<char*>(dst_host);
+  const uint64_t slot = e->slot_bytes;
+  const uint64_t n_chunks = (nbytes + slot - 1) / slot;
+  const uint64_t n_slots = e->slots.size();
+  auto issue = [&](uint64_t c) -> int {
+    const uint64_t off = c * slot, len = std::min(slot, nbytes - off);
+    const uint64_t s = c % n_slots;
+    hipStream_t st = e->streams[c & 1];
+    HIP_TRY(hipMemcpyAsync(e->slots[s], src + off, len, hipMemcpyDeviceToHost, st));
+    HIP_TRY(hipEventRecord(e->slot_done[s], st));
+    return MLF_HIP_OK;
+  };
+  for (uint64_t c = 0; c < std::min(n_chunks, n_slots); ++c)
+    if (int rc = issue(c)) return rc;
+  double wait = 0;
+  for (uint64_t c = 0; c < n_chunks; ++c) {
+    const uint64_t off = c * slot, len = std::min(slot, nbytes - off);
+    const uint64_t s = c % n_slots;
+    const double w0 = now_s();
+    HIP_TRY(hipEventSynchronize(e->slot_done[s]));
+    if (c == 0) wait = now_s() - w0;
+    pool_memcpy(*e->pool, dst + off, e->slots[s], len);
+    if (c + n_slots < n_chunks)
+      if (int rc = issue(c + n_slots)) return rc;
+  }
+  if (stats) {
+    stats->seconds = now_s() - t0;
+    stats->wait_seconds = wait;
+    stats->bytes = nbytes;
+    stats->chunks = n_chunks;
+  }
+  return MLF_HIP_OK;
+}
+
+int mlf_engine_h2d(mlf_engine* e, const void* src_host, void* dst_dev, uint64_t nbytes, void* consumer_stream,
+                   mlf_xfer_stats* stats) {
+  if (!e) return fail(MLF_HIP_BAD_ARG, "null engine");
+  if (nbytes && (!src_host || !dst_dev)) return fail(MLF_HIP_BAD_ARG, "null pointer");
+  std::lock_guard<std::mutex> g(e->busy);
+  HIP_TRY(hipSetDevice(e->device));
+  const double t0 = now_s();
+  const char* src = static_cast<const char*>(src_host);
+  char* dst = static_cast<char*>(dst_dev);
+  const uint64_t slot = e->slot_bytes;
+  const uint64_t n_chunks = (nbytes + slot - 1) / slot;
+  const uint64_t n_slots = e->slots.size();
+  for (uint64_t c = 0; c < n_chunks; ++c) {
+    const uint64_t off = c * slot, len = std::min(slot, nbytes - off);
+    const uint64_t s = c % n_slots;
+    if (c >= n_slots) HIP_TRY(hipEventSynchronize(e->slot_done[s]));  // the slot's previous upload has left it
+    pool_memcpy(*e->pool, e->slots[s], src + off, len);
+    hipStream_t st = e->streams[c & 1];
+    HIP_TRY(hipMemcpyAsync(dst + off, e->slots[s], len, hipMemcpyHostToDevice, st));
+    HIP_TRY(hipEventRecord(e->slot_done[s], st));
+  }
+  // the consumer (unpack) waits for both copy streams; the host waits too, so the slots are reusable
+  for (hipStream_t s : e->streams) {
+    HIP_TRY(hipEventRecord(e->gate, s));
+    HIP_TRY(hipStreamWaitEvent(static_cast<hipStream_t>(consumer_stream), e->gate, 0));
+    HIP_TRY(hipStreamSynchronize(s));
+  }
+  if (stats) {
+    stats->seconds = now_s() - t0;
+    stats->wait_seconds = 0;
+    stats->bytes = nbytes;
+    stats->chunks = n_chunks;
+  }
+  return MLF_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,283 @@
+"""Python face of the native plan / copy-engine / CRC entry points, plus the host-side layout rules.
+
+The *layout* of a checkpoint object's data section is decided here, on the host, and is exactly the reference's:
+records ``<u32 len><pickled TensorHeader><payload>`` back to back from offset 0, tensors first, then byte blobs
+(reference: src/ml_flashpoint/core/checkpoint_saver.py:667-698,764-800).  The bytes themselves are moved by the
+gfx950 kernels: this module only fills the descriptor table that drives them.
+"""
+
+import ctypes
+import dataclasses
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from ml_flashpoint.core.tensor_header import TensorHeader
+from ml_flashpoint.hip import _lib
+from ml_flashpoint.hip._lib import ITEM_BLOB, ITEM_DEVICE, ITEM_DTYPE, MAX_DIMS
+
+_HEADER_CACHE: Dict[Tuple[torch.dtype, Tuple[int, ...]], bytes] = {}
+
+
+def header_bytes(dtype: torch.dtype, shape: Sequence[int]) -> bytes:
+    """``TensorHeader(dtype, shape).to_bytes()``, memoised: a state dict repeats few distinct (dtype, shape)."""
+    key = (dtype, tuple(shape))
+    raw = _HEADER_CACHE.get(key)
+    if raw is None:
+        raw = TensorHeader(dtype=dtype, shape=torch.Size(key[1])).to_bytes()
+        if len(_HEADER_CACHE) < 1 << 16:
+            _HEADER_CACHE[key] = raw
+    return raw
+
+
+def _contiguous_strides(shape: Sequence[int]) -> List[int]:
+    strides = [1] * len(shape)
+    for d in range(len(shape) - 2, -1, -1):
+        strides[d] = strides[d + 1] * shape[d + 1]
+    return strides
+
+
+class ItemTable:
+    """Column-wise builder of an ``mlf_item`` array (filled per column at the end: cheaper than per-row numpy)."""
+
+    def __init__(self):
+        self._rows: List[tuple] = []
+
+    def __len__(self):
+        return len(self._rows)
+
+    def add_blob(self, blob_off: int, image_off: int, nbytes: int) -> None:
+        self._rows.append((blob_off, image_off, nbytes, ITEM_BLOB, 1, 0, (), (), ()))
+
+    def add_device(
+        self,
+        ptr: int,
+        image_off: int,
+        elem_size: int,
+        shape: Sequence[int],
+        stride: Sequence[int],
+        image_stride: Optional[Sequence[int]] = None,
+    ) -> None:
+        if len(shape) > MAX_DIMS:
+            raise NotImplementedError(f"tensors of rank > {MAX_DIMS} that are not contiguous are not supported")
+        numel = 1
+        for s in shape:
+            numel *= s
+        if image_stride is None:
+            image_stride = _contiguous_strides(shape)
+        self._rows.append(
+            (ptr, image_off, numel * elem_size, ITEM_DEVICE, elem_size, len(shape), tuple(shape), tuple(stride), tuple(image_stride))
+        )
+
+    def to_array(self) -> np.ndarray:
+        n = len(self._rows)
+        arr = np.zeros(n, dtype=ITEM_DTYPE)
+        if n == 0:
+            return arr
+        cols = list(zip(*self._rows))
+        arr["ptr"] = cols[0]
+        arr["image_off"] = cols[1]
+        arr["nbytes"] = cols[2]
+        arr["kind"] = cols[3]
+        arr["elem_size"] = cols[4]
+        arr["ndim"] = cols[5]
+        pad = (0,) * MAX_DIMS
+        arr["shape"] = [(s + pad)[:MAX_DIMS] for s in cols[6]]
+        arr["stride"] = [(s + pad)[:MAX_DIMS] for s in cols[7]]
+        arr["image_stride"] = [(s + pad)[:MAX_DIMS] for s in cols[8]]
+        return arr
+
+
+@dataclasses.dataclass
+class SaveLayout:
+    """Where every item of one checkpoint object lies, and the table that packs it."""
+
+    image_bytes: int
+    spans: List[Tuple[int, int]]  # (offset, length) of each record: tensors in order, then byte blobs in order
+    items: np.ndarray
+    blob: bytes
+    device_payload_bytes: int
+    device_tensors: List[torch.Tensor]  # kept alive while the plan may run
+
+
+def build_save_layout(tensors: Sequence[torch.Tensor], blobs: Sequence[bytes] = ()) -> SaveLayout:
+    """Lays out records for ``tensors`` (device or host) followed by ``blobs`` and returns the descriptor table.
+
+    Device tensors become DEVICE items (any strides; the image side is the C-contiguous payload).  Record headers,
+    payloads of host-resident tensors and byte blobs are collected into one host blob that the plan uploads once.
+    """
+    table = ItemTable()
+    blob = bytearray()
+    spans: List[Tuple[int, int]] = []
+    keep: List[torch.Tensor] = []
+    pos = 0
+    device_bytes = 0
+    for t in tensors:
+        start = pos
+        hdr = header_bytes(t.dtype, t.shape)
+        table.add_blob(len(blob), pos, len(hdr))
+        blob += hdr
+        pos += len(hdr)
+        nbytes = t.numel() * t.element_size()
+        if nbytes:
+            if t.device.type == "cpu":
+                # host-resident item (step counters, RNG state ...): its bytes travel with the headers
+                flat = t.detach().contiguous().reshape(-1).view(torch.uint8)
+                table.add_blob(len(blob), pos, nbytes)
+                blob += flat.numpy().tobytes()
+            else:
+                shape, stride = tuple(t.shape), tuple(t.stride())
+                if len(shape) > MAX_DIMS:
+                    if not t.is_contiguous():
+                        raise NotImplementedError(f"non-contiguous tensor of rank {len(shape)} > {MAX_DIMS}")
+                    shape, stride = (t.numel(),), (1,)
+                table.add_device(t.data_ptr(), pos, t.element_size(), shape, stride)
+                keep.append(t)
+                device_bytes += nbytes
+            pos += nbytes
+        spans.append((start, pos - start))
+    for data in blobs:
+        if len(data):
+            table.add_blob(len(blob), pos, len(data))
+            blob += data
+        spans.append((pos, len(data)))
+        pos += len(data)
+    return SaveLayout(
+        image_bytes=pos,
+        spans=spans,
+        items=table.to_array(),
+        blob=bytes(blob),
+        device_payload_bytes=device_bytes,
+        device_tensors=keep,
+    )
+
+
+class Plan:
+    """Owns a native ``mlf_plan``: device-resident descriptor and work tables for one set of items."""
+
+    def __init__(
+        self,
+        items: np.ndarray,
+        blob: bytes,
+        image_bytes: int,
+        *,
+        tile_bytes: int = 0,
+        block_threads: int = 0,
+        align_to_tensor: bool = False,
+    ):
+        lib = _lib.load()
+        assert items.dtype == ITEM_DTYPE and items.flags["C_CONTIGUOUS"]
+        opts = _lib.PlanOpts(tile_bytes, block_threads, 1 if align_to_tensor else 0, 0)
+        handle = ctypes.c_void_p()
+        blob_buf = (ctypes.c_char * len(blob)).from_buffer_copy(blob) if blob else None
+        _lib.check(
+            lib.mlf_plan_create(
+                items.ctypes.data if len(items) else None,
+                len(items),
+                ctypes.addressof(blob_buf) if blob_buf is not None else None,
+                len(blob),
+                image_bytes,
+                ctypes.byref(opts),
+                ctypes.byref(handle),
+            ),
+            "mlf_plan_create",
+        )
+        self._handle = handle
+        self.image_bytes = image_bytes
+
+    @property
+    def info(self) -> _lib.PlanInfo:
+        out = _lib.PlanInfo()
+        _lib.check(_lib.load().mlf_plan_get_info(self._handle, ctypes.byref(out)), "mlf_plan_get_info")
+        return out
+
+    def pack(self, image: torch.Tensor, stream: Optional[int] = None) -> None:
+        """Enqueues tensors -> image on ``stream`` (default: torch's current stream)."""
+        self._launch(_lib.load().mlf_pack_launch, image, stream, "mlf_pack_launch")
+
+    def unpack(self, image: torch.Tensor, stream: Optional[int] = None) -> None:
+        """Enqueues image -> tensors on ``stream`` (default: torch's current stream)."""
+        self._launch(_lib.load().mlf_unpack_launch, image, stream, "mlf_unpack_launch")
+
+    def _launch(self, fn, image: torch.Tensor, stream: Optional[int], what: str) -> None:
+        if self._handle is None:
+            raise ValueError("plan already destroyed")
+        if image.dtype != torch.uint8 or not image.is_contiguous() or image.device.type != "cuda":
+            raise ValueError("image must be a contiguous uint8 device tensor")
+        if image.numel() < self.image_bytes:
+            raise ValueError(f"image holds {image.numel()} bytes, plan needs {self.image_bytes}")
+        if stream is None:
+            stream = torch.cuda.current_stream(image.device).cuda_stream
+        _lib.check(fn(self._handle, image.data_ptr() if image.numel() else None, stream), what)
+
+    def destroy(self) -> None:
+        if getattr(self, "_handle", None) is not None:
+            _lib.load().mlf_plan_destroy(self._handle)
+            self._handle = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+class CopyEngine:
+    """Ring of pinned slots + copy streams + host threads between device images and pageable host memory."""
+
+    def __init__(self, slot_bytes: int = 32 << 20, n_slots: int = 4, n_threads: int = 8):
+        handle = ctypes.c_void_p()
+        _lib.check(_lib.load().mlf_engine_create(slot_bytes, n_slots, n_threads, ctypes.byref(handle)), "mlf_engine_create")
+        self._handle = handle
+        self.slot_bytes, self.n_slots, self.n_threads = slot_bytes, n_slots, n_threads
+
+    def d2h(self, src_dev_ptr: int, dst_host_ptr: int, nbytes: int, producer_stream: int = 0) -> _lib.XferStats:
+        stats = _lib.XferStats()
+        _lib.check(
+            _lib.load().mlf_engine_d2h(self._handle, src_dev_ptr, dst_host_ptr, nbytes, producer_stream, ctypes.byref(stats)),
+            "mlf_engine_d2h",
+        )
+        return stats
+
+    def h2d(self, src_host_ptr: int, dst_dev_ptr: int, nbytes: int, consumer_stream: int = 0) -> _lib.XferStats:
+        stats = _lib.XferStats()
+        _lib.check(
+            _lib.load().mlf_engine_h2d(self._handle, src_host_ptr, dst_dev_ptr, nbytes, consumer_stream, ctypes.byref(stats)),
+            "mlf_engine_h2d",
+        )
+        return stats
+
+    def destroy(self) -> None:
+        if getattr(self, "_handle", None) is not None:
+            _lib.load().mlf_engine_destroy(self._handle)
+            self._handle = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+def crc32c_device(buf: torch.Tensor, nbytes: int, chunk_bytes: int, stream: Optional[int] = None) -> np.ndarray:
+    """CRC-32C of each ``chunk_bytes`` piece of the first ``nbytes`` of a device uint8 tensor."""
+    if nbytes == 0:
+        return np.zeros(0, dtype=np.uint32)
+    if stream is None:
+        stream = torch.cuda.current_stream(buf.device).cuda_stream
+    n_chunks = (nbytes + chunk_bytes - 1) // chunk_bytes
+    out = np.zeros(n_chunks, dtype=np.uint32)
+    _lib.check(
+        _lib.load().mlf_crc32c_device(buf.data_ptr(), nbytes, chunk_bytes, out.ctypes.data, n_chunks, stream),
+        "mlf_crc32c_device",
+    )
+    return out
+
+
+def crc32c_host(ptr: int, nbytes: int) -> int:
+    return int(_lib.load().mlf_crc32c_host(ptr, nbytes))
+
+
+def crc32c_combine(crc_a: int, crc_b: int, len_b: int) -> int:
+    return int(_lib.load().mlf_crc32c_combine(crc_a, crc_b, len_b))

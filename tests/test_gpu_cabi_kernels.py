@@ -1,0 +1,262 @@
+"""GPU parity of the C-ABI kernels against the CPU oracle: pack, unpack, CRC-32C, copy engine.
+
+Bit-exact is the bar everywhere (byte movement and integer arithmetic only).
+"""
+
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import mlf_format as oracle_fmt
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _rand_tensor(gen, shape, dtype):
+    """Seeded tensor whose *bytes* are uniform random (so every bit pattern, NaNs included, must survive)."""
+    numel = int(np.prod(shape)) if len(shape) else 1
+    esz = torch.empty((), dtype=dtype).element_size()
+    raw = torch.randint(0, 256, (max(numel, 1) * esz,), dtype=torch.uint8, generator=gen)
+    return raw[: numel * esz].view(dtype).reshape(shape).clone()
+
+
+def _pack_image(tensors, blobs=(), **plan_kw):
+    from ml_flashpoint.hip import plan as P
+
+    layout = P.build_save_layout(tensors, blobs)
+    plan = P.Plan(layout.items, layout.blob, layout.image_bytes, **plan_kw)
+    image = torch.empty(max(layout.image_bytes, 1) + 512, dtype=torch.uint8, device=DEV)
+    image.fill_(0xAB)
+    plan.pack(image)
+    torch.cuda.synchronize()
+    host = image.cpu().numpy()
+    assert (host[layout.image_bytes :] == 0xAB).all(), "pack wrote past the end of the image"
+    return layout, plan, image, host[: layout.image_bytes].tobytes()
+
+
+MIXED = [
+    ((), torch.float32),
+    ((0,), torch.float32),
+    ((1,), torch.int64),
+    ((2, 2), torch.float32),
+    ((7,), torch.bfloat16),
+    ((13, 5), torch.float16),
+    ((3, 5, 7), torch.int32),
+    ((1023,), torch.uint8),
+    ((1025,), torch.int8),
+    ((17,), torch.bool),
+    ((64, 257), torch.float8_e4m3fn),
+    ((300, 1001), torch.bfloat16),
+    ((4, 0, 3), torch.int16),
+    ((2, 3), torch.complex64),
+    ((5,), torch.complex128),
+    ((1 << 20,), torch.float32),
+    ((777, 513), torch.float64),
+]
+
+
+def test_pack_contiguous_mixed_dtypes_matches_oracle():
+    gen = torch.Generator().manual_seed(11)
+    cpu = [_rand_tensor(gen, s, d) for s, d in MIXED]
+    dev = [t.to(DEV) for t in cpu]
+    blobs = [b"", b"x", bytes(range(256)) * 5]
+    layout, plan, image, got = _pack_image(dev, blobs)
+    want, spans = oracle_fmt.data_section(cpu, blobs)
+    assert layout.spans == spans
+    assert got == want
+
+
+@pytest.mark.parametrize("tile_bytes,threads", [(1024, 64), (4096, 256), (65536, 512), (1 << 20, 1024)])
+def test_pack_tile_and_block_shapes(tile_bytes, threads):
+    gen = torch.Generator().manual_seed(12)
+    cpu = [_rand_tensor(gen, s, d) for s, d in [((100003,), torch.uint8), ((513, 1027), torch.bfloat16), ((3,), torch.int64)]]
+    dev = [t.to(DEV) for t in cpu]
+    _, _, _, got = _pack_image(dev, tile_bytes=tile_bytes, block_threads=threads)
+    assert got == oracle_fmt.data_section(cpu)[0]
+
+
+def test_pack_misaligned_sources():
+    """Views that start at odd element offsets: the source address is not 16-byte aligned."""
+    gen = torch.Generator().manual_seed(13)
+    base8 = _rand_tensor(gen, (70001,), torch.uint8)
+    base16 = _rand_tensor(gen, (50001,), torch.bfloat16)
+    cpu = [base8[k : k + 60000] for k in (1, 2, 3, 5, 15)] + [base16[k : k + 40000] for k in (1, 3, 7)]
+    dev8, dev16 = base8.to(DEV), base16.to(DEV)
+    dev = [dev8[k : k + 60000] for k in (1, 2, 3, 5, 15)] + [dev16[k : k + 40000] for k in (1, 3, 7)]
+    _, _, _, got = _pack_image(dev)
+    assert got == oracle_fmt.data_section(cpu)[0]
+
+
+def _views(base):
+    """Non-contiguous views of a 3-D base, the kinds BASELINE's strided config names plus a few more."""
+    m = base[0]
+    return [
+        m.t(),  # transposed
+        m[:, ::2],  # every other column
+        m[16:48, :],  # row block (contiguous)
+        m[:, 8:40],  # column block (row-contiguous pieces)
+        base.permute(2, 0, 1),
+        base[::2, 1:, ::3],
+        base[1].t()[3:, ::2],
+        m[5],  # one row
+        m[:, 5],  # one column
+        base.expand(2, *base.shape)[1],  # stride-0 parent
+    ]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float8_e4m3fn, torch.float32, torch.int64, torch.complex128])
+def test_pack_strided_views_match_bruteforce_oracle(dtype):
+    gen = torch.Generator().manual_seed(14)
+    base_cpu = _rand_tensor(gen, (3, 64, 96), dtype)
+    base_dev = base_cpu.to(DEV)
+    cpu, dev = _views(base_cpu), _views(base_dev)
+    layout, plan, _, got = _pack_image(dev)
+    want = b"".join(
+        oracle_fmt.header_bytes(oracle_fmt.dtype_name(t.dtype), tuple(t.shape)) + oracle_fmt.payload_bytes_bruteforce(t)
+        for t in cpu
+    )
+    assert got == want
+    assert got == oracle_fmt.data_section(cpu)[0]
+    assert plan.info.n_strided_items > 0
+
+
+def test_pack_large_rows_go_through_flat_kernel():
+    gen = torch.Generator().manual_seed(15)
+    base_cpu = _rand_tensor(gen, (64, 8192), torch.bfloat16)
+    base_dev = base_cpu.to(DEV)
+    cpu, dev = [base_cpu[:, 1024:5120]], [base_dev[:, 1024:5120]]
+    _, plan, _, got = _pack_image(dev)
+    assert got == oracle_fmt.data_section(cpu)[0]
+    assert plan.info.n_strided_items == 0 and plan.info.n_flat_tiles >= 64
+
+
+def test_pack_host_resident_tensors_travel_in_blob():
+    gen = torch.Generator().manual_seed(16)
+    cpu = [_rand_tensor(gen, (33, 3), torch.float32), _rand_tensor(gen, (5000,), torch.int64).t(), _rand_tensor(gen, (), torch.int64)]
+    mixed = [cpu[0].to(DEV), cpu[1], cpu[2]]
+    _, _, _, got = _pack_image(mixed, [b"tail"])
+    assert got == oracle_fmt.data_section(cpu, [b"tail"])[0]
+
+
+def test_unpack_restores_full_tensors_bit_exact():
+    from ml_flashpoint.hip import plan as P
+
+    gen = torch.Generator().manual_seed(21)
+    cpu = [_rand_tensor(gen, s, d) for s, d in MIXED]
+    data, spans = oracle_fmt.data_section(cpu)
+    image = torch.frombuffer(bytearray(data), dtype=torch.uint8).to(DEV)
+    targets = [torch.zeros_like(t, device=DEV) for t in cpu]
+    table = P.ItemTable()
+    for t, tgt, (off, length) in zip(cpu, targets, spans):
+        nbytes = t.numel() * t.element_size()
+        if nbytes:
+            table.add_device(tgt.data_ptr(), off + length - nbytes, t.element_size(), tuple(t.shape), tuple(tgt.stride()))
+    plan = P.Plan(table.to_array(), b"", len(data), align_to_tensor=True)
+    padded = torch.empty(len(data) + 256, dtype=torch.uint8, device=DEV)
+    padded[: len(data)] = image
+    plan.unpack(padded)
+    torch.cuda.synchronize()
+    for t, tgt in zip(cpu, targets):
+        assert torch.equal(tgt.cpu().contiguous().reshape(-1).view(torch.uint8), t.contiguous().reshape(-1).view(torch.uint8))
+
+
+def test_unpack_sub_boxes_into_strided_targets():
+    """Restore of a narrowed box of the stored tensor into a non-contiguous target (resharding reads)."""
+    from ml_flashpoint.hip import plan as P
+
+    gen = torch.Generator().manual_seed(22)
+    stored = _rand_tensor(gen, (12, 20, 10), torch.float32)
+    data, spans = oracle_fmt.data_section([stored])
+    payload_off = spans[0][0] + spans[0][1] - stored.numel() * 4
+    image = torch.zeros(len(data) + 256, dtype=torch.uint8, device=DEV)
+    image[: len(data)] = torch.frombuffer(bytearray(data), dtype=torch.uint8).to(DEV)
+    cases = [((0, 0, 0), (12, 20, 10)), ((1, 0, 3), (2, 2, 2)), ((4, 5, 0), (8, 15, 10)), ((0, 19, 9), (12, 1, 1))]
+    for offsets, lengths in cases:
+        want = oracle_fmt.read_item(data[spans[0][0] : spans[0][0] + spans[0][1]], offsets, lengths)
+        parent = torch.zeros((lengths[0], lengths[1] * 2, lengths[2] + 3), dtype=torch.float32, device=DEV)
+        target = parent[:, ::2, 3:]
+        src_strides = (200, 10, 1)
+        box_off = sum(o * s for o, s in zip(offsets, src_strides)) * 4
+        table = P.ItemTable()
+        table.add_device(target.data_ptr(), payload_off + box_off, 4, lengths, tuple(target.stride()), image_stride=src_strides)
+        plan = P.Plan(table.to_array(), b"", len(data), align_to_tensor=True)
+        plan.unpack(image)
+        torch.cuda.synchronize()
+        assert torch.equal(target.cpu().view(torch.int32), want.contiguous().view(torch.int32))
+        assert int(parent[:, 1::2, :].abs().sum()) == 0 and int(parent[:, :, :3].abs().sum()) == 0
+
+
+def test_plan_rejects_items_outside_image():
+    from ml_flashpoint.hip import _lib, plan as P
+
+    t = torch.zeros(100, dtype=torch.float32, device=DEV)
+    table = P.ItemTable()
+    table.add_device(t.data_ptr(), 10, 4, (100,), (1,))
+    with pytest.raises(_lib.HipError, match="does not fit in the image"):
+        P.Plan(table.to_array(), b"", 400)
+    table = P.ItemTable()
+    table.add_blob(0, 0, 16)
+    with pytest.raises(_lib.HipError, match="outside the host blob"):
+        P.Plan(table.to_array(), b"12345678", 64)
+
+
+@pytest.mark.parametrize("nbytes", [1, 15, 1023, 1024, 65535, 65536, 65537, 3 * 65536 + 1024 + 7, (5 << 20) + 13])
+def test_crc32c_device_matches_oracle(nbytes, oracle_c):
+    from ml_flashpoint.hip import plan as P
+
+    gen = torch.Generator().manual_seed(nbytes)
+    host = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=gen)
+    dev = host.to(DEV)
+    for chunk in (65536, 1 << 20):
+        got = P.crc32c_device(dev, nbytes, chunk)
+        n_chunks = (nbytes + chunk - 1) // chunk
+        want = np.zeros(n_chunks, dtype=np.uint32)
+        raw = host.numpy().tobytes()
+        oracle_c.oracle_crc32c_chunks(raw, nbytes, chunk, want.ctypes.data)
+        assert got.tolist() == want.tolist()
+        # checksum of checksums: chaining the chunk CRCs reproduces the CRC of the whole buffer
+        whole = int(got[0])
+        for k in range(1, n_chunks):
+            whole = P.crc32c_combine(whole, int(got[k]), min(chunk, nbytes - k * chunk))
+        assert whole == oracle_c.oracle_crc32c(raw, nbytes)
+
+
+def test_crc32c_known_vectors_on_device(oracle_c):
+    from ml_flashpoint.hip import plan as P
+
+    for data, want in [
+        (b"123456789", 0xE3069283),
+        (bytes(32), 0x8A9136AA),
+        (b"\xff" * 32, 0x62A8AB43),
+        (bytes(range(32)), 0x46DD794E),
+        (bytes(range(31, -1, -1)), 0x113FDB5C),
+    ]:
+        dev = torch.frombuffer(bytearray(data), dtype=torch.uint8).to(DEV)
+        assert int(P.crc32c_device(dev, len(data), 65536)[0]) == want
+
+
+@pytest.mark.parametrize("nbytes", [1, 4097, (1 << 20) + 5, (9 << 20) + 12345])
+def test_copy_engine_round_trip(nbytes, shm_dir):
+    """Device -> mapped tmpfs file -> device through the pinned ring, several chunks, ragged tail."""
+    from ml_flashpoint.checkpoint_object_manager.buffer_object.buffer_object_ext import BufferObject
+    from ml_flashpoint.hip import plan as P
+
+    gen = torch.Generator().manual_seed(nbytes)
+    host = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=gen)
+    dev = host.to(DEV)
+    engine = P.CopyEngine(slot_bytes=1 << 20, n_slots=3, n_threads=4)
+    bo = BufferObject(f"{shm_dir}/obj.bin", 4096 + nbytes, True)
+    stream = torch.cuda.current_stream().cuda_stream
+    stats = engine.d2h(dev.data_ptr(), bo.get_data_ptr() + 4096, nbytes, stream)
+    assert stats.bytes == nbytes and stats.chunks == (nbytes + (1 << 20) - 1) // (1 << 20)
+    assert bytes(memoryview(bo)[4096:]) == host.numpy().tobytes()
+    back = torch.zeros(nbytes + 64, dtype=torch.uint8, device=DEV)
+    engine.h2d(bo.get_data_ptr() + 4096, back.data_ptr(), nbytes, stream)
+    torch.cuda.synchronize()
+    assert torch.equal(back[:nbytes].cpu(), host) and int(back[nbytes:].sum()) == 0
+    bo.close()
+    engine.destroy()
