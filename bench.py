@@ -1,0 +1,365 @@
+"""Benchmark of the save/restore data path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload llama3-8b-shard] [--scale S]
+
+A *step* is one full save of the workload's state dict (resident in HBM) into a pooled tmpfs buffer object, followed
+by one full restore of that object into the (zeroed) live tensors, both driven through the PyTorch DCP adapters
+(``MemoryStorageWriter`` / ``MemoryStorageReader``) with the gfx950 saver/loader plugged in.  Prints ONE JSON line:
+
+* ``value``          GB/s moved through the path per step: (bytes saved + bytes restored) / step time
+* ``save_GBps`` / ``restore_GBps`` / ``blocking_save_ms`` (save entry -> training stream may continue) and the
+  stage breakdown (pack / unpack kernel GB/s from HIP events, D2H / H2D GB/s of the copy engine)
+* ``roofline``       the pack kernel against HBM peak: algorithmic bytes = 2 x payload bytes per launch
+* ``cpu_baseline``   the CPU oracle (restating the reference's per-tensor path) timed on this box's host cores on a
+                     bounded sample of the same state dict
+
+Synthetic data, seeded; the restored tensors are checked against fingerprints of the originals after the timed region.
+"""
+
+import argparse
+import concurrent.futures
+import json
+import os
+import shutil
+import sys
+import tempfile
+import time
+
+REPO = os.path.dirname(os.path.abspath(__file__))
+for _p in (REPO, os.path.join(REPO, "ml-flashpoint_amd"), os.path.join(REPO, "tests")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, vendor figure
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--workload", default="llama3-8b-shard",
+                    choices=["llama3-8b-shard", "many-small", "mixtral-expert-shard", "strided-views", "gpt2-small"])
+    ap.add_argument("--scale", type=float, default=1.0, help="fraction of the workload's layers/tensors (debugging)")
+    ap.add_argument("--tile-bytes", type=int, default=0)
+    ap.add_argument("--block-threads", type=int, default=0)
+    ap.add_argument("--slot-mib", type=int, default=32)
+    ap.add_argument("--slots", type=int, default=4)
+    ap.add_argument("--copy-threads", type=int, default=8)
+    ap.add_argument("--crc-chunk-mib", type=int, default=0, help="> 0: CRC-32C per chunk on save, verified on restore")
+    ap.add_argument("--cpu-baseline-gb", type=float, default=12.0, help="size of the CPU baseline's sample (0 = skip)")
+    ap.add_argument("--root", default=None, help="directory on tmpfs for the pool and checkpoints")
+    return ap.parse_args()
+
+
+def build_workload(name, device, scale):
+    import workloads
+
+    if name == "llama3-8b-shard":
+        layers = max(1, round(32 * scale))
+        sd = workloads.llama3_8b_shard(device, layers=layers) if scale >= 1.0 else workloads.llama3_8b_shard(
+            device, layers=layers, vocab=max(1024, int(128256 * scale)))
+        label = "Llama-3-8B-shaped shard: bf16 weights + fp32 master + fp32 Adam m,v"
+    elif name == "many-small":
+        sd = workloads.many_small(device, count=max(1, int(20000 * scale)))
+        label = "20,000 tensors, 64 B..4 MB log-uniform, fp32/bf16/int64"
+    elif name == "mixtral-expert-shard":
+        sd = workloads.mixtral_expert_shard(device, layers=max(1, round(32 * scale)))
+        label = "Mixtral-8x7B-shaped expert shard, bf16"
+    elif name == "strided-views":
+        sd, parents = workloads.strided_views(device, count=max(3, int(2000 * scale)))
+        sd = dict(sd)
+        sd["__parents__"] = parents  # keep alive; not a tensor entry
+        label = "2,000 transposed / strided / row-block views of bf16/fp8/fp32 parents"
+    else:
+        sd = workloads.gpt2_small(device)
+        label = "GPT-2-small fp32"
+    parents = sd.pop("__parents__", None)
+    return sd, label, parents
+
+
+def cpu_baseline(sd, sample_bytes, root, device):
+    """The reference's CPU path, restated by the oracle, on a prefix of the state dict of about ``sample_bytes``."""
+    import torch
+
+    from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId, CheckpointObjectId
+    from oracle import cpu_path
+
+    sample, total = {}, 0
+    for k, v in sd.items():
+        if total >= sample_bytes:
+            break
+        sample[k] = v
+        total += v.numel() * v.element_size()
+    saver = cpu_path.OracleCheckpointSaver(initial_buffer_size_bytes=total + (1 << 20))
+    threads = saver.torch_thread_count(1)
+    cid = CheckpointContainerId(os.path.join(root, "cpu_baseline", "step-0_ckpt"))
+    path = os.path.join(cid.data, "sample.distcp")
+    tensors = list(sample.values())
+    times = {"stage": [], "write": [], "restore": []}
+    for rep in range(2):  # the first pass faults the tmpfs pages in, like the GPU path's warm-up
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        staged = saver.stage_data(cid, sample, non_blocking=True)
+        t1 = time.perf_counter()
+        original = torch.get_num_threads()
+        torch.set_num_threads(threads)
+        try:
+            if rep == 0:
+                spans = cpu_path.write_object(path, list(staged.values()), [], total + (1 << 20))
+                t2 = time.perf_counter()
+            else:
+                # rewrite in place over warm pages: what a pooled buffer gives the reference from the second save on
+                spans = _rewrite_warm(path, list(staged.values()))
+                t2 = time.perf_counter()
+        finally:
+            torch.set_num_threads(original)
+        del staged
+        # restore: read() copy, frombuffer, copy_ to the device tensor
+        import mmap
+
+        from oracle import mlf_format as fmt
+
+        targets = [torch.empty_like(t) for t in tensors]
+        torch.cuda.synchronize()
+        t3 = time.perf_counter()
+        with open(path, "rb") as f:
+            mm = mmap.mmap(f.fileno(), 0, mmap.MAP_SHARED, mmap.PROT_READ)
+            for (off, length), tgt in zip(spans, targets):
+                record = mm[fmt.METADATA_SIZE + off : fmt.METADATA_SIZE + off + length]
+                tgt.copy_(fmt.read_item(record, (0,) * tgt.dim(), tuple(tgt.shape)))
+            mm.close()
+        torch.cuda.synchronize()
+        t4 = time.perf_counter()
+        ok = all(torch.equal(a.view(torch.uint8), b.contiguous().view(torch.uint8)) for a, b in zip(targets[:8], tensors[:8]))
+        del targets
+        times["stage"].append(t1 - t0)
+        times["write"].append(t2 - t1)
+        times["restore"].append(t4 - t3)
+    shutil.rmtree(os.path.join(root, "cpu_baseline"), ignore_errors=True)
+    stage, write, restore = times["stage"][-1], times["write"][-1], times["restore"][-1]
+    gb = total / 1e9
+    return {
+        "value": round(2 * gb / (stage + write + restore), 3),
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"first {len(sample)} tensors ({gb:.2f} GB) of the same state dict, second pass (warm tmpfs pages)",
+        "save_GBps": round(gb / (stage + write), 3),
+        "restore_GBps": round(gb / restore, 3),
+        "blocking_stage_ms": round(stage * 1e3, 1),
+        "write_GBps": round(gb / write, 3),
+        "host_cpus": os.cpu_count(),
+        "restored_ok": bool(ok),
+    }
+
+
+def _rewrite_warm(path, tensors):
+    """Second write of the CPU baseline: same records into the already-populated file (no truncation)."""
+    import mmap
+
+    import torch
+
+    from oracle import mlf_format as fmt
+
+    spans, pos = [], 0
+    with open(path, "r+b") as f:
+        mm = mmap.mmap(f.fileno(), 0, mmap.MAP_SHARED, mmap.PROT_READ | mmap.PROT_WRITE)
+        mv = memoryview(mm)
+        for t in tensors:
+            start = pos
+            hdr = fmt.header_bytes(fmt.dtype_name(t.dtype), tuple(t.shape))
+            mv[fmt.METADATA_SIZE + pos : fmt.METADATA_SIZE + pos + len(hdr)] = hdr
+            pos += len(hdr)
+            nbytes = t.numel() * t.element_size()
+            if nbytes:
+                dest = mv[fmt.METADATA_SIZE + pos : fmt.METADATA_SIZE + pos + nbytes]
+                torch.frombuffer(dest, dtype=t.dtype, count=t.numel()).reshape(t.shape).copy_(t)
+                del dest
+                pos += nbytes
+            spans.append((start, pos - start))
+        mv.release()
+        mm.close()
+    return spans
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU's share of the save/restore path; runs with --gpus > 1 are not part of this "
+              "build (each rank would run this same pipeline independently on its own shard).", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import torch.distributed.checkpoint as dcp
+    import torch.multiprocessing as torch_mp
+    from torch.distributed.checkpoint import DefaultSavePlanner
+
+    import workloads
+    from ml_flashpoint.adapter.pytorch.memory_storage_reader import MemoryStorageReader
+    from ml_flashpoint.adapter.pytorch.memory_storage_writer import MemoryStorageWriter
+    from ml_flashpoint.checkpoint_object_manager.buffer_metadata import METADATA_SIZE
+    from ml_flashpoint.checkpoint_object_manager.checkpoint_object_manager import CheckpointObjectManager
+    from ml_flashpoint.core.buffer_pool import BufferPoolConfig
+    from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId
+    from ml_flashpoint.core.checkpoint_loader import DefaultMLFlashpointCheckpointLoader
+    from ml_flashpoint.core.checkpoint_saver import DefaultMLFlashpointCheckpointSaver
+    from ml_flashpoint.hip.checkpoint_saver import EngineConfig
+
+    import warnings
+
+    warnings.filterwarnings("ignore", message="torch.distributed is disabled")
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+    t_setup = time.perf_counter()
+    sd, label, parents = build_workload(args.workload, device, args.scale)
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    payload = workloads.payload_bytes(sd)
+    prints = {k: workloads.fingerprint(v) for k, v in sd.items()}
+    torch.cuda.synchronize()
+    print(f"[bench] workload {args.workload}: {len(sd)} tensors, {payload / 1e9:.2f} GB payload, built in "
+          f"{time.perf_counter() - t_setup:.1f}s", file=sys.stderr, flush=True)
+
+    base = args.root or ("/dev/shm" if os.access("/dev/shm", os.W_OK) else None)
+    root = tempfile.mkdtemp(prefix="mlf_bench_", dir=base)
+    mgr = torch_mp.get_context("spawn").Manager()
+    fut = concurrent.futures.Future()
+    fut.set_result(mgr)
+    engine_cfg = EngineConfig(slot_bytes=args.slot_mib << 20, n_slots=args.slots, copy_threads=args.copy_threads)
+    # one pooled buffer: the previous step's object is deleted before the next save, as finalize_checkpoint's
+    # background cleanup would have done, so the same warm tmpfs pages are reused every step
+    CheckpointObjectManager._worker_pool = None
+    manager = CheckpointObjectManager(BufferPoolConfig(os.path.join(root, "pool"), 0, 1, METADATA_SIZE + (1 << 20)))
+    saver = DefaultMLFlashpointCheckpointSaver(
+        lambda: 0, lambda: 0, lambda: None, manager, None, initial_buffer_size_bytes=1 << 20,
+        engine_config=engine_cfg, tile_bytes=args.tile_bytes, block_threads=args.block_threads,
+        crc_chunk_bytes=args.crc_chunk_mib << 20)
+    loader = DefaultMLFlashpointCheckpointLoader(manager, None, engine_config=engine_cfg, tile_bytes=args.tile_bytes,
+                                                 block_threads=args.block_threads)
+    saver.record_kernel_events = loader.record_kernel_events = True
+    result = None
+    try:
+        rec = {k: [] for k in ("step", "save", "restore", "blocking", "plan", "pack_launch", "d2h", "h2d")}
+        file_bytes = 0
+        prev = None
+        for it in range(args.warmup + args.steps):
+            timed = it >= args.warmup
+            cid = CheckpointContainerId(os.path.join(root, "run", f"step-{it}_ckpt"))
+            if prev is not None:
+                manager.delete_container(prev)
+            saver.kernel_events.clear()
+            loader.kernel_events.clear()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            # ---- save: plan -> pack (blocking part ends at the synchronize) -> D2H -> metadata -> finalize ----
+            saver.initialize_checkpoint(cid)
+            writer = MemoryStorageWriter(saver, fut)
+            writer.reset(cid.data)
+            planner = DefaultSavePlanner()
+            planner.set_up_planner(sd, is_coordinator=True)
+            local = writer.prepare_local_plan(planner.create_local_plan())
+            plans, metadata = planner.create_global_plan([local])
+            plan = planner.finish_plan(writer.prepare_global_plan(plans)[0])
+            t_plan = time.perf_counter()
+            buckets = writer.prepare_write_data_buckets(cid, plan, planner)
+            t_launch = time.perf_counter()
+            staged = MemoryStorageWriter.stage_write_data_buckets(cid, buckets, non_blocking=True)
+            t_block = time.perf_counter()
+            results = writer.write_staged_data_buckets(cid, staged, replicate_after_write=False).wait()
+            writer.finish_checkpoint(cid, metadata, [results])
+            saver.finalize_checkpoint(cid)
+            t_saved = time.perf_counter()
+            d2h = dict(saver.last_save_stats)
+            pack_ms = sum(b.elapsed_time(e) for b, e, _ in saver.kernel_events)
+            pack_bytes = sum(n for _, _, n in saver.kernel_events)
+            del buckets, staged, results
+            # ---- restore into zeroed live tensors ----
+            for v in sd.values():
+                v.zero_() if v.is_contiguous() else v.fill_(0)
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            dcp.load(sd, checkpoint_id=cid.data, storage_reader=MemoryStorageReader(cid.data, loader), no_dist=True)
+            torch.cuda.synchronize()
+            t2 = time.perf_counter()
+            unpack_ms = sum(b.elapsed_time(e) for b, e, _ in loader.kernel_events)
+            unpack_bytes = sum(n for _, _, n in loader.kernel_events)
+            file_bytes = os.path.getsize(os.path.join(cid.data, "__0__0_src0.distcp"))
+            prev = cid
+            line = (f"[bench] it {it} {'timed ' if timed else 'warmup'} save {t_saved - t0:.3f}s (blocking "
+                    f"{(t_block - t0) * 1e3:.1f} ms, pack kernel {pack_ms:.2f} ms, d2h {d2h.get('d2h_s', 0):.3f}s) "
+                    f"restore {t2 - t1:.3f}s (h2d {loader.last_load_stats.get('h2d_s', 0):.3f}s, unpack {unpack_ms:.2f} ms)")
+            print(line, file=sys.stderr, flush=True)
+            if timed:
+                rec["step"].append((t_saved - t0) + (t2 - t1))
+                rec["save"].append(t_saved - t0)
+                rec["restore"].append(t2 - t1)
+                rec["blocking"].append(t_block - t0)
+                rec["plan"].append(t_plan - t0)
+                rec["pack_launch"].append(t_launch - t_plan)
+                rec["d2h"].append(d2h.get("d2h_s", 0.0))
+                rec["h2d"].append(loader.last_load_stats.get("h2d_s", 0.0))
+                rec.setdefault("pack_ms", []).append(pack_ms)
+                rec.setdefault("unpack_ms", []).append(unpack_ms)
+                rec.setdefault("pack_bytes", []).append(pack_bytes)
+                rec.setdefault("unpack_bytes", []).append(unpack_bytes)
+        # parity after the timed region: restored bits == original bits
+        mismatched = [k for k, v in sd.items() if workloads.fingerprint(v) != prints[k]]
+        assert not mismatched, f"restored tensors differ from the originals: {mismatched[:5]}"
+        manager.delete_container(prev)
+
+        mean = lambda xs: sum(xs) / len(xs)  # noqa: E731
+        step_s = mean(rec["step"])
+        gb = file_bytes / 1e9
+        pack_s = mean(rec["pack_ms"]) * 1e-3
+        unpack_s = mean(rec["unpack_ms"]) * 1e-3
+        pack_gbps = 2 * mean(rec["pack_bytes"]) / 1e9 / pack_s if pack_s > 0 else 0.0
+        result = {
+            "metric": "save+restore GB/s through the shm buffer path (with blocking save ms), 1 MI355X",
+            "value": round(2 * gb / step_s, 3),
+            "unit": "GB/s",
+            "n_gpus": 1,
+            "steps": args.steps,
+            "warmup": args.warmup,
+            "ms_per_step": round(step_s * 1e3, 2),
+            "higher_is_better": True,
+            "scaling": "weak",
+            "vs_baseline": None,
+            "dtype": "u8",
+            "data": "synthetic",
+            "config": {"workload": f"{args.workload}: {label}", "tensors": len(sd), "payload_bytes": payload,
+                       "file_bytes": file_bytes, "scale": args.scale, "tile_bytes": args.tile_bytes or 4096,
+                       "engine": {"slot_mib": args.slot_mib, "slots": args.slots, "copy_threads": args.copy_threads},
+                       "crc_chunk_mib": args.crc_chunk_mib},
+            "save_GBps": round(gb / mean(rec["save"]), 3),
+            "restore_GBps": round(gb / mean(rec["restore"]), 3),
+            "blocking_save_ms": round(mean(rec["blocking"]) * 1e3, 2),
+            "blocking_breakdown_ms": {"dcp_plan": round(mean(rec["plan"]) * 1e3, 2),
+                                      "layout_and_pack_launch": round(mean(rec["pack_launch"]) * 1e3, 2),
+                                      "pack_kernel": round(pack_s * 1e3, 3)},
+            "pack_GBps": round(pack_gbps, 1),
+            "unpack_GBps": round(2 * mean(rec["unpack_bytes"]) / 1e9 / unpack_s, 1) if unpack_s > 0 else None,
+            "d2h_GBps": round(gb / mean(rec["d2h"]), 2) if mean(rec["d2h"]) > 0 else None,
+            "h2d_GBps": round(gb / mean(rec["h2d"]), 2) if mean(rec["h2d"]) > 0 else None,
+            "parity": "restored tensors bit-identical to originals (fingerprints)",
+            "roofline": {"bound": "hbm", "kernel": "mlf_flat_kernel<pack>", "achieved": round(pack_gbps, 1),
+                         "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(pack_gbps / HBM_PEAK_GBPS, 4),
+                         "traffic": None,
+                         "algorithmic_bytes_per_launch": int(2 * mean(rec["pack_bytes"])),
+                         "avg_launch_ms": round(pack_s * 1e3, 3)},
+        }
+        if args.cpu_baseline_gb > 0:
+            result["cpu_baseline"] = cpu_baseline(sd, args.cpu_baseline_gb * 1e9, root, device)
+    finally:
+        try:
+            manager.teardown_pool()
+        except Exception:
+            pass
+        mgr.shutdown()
+        shutil.rmtree(root, ignore_errors=True)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -59,15 +59,15 @@ typedef struct mlf_item {
 } mlf_item;
 
 typedef struct mlf_plan_opts {
-  uint32_t tile_bytes;       /* bytes one wavefront copies per work item (multiple of 1024; 0 = default)       */
+  uint32_t tile_bytes;       /* bytes one workgroup copies per work item (multiple of 1024; 0 = default)       */
   uint32_t block_threads;    /* threads per workgroup for the copy kernels (multiple of 64; 0 = default)       */
   uint32_t align_to_tensor;  /* 0: cut tiles at 16-byte boundaries of the image (pack); 1: of the tensor (unpack) */
-  uint32_t reserved;
+  uint32_t unroll;           /* 16-byte vectors in flight per thread in the copy loop: 1, 2, 4, 8 (0 = default) */
 } mlf_plan_opts;
 
 typedef struct mlf_plan_info {
   uint64_t n_items;
-  uint64_t n_flat_tiles;      /* wavefront work items of the flat (byte-segment) kernel                        */
+  uint64_t n_flat_tiles;      /* workgroup work items of the flat (byte-segment) kernel                        */
   uint64_t n_strided_items;   /* items that go through the generic strided kernel                              */
   uint64_t n_strided_work;
   uint64_t n_transposed_items;/* items that go through the LDS-tiled transpose kernel                          */

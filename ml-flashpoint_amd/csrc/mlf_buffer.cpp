@@ -11,6 +11,9 @@
 #include <errno.h>
 #include <fcntl.h>
 #include <string.h>
+#ifndef _GNU_SOURCE
+#define _GNU_SOURCE
+#endif
 #include <sys/mman.h>
 #include <sys/stat.h>
 #include <unistd.h>
@@ -184,18 +187,31 @@ int mlf_buffer_resize(mlf_buffer* b, size_t new_capacity) {
   if (!b->writable) return fail(MLF_FAILED_PRECONDITION, "Cannot resize a read-only buffer.");
   if (new_capacity == 0) return fail(MLF_INVALID_ARGUMENT, "Cannot resize buffer to 0.");
   if (new_capacity == b->cap) return MLF_OK;
-  if (munmap(b->ptr, b->cap) == -1) return fail_errno("munmap() failed during resize", errno);
-  b->ptr = nullptr;
-  if (ftruncate(b->fd, (off_t)new_capacity) == -1) {
-    int e = errno;
-    b->closed = true;  // mapping is gone; the handle cannot be used any more
-    return fail_errno("ftruncate() failed during resize", e);
-  }
-  void* p = mmap(nullptr, new_capacity, PROT_READ | PROT_WRITE, MAP_SHARED, b->fd, 0);
+  // Same outcome as munmap + ftruncate + mmap (the file and the mapping both get the new size, the address may
+  // change), but mremap carries the page-table entries of the surviving range over, so a pooled buffer that is
+  // trimmed after one save and grown again for the next is written without taking a minor fault per page.
+  const bool shrinking = new_capacity < b->cap;
+  if (!shrinking && ftruncate(b->fd, (off_t)new_capacity) == -1) return fail_errno("ftruncate() failed during resize", errno);
+  void* p = mremap(b->ptr, b->cap, new_capacity, MREMAP_MAYMOVE);
   if (p == MAP_FAILED) {
     int e = errno;
-    b->closed = true;
-    return fail_errno("mmap() failed during resize", e);
+    // fall back to the plain sequence
+    if (munmap(b->ptr, b->cap) == -1) return fail_errno("munmap() failed during resize", errno);
+    b->ptr = nullptr;
+    if (ftruncate(b->fd, (off_t)new_capacity) == -1) {
+      b->closed = true;
+      return fail_errno("ftruncate() failed during resize", errno);
+    }
+    p = mmap(nullptr, new_capacity, PROT_READ | PROT_WRITE, MAP_SHARED, b->fd, 0);
+    if (p == MAP_FAILED) {
+      b->closed = true;
+      return fail_errno(std::string("mmap() failed during resize (after mremap: ") + strerror(e) + ")", errno);
+    }
+  } else if (shrinking && ftruncate(b->fd, (off_t)new_capacity) == -1) {
+    int e2 = errno;
+    b->ptr = p;
+    b->cap = new_capacity;
+    return fail_errno("ftruncate() failed during resize", e2);
   }
   b->ptr = p;
   b->cap = new_capacity;

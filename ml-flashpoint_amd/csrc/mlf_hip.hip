@@ -7,10 +7,14 @@
 //
 // Everything on this path is integer byte movement, so the bound is HBM bandwidth (pack/unpack/crc) or the
 // host link (engine).  Kernels are written for 64-wide wavefronts and 16-byte accesses:
-//   * flat kernel: one wavefront per work item ("tile": <= tile_bytes of one contiguous item).  The
+//   * flat kernel: one small workgroup per tile (default 256 threads x one 16-byte vector = 4 KiB).  The
 //     destination is peeled to a 16-byte boundary, the body is non-temporal dwordx4 stores fed by dwordx4
 //     loads from a possibly misaligned source (gfx950 runs in unaligned-access mode), the tail is bytes.
-//     No LDS, no barriers; tiles of one item are consecutive so neighbouring waves stream neighbouring lines.
+//     No LDS, no barriers.  Workgroups are short-lived and consecutive workgroups copy consecutive tiles, so
+//     the set of tiles in flight at any moment is a compact, sequential window of HBM; measured on MI355X
+//     this ordering is worth ~25 % over long-running workgroups that each stream a large private region.
+//     Tiles are not listed one by one: a table entry ("span") describes up to 128 (or 16, or 1) consecutive
+//     tiles of one contiguous item and the workgroups that share it derive their tile from blockIdx.
 //   * strided kernel: generic N-d index walk for non-contiguous sources/targets and sub-box restores.
 //   * crc kernel: per wavefront a 64 KiB segment is read as coalesced 1 KiB rows; every lane keeps four
 //     Horner accumulators advanced by x^8192 through LDS tables, then lanes are folded with GF(2) multiplies.
@@ -62,7 +66,7 @@ double now_s() {
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef u32x4 u32x4_u __attribute__((aligned(1)));  // dwordx4 access at any byte address
 
-struct FlatTile {   // one wavefront's work: copy n bytes between a tensor address and an image offset
+struct Span {       // n bytes of one contiguous item, copied by the (1 << shift) workgroups that share the entry
   uint64_t tensor;  // absolute device address on the tensor (or blob) side
   uint64_t image;   // byte offset in the image
   uint32_t n;
@@ -85,50 +89,59 @@ struct StridedWork {  // one workgroup's work: elements [start, start+count) of 
   uint32_t desc;
 };
 
-constexpr int kWave = 64;
-constexpr int kUnroll = 4;  // dwordx4 per lane in flight: 4 KiB per wavefront per loop trip
 
 // ---------------------------------------------------------------------------------------------------------
 // flat kernel
 // ---------------------------------------------------------------------------------------------------------
-template <bool PACK>
-__global__ void __launch_bounds__(1024) mlf_flat_kernel(const FlatTile* __restrict__ tiles, uint32_t n_tiles,
-                                                        char* __restrict__ image) {
-  const uint32_t waves_per_block = blockDim.x >> 6;
-  const uint32_t wave = blockIdx.x * waves_per_block + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  if (wave >= n_tiles) return;
-  const uint32_t lane = threadIdx.x & (kWave - 1);
-  const FlatTile t = tiles[wave];
-  const char* src = PACK ? reinterpret_cast<const char*>(t.tensor) : image + t.image;
-  char* dst = PACK ? image + t.image : reinterpret_cast<char*>(t.tensor);
-  uint32_t n = t.n;
+// Workgroup b serves tile (b & mask) of span (b >> shift).  Tile boundaries inside a span sit at 16-byte
+// boundaries of the destination: tile 0 is [0, head + T), tile j is [head + j*T, head + (j+1)*T), the last one
+// is cut at the span's end, where head = bytes from the span's first destination byte to the next boundary.
+// Threads interleave at 16-byte granularity, so a wavefront moves 1 KiB of consecutive bytes per access.
+template <bool PACK, int U>
+__global__ void __launch_bounds__(1024) mlf_flat_kernel(const Span* __restrict__ spans, uint32_t shift,
+                                                        uint32_t tile_bytes, char* __restrict__ image) {
+  const Span sp = spans[blockIdx.x >> shift];
+  const uint32_t sub = blockIdx.x & ((1u << shift) - 1u);
+  const char* src0 = PACK ? reinterpret_cast<const char*>(sp.tensor) : image + sp.image;
+  char* dst0 = PACK ? image + sp.image : reinterpret_cast<char*>(sp.tensor);
+  uint32_t head0 = (16u - (uint32_t)(reinterpret_cast<uintptr_t>(dst0) & 15u)) & 15u;
+  head0 = head0 < sp.n ? head0 : sp.n;
+  const uint32_t start = sub ? head0 + sub * tile_bytes : 0u;
+  if (start >= sp.n) return;  // unused slot of a partly filled span
+  uint32_t end = head0 + (sub + 1u) * tile_bytes;
+  end = end < sp.n ? end : sp.n;
 
-  // bytes up to the first 16-byte boundary of the destination
-  uint32_t head = (16u - (uint32_t)(reinterpret_cast<uintptr_t>(dst) & 15u)) & 15u;
-  head = head < n ? head : n;
-  if (lane < head) dst[lane] = src[lane];
+  const char* src = src0 + start;
+  char* dst = dst0 + start;
+  uint32_t n = end - start;
+  const uint32_t tid = threadIdx.x;
+  const uint32_t bd = blockDim.x;
+  const uint32_t head = sub ? 0u : head0;  // only a span's first tile starts off a boundary
+  if (tid < head) dst[tid] = src[tid];
   src += head;
   dst += head;
   n -= head;
 
   const uint32_t nvec = n >> 4;
   u32x4* __restrict__ d = reinterpret_cast<u32x4*>(dst);
-  uint32_t i = lane;
-  for (; i + (kUnroll - 1) * kWave < nvec; i += kUnroll * kWave) {
-    u32x4 v[kUnroll];
+  uint32_t i = tid;
+  if (U > 1) {
+    for (; i + (U - 1) * bd < nvec; i += U * bd) {
+      u32x4 v[U];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
-      v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_u*>(src + (size_t)(i + u * kWave) * 16));
+      for (int u = 0; u < U; ++u)
+        v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_u*>(src + (size_t)(i + u * bd) * 16));
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) __builtin_nontemporal_store(v[u], &d[i + u * kWave]);
+      for (int u = 0; u < U; ++u) __builtin_nontemporal_store(v[u], &d[i + u * bd]);
+    }
   }
-  for (; i < nvec; i += kWave) {
+  for (; i < nvec; i += bd) {
     u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_u*>(src + (size_t)i * 16));
     __builtin_nontemporal_store(v, &d[i]);
   }
   const uint32_t tail = n & 15u;
-  if (lane < tail) {
-    const uint32_t o = (nvec << 4) + lane;
+  if (tid < tail) {
+    const uint32_t o = (nvec << 4) + tid;
     dst[o] = src[o];
   }
 }
@@ -384,30 +397,54 @@ void pool_memcpy(WorkerPool& pool, char* dst, const char* src, size_t n) {
 // ---------------------------------------------------------------------------------------------------------
 // plan
 // ---------------------------------------------------------------------------------------------------------
+constexpr int kSpanClasses = 3;
+constexpr uint32_t kSpanShift[kSpanClasses] = {7, 4, 0};  // 128, 16 or 1 tiles per table entry
+
 struct mlf_plan {
   int device = 0;
-  FlatTile* d_tiles = nullptr;
+  Span* d_spans[kSpanClasses] = {nullptr, nullptr, nullptr};
+  uint64_t n_spans[kSpanClasses] = {0, 0, 0};
+  uint32_t tile_bytes = 4096;
   StridedDesc* d_descs = nullptr;
   StridedWork* d_work = nullptr;
   char* d_blob = nullptr;
   uint32_t block_threads = 256;
+  uint32_t unroll = 1;
   mlf_plan_info info{};
 };
 
 namespace {
 
-constexpr uint32_t kDefaultTileBytes = 64 * 1024;
+constexpr uint32_t kDefaultTileBytes = 4096;
 constexpr uint32_t kStridedElemsPerBlock = 32 * 1024;
 
-// Cuts [0, n) of one contiguous item into tiles whose destination starts are 16-byte aligned (except the first).
-void cut_tiles(std::vector<FlatTile>& out, uint64_t tensor_addr, uint64_t image_off, uint64_t n, uint32_t tile,
+struct SpanTables {
+  std::vector<Span> cls[kSpanClasses];
+};
+
+// Covers [0, n) of one contiguous item with spans: as many 128-tile entries as fit, then 16-tile entries, then
+// single tiles.  Every entry is self-contained (the kernel derives tile cuts from the entry's own first
+// destination address), so pieces may start anywhere.
+void cut_spans(SpanTables& out, uint64_t tensor_addr, uint64_t image_off, uint64_t n, uint32_t tile,
                bool align_to_tensor) {
-  const uint64_t dst_addr = align_to_tensor ? tensor_addr : image_off;  // image base is 256-byte aligned
-  const uint64_t head = (16 - (dst_addr & 15)) & 15;
   uint64_t done = 0;
   while (done < n) {
-    uint64_t len = std::min<uint64_t>(n - done, done == 0 ? tile + head : tile);
-    out.push_back(FlatTile{tensor_addr + done, image_off + done, (uint32_t)len, 0});
+    const uint64_t dst_addr = (align_to_tensor ? tensor_addr : image_off) + done;  // image base is 256-byte aligned
+    const uint64_t head = (16 - (dst_addr & 15)) & 15;
+    const uint64_t left = n - done;
+    int c = kSpanClasses - 1;
+    for (int k = 0; k < kSpanClasses; ++k) {
+      if (left >= ((uint64_t)tile << kSpanShift[k])) {
+        c = k;
+        break;
+      }
+    }
+    // a full entry of class c holds (tile << shift) bytes; the single-tile class also takes the short rest,
+    // and its first tile may carry the head bytes on top
+    uint64_t len = (uint64_t)tile << kSpanShift[c];
+    if (c == kSpanClasses - 1) len = std::min<uint64_t>(left, tile + head);
+    len = std::min(len, left);
+    out.cls[c].push_back(Span{tensor_addr + done, image_off + done, (uint32_t)len, 0});
     done += len;
   }
 }
@@ -481,19 +518,23 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
   uint32_t tile = opts && opts->tile_bytes ? opts->tile_bytes : kDefaultTileBytes;
   uint32_t threads = opts && opts->block_threads ? opts->block_threads : 256;
   const bool align_to_tensor = opts && opts->align_to_tensor;
-  if (tile % 1024 || tile > (64u << 20)) return fail(MLF_HIP_BAD_ARG, "tile_bytes must be a multiple of 1024, at most 64 MiB");
+  if (tile % 1024 || tile > (1u << 20)) return fail(MLF_HIP_BAD_ARG, "tile_bytes must be a multiple of 1024, at most 1 MiB");
   if (threads % 64 || threads > 1024) return fail(MLF_HIP_BAD_ARG, "block_threads must be a multiple of 64, at most 1024");
 
   std::unique_ptr<mlf_plan> plan(new mlf_plan());
   HIP_TRY(hipGetDevice(&plan->device));
   plan->block_threads = threads;
+  plan->tile_bytes = tile;
+  plan->unroll = opts && opts->unroll ? opts->unroll : 1;
+  if (plan->unroll != 1 && plan->unroll != 2 && plan->unroll != 4 && plan->unroll != 8)
+    return fail(MLF_HIP_BAD_ARG, "unroll must be 1, 2, 4 or 8");
   if (blob_bytes) {
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&plan->d_blob), blob_bytes));
     HIP_TRY(hipMemcpy(plan->d_blob, host_blob, blob_bytes, hipMemcpyHostToDevice));
   }
   const uint64_t blob_base = reinterpret_cast<uint64_t>(plan->d_blob);
 
-  std::vector<FlatTile> tiles;
+  SpanTables tiles;
   std::vector<StridedDesc> descs;
   std::vector<StridedWork> work;
   mlf_plan_info& info = plan->info;
@@ -512,7 +553,7 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
         rc = fail(MLF_HIP_BAD_ARG, "blob item " + std::to_string(k) + " lies outside the host blob");
         break;
       }
-      cut_tiles(tiles, blob_base + it.ptr, it.image_off, it.nbytes, tile, false);
+      cut_spans(tiles, blob_base + it.ptr, it.image_off, it.nbytes, tile, false);
       info.blob_bytes += it.nbytes;
       continue;
     }
@@ -552,7 +593,7 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
     info.device_bytes += it.nbytes;
     const Collapsed c = collapse_dims(it);
     if (c.ndim == 0 || (c.ndim == 1 && c.ts[0] == 1 && c.is[0] == 1)) {
-      cut_tiles(tiles, it.ptr, it.image_off, it.nbytes, tile, align_to_tensor);
+      cut_spans(tiles, it.ptr, it.image_off, it.nbytes, tile, align_to_tensor);
       continue;
     }
     // rows that are contiguous on both sides and long enough go through the flat kernel, one row at a time
@@ -567,7 +608,7 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
           toff += idx[d] * c.ts[d];
           ioff += idx[d] * c.is[d];
         }
-        cut_tiles(tiles, it.ptr + (uint64_t)(toff * (int64_t)esz), it.image_off + (uint64_t)(ioff * (int64_t)esz),
+        cut_spans(tiles, it.ptr + (uint64_t)(toff * (int64_t)esz), it.image_off + (uint64_t)(ioff * (int64_t)esz),
                   row_bytes, tile, align_to_tensor);
         for (int d = last - 1; d >= 0; --d) {
           if (++idx[d] < c.shape[d]) break;
@@ -592,8 +633,10 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
       work.push_back(StridedWork{s, (uint32_t)std::min<uint64_t>(kStridedElemsPerBlock, numel - s), desc_idx});
     ++info.n_strided_items;
   }
-  if (rc == MLF_HIP_OK && tiles.size() > 0xFFFFFFF0ull) rc = fail(MLF_HIP_BAD_ARG, "too many tiles: raise tile_bytes");
-  if (rc == MLF_HIP_OK) rc = upload(tiles, &plan->d_tiles);
+  for (int c = 0; c < kSpanClasses && rc == MLF_HIP_OK; ++c) {
+    if (rc == MLF_HIP_OK) rc = upload(tiles.cls[c], &plan->d_spans[c]);
+    plan->n_spans[c] = tiles.cls[c].size();
+  }
   if (rc == MLF_HIP_OK) rc = upload(descs, &plan->d_descs);
   if (rc == MLF_HIP_OK) rc = upload(work, &plan->d_work);
   if (rc != MLF_HIP_OK) {
@@ -602,17 +645,20 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
     g_err = keep;
     return rc;
   }
-  info.n_flat_tiles = tiles.size();
+  info.n_flat_tiles = 0;
+  info.table_bytes = descs.size() * sizeof(StridedDesc) + work.size() * sizeof(StridedWork) + blob_bytes;
+  for (int c = 0; c < kSpanClasses; ++c) {
+    info.n_flat_tiles += plan->n_spans[c] << kSpanShift[c];
+    info.table_bytes += plan->n_spans[c] * sizeof(Span);
+  }
   info.n_strided_work = work.size();
-  info.table_bytes = tiles.size() * sizeof(FlatTile) + descs.size() * sizeof(StridedDesc) +
-                     work.size() * sizeof(StridedWork) + blob_bytes;
   *out = plan.release();
   return MLF_HIP_OK;
 }
 
 int mlf_plan_destroy(mlf_plan* plan) {
   if (!plan) return MLF_HIP_OK;
-  (void)hipFree(plan->d_tiles);
+  for (Span* t : plan->d_spans) (void)hipFree(t);
   (void)hipFree(plan->d_descs);
   (void)hipFree(plan->d_work);
   (void)hipFree(plan->d_blob);
@@ -635,17 +681,28 @@ int launch_plan(const mlf_plan* plan, char* image, hipStream_t stream) {
   if (!plan) return fail(MLF_HIP_BAD_ARG, "null plan");
   if (!image && plan->info.image_bytes) return fail(MLF_HIP_BAD_ARG, "null image");
   if (reinterpret_cast<uintptr_t>(image) & 255) return fail(MLF_HIP_BAD_ARG, "image must be 256-byte aligned");
-  const uint32_t n_tiles = (uint32_t)plan->info.n_flat_tiles;
-  if (n_tiles) {
-    const uint32_t waves = plan->block_threads / 64;
-    const uint32_t grid = (n_tiles + waves - 1) / waves;
-    hipLaunchKernelGGL((mlf_flat_kernel<PACK>), dim3(grid), dim3(plan->block_threads), 0, stream, plan->d_tiles,
-                       n_tiles, image);
-    HIP_TRY(hipGetLastError());
+  // a launch may not exceed 2^32 - 1 threads in total, so large tables go out in several launches
+  const uint64_t max_blocks = 0xFFFFFFFFull / plan->block_threads;
+  for (int c = 0; c < kSpanClasses; ++c) {
+    const uint32_t shift = kSpanShift[c], tile = plan->tile_bytes;
+    const uint64_t per_launch = std::max<uint64_t>(1, max_blocks >> shift);
+    for (uint64_t first = 0; first < plan->n_spans[c]; first += per_launch) {
+      const uint64_t count = std::min(per_launch, plan->n_spans[c] - first);
+      const dim3 grid((uint32_t)(count << shift)), block(plan->block_threads);
+      const Span* table = plan->d_spans[c] + first;
+      switch (plan->unroll) {
+        case 2: hipLaunchKernelGGL((mlf_flat_kernel<PACK, 2>), grid, block, 0, stream, table, shift, tile, image); break;
+        case 4: hipLaunchKernelGGL((mlf_flat_kernel<PACK, 4>), grid, block, 0, stream, table, shift, tile, image); break;
+        case 8: hipLaunchKernelGGL((mlf_flat_kernel<PACK, 8>), grid, block, 0, stream, table, shift, tile, image); break;
+        default: hipLaunchKernelGGL((mlf_flat_kernel<PACK, 1>), grid, block, 0, stream, table, shift, tile, image); break;
+      }
+      HIP_TRY(hipGetLastError());
+    }
   }
-  if (plan->info.n_strided_work) {
-    hipLaunchKernelGGL((mlf_strided_kernel<PACK>), dim3((uint32_t)plan->info.n_strided_work), dim3(256), 0, stream,
-                       plan->d_descs, plan->d_work, image);
+  for (uint64_t first = 0; first < plan->info.n_strided_work; first += (1u << 23)) {
+    const uint64_t count = std::min<uint64_t>(1u << 23, plan->info.n_strided_work - first);
+    hipLaunchKernelGGL((mlf_strided_kernel<PACK>), dim3((uint32_t)count), dim3(256), 0, stream, plan->d_descs,
+                       plan->d_work + first, image);
     HIP_TRY(hipGetLastError());
   }
   return MLF_HIP_OK;

@@ -211,6 +211,17 @@ class BufferIO:
             raise ValueError(f"Format signature must be at most 8 bytes, got {len(signature)}")
         self._metadata.format_signature = signature
 
+    @property
+    def len_written_data(self) -> int:
+        """High-water mark of the data section, in bytes."""
+        self._check_validity()
+        return self._metadata.len_written_data
+
+    def raw_view(self) -> memoryview:
+        """The whole mapping, metadata block included (no copy).  Valid until close() or resize()."""
+        self._check_validity()
+        return self._mv
+
     def data_address(self, pos: int = 0) -> int:
         """Raw address of data-section byte ``pos`` (for native copy engines that write around the stream)."""
         self._check_validity()

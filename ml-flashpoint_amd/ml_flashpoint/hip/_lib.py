@@ -37,7 +37,7 @@ class PlanOpts(ctypes.Structure):
         ("tile_bytes", ctypes.c_uint32),
         ("block_threads", ctypes.c_uint32),
         ("align_to_tensor", ctypes.c_uint32),
-        ("reserved", ctypes.c_uint32),
+        ("unroll", ctypes.c_uint32),
     ]
 
 

@@ -1,0 +1,305 @@
+"""gfx950 implementation of the loader plug-in interface.
+
+The reference reads item by item: ``read()`` copies the record out of the mapping, ``torch.frombuffer`` wraps it,
+``narrow_tensor_by_index`` selects the requested box and ``target.copy_()`` moves it (pageable H2D when the target
+is on the GPU); src/ml_flashpoint/core/checkpoint_loader.py:177-219,300-336.  Here, per object:
+
+1. record headers are parsed straight from the mapping (a few hundred bytes per item, no payload copy),
+2. the byte range that covers all requested payloads is streamed into HBM through pinned slots,
+3. one batched scatter kernel writes every requested box into its target tensor, whatever the target's strides.
+
+Items whose target lives on the host, byte-blob items, and objects in the legacy ``torch.save`` format are served
+on the host, the way the reference serves them.
+"""
+
+import io
+import logging
+import os
+import pickle
+import struct
+import time
+from pathlib import Path
+from typing import IO, Callable, List, Optional, cast
+
+import torch
+from torch.distributed._shard._utils import narrow_tensor_by_index
+from torch.distributed.checkpoint import Metadata
+from torch.distributed.checkpoint.filesystem import _StorageInfo
+from torch.distributed.checkpoint.planner import LoadItemType, LoadPlanner, ReadItem
+from torch.distributed.checkpoint.utils import _create_file_view
+from typing_extensions import override
+
+from ml_flashpoint.checkpoint_object_manager.buffer_metadata import METADATA_SIZE
+from ml_flashpoint.checkpoint_object_manager.checkpoint_object_manager import CheckpointObjectManager
+from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId, CheckpointObjectId
+from ml_flashpoint.core.checkpoint_loader import MLFlashpointCheckpointLoader
+from ml_flashpoint.core.defaults import DIRTY_MARKER_SUFFIX, CheckpointFormat, default_metadata_object_name
+from ml_flashpoint.core.mlf_logging import get_logger
+from ml_flashpoint.core.utils import log_execution_time
+from ml_flashpoint.hip import _lib, integrity
+from ml_flashpoint.hip import plan as hip_plan
+from ml_flashpoint.hip.checkpoint_saver import EngineConfig
+
+_LOGGER = get_logger(__name__)
+
+_MAX_HEADER_LEN = 1024 * 1024  # a larger "length" means the record is not in the MLF_TENS format
+_UPLOAD_ALIGN = 4096
+
+
+class HipMLFlashpointCheckpointLoader(MLFlashpointCheckpointLoader):
+    def __init__(
+        self,
+        checkpoint_object_manager: CheckpointObjectManager,
+        replication_manager=None,
+        *,
+        global_rank_getter: Callable[[], int] = lambda: 0,
+        local_rank_getter: Callable[[], int] = lambda: 0,
+        broadcast_object_list_func: Optional[Callable[..., None]] = None,
+        all_gather_object_func: Optional[Callable[..., None]] = None,
+        world_size_getter: Callable[[], int] = lambda: 1,
+        engine_config: Optional[EngineConfig] = None,
+        tile_bytes: int = 0,
+        block_threads: int = 0,
+        verify_crc: bool = True,
+    ):
+        """Arguments as the reference's default loader (checkpoint_loader.py:126-158), plus the copy-engine and
+        kernel work-split knobs and ``verify_crc`` (check the CRC-32C sidecar of an object, when it has one)."""
+        _lib.load()
+        self._checkpoint_object_manager = checkpoint_object_manager
+        self._replication_manager = replication_manager
+        self._global_rank_getter = global_rank_getter
+        self._local_rank_getter = local_rank_getter
+        self._broadcast_object_list_func = broadcast_object_list_func
+        self._all_gather_object_func = all_gather_object_func
+        self._world_size_getter = world_size_getter
+        self._engine_config = engine_config or EngineConfig()
+        self._tile_bytes = tile_bytes
+        self._block_threads = block_threads
+        self._verify_crc = verify_crc
+        self._engine: Optional[hip_plan.CopyEngine] = None
+        self.last_load_stats: dict = {}
+        # set to True to bracket every unpack launch with timing events; see the saver's attribute of the same name
+        self.record_kernel_events = False
+        self.kernel_events: list = []
+
+    def _get_engine(self) -> hip_plan.CopyEngine:
+        if self._engine is None:
+            cfg = self._engine_config
+            self._engine = hip_plan.CopyEngine(cfg.slot_bytes, cfg.n_slots, cfg.copy_threads)
+        return self._engine
+
+    @override
+    @log_execution_time(logger=_LOGGER, name="read_metadata")
+    def read_metadata(
+        self,
+        checkpoint_id: CheckpointContainerId,
+        object_name: str = default_metadata_object_name(),
+    ) -> Metadata:
+        path = Path(checkpoint_id.data) / object_name
+        try:
+            with open(path, "rb") as f:
+                return pickle.load(f)
+        except Exception:
+            _LOGGER.exception("Error reading metadata from '%s'", path)
+            raise
+
+    # ---- host-side record access ----------------------------------------------------------------------
+    def read_tensor(self, buffer_slice: IO[bytes], req: ReadItem, use_optimized_loader: bool = False) -> torch.Tensor:
+        """Host read of one record into a CPU tensor, narrowed to the requested box.  Used for host-resident
+        targets and for objects in the legacy format (same steps as checkpoint_loader.py:177-219)."""
+        pos = buffer_slice.tell()
+        tensor: Optional[torch.Tensor] = None
+        if use_optimized_loader:
+            raw_len = buffer_slice.read(4)
+            if len(raw_len) == 4:
+                (header_len,) = struct.unpack("<I", raw_len)
+                if header_len < _MAX_HEADER_LEN:
+                    try:
+                        header = pickle.loads(buffer_slice.read(header_len))
+                        data = buffer_slice.read()
+                        tensor = torch.frombuffer(data, dtype=header.dtype).reshape(header.shape)
+                    except Exception:
+                        _LOGGER.exception("Failed to parse tensor header")
+                        raise
+        if tensor is None:
+            buffer_slice.seek(pos)
+            tensor = cast(torch.Tensor, torch.load(cast(IO[bytes], buffer_slice), map_location="cpu", weights_only=True))
+        return narrow_tensor_by_index(tensor, req.storage_offsets, req.lengths)
+
+    @staticmethod
+    def _parse_header(view: memoryview, offset: int, length: int):
+        """(dtype, shape, payload offset) of the record at data-section ``offset``; None if it is not MLF_TENS."""
+        base = METADATA_SIZE + offset
+        if length < 4:
+            return None
+        (header_len,) = struct.unpack_from("<I", view, base)
+        if header_len >= _MAX_HEADER_LEN or 4 + header_len > length:
+            return None
+        header = pickle.loads(view[base + 4 : base + 4 + header_len])
+        return header.dtype, header.shape, offset + 4 + header_len
+
+    # ---- read_data ------------------------------------------------------------------------------------
+    @override
+    @log_execution_time(logger=_LOGGER, name="read_data", level=logging.INFO)
+    def read_data(
+        self,
+        checkpoint_object_id: CheckpointObjectId,
+        read_items: List[ReadItem],
+        planner: LoadPlanner,
+        storage_data: dict[int, _StorageInfo],
+    ) -> None:
+        if not os.path.exists(checkpoint_object_id.data):
+            msg = f"Checkpoint object '{checkpoint_object_id.data}' does not exist on any node in the cluster"
+            _LOGGER.error(msg)
+            raise FileNotFoundError(msg)
+        t_start = time.perf_counter()
+        stats = {"h2d_s": 0.0, "h2d_bytes": 0, "device_payload_bytes": 0, "host_items": 0, "device_items": 0}
+        with self._checkpoint_object_manager.get_buffer(checkpoint_object_id) as stream:
+            optimized = stream.format_signature == CheckpointFormat.MLF_FORMAT
+            device_reqs = []  # (req, target, dtype, shape, payload_off)
+            for req in read_items:
+                item_md = storage_data[req.storage_index]
+                if req.type == LoadItemType.BYTE_IO:
+                    view = cast(IO[bytes], _create_file_view(stream, item_md.offset, item_md.length))
+                    data = io.BytesIO(view.read(item_md.length))
+                    data.seek(0)
+                    planner.load_bytes(req, data)
+                    continue
+                target = planner.resolve_tensor(req).detach()
+                parsed = self._parse_header(stream.raw_view(), item_md.offset, item_md.length) if optimized else None
+                if parsed is None or target.device.type == "cpu":
+                    view = cast(IO[bytes], _create_file_view(stream, item_md.offset, item_md.length))
+                    tensor = self.read_tensor(view, req, use_optimized_loader=optimized)
+                    assert target.size() == tensor.size(), (
+                        f"req {req.storage_index} mismatch sizes {target.size()} vs {tensor.size()}"
+                    )
+                    target.copy_(tensor)
+                    planner.commit_tensor(req, target)
+                    stats["host_items"] += 1
+                    continue
+                device_reqs.append((req, target) + parsed)
+            if device_reqs:
+                self._read_device_items(checkpoint_object_id, stream, device_reqs, planner, stats)
+        stats["read_s"] = time.perf_counter() - t_start
+        self.last_load_stats = stats
+
+    def _read_device_items(self, object_id, stream, device_reqs, planner, stats) -> None:
+        devices = {t.device for _, t, *_ in device_reqs}
+        if len(devices) != 1:
+            raise ValueError("all device targets of one checkpoint object must live on the same device")
+        device = devices.pop()
+        written = stream.len_written_data
+        sidecar = integrity.read_sidecar(object_id.data) if self._verify_crc else None
+
+        # box of the stored tensor each request wants, as offsets/strides over the stored C-contiguous payload
+        boxes = []
+        lo, hi = None, 0
+        for req, target, dtype, shape, payload_off in device_reqs:
+            esz = torch.empty((), dtype=dtype).element_size()
+            stored_strides = hip_plan._contiguous_strides(tuple(shape))
+            # a dimension is narrowed only where the requested length is smaller than the stored size
+            lengths = [l if l < s else s for l, s in zip(req.lengths, shape)]
+            offsets = [o if l < s else 0 for o, l, s in zip(req.storage_offsets, req.lengths, shape)]
+            lengths += list(shape[len(lengths):])
+            offsets += [0] * (len(shape) - len(offsets))
+            box_shape = torch.Size(lengths)
+            assert target.size() == box_shape, f"req {req.storage_index} mismatch sizes {target.size()} vs {box_shape}"
+            if target.dtype != dtype:
+                raise TypeError(f"req {req.storage_index}: stored dtype {dtype} differs from target dtype {target.dtype}")
+            numel = box_shape.numel()
+            nbytes_stored = torch.Size(shape).numel() * esz
+            if payload_off + nbytes_stored > written:
+                raise ValueError(f"req {req.storage_index}: record reaches past the written data of '{object_id.data}'")
+            if numel:
+                first = payload_off + sum(o * s for o, s in zip(offsets, stored_strides)) * esz
+                last = first + (sum((l - 1) * s for l, s in zip(lengths, stored_strides)) + 1) * esz
+                lo = first if lo is None else min(lo, first)
+                hi = max(hi, last)
+            boxes.append((target, esz, lengths, stored_strides, payload_off, offsets, numel))
+        if lo is None:
+            for req, target, *_ in device_reqs:
+                planner.commit_tensor(req, target)
+            return
+        if sidecar is not None:
+            lo, hi = 0, written  # checksums cover the whole data section
+        lo = lo // _UPLOAD_ALIGN * _UPLOAD_ALIGN
+        span = hi - lo
+
+        table = hip_plan.ItemTable()
+        for target, esz, lengths, stored_strides, payload_off, offsets, numel in boxes:
+            if not numel:
+                continue
+            first = payload_off + sum(o * s for o, s in zip(offsets, stored_strides)) * esz
+            shape, tstride, istride = tuple(lengths), tuple(target.stride()), tuple(stored_strides)
+            if len(shape) > _lib.MAX_DIMS:
+                if not (target.is_contiguous() and all(o == 0 for o in offsets) and istride == tuple(
+                        hip_plan._contiguous_strides(shape))):
+                    raise NotImplementedError(f"rank > {_lib.MAX_DIMS} targets must be contiguous full tensors")
+                shape, tstride, istride = (numel,), (1,), (1,)
+            table.add_device(target.data_ptr(), first - lo, esz, shape, tstride, image_stride=istride)
+            stats["device_payload_bytes"] += numel * esz
+        with torch.cuda.device(device):
+            _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
+            image = torch.empty(span, dtype=torch.uint8, device=device)
+            cur = torch.cuda.current_stream(device)
+            st = self._get_engine().h2d(stream.data_address(lo), image.data_ptr(), span, cur.cuda_stream)
+            stats["h2d_s"] += st.seconds
+            stats["h2d_bytes"] += span
+            if sidecar is not None:
+                chunk_bytes, data_bytes, want = sidecar
+                if data_bytes != written:
+                    raise integrity.ChecksumMismatchError(
+                        f"'{object_id.data}': sidecar covers {data_bytes} bytes, object holds {written}")
+                got = hip_plan.crc32c_device(image, written, chunk_bytes, cur.cuda_stream)
+                bad = [int(i) for i in (got != want).nonzero()[0]]
+                if bad:
+                    raise integrity.ChecksumMismatchError(
+                        f"'{object_id.data}': CRC-32C mismatch in chunk(s) {bad[:8]} of {len(want)} "
+                        f"(chunk size {chunk_bytes})")
+            plan = hip_plan.Plan(table.to_array(), b"", span, tile_bytes=self._tile_bytes,
+                                 block_threads=self._block_threads, align_to_tensor=True)
+            if self.record_kernel_events:
+                begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                begin.record(cur)
+                plan.unpack(image, cur.cuda_stream)
+                end.record(cur)
+                self.kernel_events.append((begin, end, stats["device_payload_bytes"]))
+            else:
+                plan.unpack(image, cur.cuda_stream)
+            cur.synchronize()  # targets are complete (and the image may be freed) when read_data returns
+            plan.destroy()
+        for req, target, *_ in device_reqs:
+            planner.commit_tensor(req, target)
+        stats["device_items"] += len(device_reqs)
+
+    # ---- discovery --------------------------------------------------------------------------------------
+    @override
+    def get_latest_complete_checkpoint(
+        self, checkpoint_base_container: CheckpointContainerId
+    ) -> Optional[CheckpointContainerId]:
+        """Single-node form of the reference's discovery (checkpoint_loader.py:507-577): the highest
+        ``step-N_ckpt`` directory under the base that has no ``*unfinished`` marker beside it.  Agreement across
+        nodes and retrieval of missing objects from peers belong to the replication layer, which this package
+        does not implement."""
+        base = checkpoint_base_container.data
+        if not os.path.isdir(base):
+            return None
+        names = os.listdir(base)
+        dirty_pattern = CheckpointContainerId.get_dirty_version_checkpoint_container_pattern()
+        dirty_steps = set()
+        for name in names:
+            m = dirty_pattern.match(name)
+            if m and name.endswith(DIRTY_MARKER_SUFFIX):
+                dirty_steps.add(int(m.group(1)))
+        best = None
+        for name in names:
+            step = CheckpointContainerId.parse_version_container_step(name)
+            if step is None or step in dirty_steps or not os.path.isdir(os.path.join(base, name)):
+                continue
+            if best is None or step > best:
+                best = step
+        if best is None:
+            return None
+        return CheckpointContainerId.create_child(
+            checkpoint_base_container, CheckpointContainerId.format_version_container(best)
+        )

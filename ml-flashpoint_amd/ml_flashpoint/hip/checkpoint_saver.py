@@ -1,0 +1,468 @@
+"""gfx950 implementation of the saver plug-in interface.
+
+Where the reference's default saver copies tensor by tensor (``Tensor.to("cpu")``, then header +
+``frombuffer().copy_()`` into the mapping; src/ml_flashpoint/core/checkpoint_saver.py:347-360,622-707,764-800),
+this saver
+
+1. lays the whole object out on the host (same record format, same offsets),
+2. packs every device tensor and every header into a byte-exact *image* of the object's data section in HBM with
+   one batched kernel launch (``prepare_write_data`` - the training stream is free again once that kernel ends),
+3. streams the image into the mapped buffer file through pinned slots (``write_data``),
+
+so the bytes on tmpfs are identical to the reference's while the blocking part shrinks to an HBM-to-HBM copy.
+Host-only duties (dirty marker, metadata file, finalize + removal of older steps) are kept as the reference has
+them (checkpoint_saver.py:340-343,533-619,709-762).
+"""
+
+import concurrent.futures
+import dataclasses
+import io
+import logging
+import os
+import pickle
+import subprocess
+import threading
+import time
+from typing import Callable, Optional, Union
+
+import torch
+from torch.distributed.checkpoint import metadata as torchdistmeta
+from torch.distributed.checkpoint.filesystem import _split_by_size_and_type, _StorageInfo
+from torch.distributed.checkpoint.planner import WriteItem, WriteItemType
+from torch.distributed.checkpoint.storage import WriteResult
+from typing_extensions import override
+
+from ml_flashpoint.checkpoint_object_manager.checkpoint_object_manager import CheckpointObjectManager
+from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId, CheckpointObjectId
+from ml_flashpoint.core.checkpoint_saver import (
+    _DEFAULT_OBJ_NAME_SUFFIX,
+    DEFAULT_INITIAL_BUFFER_SIZE_BYTES,
+    MLFlashpointCheckpointSaver,
+    ObjectWriteBucket,
+    WriteItemResolver,
+)
+from ml_flashpoint.core.defaults import DIRTY_MARKER_SUFFIX, CheckpointFormat, default_metadata_object_name
+from ml_flashpoint.core.mlf_logging import get_logger
+from ml_flashpoint.core.utils import log_execution_time
+from ml_flashpoint.hip import _lib, integrity
+from ml_flashpoint.hip import plan as hip_plan
+
+_LOGGER = get_logger(__name__)
+
+_STAGE_ALIGN = 64
+
+
+@dataclasses.dataclass
+class EngineConfig:
+    """Shape of the pinned ring between HBM and the buffer file."""
+
+    slot_bytes: int = 32 << 20
+    n_slots: int = 4
+    copy_threads: int = 8
+
+
+class StagedObject:
+    """Image of one checkpoint object in HBM, with the layout that produced it."""
+
+    def __init__(self, layout: hip_plan.SaveLayout, plan: Optional[hip_plan.Plan], image: Optional[torch.Tensor],
+                 device_index: int, stream: int, items: list):
+        self.layout = layout
+        self.plan = plan
+        self.image = image
+        self.device_index = device_index
+        self.stream = stream
+        self.items = items  # WriteItems in span order: tensors, then byte blobs
+        self.consumed = False
+
+
+class StagedTensorRef:
+    """Placeholder that replaces a tensor in ``ObjectWriteBucket.tensor_data`` once its bytes are in the image.
+
+    Generic staging code that calls ``tensor.to("cpu")`` on bucket entries gets the same object back: there is
+    nothing left to move, the bytes already sit in the packed image.
+    """
+
+    __slots__ = ("staged", "index", "dtype", "shape")
+    device = torch.device("cpu")
+    is_cuda = False
+
+    def __init__(self, staged: StagedObject, index: int, dtype: torch.dtype, shape: torch.Size):
+        self.staged, self.index, self.dtype, self.shape = staged, index, dtype, shape
+
+    def to(self, *args, **kwargs):
+        return self
+
+    def detach(self):
+        return self
+
+    def numel(self) -> int:
+        return self.shape.numel()
+
+    def element_size(self) -> int:
+        return torch.empty((), dtype=self.dtype).element_size()
+
+
+class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
+    def __init__(
+        self,
+        global_rank_getter: Callable[[], int],
+        local_rank_getter: Callable[[], int],
+        global_barrier_func: Callable[[], None],
+        ckpt_obj_manager: CheckpointObjectManager,
+        replication_manager=None,
+        initial_buffer_size_bytes: int = DEFAULT_INITIAL_BUFFER_SIZE_BYTES,
+        use_optimized_save: bool = True,
+        *,
+        engine_config: Optional[EngineConfig] = None,
+        tile_bytes: int = 0,
+        block_threads: int = 0,
+        crc_chunk_bytes: int = 0,
+    ):
+        """Same positional arguments as the reference's default saver (checkpoint_saver.py:290-321).
+
+        Keyword-only extras: ``engine_config`` (pinned ring), ``tile_bytes`` / ``block_threads`` (pack kernel work
+        split, 0 = library default), ``crc_chunk_bytes`` (> 0: compute a CRC-32C per chunk of every object on the
+        GPU and keep it beside the object).
+        """
+        if not use_optimized_save:
+            raise ValueError(
+                "use_optimized_save=False asks for torch.save records, which are produced on the CPU only; "
+                "the gfx950 saver writes the MLF_TENS format."
+            )
+        _lib.load()  # fail now, loudly, if the native library is not there
+        self._global_rank_getter = global_rank_getter
+        self._local_rank_getter = local_rank_getter
+        self._barrier_func = global_barrier_func
+        self._chkpt_obj_manager = ckpt_obj_manager
+        self._replication_manager = replication_manager
+        self._initial_buffer_size_bytes = initial_buffer_size_bytes
+        self._use_optimized_save = True
+        self._engine_config = engine_config or EngineConfig()
+        self._tile_bytes = tile_bytes
+        self._block_threads = block_threads
+        self._crc_chunk_bytes = crc_chunk_bytes
+        self._init_runtime_state()
+
+    def _init_runtime_state(self):
+        self._engine: Optional[hip_plan.CopyEngine] = None
+        self._engine_lock = threading.Lock()
+        self.last_save_stats: dict = {}
+        # set to True to bracket every pack launch with timing events on its stream; (start, end, payload bytes)
+        # tuples are appended to kernel_events for the caller to read after a synchronize
+        self.record_kernel_events = False
+        self.kernel_events: list = []
+
+    # ---- pickling: only configuration crosses a process boundary --------------------------------------
+    def __getstate__(self):
+        state = self.__dict__.copy()
+        for key in ("_replication_manager", "_engine", "_engine_lock", "last_save_stats", "kernel_events"):
+            state.pop(key, None)
+        return state
+
+    def __setstate__(self, state):
+        self.__dict__.update(state)
+        self._replication_manager = None
+        self._init_runtime_state()
+
+    def _get_engine(self) -> hip_plan.CopyEngine:
+        with self._engine_lock:
+            if self._engine is None:
+                cfg = self._engine_config
+                self._engine = hip_plan.CopyEngine(cfg.slot_bytes, cfg.n_slots, cfg.copy_threads)
+            return self._engine
+
+    # ---- dirty marker / directory ----------------------------------------------------------------------
+    @override
+    @log_execution_time(logger=_LOGGER, name="initialize_checkpoint")
+    def initialize_checkpoint(self, checkpoint_id: CheckpointContainerId) -> None:
+        self._create_dirty_checkpoint_marker(checkpoint_id)
+        os.makedirs(checkpoint_id.data, exist_ok=True)
+
+    def _get_dirty_marker_file_path(self, checkpoint_id: CheckpointContainerId) -> str:
+        if str(checkpoint_id) == "/":
+            raise ValueError("CheckpointContainerId cannot be the root path '/'")
+        return f"{str(checkpoint_id).rstrip('/')}__{self._local_rank_getter()}__{DIRTY_MARKER_SUFFIX}"
+
+    def _create_dirty_checkpoint_marker(self, checkpoint_id: CheckpointContainerId) -> None:
+        path = self._get_dirty_marker_file_path(checkpoint_id)
+        os.makedirs(os.path.dirname(path), exist_ok=True)
+        with open(path, "w"):
+            pass
+
+    def _remove_dirty_checkpoint_marker(self, checkpoint_id: CheckpointContainerId) -> None:
+        path = self._get_dirty_marker_file_path(checkpoint_id)
+        if not os.path.exists(path):
+            _LOGGER.warning("Dirty marker file path: '%s' does not exist, skipping removal.", path)
+            return
+        os.remove(path)
+
+    # ---- stage_data ---------------------------------------------------------------------------------
+    @override
+    @log_execution_time(logger=_LOGGER, name="stage_data", level=logging.INFO)
+    def stage_data(self, checkpoint_id: CheckpointContainerId, state_dict: dict, non_blocking: bool = True) -> dict:
+        """Host-resident copy of a flat state dict: one batched gather in HBM and one pinned-ring transfer into a
+        single host arena, instead of one pageable D2H copy per tensor.  Host tensors and non-tensors pass through.
+        Blocking either way (``non_blocking`` is accepted for interface compatibility)."""
+        device_entries = [(k, v) for k, v in state_dict.items() if isinstance(v, torch.Tensor) and v.device.type != "cpu"]
+        staged = dict(state_dict)
+        by_device: dict = {}
+        for k, v in device_entries:
+            by_device.setdefault(v.device, []).append((k, v))
+        for device, entries in by_device.items():
+            table = hip_plan.ItemTable()
+            offsets, pos = [], 0
+            for _, t in entries:
+                offsets.append(pos)
+                nbytes = t.numel() * t.element_size()
+                if nbytes:
+                    shape, stride = tuple(t.shape), tuple(t.stride())
+                    if len(shape) > _lib.MAX_DIMS and t.is_contiguous():
+                        shape, stride = (t.numel(),), (1,)
+                    table.add_device(t.data_ptr(), pos, t.element_size(), shape, stride)
+                pos = (pos + nbytes + _STAGE_ALIGN - 1) // _STAGE_ALIGN * _STAGE_ALIGN
+            arena = torch.empty(max(pos, 1), dtype=torch.uint8)
+            if pos:
+                with torch.cuda.device(device):
+                    _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
+                    plan = hip_plan.Plan(table.to_array(), b"", pos, tile_bytes=self._tile_bytes,
+                                         block_threads=self._block_threads)
+                    image = torch.empty(pos, dtype=torch.uint8, device=device)
+                    stream = torch.cuda.current_stream(device).cuda_stream
+                    plan.pack(image, stream)
+                    self._get_engine().d2h(image.data_ptr(), arena.data_ptr(), pos, stream)
+                    plan.destroy()
+            for (k, t), off in zip(entries, offsets):
+                n = t.numel()
+                if n == 0:
+                    staged[k] = torch.empty(t.shape, dtype=t.dtype)
+                else:
+                    staged[k] = arena[off : off + n * t.element_size()].view(t.dtype).reshape(t.shape)
+        return staged
+
+    # ---- prepare_write_data (+ the pack) ------------------------------------------------------------
+    @override
+    @log_execution_time(logger=_LOGGER, name="prepare_write_data")
+    def prepare_write_data(
+        self,
+        checkpoint_id: CheckpointContainerId,
+        write_items: list[WriteItem],
+        write_item_resolver: WriteItemResolver,
+        object_name_prefix: str,
+        bucket_count: int,
+    ) -> list[ObjectWriteBucket]:
+        """Groups the items exactly as the reference does (same bucketing routine, same object names) and, per
+        object, enqueues the pack of its image on the current stream.  The returned buckets carry
+        ``StagedTensorRef`` placeholders; ``write_data`` finds the image through them."""
+        t_start = time.perf_counter()
+        bucket_count = max(bucket_count, 1)
+        rank = self._global_rank_getter()
+        write_buckets: list[ObjectWriteBucket] = []
+        stats = {"plan_build_s": 0.0, "objects": 0, "device_payload_bytes": 0, "image_bytes": 0}
+        for bucket in _split_by_size_and_type(bucket_count, write_items):
+            if not bucket:
+                continue
+            bytes_data = [
+                (item, write_item_resolver.resolve_data(item)) for item in bucket if item.type == WriteItemType.BYTE_IO
+            ]
+            tensor_data = [
+                (item, write_item_resolver.resolve_data(item).detach()) for item in bucket if item.type != WriteItemType.BYTE_IO
+            ]
+            if not bytes_data and not tensor_data:
+                continue
+            object_name = f"{object_name_prefix}_{len(write_buckets)}_src{rank}{_DEFAULT_OBJ_NAME_SUFFIX}"
+            object_id = CheckpointObjectId.from_container(checkpoint_id, object_name)
+            staged = self._stage_object(tensor_data, bytes_data, stats)
+            refs = [
+                (item, StagedTensorRef(staged, i, t.dtype, t.shape)) for i, (item, t) in enumerate(tensor_data)
+            ]
+            write_buckets.append(
+                ObjectWriteBucket(object_id=object_id, object_name=object_name, bytesio_data=bytes_data, tensor_data=refs)
+            )
+        stats["prepare_s"] = time.perf_counter() - t_start
+        self.last_save_stats = stats
+        return write_buckets
+
+    def _stage_object(self, tensor_data, bytes_data, stats: dict) -> StagedObject:
+        blobs = []
+        for _, data in bytes_data:
+            data.seek(0)
+            blobs.append(data.read())
+        tensors = [t for _, t in tensor_data]
+        t0 = time.perf_counter()
+        layout = hip_plan.build_save_layout(tensors, blobs)
+        device = next((t.device for t in tensors if t.device.type != "cpu"), None)
+        if any(t.device != device for t in tensors if t.device.type != "cpu"):
+            raise ValueError("all device tensors of one checkpoint object must live on the same device")
+        if device is None:
+            device = torch.device("cuda", torch.cuda.current_device())
+        items = [item for item, _ in tensor_data] + [item for item, _ in bytes_data]
+        plan = image = None
+        stream = 0
+        if layout.image_bytes:
+            with torch.cuda.device(device):
+                _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
+                plan = hip_plan.Plan(layout.items, layout.blob, layout.image_bytes, tile_bytes=self._tile_bytes,
+                                     block_threads=self._block_threads)
+                image = torch.empty(layout.image_bytes, dtype=torch.uint8, device=device)
+                stream = torch.cuda.current_stream(device).cuda_stream
+                stats["plan_build_s"] += time.perf_counter() - t0
+                if self.record_kernel_events:
+                    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    begin.record()
+                    plan.pack(image, stream)
+                    end.record()
+                    self.kernel_events.append((begin, end, layout.device_payload_bytes))
+                else:
+                    plan.pack(image, stream)
+        stats["objects"] += 1
+        stats["device_payload_bytes"] += layout.device_payload_bytes
+        stats["image_bytes"] += layout.image_bytes
+        return StagedObject(layout, plan, image, device.index or 0, stream, items)
+
+    # ---- write_data -----------------------------------------------------------------------------
+    @override
+    @log_execution_time(logger=_LOGGER, name="write_data", level=logging.INFO)
+    def write_data(
+        self,
+        checkpoint_id: CheckpointContainerId,
+        write_buckets: list[ObjectWriteBucket],
+        replicate_after_write: bool,
+        thread_count: int = 1,
+    ) -> list[WriteResult]:
+        """Moves each bucket's image into its buffer object and returns the WriteResults.
+
+        Buckets are processed one after another on the calling thread: the transfer is link-bound and the copy
+        engine already spreads the host-side copy over its own threads, so ``thread_count`` adds nothing here.
+        Buckets that still hold plain tensors (not produced by ``prepare_write_data`` of this class) are packed
+        first."""
+        all_results: list[WriteResult] = []
+        errors: list[Exception] = []
+        xfer = {"d2h_s": 0.0, "d2h_wait_s": 0.0, "d2h_bytes": 0, "crc_s": 0.0}
+        for bucket in write_buckets:
+            try:
+                all_results.extend(self._write_bucket(bucket, replicate_after_write, xfer))
+            except Exception as e:  # collected, first one re-raised: same contract as the reference's workers
+                _LOGGER.exception("Error writing object '%s'", bucket.object_id)
+                errors.append(e)
+        self.last_save_stats = {**self.last_save_stats, **xfer}
+        if errors:
+            raise errors[0]
+        return all_results
+
+    def _staged_of(self, bucket: ObjectWriteBucket) -> StagedObject:
+        refs = [t for _, t in bucket.tensor_data]
+        if refs and all(isinstance(r, StagedTensorRef) for r in refs):
+            staged = refs[0].staged
+            if all(r.staged is staged for r in refs) and not staged.consumed:
+                return staged
+            raise ValueError(f"bucket for '{bucket.object_id}' refers to a staged image that was already written")
+        if any(isinstance(r, StagedTensorRef) for r in refs):
+            raise ValueError("bucket mixes staged placeholders and tensors")
+        return self._stage_object(bucket.tensor_data, bucket.bytesio_data, {"plan_build_s": 0.0, "objects": 0,
+                                                                            "device_payload_bytes": 0, "image_bytes": 0})
+
+    def _write_bucket(self, bucket: ObjectWriteBucket, replicate_after_write: bool, xfer: dict) -> list[WriteResult]:
+        staged = self._staged_of(bucket)
+        layout = staged.layout
+        nbytes = layout.image_bytes
+        crcs = None
+        with self._chkpt_obj_manager.acquire_buffer(
+            bucket.object_id, max(self._initial_buffer_size_bytes, nbytes, 1)
+        ) as writer:
+            writer.set_format_signature(CheckpointFormat.MLF_FORMAT)
+            if nbytes:
+                ensure = getattr(writer, "ensure_capacity", None)
+                if ensure is not None:
+                    ensure(nbytes)  # pooled buffers grow once, to the exact total
+                with torch.cuda.device(staged.device_index):
+                    _lib.check(_lib.load().mlf_hip_set_device(staged.device_index), "mlf_hip_set_device")
+                    if self._crc_chunk_bytes:
+                        t0 = time.perf_counter()
+                        crcs = hip_plan.crc32c_device(staged.image, nbytes, self._crc_chunk_bytes, staged.stream)
+                        xfer["crc_s"] += time.perf_counter() - t0
+                    start = writer.tell()
+                    writer.next_buffer_slice(nbytes).release()  # bounds check + position/high-water mark
+                    st = self._get_engine().d2h(staged.image.data_ptr(), writer.data_address(start), nbytes, staged.stream)
+                    xfer["d2h_s"] += st.seconds
+                    xfer["d2h_wait_s"] += st.wait_seconds
+                    xfer["d2h_bytes"] += nbytes
+        staged.consumed = True
+        staged.image = None
+        if staged.plan is not None:
+            staged.plan.destroy()
+        if crcs is not None:
+            integrity.write_sidecar(str(bucket.object_id), self._crc_chunk_bytes, nbytes, crcs)
+        results = [
+            WriteResult(
+                index=item.index,
+                size_in_bytes=length,
+                storage_data=_StorageInfo(relative_path=bucket.object_name, offset=offset, length=length),
+            )
+            for item, (offset, length) in zip(staged.items, layout.spans)
+        ]
+        if replicate_after_write and self._replication_manager is not None:
+            # without a replication manager (single node, or this package used on its own) there is no peer to
+            # send to; an explicit async_replicate_object() call still raises
+            self.async_replicate_object(bucket.object_id)
+        return results
+
+    # ---- replication hand-off, metadata, finalize (host logic kept as in the reference) -------------------
+    @log_execution_time(logger=_LOGGER, name="async_replicate_object")
+    def async_replicate_object(self, object_id: CheckpointObjectId) -> list[concurrent.futures.Future]:
+        if self._replication_manager is None:
+            raise RuntimeError("ReplicationManager is not available (None). Cannot replicate object.")
+        return self._replication_manager.async_replicate(self._chkpt_obj_manager.get_buffer(object_id))
+
+    @override
+    @log_execution_time(logger=_LOGGER, name="write_metadata")
+    def write_metadata(
+        self,
+        checkpoint_id: CheckpointContainerId,
+        metadata: torchdistmeta.Metadata,
+        md_object_name: str = default_metadata_object_name(),
+    ):
+        final_path = os.path.join(checkpoint_id.data, md_object_name)
+        tmp_path = final_path + ".tmp"
+        os.makedirs(os.path.dirname(final_path), exist_ok=True)
+        with open(tmp_path, "wb") as f:
+            pickle.dump(metadata, f)
+        os.rename(tmp_path, final_path)
+
+    @override
+    @log_execution_time(logger=_LOGGER, name="finalize_checkpoint")
+    def finalize_checkpoint(self, checkpoint_id: CheckpointContainerId) -> Union[subprocess.Popen, None]:
+        self._remove_dirty_checkpoint_marker(checkpoint_id)
+        self._barrier_func()
+        if self._local_rank_getter() == 0:
+            return self._remove_older_checkpoints(older_than=checkpoint_id)
+        return None
+
+    def _remove_older_checkpoints(self, older_than: CheckpointContainerId) -> Optional[subprocess.Popen]:
+        parent = os.path.dirname(older_than.data)
+        limit = CheckpointContainerId.parse_version_container_step(os.path.basename(older_than.data))
+        if limit is None:
+            _LOGGER.warning("Could not parse step from 'older_than' checkpoint container: '%s'. "
+                            "Skipping removal of older checkpoints.", older_than)
+            return None
+        doomed = []
+        for name in os.listdir(parent):
+            step = CheckpointContainerId.parse_version_container_step(name)
+            path = os.path.join(parent, name)
+            if step is not None and step < limit and os.path.isdir(path):
+                doomed.append(path)
+        if not doomed:
+            return None
+        try:
+            # detached `rm -rf`: does not hold the GIL and survives signals sent to the training job's group
+            return subprocess.Popen(["rm", "-rf"] + doomed, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL,
+                                    start_new_session=True)
+        except Exception as e:
+            _LOGGER.exception("Background deletion of old checkpoints failed: %s", e)
+            return None
+
+    def release_device_memory(self) -> None:
+        """Destroys the copy engine (pinned slots, streams); it is rebuilt on the next save."""
+        with self._engine_lock:
+            if self._engine is not None:
+                self._engine.destroy()
+                self._engine = None

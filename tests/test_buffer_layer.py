@@ -1,0 +1,322 @@
+"""Host buffer layer: native BufferObject, BufferIO, BufferPool, CheckpointObjectManager.
+
+Behaviours are the ones the reference's tests pin (tests/checkpoint_object_manager/test_buffer_io.py,
+test_checkpoint_object_manager.py, buffer_object/test_buffer_object_bindings.py, tests/core/test_buffer_pool.py),
+re-expressed against this package.
+"""
+
+import io
+import os
+import struct
+
+import pytest
+
+from ml_flashpoint.checkpoint_object_manager.buffer_io import BufferIO
+from ml_flashpoint.checkpoint_object_manager.buffer_metadata import METADATA_SIZE, BufferMetadataType
+from ml_flashpoint.checkpoint_object_manager.buffer_object.buffer_object_ext import BufferObject
+from ml_flashpoint.checkpoint_object_manager.checkpoint_object_manager import CheckpointObjectManager
+from ml_flashpoint.core.buffer_pool import BufferPool, BufferPoolConfig, PooledBufferIO
+from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId, CheckpointObjectId
+
+
+# ---- native object ------------------------------------------------------------------------------------------
+def test_create_properties_and_memoryview(tmp_path):
+    p = str(tmp_path / "sub" / "dir" / "buf")  # parents are created
+    bo = BufferObject(p, capacity=1024, overwrite=False)
+    assert bo.get_id() == p and bo.get_capacity() == 1024 and bo.closed is False and bo.is_readonly is False
+    mv = memoryview(bo)
+    assert mv.nbytes == 1024 and not mv.readonly and mv.format == "B" and mv.ndim == 1
+    assert bo.get_data_ptr() != 0
+    mv.release()
+    bo.close()
+    assert bo.closed and bo.get_capacity() == 0
+    with pytest.raises(RuntimeError, match="Buffer is closed"):
+        bo.get_data_ptr()
+
+
+def test_overwrite_flag_and_error_text(tmp_path):
+    p = str(tmp_path / "x")
+    BufferObject(p, capacity=32, overwrite=False).close()
+    with pytest.raises(RuntimeError, match="File already exists and overwrite is set to false"):
+        BufferObject(p, capacity=32, overwrite=False)
+    bo = BufferObject(p, capacity=64, overwrite=True)
+    assert bo.get_capacity() == 64
+    bo.close()
+    with pytest.raises(RuntimeError, match="requires a size greater than 0"):
+        BufferObject(str(tmp_path / "zero"), capacity=0, overwrite=True)
+
+
+def test_write_close_reopen_readonly(tmp_path):
+    p = str(tmp_path / "rw")
+    bo = BufferObject(p, capacity=128, overwrite=True)
+    mv = memoryview(bo)
+    mv[:20] = b"Hello, BufferObject!"
+    mv.release()
+    bo.close()
+    ro = BufferObject(p)
+    mv = memoryview(ro)
+    assert ro.get_capacity() == 128 and ro.is_readonly and mv.readonly and mv[:20].tobytes() == b"Hello, BufferObject!"
+    with pytest.raises(TypeError):
+        mv[0] = 65
+    with pytest.raises(RuntimeError, match="read-only"):
+        ro.resize(256)
+    mv.release()
+    ro.close(truncate_size=10)  # ignored for read-only mappings
+    assert os.path.getsize(p) == 128
+
+
+def test_open_errors(tmp_path):
+    with pytest.raises(RuntimeError, match="Path is a directory, not a file"):
+        BufferObject(str(tmp_path))
+    empty = tmp_path / "empty"
+    empty.write_bytes(b"")
+    with pytest.raises(RuntimeError, match="File cannot be empty"):
+        BufferObject(str(empty))
+    with pytest.raises(RuntimeError, match="No such file or directory"):
+        BufferObject(str(tmp_path / "missing"))
+
+
+def test_closed_object_buffer_error_and_idempotent_close(tmp_path):
+    bo = BufferObject(str(tmp_path / "c"), capacity=16, overwrite=True)
+    bo.close()
+    bo.close()
+    bo.close()
+    with pytest.raises(BufferError) as exc:
+        memoryview(bo)
+    assert isinstance(exc.value.__cause__, RuntimeError)
+    assert "Cannot create buffer view on a closed BufferObject" in str(exc.value.__cause__)
+    with pytest.raises(RuntimeError, match="closed buffer"):
+        bo.resize(32)
+
+
+def test_close_truncates_and_resize_keeps_contents(tmp_path):
+    p = str(tmp_path / "t")
+    bo = BufferObject(p, capacity=8192, overwrite=True)
+    mv = memoryview(bo)
+    mv[:4] = b"abcd"
+    mv.release()
+    bo.resize(16384)
+    assert bo.get_capacity() == 16384 and os.path.getsize(p) == 16384
+    assert memoryview(bo)[:4].tobytes() == b"abcd"
+    with pytest.raises(RuntimeError, match="resize buffer to 0"):
+        bo.resize(0)
+    bo.close(truncate_size=100)
+    assert os.path.getsize(p) == 100
+
+
+# ---- BufferIO -------------------------------------------------------------------------------------------------
+@pytest.fixture
+def rw(tmp_path):
+    stream = BufferIO(BufferObject(str(tmp_path / "io.bin"), METADATA_SIZE + 1024, True))
+    yield stream
+    stream.close()
+
+
+def test_data_lands_after_the_metadata_block(rw, tmp_path):
+    assert rw.write(b"payload!") == 8
+    raw = rw.raw_view()
+    assert raw[METADATA_SIZE : METADATA_SIZE + 8].tobytes() == b"payload!"
+    assert struct.unpack_from("<Q", raw, 0)[0] == 8
+    rw.set_format_signature(b"MLF_TENS")
+    assert raw[8:16].tobytes() == b"MLF_TENS" and rw.format_signature == b"MLF_TENS"
+    with pytest.raises(ValueError, match="at most 8 bytes"):
+        rw.set_format_signature(b"123456789")
+
+
+def test_high_water_mark_seek_and_read_clamping(rw):
+    rw.write(b"0123456789")
+    assert rw.tell() == 10 and rw.len_written_data == 10
+    rw.seek(2)
+    rw.write(b"AB")
+    assert rw.len_written_data == 10  # overwrite inside: mark unchanged
+    assert rw.seek(0) == 0 and rw.read() == b"01AB456789"
+    assert rw.read() == b"" and rw.read(5) == b""
+    assert rw.seek(-3, io.SEEK_END) == 7 and rw.read(100) == b"789"
+    assert rw.seek(1, io.SEEK_SET) == 1 and rw.seek(2, io.SEEK_CUR) == 3
+    rw.seek(50)
+    assert rw.read(4) == b""  # beyond the mark
+    with pytest.raises(ValueError, match="invalid whence"):
+        rw.seek(0, 9)
+    with pytest.raises(ValueError, match="Negative seek position"):
+        rw.seek(-1)
+    assert rw.write(b"") == 0
+
+
+def test_readinto(rw):
+    rw.write(b"abcdefgh")
+    rw.seek(2)
+    target = bytearray(4)
+    assert rw.readinto(target) == 4 and bytes(target) == b"cdef"
+    big = bytearray(10)
+    assert rw.readinto(big) == 2 and bytes(big[:2]) == b"gh"
+    assert rw.readinto(bytearray(3)) == 0 and rw.readinto(bytearray(0)) == 0
+    with pytest.raises(TypeError, match="writable bytes-like"):
+        rw.readinto(b"immutable")
+    with pytest.raises(TypeError):
+        rw.readinto(memoryview(b"ro"))
+
+
+def test_capacity_is_enforced(rw):
+    with pytest.raises(ValueError, match="exceeds buffer capacity"):
+        rw.write(b"x" * 1025)
+    rw.write(b"x" * 1000)
+    with pytest.raises(ValueError, match="exceeds buffer capacity"):
+        rw.next_buffer_slice(25)
+    with pytest.raises(ValueError, match="non-negative"):
+        rw.next_buffer_slice(-1)
+    view = rw.next_buffer_slice(24)
+    view[:] = b"y" * 24
+    view.release()
+    assert rw.tell() == 1024 and rw.len_written_data == 1024
+    assert rw.data_address(4) == rw.buffer_obj.get_data_ptr() + METADATA_SIZE + 4
+
+
+def test_close_truncates_file_to_written_size(tmp_path):
+    p = str(tmp_path / "trunc.bin")
+    stream = BufferIO(BufferObject(p, METADATA_SIZE + 4096, True))
+    stream.write(b"z" * 123)
+    stream.close()
+    assert os.path.getsize(p) == METADATA_SIZE + 123
+    assert stream.closed
+    stream.close()  # idempotent
+    with pytest.raises(ValueError, match="closed BufferIO"):
+        stream.tell()
+    keep = BufferIO(BufferObject(str(tmp_path / "keep.bin"), METADATA_SIZE + 4096, True))
+    keep.write(b"q")
+    keep.close(truncate=False)
+    assert os.path.getsize(str(tmp_path / "keep.bin")) == METADATA_SIZE + 4096
+
+
+def test_readonly_stream(tmp_path):
+    p = str(tmp_path / "ro.bin")
+    with BufferIO(BufferObject(p, METADATA_SIZE + 64, True)) as w:
+        w.set_format_signature(b"TORCH___")
+        w.write(b"readonly-data")
+    with BufferIO(BufferObject(p)) as r:
+        assert r.is_readonly and r.format_signature == b"TORCH___" and r.read() == b"readonly-data"
+        for op, args in (("write", (b"x",)), ("next_buffer_slice", (1,)), ("set_format_signature", (b"A",)), ("resize", (8192,))):
+            with pytest.raises(TypeError, match="not supported in read-only mode"):
+                getattr(r, op)(*args)
+    assert os.path.getsize(p) == METADATA_SIZE + 13  # a read-only close never truncates
+
+
+def test_resize_keeps_the_whole_metadata_block(tmp_path):
+    stream = BufferIO(BufferObject(str(tmp_path / "rs.bin"), METADATA_SIZE + 100, True))
+    stream.set_format_signature(b"MLF_TENS")
+    stream.write(b"k" * 100)
+    before = stream.raw_view()[:METADATA_SIZE].tobytes()
+    stream.resize(METADATA_SIZE + 100000)
+    assert stream.raw_view()[:METADATA_SIZE].tobytes() == before
+    stream.write(b"m" * 50000)  # the live metadata view follows the new mapping
+    assert stream.len_written_data == 50100
+    with pytest.raises(ValueError, match="at least 4096"):
+        stream.resize(100)
+    stream.close()
+
+
+def test_constructor_validation(tmp_path):
+    closed = BufferObject(str(tmp_path / "c.bin"), 8192, True)
+    closed.close()
+    with pytest.raises(ValueError, match="closed BufferObject"):
+        BufferIO(closed)
+    with pytest.raises(ValueError, match="at least 4096"):
+        BufferIO(BufferObject(str(tmp_path / "small.bin"), 100, True))
+    assert BufferMetadataType.len_written_data.offset == 0 and BufferMetadataType.format_signature.offset == 8
+
+
+# ---- pool -------------------------------------------------------------------------------------------------------
+def test_pool_preallocates_named_files_and_links(tmp_path):
+    pool = BufferPool(str(tmp_path / "pool"), rank=3, num_buffers=2, buffer_size=METADATA_SIZE + 1000)
+    names = sorted(os.listdir(tmp_path / "pool"))
+    assert names == ["buffer_3_0.dist", "buffer_3_1.dist"]
+    assert all(os.path.getsize(tmp_path / "pool" / n) == METADATA_SIZE + 1000 for n in names)
+    link = str(tmp_path / "obj_a.distcp")
+    buf = pool.acquire(link)
+    assert isinstance(buf, PooledBufferIO) and os.path.islink(link)
+    assert os.path.dirname(os.readlink(link)) == str(tmp_path / "pool")
+    buf.write(b"hello")
+    buf.close()
+    assert buf.closed and os.path.getsize(link) == METADATA_SIZE + 5  # truncated, mapping kept by the pool
+    pool.acquire(str(tmp_path / "obj_b.distcp"))
+    with pytest.raises(RuntimeError, match="BufferPool exhausted. All 2 buffers are in use."):
+        pool.acquire(str(tmp_path / "obj_c.distcp"))
+    os.remove(link)  # deleting the checkpoint object frees its buffer
+    again = pool.acquire(str(tmp_path / "obj_c.distcp"))
+    assert again.tell() == 0 and again.len_written_data == 0
+    pool.teardown()
+
+
+def test_pool_auto_resize_formula(tmp_path):
+    pool = BufferPool(str(tmp_path / "pool"), num_buffers=1, buffer_size=METADATA_SIZE + 100)
+    buf = pool.acquire(str(tmp_path / "o.distcp"))
+    buf.write(b"a" * 100)  # fits exactly: no growth
+    assert buf.buffer_obj.get_capacity() == METADATA_SIZE + 100
+    buf.write(b"b" * 10)
+    expected = int(max((METADATA_SIZE + 100) * 1.1, METADATA_SIZE + 100 + 10 + 1024 * 1024))
+    assert buf.buffer_obj.get_capacity() == expected
+    view = buf.next_buffer_slice(3 * 1024 * 1024)
+    view.release()
+    assert buf.buffer_obj.get_capacity() >= METADATA_SIZE + 110 + 3 * 1024 * 1024
+    buf.seek(0)
+    assert buf.read(105) == b"a" * 100 + b"b" * 5
+    buf.close()
+    pool.teardown()
+
+
+def test_pool_symlink_failure_returns_buffer(tmp_path):
+    pool = BufferPool(str(tmp_path / "pool"), num_buffers=1, buffer_size=METADATA_SIZE + 10)
+    with pytest.raises(OSError):
+        pool.acquire(str(tmp_path / "no_such_dir" / "o.distcp"))
+    assert len(pool.free_buffers) == 1 and not pool.active_buffers
+    pool.teardown()
+    with pytest.raises(ValueError):
+        BufferPool("", num_buffers=1, buffer_size=10)
+    with pytest.raises(ValueError):
+        BufferPool(str(tmp_path), num_buffers=0, buffer_size=10)
+    with pytest.raises(ValueError):
+        BufferPoolConfig(str(tmp_path), rank=-1, num_buffers=1, buffer_size=1)
+
+
+# ---- manager ----------------------------------------------------------------------------------------------------
+@pytest.fixture
+def no_pool():
+    CheckpointObjectManager._worker_pool = None
+    yield
+    CheckpointObjectManager().teardown_pool()
+
+
+def test_manager_acquire_adds_metadata_block_and_overwrites(tmp_path, no_pool):
+    mgr = CheckpointObjectManager()
+    oid = CheckpointObjectId(str(tmp_path / "step-1_ckpt" / "o.distcp"))
+    with mgr.acquire_buffer(oid, 1000) as w:
+        assert w.buffer_obj.get_capacity() == 1000 + METADATA_SIZE
+        w.write(b"first")
+    with pytest.raises(FileExistsError):
+        mgr.acquire_buffer(oid, 1000, overwrite=False)
+    with mgr.acquire_buffer(oid, 10) as w:  # default: overwrite
+        w.write(b"second")
+    with mgr.get_buffer(oid) as r:
+        assert r.read() == b"second"
+    with pytest.raises(ValueError, match="positive integer"):
+        mgr.acquire_buffer(oid, 0)
+    assert mgr.get_buffer(CheckpointObjectId(str(tmp_path / "absent"))) is None
+    assert mgr.get_buffer(CheckpointObjectId(str(tmp_path / "step-1_ckpt"))) is None  # a directory
+    mgr.delete_object(oid)
+    assert not os.path.exists(str(oid))
+    mgr.delete_container(CheckpointContainerId(str(tmp_path / "step-1_ckpt")))
+    assert not os.path.exists(str(tmp_path / "step-1_ckpt"))
+
+
+def test_manager_prefers_pool_then_falls_back(tmp_path, no_pool):
+    mgr = CheckpointObjectManager(BufferPoolConfig(str(tmp_path / "pool"), 0, 1, METADATA_SIZE + 64))
+    a = CheckpointObjectId(str(tmp_path / "ck" / "a.distcp"))
+    b = CheckpointObjectId(str(tmp_path / "ck" / "b.distcp"))
+    wa = mgr.acquire_buffer(a, 64)
+    assert isinstance(wa, PooledBufferIO) and os.path.islink(str(a))
+    wb = mgr.acquire_buffer(b, 64)  # pool exhausted: standalone file
+    assert isinstance(wb, BufferIO) and not os.path.islink(str(b))
+    wa.close()
+    wb.close()
+    mgr.close_buffer(wb)  # closing a closed buffer is ignored
+    # another manager in the same process shares the pool
+    assert CheckpointObjectManager()._get_or_create_buffer_pool() is CheckpointObjectManager._worker_pool

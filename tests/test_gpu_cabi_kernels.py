@@ -134,6 +134,32 @@ def test_pack_large_rows_go_through_flat_kernel():
     assert plan.info.n_strided_items == 0 and plan.info.n_flat_tiles >= 64
 
 
+def test_pack_and_unpack_tables_larger_than_one_launch():
+    """5 GiB through 1 KiB tiles of 1024 threads needs more than 2^32 threads: the work goes out in several
+    launches.  Checked on the device (payload region of the image == source; round trip restores the source)."""
+    from ml_flashpoint.hip import plan as P
+
+    n = 5 * (1 << 30) + 12345
+    src = torch.empty(n, dtype=torch.uint8, device=DEV)
+    src[: n // 8 * 8].view(torch.int64).random_()
+    src[n // 8 * 8 :] = 7
+    layout = P.build_save_layout([src])
+    hdr = layout.spans[0][1] - n
+    image = torch.zeros(layout.image_bytes + 256, dtype=torch.uint8, device=DEV)
+    plan = P.Plan(layout.items, layout.blob, layout.image_bytes, tile_bytes=1024, block_threads=1024)
+    assert plan.info.n_flat_tiles * 1024 > 1 << 32
+    plan.pack(image)
+    torch.cuda.synchronize()
+    assert torch.equal(image[hdr : hdr + n], src)
+    assert bytes(image[:hdr].cpu().numpy()) == oracle_fmt.header_bytes("uint8", (n,)) and int(image[hdr + n :].sum()) == 0
+    back = torch.zeros_like(src)
+    table = P.ItemTable()
+    table.add_device(back.data_ptr(), hdr, 1, (n,), (1,))
+    P.Plan(table.to_array(), b"", layout.image_bytes, tile_bytes=1024, block_threads=1024, align_to_tensor=True).unpack(image)
+    torch.cuda.synchronize()
+    assert torch.equal(back, src)
+
+
 def test_pack_host_resident_tensors_travel_in_blob():
     gen = torch.Generator().manual_seed(16)
     cpu = [_rand_tensor(gen, (33, 3), torch.float32), _rand_tensor(gen, (5000,), torch.int64).t(), _rand_tensor(gen, (), torch.int64)]

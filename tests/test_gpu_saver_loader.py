@@ -1,0 +1,398 @@
+"""GPU parity of the saver/loader plug-ins behind the DCP adapters: file bytes and restored tensors are compared
+with the CPU oracle on the same seeded state dicts (bit-exact)."""
+
+import concurrent.futures
+import io
+import os
+import pickle
+
+import pytest
+import torch
+import torch.distributed.checkpoint as dcp
+import torch.multiprocessing as torch_mp
+from torch.distributed.checkpoint.filesystem import _StorageInfo
+from torch.distributed.checkpoint.metadata import MetadataIndex
+from torch.distributed.checkpoint.planner import LoadItemType, ReadItem, WriteItemType
+
+import workloads
+from ml_flashpoint.adapter.pytorch.memory_storage_reader import MemoryStorageReader
+from ml_flashpoint.adapter.pytorch.memory_storage_writer import MemoryStorageWriter
+from ml_flashpoint.checkpoint_object_manager.buffer_metadata import METADATA_SIZE
+from ml_flashpoint.checkpoint_object_manager.checkpoint_object_manager import CheckpointObjectManager
+from ml_flashpoint.core.buffer_pool import BufferPoolConfig
+from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId, CheckpointObjectId
+from oracle import mlf_format as fmt
+from oracle.cpu_path import OracleCheckpointLoader, OracleCheckpointSaver
+
+pytestmark = [pytest.mark.gpu, pytest.mark.filterwarnings("ignore:torch.distributed is disabled")]
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def manager_future():
+    mgr = torch_mp.get_context("spawn").Manager()
+    fut = concurrent.futures.Future()
+    fut.set_result(mgr)
+    yield fut
+    mgr.shutdown()
+
+
+@pytest.fixture(autouse=True)
+def _fresh_pool():
+    CheckpointObjectManager._worker_pool = None
+    yield
+    CheckpointObjectManager().teardown_pool()
+
+
+def _saver(manager=None, **kw):
+    from ml_flashpoint.core.checkpoint_saver import DefaultMLFlashpointCheckpointSaver
+
+    return DefaultMLFlashpointCheckpointSaver(
+        global_rank_getter=lambda: 0,
+        local_rank_getter=lambda: 0,
+        global_barrier_func=lambda: None,
+        ckpt_obj_manager=manager or CheckpointObjectManager(),
+        replication_manager=None,
+        initial_buffer_size_bytes=kw.pop("initial_buffer_size_bytes", 1 << 20),
+        **kw,
+    )
+
+
+def _loader(**kw):
+    from ml_flashpoint.core.checkpoint_loader import DefaultMLFlashpointCheckpointLoader
+
+    return DefaultMLFlashpointCheckpointLoader(CheckpointObjectManager(), None, **kw)
+
+
+def _bits(t):
+    return t.detach().cpu().contiguous().reshape(-1).view(torch.uint8)
+
+
+def _expected_file(sd_cpu, metadata, raw):
+    """Oracle image for the item order the plan chose; byte blobs (pickled non-tensors) are taken as written."""
+    by_offset = sorted(metadata.storage_data.items(), key=lambda kv: kv[1].offset)
+    tensors = [sd_cpu[i.fqn] for i, _ in by_offset if isinstance(sd_cpu[i.fqn], torch.Tensor)]
+    blobs = [raw[METADATA_SIZE + s.offset : METADATA_SIZE + s.offset + s.length] for i, s in by_offset
+             if not isinstance(sd_cpu[i.fqn], torch.Tensor)]
+    image, spans = fmt.file_image(tensors, blobs)
+    return image, spans, [(s.offset, s.length) for _, s in by_offset]
+
+
+def _mixed_state_dict():
+    g = torch.Generator().manual_seed(99)
+    rb = lambda n: torch.randint(0, 256, (n,), dtype=torch.uint8, generator=g)  # noqa: E731
+    base = rb(64 * 96 * 2).view(torch.bfloat16).reshape(64, 96)
+    sd = {
+        "w.fp32": torch.randn(257, 33, generator=g) * 0.02,
+        "w.bf16": rb(1000 * 2).view(torch.bfloat16).reshape(10, 100),
+        "w.fp8": rb(4096).view(torch.float8_e4m3fn).reshape(64, 64),
+        "w.i64": torch.randint(-(2**62), 2**62, (513,), generator=g),
+        "w.scalar": torch.tensor(3.25),
+        "w.empty": torch.empty(0, 7),
+        "w.bool": torch.rand(40, generator=g) > 0.5,
+        "v.transposed": base.t(),
+        "v.cols": base[:, ::2],
+        "v.rows": base[16:48],
+        "obj.step": 123,
+        "obj.cfg": "lr=1e-3;name=x",
+    }
+    return sd
+
+
+def _to_dev(sd, keep_on_host=()):
+    out = {}
+    for k, v in sd.items():
+        if isinstance(v, torch.Tensor) and k not in keep_on_host:
+            if v.is_contiguous():
+                out[k] = v.to(DEV)
+            else:  # rebuild the same view over a device copy of the base
+                base = torch.empty(v.untyped_storage().size(), dtype=torch.uint8)
+                base.untyped_storage().copy_(v.untyped_storage())
+                dev_base = base.to(DEV)
+                out[k] = torch.as_strided(dev_base.view(v.dtype), v.shape, v.stride(), v.storage_offset())
+        else:
+            out[k] = v
+    return out
+
+
+def test_dcp_save_bytes_equal_oracle_and_load_is_bit_exact(shm_dir, manager_future):
+    sd_cpu = _mixed_state_dict()
+    sd_dev = _to_dev(sd_cpu, keep_on_host=("w.i64",))  # one host-resident tensor among device tensors
+    ckpt = os.path.join(shm_dir, "step-5_ckpt")
+    saver = _saver()
+    dcp.save(sd_dev, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(saver, manager_future), no_dist=True)
+    assert sorted(os.listdir(ckpt)) == [".metadata", "__0__0_src0.distcp"]
+    raw = open(os.path.join(ckpt, "__0__0_src0.distcp"), "rb").read()
+    metadata = pickle.load(open(os.path.join(ckpt, ".metadata"), "rb"))
+    image, spans, got_spans = _expected_file(sd_cpu, metadata, raw)
+    assert raw == image and got_spans == spans
+    assert saver.last_save_stats["d2h_bytes"] == len(raw) - METADATA_SIZE
+
+    # the oracle's CPU saver writes the very same file for the host copy of the state dict
+    ckpt2 = os.path.join(shm_dir, "oracle", "step-5_ckpt")
+    dcp.save(sd_cpu, checkpoint_id=ckpt2, storage_writer=MemoryStorageWriter(OracleCheckpointSaver(), manager_future), no_dist=True)
+    assert open(os.path.join(ckpt2, "__0__0_src0.distcp"), "rb").read() == raw
+
+    for src_ckpt in (ckpt, ckpt2):  # restore from our file and from the oracle's file
+        target = {}
+        for k, v in sd_dev.items():
+            if isinstance(v, torch.Tensor):
+                target[k] = torch.zeros(v.shape, dtype=torch.uint8 if v.dtype == torch.float8_e4m3fn else v.dtype, device=v.device)
+                if v.dtype == torch.float8_e4m3fn:
+                    target[k] = target[k].view(torch.float8_e4m3fn)
+            else:
+                target[k] = None
+        loader = _loader()
+        dcp.load(target, checkpoint_id=src_ckpt, storage_reader=MemoryStorageReader(src_ckpt, loader), no_dist=True)
+        assert target["obj.step"] == 123 and target["obj.cfg"] == "lr=1e-3;name=x"
+        for k, v in sd_cpu.items():
+            if isinstance(v, torch.Tensor):
+                assert torch.equal(_bits(target[k]), _bits(v)), k
+        assert loader.last_load_stats["device_items"] >= 8 and loader.last_load_stats["host_items"] == 1
+
+    # and the oracle's CPU loader restores our file
+    target = {k: (torch.zeros_like(v) if isinstance(v, torch.Tensor) else None) for k, v in sd_cpu.items()}
+    dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, OracleCheckpointLoader()), no_dist=True)
+    for k, v in sd_cpu.items():
+        if isinstance(v, torch.Tensor):
+            assert torch.equal(_bits(target[k]), _bits(v)), k
+
+
+def test_gpt2_small_config_on_device(shm_dir, manager_future):
+    """BASELINE config 1's state dict, resident on the GPU, saved by the gfx950 saver: same bytes as the oracle."""
+    sd_dev = workloads.gpt2_small(device=DEV, layers=3, d=256, vocab=5003, ctx=128)
+    sd_cpu = {k: v.cpu() for k, v in sd_dev.items()}
+    ckpt = os.path.join(shm_dir, "step-1_ckpt")
+    dcp.save(sd_dev, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(_saver(), manager_future), no_dist=True)
+    raw = open(os.path.join(ckpt, "__0__0_src0.distcp"), "rb").read()
+    metadata = pickle.load(open(os.path.join(ckpt, ".metadata"), "rb"))
+    image, spans, got_spans = _expected_file(sd_cpu, metadata, raw)
+    assert raw == image and got_spans == spans
+    target = {k: torch.zeros_like(v) for k, v in sd_dev.items()}
+    dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, _loader()), no_dist=True)
+    assert all(torch.equal(target[k].view(torch.int32), sd_dev[k].view(torch.int32)) for k in sd_dev)
+
+
+def test_megatron_style_sequence_with_pool_and_finalize(shm_dir, manager_future):
+    """initialize -> prepare buckets (pack) -> generic stage step -> write -> finish -> finalize, into pooled buffers,
+    twice (the second save reuses a pool buffer and removes the first step)."""
+    from torch.distributed.checkpoint import DefaultSavePlanner
+    from torch.distributed.checkpoint.default_planner import create_default_local_save_plan
+
+    pool_cfg = BufferPoolConfig(os.path.join(shm_dir, "pool"), 0, 2, METADATA_SIZE + 4096)
+    manager = CheckpointObjectManager(pool_cfg)
+    saver = _saver(manager)
+    sd_cpu = {k: v for k, v in _mixed_state_dict().items() if isinstance(v, torch.Tensor)}
+    sd_dev = _to_dev(sd_cpu)
+    for step in (10, 20):
+        cid = CheckpointContainerId(os.path.join(shm_dir, "run", f"step-{step}_ckpt"))
+        saver.initialize_checkpoint(cid)
+        marker = f"{cid}__0__unfinished"
+        assert os.path.exists(marker)
+        writer = MemoryStorageWriter(saver, manager_future)
+        writer.reset(cid.data)
+        planner = DefaultSavePlanner()
+        planner.set_up_planner(sd_dev, is_coordinator=True)
+        local = writer.prepare_local_plan(planner.create_local_plan())
+        plans, metadata = planner.create_global_plan([local])
+        plan = planner.finish_plan(writer.prepare_global_plan(plans)[0])
+        buckets = writer.prepare_write_data_buckets(cid, plan, planner)
+        staged = MemoryStorageWriter.stage_write_data_buckets(cid, buckets, non_blocking=True)
+        assert all(a is b for (_, a), (_, b) in zip(buckets[0].tensor_data, staged[0].tensor_data))
+        for t in sd_dev.values():  # training may overwrite the live tensors as soon as staging returned
+            if t.numel() and t.is_contiguous() and t.dtype not in (torch.bool, torch.float8_e4m3fn):
+                t.add_(1)
+        results = writer.write_staged_data_buckets(cid, staged, replicate_after_write=False).wait()
+        assert writer.get_write_results(cid) is not None
+        writer.finish_checkpoint(cid, metadata, [results])
+        proc = saver.finalize_checkpoint(cid)
+        assert not os.path.exists(marker)
+        if proc is not None:
+            proc.wait()
+        obj = os.path.join(cid.data, "__0__0_src0.distcp")
+        assert os.path.islink(obj)
+        raw = open(obj, "rb").read()
+        md = pickle.load(open(os.path.join(cid.data, ".metadata"), "rb"))
+        image, spans, got_spans = _expected_file(sd_cpu, md, raw)
+        assert raw == image and got_spans == spans  # the bytes are those of the moment prepare returned
+        sd_cpu = {k: v.cpu() for k, v in sd_dev.items()}  # what the next save must capture
+    assert not os.path.exists(os.path.join(shm_dir, "run", "step-10_ckpt"))
+    assert _loader().get_latest_complete_checkpoint(CheckpointContainerId(os.path.join(shm_dir, "run"))).data.endswith("step-20_ckpt")
+
+
+def test_crc_sidecar_written_and_corruption_detected(shm_dir, manager_future):
+    from ml_flashpoint.hip import integrity
+
+    sd = {"a": torch.randn(300_000, device=DEV), "b": torch.randn(7, 9, device=DEV).to(torch.bfloat16)}
+    ckpt = os.path.join(shm_dir, "step-2_ckpt")
+    dcp.save(sd, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(_saver(crc_chunk_bytes=1 << 18), manager_future), no_dist=True)
+    obj = os.path.join(ckpt, "__0__0_src0.distcp")
+    chunk, nbytes, crcs = integrity.read_sidecar(obj)
+    raw = open(obj, "rb").read()
+    assert chunk == 1 << 18 and nbytes == len(raw) - METADATA_SIZE and len(crcs) == -(-nbytes // chunk)
+    import ctypes
+
+    from ml_flashpoint.hip import plan as P
+
+    for k, c in enumerate(crcs):  # the GPU's values are the CRCs of the bytes that landed in the file
+        piece = raw[METADATA_SIZE + k * chunk : METADATA_SIZE + (k + 1) * chunk]
+        buf = ctypes.create_string_buffer(piece, len(piece))
+        assert P.crc32c_host(ctypes.addressof(buf), len(piece)) == int(c)
+    target = {k: torch.zeros_like(v) for k, v in sd.items()}
+    dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, _loader()), no_dist=True)
+    assert all(torch.equal(target[k], sd[k]) for k in sd)
+    with open(obj, "r+b") as f:  # flip one payload bit in the third chunk
+        f.seek(METADATA_SIZE + 2 * chunk + 1000)
+        byte = f.read(1)
+        f.seek(-1, os.SEEK_CUR)
+        f.write(bytes([byte[0] ^ 0x10]))
+    with pytest.raises(BaseException) as exc:
+        dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, _loader()), no_dist=True)
+    cause = exc.value.failures[0][0] if hasattr(exc.value, "failures") else exc.value
+    assert isinstance(cause, integrity.ChecksumMismatchError) and "chunk(s) [2]" in str(cause)
+    dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, _loader(verify_crc=False)), no_dist=True)
+
+
+def test_stage_data_returns_host_copies(shm_dir):
+    sd_cpu = _mixed_state_dict()
+    sd_dev = _to_dev(sd_cpu, keep_on_host=("w.i64",))
+    staged = _saver().stage_data(CheckpointContainerId(os.path.join(shm_dir, "step-1_ckpt")), sd_dev)
+    assert list(staged) == list(sd_dev)
+    for k, v in sd_cpu.items():
+        if isinstance(v, torch.Tensor):
+            assert staged[k].device.type == "cpu" and staged[k].shape == v.shape and staged[k].dtype == v.dtype
+            assert torch.equal(_bits(staged[k]), _bits(v)), k
+        else:
+            assert staged[k] == v
+    assert staged["w.i64"] is sd_dev["w.i64"]
+
+
+class _Resolver:
+    def __init__(self, data):
+        self.data = data
+
+    def resolve_data(self, item):
+        return self.data[item.index.fqn]
+
+
+class _Planner:
+    """Minimal LoadPlanner stand-in: hands out targets by fqn and records commits / loaded bytes."""
+
+    def __init__(self, targets):
+        self.targets, self.committed, self.loaded = targets, [], {}
+
+    def resolve_tensor(self, req):
+        return self.targets[req.dest_index.fqn]
+
+    def commit_tensor(self, req, tensor):
+        self.committed.append(req.dest_index.fqn)
+
+    def load_bytes(self, req, value):
+        self.loaded[req.dest_index.fqn] = value.read()
+
+
+def _write_direct(shm_dir, data, bucket_count=1):
+    saver = _saver()
+    cid = CheckpointContainerId(os.path.join(shm_dir, "step-7_ckpt"))
+    from torch.distributed.checkpoint.planner_helpers import _create_write_items
+
+    items = [wi for k, v in data.items() for wi in _create_write_items(k, v)]
+    assert all((wi.type == WriteItemType.BYTE_IO) == isinstance(data[wi.index.fqn], io.BytesIO) for wi in items)
+    buckets = saver.prepare_write_data(cid, items, _Resolver(data), "data", bucket_count)
+    results = saver.write_data(cid, buckets, replicate_after_write=False, thread_count=bucket_count)
+    return cid, buckets, {r.index.fqn: r.storage_data for r in results}
+
+
+def test_direct_saver_calls_offsets_names_and_sub_box_reads(shm_dir):
+    g = torch.Generator().manual_seed(5)
+    stored = torch.randn(12, 20, 10, generator=g)
+    data = {"t3": stored.to(DEV), "blob": io.BytesIO(b"some-bytes"), "t1": torch.arange(20, dtype=torch.float32, device=DEV)}
+    cid, buckets, info = _write_direct(shm_dir, data)
+    assert [b.object_name for b in buckets] == ["data_0_src0.distcp"]
+    hdr3 = len(fmt.header_bytes("float32", (12, 20, 10)))
+    hdr1 = len(fmt.header_bytes("float32", (20,)))
+    assert (info["t3"].offset, info["t3"].length) == (0, hdr3 + stored.numel() * 4)  # tensors first ...
+    assert (info["t1"].offset, info["t1"].length) == (info["t3"].length, hdr1 + 80)
+    assert (info["blob"].offset, info["blob"].length) == (info["t3"].length + info["t1"].length, 10)  # ... then blobs
+    oid = CheckpointObjectId.from_container(cid, "data_0_src0.distcp")
+    assert os.path.getsize(oid.data) == METADATA_SIZE + info["blob"].offset + 10
+
+    storage = {0: info["t3"], 1: info["t1"], 2: info["blob"]}
+    parent = torch.zeros(2, 4, 5, device=DEV)
+    targets = {"box": parent[:, ::2, 3:], "slice": torch.zeros(10, device=DEV), "host": torch.zeros(8, 15, 10), "blob": None}
+    reqs = [
+        ReadItem(type=LoadItemType.TENSOR, dest_index=MetadataIndex("box"), dest_offsets=torch.Size([0, 0, 0]), storage_index=0,
+                 storage_offsets=torch.Size([1, 0, 3]), lengths=torch.Size([2, 2, 2])),
+        ReadItem(type=LoadItemType.TENSOR, dest_index=MetadataIndex("slice"), dest_offsets=torch.Size([0]), storage_index=1,
+                 storage_offsets=torch.Size([5]), lengths=torch.Size([10])),
+        ReadItem(type=LoadItemType.TENSOR, dest_index=MetadataIndex("host"), dest_offsets=torch.Size([0, 0, 0]), storage_index=0,
+                 storage_offsets=torch.Size([4, 5, 0]), lengths=torch.Size([8, 15, 10])),
+        ReadItem(type=LoadItemType.BYTE_IO, dest_index=MetadataIndex("blob"), dest_offsets=torch.Size([0]), storage_index=2,
+                 storage_offsets=torch.Size([0]), lengths=torch.Size([0])),
+    ]
+    planner = _Planner(targets)
+    _loader().read_data(oid, reqs, planner, storage)
+    assert torch.equal(targets["box"].cpu(), stored[1:3, 0:2, 3:5])
+    assert torch.equal(targets["slice"].cpu(), torch.arange(5, 15, dtype=torch.float32))  # the reference's known answer
+    assert torch.equal(targets["host"], stored[4:12, 5:20, :])
+    assert planner.loaded == {"blob": b"some-bytes"} and sorted(planner.committed) == ["box", "host", "slice"]
+    assert float(parent[:, 1::2].abs().sum()) == 0 and float(parent[:, :, :3].abs().sum()) == 0
+
+    with pytest.raises(AssertionError, match="mismatch sizes"):
+        _loader().read_data(oid, [reqs[1]], _Planner({"slice": torch.zeros(11, device=DEV)}), storage)
+    with pytest.raises(FileNotFoundError, match="does not exist on any node in the cluster"):
+        _loader().read_data(CheckpointObjectId(oid.data + ".gone"), reqs, planner, storage)
+
+
+def test_multiple_buckets_and_overwrite_of_existing_object(shm_dir):
+    data = {f"t{i}": torch.full((1000 + i,), float(i), device=DEV) for i in range(5)}
+    data["b0"], data["b1"] = io.BytesIO(b"zero"), io.BytesIO(b"one")
+    cid, buckets, info = _write_direct(shm_dir, data, bucket_count=3)
+    names = sorted(b.object_name for b in buckets)
+    assert names == ["data_0_src0.distcp", "data_1_src0.distcp", "data_2_src0.distcp"]
+    assert sum(len(b.tensor_data) + len(b.bytesio_data) for b in buckets) == 7
+    for b in buckets:  # every object parses as a sequence of records + blobs the oracle agrees with
+        raw = open(b.object_id.data, "rb").read()
+        tensors = [data[i.index.fqn].cpu() for i, _ in b.tensor_data]
+        blobs = [d.getvalue() for _, d in b.bytesio_data]
+        assert raw == fmt.file_image(tensors, blobs)[0]
+    _write_direct(shm_dir, {"t0": torch.ones(3, device=DEV)})  # same object id again: overwritten, not an error
+    raw = open(os.path.join(cid.data, "data_0_src0.distcp"), "rb").read()
+    assert raw == fmt.file_image([torch.ones(3)])[0]
+
+
+def test_legacy_torch_save_objects_are_still_readable(shm_dir):
+    """An object whose signature is TORCH___ holds torch.save records; the loader reads it on the host."""
+    from ml_flashpoint.core.defaults import CheckpointFormat
+
+    t = torch.tensor([4.0, 5.0, 6.0])
+    oid = CheckpointObjectId(os.path.join(shm_dir, "step-1_ckpt", "legacy.distcp"))
+    with CheckpointObjectManager().acquire_buffer(oid, 1 << 16) as w:
+        w.set_format_signature(CheckpointFormat.TORCH_SAVE)
+        torch.save(t, w)
+        length = w.tell()
+    target = torch.zeros(3, device=DEV)
+    req = ReadItem(type=LoadItemType.TENSOR, dest_index=MetadataIndex("x"), dest_offsets=torch.Size([0]), storage_index=0,
+                   storage_offsets=torch.Size([0]), lengths=torch.Size([3]))
+    _loader().read_data(oid, [req], _Planner({"x": target}), {0: _StorageInfo("legacy.distcp", 0, length)})
+    assert torch.equal(target.cpu(), t)
+
+
+def test_saver_rejects_cpu_only_format_and_is_picklable():
+    with pytest.raises(ValueError, match="MLF_TENS"):
+        _saver(use_optimized_save=False)
+    from ml_flashpoint.hip.checkpoint_saver import HipMLFlashpointCheckpointSaver
+
+    s = HipMLFlashpointCheckpointSaver(_zero, _zero, _none, CheckpointObjectManager(), replication_manager=object())
+    clone = pickle.loads(pickle.dumps(s))
+    assert clone._replication_manager is None and clone._engine is None
+    with pytest.raises(RuntimeError, match="ReplicationManager is not available"):
+        clone.async_replicate_object(CheckpointObjectId("/x/y"))
+
+
+def _zero():
+    return 0
+
+
+def _none():
+    return None
