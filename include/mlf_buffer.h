@@ -64,6 +64,8 @@ size_t mlf_buffer_capacity(const mlf_buffer* b);
 int mlf_buffer_is_closed(const mlf_buffer* b);
 int mlf_buffer_is_readonly(const mlf_buffer* b);
 const char* mlf_buffer_id(const mlf_buffer* b);
+/* The descriptor the mapping was made from (-1 once closed); stays owned by the buffer object. */
+int mlf_buffer_fd(const mlf_buffer* b);
 
 /* Message of the last failure on the calling thread ("" if none). */
 const char* mlf_buffer_last_error(void);

@@ -148,6 +148,16 @@ int mlf_engine_d2h(mlf_engine* engine, const void* src_dev, void* dst_host, uint
 int mlf_engine_h2d(mlf_engine* engine, const void* src_host, void* dst_dev, uint64_t nbytes,
                    void* consumer_stream, mlf_xfer_stats* stats);
 
+/* The same two transfers with the pageable end given as a byte range of an open file instead of a pointer:
+ * the host threads pwrite()/pread() the pinned slots straight to/from the buffer file (`fd` from
+ * mlf_buffer_fd(), `file_offset` = 4096 + position in the data section).  The bytes land in the same page-cache
+ * pages a MAP_SHARED mapping shows (buffer_helper.cpp:96-103), but no page-table entry is built or torn down per
+ * 4 KiB of the object, which for a 100 GB object costs more than the copy itself. */
+int mlf_engine_d2h_fd(mlf_engine* engine, const void* src_dev, int fd, uint64_t file_offset, uint64_t nbytes,
+                      void* producer_stream, mlf_xfer_stats* stats);
+int mlf_engine_h2d_fd(mlf_engine* engine, int fd, uint64_t file_offset, void* dst_dev, uint64_t nbytes,
+                      void* consumer_stream, mlf_xfer_stats* stats);
+
 #ifdef __cplusplus
 }
 #endif

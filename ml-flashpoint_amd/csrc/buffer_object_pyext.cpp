@@ -128,6 +128,15 @@ PyObject* bo_get_data_ptr(PyObject* self_, PyObject*) {
   return PyLong_FromVoidPtr(mlf_buffer_data_ptr(self->handle));
 }
 
+PyObject* bo_fileno(PyObject* self_, PyObject*) {
+  auto* self = reinterpret_cast<PyBufferObject*>(self_);
+  if (mlf_buffer_is_closed(self->handle)) {
+    PyErr_SetString(PyExc_RuntimeError, "Buffer is closed: no file descriptor.");
+    return nullptr;
+  }
+  return PyLong_FromLong(mlf_buffer_fd(self->handle));
+}
+
 PyObject* bo_closed(PyObject* self_, void*) {
   auto* self = reinterpret_cast<PyBufferObject*>(self_);
   return PyBool_FromLong(mlf_buffer_is_closed(self->handle));
@@ -164,6 +173,7 @@ PyMethodDef bo_methods[] = {
     {"get_id", bo_get_id, METH_NOARGS, "Gets the buffer object id."},
     {"get_capacity", bo_get_capacity, METH_NOARGS, "Gets the buffer object capacity."},
     {"get_data_ptr", bo_get_data_ptr, METH_NOARGS, "Returns the raw memory address of the buffer as an integer."},
+    {"fileno", bo_fileno, METH_NOARGS, "Returns the descriptor of the mapped file (owned by the buffer object)."},
     {nullptr, nullptr, 0, nullptr}};
 
 PyGetSetDef bo_getset[] = {{"closed", bo_closed, nullptr, "True once closed.", nullptr},

@@ -223,6 +223,7 @@ size_t mlf_buffer_capacity(const mlf_buffer* b) { return is_open(b) ? b->cap : 0
 int mlf_buffer_is_closed(const mlf_buffer* b) { return is_open(b) ? 0 : 1; }
 int mlf_buffer_is_readonly(const mlf_buffer* b) { return (b && b->writable) ? 0 : 1; }
 const char* mlf_buffer_id(const mlf_buffer* b) { return b ? b->id.c_str() : ""; }
+int mlf_buffer_fd(const mlf_buffer* b) { return is_open(b) ? b->fd : -1; }
 
 int mlf_host_parallel_memcpy(void* dst, const void* src, size_t n, int threads) {
   if (n == 0) return MLF_OK;

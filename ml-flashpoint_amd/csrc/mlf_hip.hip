@@ -21,8 +21,10 @@
 #include "mlf_hip.h"
 
 #include <hip/hip_runtime.h>
+#include <errno.h>
 #include <nmmintrin.h>
 #include <string.h>
+#include <unistd.h>
 
 #include <algorithm>
 #include <atomic>
@@ -390,6 +392,66 @@ void pool_memcpy(WorkerPool& pool, char* dst, const char* src, size_t n) {
     const size_t off = (size_t)i * per;
     if (off < n) memcpy(dst + off, src + off, std::min(per, n - off));
   });
+}
+
+// The pageable end of a transfer: a plain pointer, or a byte range of an open file (pread/pwrite).  Going
+// through the file descriptor moves the same page-cache pages as a MAP_SHARED mapping would, without building
+// (and later tearing down) one page-table entry per 4 KiB of a buffer that can be 100+ GB.
+struct HostEnd {
+  char* ptr = nullptr;
+  int fd = -1;
+  uint64_t file_off = 0;
+};
+
+int full_pwrite(int fd, const char* buf, size_t len, uint64_t off) {
+  while (len) {
+    ssize_t w = pwrite(fd, buf, len, (off_t)off);
+    if (w < 0) {
+      if (errno == EINTR) continue;
+      return errno;
+    }
+    buf += w;
+    off += (uint64_t)w;
+    len -= (size_t)w;
+  }
+  return 0;
+}
+
+int full_pread(int fd, char* buf, size_t len, uint64_t off) {
+  while (len) {
+    ssize_t r = pread(fd, buf, len, (off_t)off);
+    if (r < 0) {
+      if (errno == EINTR) continue;
+      return errno;
+    }
+    if (r == 0) return ENODATA;  // file shorter than the requested range
+    buf += r;
+    off += (uint64_t)r;
+    len -= (size_t)r;
+  }
+  return 0;
+}
+
+// slot -> host end (to_host) or host end -> slot, split over the pool; returns 0 or an errno value
+int pool_host_copy(WorkerPool& pool, const HostEnd& host, uint64_t host_off, char* slot, size_t n, bool to_host) {
+  if (host.fd < 0) {
+    if (to_host) pool_memcpy(pool, host.ptr + host_off, slot, n);
+    else pool_memcpy(pool, slot, host.ptr + host_off, n);
+    return 0;
+  }
+  const unsigned parts = std::max<unsigned>(1, std::min<size_t>(pool.width(), n / ((size_t)1 << 20)));
+  size_t per = (n + parts - 1) / parts;
+  per = (per + 4095) & ~(size_t)4095;
+  std::atomic<int> err{0};
+  pool.run(parts, [&](unsigned i) {
+    const size_t off = (size_t)i * per;
+    if (off >= n) return;
+    const size_t len = std::min(per, n - off);
+    const int e = to_host ? full_pwrite(host.fd, slot + off, len, host.file_off + host_off + off)
+                          : full_pread(host.fd, slot + off, len, host.file_off + host_off + off);
+    if (e) err.store(e);
+  });
+  return err.load();
 }
 
 }  // namespace
@@ -860,10 +922,14 @@ int mlf_engine_create(uint64_t slot_bytes, uint32_t n_slots, uint32_t n_threads,
   return MLF_HIP_OK;
 }
 
-int mlf_engine_d2h(mlf_engine* e, const void* src_dev, void* dst_host, uint64_t nbytes, void* producer_stream,
-                   mlf_xfer_stats* stats) {
+}  // extern "C"
+
+namespace {
+
+int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t nbytes, void* producer_stream,
+               mlf_xfer_stats* stats) {
   if (!e) return fail(MLF_HIP_BAD_ARG, "null engine");
-  if (nbytes && (!src_dev || !dst_host)) return fail(MLF_HIP_BAD_ARG, "null pointer");
+  if (nbytes && (!src_dev || (host.fd < 0 && !host.ptr))) return fail(MLF_HIP_BAD_ARG, "null pointer");
   std::lock_guard<std::mutex> g(e->busy);
   HIP_TRY(hipSetDevice(e->device));
   const double t0 = now_s();
@@ -871,7 +937,6 @@ int mlf_engine_d2h(mlf_engine* e, const void* src_dev, void* dst_host, uint64_t 
   HIP_TRY(hipEventRecord(e->gate, static_cast<hipStream_t>(producer_stream)));
   for (hipStream_t s : e->streams) HIP_TRY(hipStreamWaitEvent(s, e->gate, 0));
   const char* src = static_cast<const char*>(src_dev);
-  char* dst = static_cast<char*>(dst_host);
   const uint64_t slot = e->slot_bytes;
   const uint64_t n_chunks = (nbytes + slot - 1) / slot;
   const uint64_t n_slots = e->slots.size();
@@ -883,6 +948,9 @@ int mlf_engine_d2h(mlf_engine* e, const void* src_dev, void* dst_host, uint64_t 
     HIP_TRY(hipEventRecord(e->slot_done[s], st));
     return MLF_HIP_OK;
   };
+  auto drain_streams = [&] {
+    for (hipStream_t s : e->streams) (void)hipStreamSynchronize(s);
+  };
   for (uint64_t c = 0; c < std::min(n_chunks, n_slots); ++c)
     if (int rc = issue(c)) return rc;
   double wait = 0;
@@ -892,7 +960,10 @@ int mlf_engine_d2h(mlf_engine* e, const void* src_dev, void* dst_host, uint64_t 
     const double w0 = now_s();
     HIP_TRY(hipEventSynchronize(e->slot_done[s]));
     if (c == 0) wait = now_s() - w0;
-    pool_memcpy(*e->pool, dst + off, e->slots[s], len);
+    if (int err = pool_host_copy(*e->pool, host, off, e->slots[s], len, true)) {
+      drain_streams();  // copies still in flight target the slots: let them land before anyone reuses them
+      return fail(MLF_HIP_RUNTIME, std::string("pwrite() to the buffer file failed: ") + strerror(err));
+    }
     if (c + n_slots < n_chunks)
       if (int rc = issue(c + n_slots)) return rc;
   }
@@ -905,14 +976,13 @@ int mlf_engine_d2h(mlf_engine* e, const void* src_dev, void* dst_host, uint64_t 
   return MLF_HIP_OK;
 }
 
-int mlf_engine_h2d(mlf_engine* e, const void* src_host, void* dst_dev, uint64_t nbytes, void* consumer_stream,
-                   mlf_xfer_stats* stats) {
+int engine_h2d(mlf_engine* e, const HostEnd& host, void* dst_dev, uint64_t nbytes, void* consumer_stream,
+               mlf_xfer_stats* stats) {
   if (!e) return fail(MLF_HIP_BAD_ARG, "null engine");
-  if (nbytes && (!src_host || !dst_dev)) return fail(MLF_HIP_BAD_ARG, "null pointer");
+  if (nbytes && (!dst_dev || (host.fd < 0 && !host.ptr))) return fail(MLF_HIP_BAD_ARG, "null pointer");
   std::lock_guard<std::mutex> g(e->busy);
   HIP_TRY(hipSetDevice(e->device));
   const double t0 = now_s();
-  const char* src = static_cast<const char*>(src_host);
   char* dst = static_cast<char*>(dst_dev);
   const uint64_t slot = e->slot_bytes;
   const uint64_t n_chunks = (nbytes + slot - 1) / slot;
@@ -921,7 +991,10 @@ int mlf_engine_h2d(mlf_engine* e, const void* src_host, void* dst_dev, uint64_t 
     const uint64_t off = c * slot, len = std::min(slot, nbytes - off);
     const uint64_t s = c % n_slots;
     if (c >= n_slots) HIP_TRY(hipEventSynchronize(e->slot_done[s]));  // the slot's previous upload has left it
-    pool_memcpy(*e->pool, e->slots[s], src + off, len);
+    if (int err = pool_host_copy(*e->pool, host, off, e->slots[s], len, false)) {
+      for (hipStream_t st : e->streams) (void)hipStreamSynchronize(st);
+      return fail(MLF_HIP_RUNTIME, std::string("pread() from the buffer file failed: ") + strerror(err));
+    }
     hipStream_t st = e->streams[c & 1];
     HIP_TRY(hipMemcpyAsync(dst + off, e->slots[s], len, hipMemcpyHostToDevice, st));
     HIP_TRY(hipEventRecord(e->slot_done[s], st));
@@ -939,6 +1012,42 @@ int mlf_engine_h2d(mlf_engine* e, const void* src_host, void* dst_dev, uint64_t 
     stats->chunks = n_chunks;
   }
   return MLF_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mlf_engine_d2h(mlf_engine* e, const void* src_dev, void* dst_host, uint64_t nbytes, void* producer_stream,
+                   mlf_xfer_stats* stats) {
+  HostEnd host;
+  host.ptr = static_cast<char*>(dst_host);
+  return engine_d2h(e, src_dev, host, nbytes, producer_stream, stats);
+}
+
+int mlf_engine_h2d(mlf_engine* e, const void* src_host, void* dst_dev, uint64_t nbytes, void* consumer_stream,
+                   mlf_xfer_stats* stats) {
+  HostEnd host;
+  host.ptr = const_cast<char*>(static_cast<const char*>(src_host));
+  return engine_h2d(e, host, dst_dev, nbytes, consumer_stream, stats);
+}
+
+int mlf_engine_d2h_fd(mlf_engine* e, const void* src_dev, int fd, uint64_t file_offset, uint64_t nbytes,
+                      void* producer_stream, mlf_xfer_stats* stats) {
+  if (fd < 0) return fail(MLF_HIP_BAD_ARG, "bad file descriptor");
+  HostEnd host;
+  host.fd = fd;
+  host.file_off = file_offset;
+  return engine_d2h(e, src_dev, host, nbytes, producer_stream, stats);
+}
+
+int mlf_engine_h2d_fd(mlf_engine* e, int fd, uint64_t file_offset, void* dst_dev, uint64_t nbytes,
+                      void* consumer_stream, mlf_xfer_stats* stats) {
+  if (fd < 0) return fail(MLF_HIP_BAD_ARG, "bad file descriptor");
+  HostEnd host;
+  host.fd = fd;
+  host.file_off = file_offset;
+  return engine_h2d(e, host, dst_dev, nbytes, consumer_stream, stats);
 }
 
 }  // extern "C"

@@ -227,6 +227,13 @@ class BufferIO:
         self._check_validity()
         return self.buffer_obj.get_data_ptr() + METADATA_SIZE + pos
 
+    def fileno(self) -> int:
+        """Descriptor of the mapped file, for engines that read/write the file directly; -1 if the underlying
+        buffer object does not expose one."""
+        self._check_validity()
+        getter = getattr(self.buffer_obj, "fileno", None)
+        return getter() if getter is not None else -1
+
     def __enter__(self):
         self._check_validity()
         return self

@@ -90,6 +90,8 @@ _SIGNATURES = {
     "mlf_engine_destroy": (_INT, [_VP]),
     "mlf_engine_d2h": (_INT, [_VP, _VP, _VP, _U64, _VP, ctypes.POINTER(XferStats)]),
     "mlf_engine_h2d": (_INT, [_VP, _VP, _VP, _U64, _VP, ctypes.POINTER(XferStats)]),
+    "mlf_engine_d2h_fd": (_INT, [_VP, _VP, _INT, _U64, _U64, _VP, ctypes.POINTER(XferStats)]),
+    "mlf_engine_h2d_fd": (_INT, [_VP, _INT, _U64, _VP, _U64, _VP, ctypes.POINTER(XferStats)]),
 }
 
 _LIB: Optional[ctypes.CDLL] = None

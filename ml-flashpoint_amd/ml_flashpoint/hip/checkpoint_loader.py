@@ -61,6 +61,7 @@ class HipMLFlashpointCheckpointLoader(MLFlashpointCheckpointLoader):
         tile_bytes: int = 0,
         block_threads: int = 0,
         verify_crc: bool = True,
+        use_file_io: bool = True,
     ):
         """Arguments as the reference's default loader (checkpoint_loader.py:126-158), plus the copy-engine and
         kernel work-split knobs and ``verify_crc`` (check the CRC-32C sidecar of an object, when it has one)."""
@@ -76,6 +77,9 @@ class HipMLFlashpointCheckpointLoader(MLFlashpointCheckpointLoader):
         self._tile_bytes = tile_bytes
         self._block_threads = block_threads
         self._verify_crc = verify_crc
+        # pread() the buffer file into the pinned slots instead of reading through the (fresh, read-only) mapping:
+        # reads of tmpfs run in parallel, and no page-table entry per 4 KiB has to be built and torn down
+        self._use_file_io = use_file_io
         self._engine: Optional[hip_plan.CopyEngine] = None
         self.last_load_stats: dict = {}
         # set to True to bracket every unpack launch with timing events; see the saver's attribute of the same name
@@ -242,7 +246,11 @@ class HipMLFlashpointCheckpointLoader(MLFlashpointCheckpointLoader):
             _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
             image = torch.empty(span, dtype=torch.uint8, device=device)
             cur = torch.cuda.current_stream(device)
-            st = self._get_engine().h2d(stream.data_address(lo), image.data_ptr(), span, cur.cuda_stream)
+            fd = stream.fileno() if self._use_file_io else -1
+            if fd >= 0:
+                st = self._get_engine().h2d_fd(fd, METADATA_SIZE + lo, image.data_ptr(), span, cur.cuda_stream)
+            else:
+                st = self._get_engine().h2d(stream.data_address(lo), image.data_ptr(), span, cur.cuda_stream)
             stats["h2d_s"] += st.seconds
             stats["h2d_bytes"] += span
             if sidecar is not None:

@@ -32,6 +32,7 @@ from torch.distributed.checkpoint.planner import WriteItem, WriteItemType
 from torch.distributed.checkpoint.storage import WriteResult
 from typing_extensions import override
 
+from ml_flashpoint.checkpoint_object_manager.buffer_metadata import METADATA_SIZE
 from ml_flashpoint.checkpoint_object_manager.checkpoint_object_manager import CheckpointObjectManager
 from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId, CheckpointObjectId
 from ml_flashpoint.core.checkpoint_saver import (
@@ -117,12 +118,15 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         tile_bytes: int = 0,
         block_threads: int = 0,
         crc_chunk_bytes: int = 0,
+        use_file_io: bool = False,
     ):
         """Same positional arguments as the reference's default saver (checkpoint_saver.py:290-321).
 
         Keyword-only extras: ``engine_config`` (pinned ring), ``tile_bytes`` / ``block_threads`` (pack kernel work
         split, 0 = library default), ``crc_chunk_bytes`` (> 0: compute a CRC-32C per chunk of every object on the
-        GPU and keep it beside the object).
+        GPU and keep it beside the object), ``use_file_io`` (False, the default: the host threads memcpy the
+        pinned slots into the mapping, whose page-table entries a pooled buffer keeps from save to save; True: they
+        pwrite() through the file descriptor, which tmpfs serialises on the inode lock - measured 5x slower).
         """
         if not use_optimized_save:
             raise ValueError(
@@ -141,6 +145,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         self._tile_bytes = tile_bytes
         self._block_threads = block_threads
         self._crc_chunk_bytes = crc_chunk_bytes
+        self._use_file_io = use_file_io
         self._init_runtime_state()
 
     def _init_runtime_state(self):
@@ -382,7 +387,11 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                         xfer["crc_s"] += time.perf_counter() - t0
                     start = writer.tell()
                     writer.next_buffer_slice(nbytes).release()  # bounds check + position/high-water mark
-                    st = self._get_engine().d2h(staged.image.data_ptr(), writer.data_address(start), nbytes, staged.stream)
+                    fd = writer.fileno() if self._use_file_io else -1
+                    if fd >= 0:
+                        st = self._get_engine().d2h_fd(staged.image.data_ptr(), fd, METADATA_SIZE + start, nbytes, staged.stream)
+                    else:
+                        st = self._get_engine().d2h(staged.image.data_ptr(), writer.data_address(start), nbytes, staged.stream)
                     xfer["d2h_s"] += st.seconds
                     xfer["d2h_wait_s"] += st.wait_seconds
                     xfer["d2h_bytes"] += nbytes

@@ -249,6 +249,24 @@ class CopyEngine:
         )
         return stats
 
+    def d2h_fd(self, src_dev_ptr: int, fd: int, file_offset: int, nbytes: int, producer_stream: int = 0) -> _lib.XferStats:
+        """Device -> byte range of an open file (pwrite from the pinned slots)."""
+        stats = _lib.XferStats()
+        _lib.check(
+            _lib.load().mlf_engine_d2h_fd(self._handle, src_dev_ptr, fd, file_offset, nbytes, producer_stream, ctypes.byref(stats)),
+            "mlf_engine_d2h_fd",
+        )
+        return stats
+
+    def h2d_fd(self, fd: int, file_offset: int, dst_dev_ptr: int, nbytes: int, consumer_stream: int = 0) -> _lib.XferStats:
+        """Byte range of an open file -> device (pread into the pinned slots)."""
+        stats = _lib.XferStats()
+        _lib.check(
+            _lib.load().mlf_engine_h2d_fd(self._handle, fd, file_offset, dst_dev_ptr, nbytes, consumer_stream, ctypes.byref(stats)),
+            "mlf_engine_h2d_fd",
+        )
+        return stats
+
     def destroy(self) -> None:
         if getattr(self, "_handle", None) is not None:
             _lib.load().mlf_engine_destroy(self._handle)

@@ -284,5 +284,20 @@ def test_copy_engine_round_trip(nbytes, shm_dir):
     engine.h2d(bo.get_data_ptr() + 4096, back.data_ptr(), nbytes, stream)
     torch.cuda.synchronize()
     assert torch.equal(back[:nbytes].cpu(), host) and int(back[nbytes:].sum()) == 0
+    # the same two transfers through the file descriptor (pwrite / pread), at an odd file offset
+    memoryview(bo)[:] = bytes(4096 + nbytes)
+    bo2 = BufferObject(f"{shm_dir}/obj2.bin", 4096 + 7 + nbytes, True)
+    stats = engine.d2h_fd(dev.data_ptr(), bo2.fileno(), 4096 + 7, nbytes, stream)
+    assert stats.bytes == nbytes
+    assert bytes(memoryview(bo2)[4096 + 7 :]) == host.numpy().tobytes() and bytes(memoryview(bo2)[: 4096 + 7]) == bytes(4096 + 7)
+    back.zero_()
+    engine.h2d_fd(bo2.fileno(), 4096 + 7, back.data_ptr(), nbytes, stream)
+    torch.cuda.synchronize()
+    assert torch.equal(back[:nbytes].cpu(), host) and int(back[nbytes:].sum()) == 0
+    from ml_flashpoint.hip import _lib
+
+    with pytest.raises(_lib.HipError, match="pread"):  # asking for more than the file holds is an error, not a hang
+        engine.h2d_fd(bo2.fileno(), 4096 + 7, back.data_ptr(), nbytes + 64, stream)
     bo.close()
+    bo2.close()
     engine.destroy()
