@@ -31,6 +31,11 @@ for _p in (REPO, os.path.join(REPO, "ml-flashpoint_amd"), os.path.join(REPO, "te
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, vendor figure
+# HBM bytes moved by one pack of the default workload, relative to its algorithmic bytes (2 x payload): measured
+# with `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`, each scaled against a torch.add kernel of known size
+# (summary: profiles/pmc_traffic_mlf_flat_kernel_llama3-8b-shard.md).  Hardware counters cannot be read from
+# inside this script, so the ratio is applied to the live algorithmic byte count of the same workload only.
+PACK_TRAFFIC_RATIO_LLAMA3_8B = 1.0205
 
 
 def parse_args():
@@ -377,7 +382,8 @@ def main():
             "parity": "restored tensors bit-identical to originals (fingerprints)",
             "roofline": {"bound": "hbm", "kernel": "mlf_flat_kernel<pack>", "achieved": round(pack_gbps, 1),
                          "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(pack_gbps / HBM_PEAK_GBPS, 4),
-                         "traffic": None,
+                         "traffic": (int(PACK_TRAFFIC_RATIO_LLAMA3_8B * 2 * mean(rec["pack_bytes"]))
+                                     if args.workload == "llama3-8b-shard" and args.scale >= 1.0 else None),
                          "algorithmic_bytes_per_launch": int(2 * mean(rec["pack_bytes"])),
                          "avg_launch_ms": round(pack_s * 1e3, 3)},
         }

@@ -24,6 +24,7 @@ known-answer sub-box reads (tests/core/test_checkpoint_loader.py:223-302).
 """
 
 import struct
+import warnings
 from typing import List, Sequence, Tuple
 
 import numpy as np
@@ -202,7 +203,7 @@ def parse_record(record: bytes) -> Tuple[torch.dtype, Tuple[int, ...], bytes]:
             break
     if strings[:2] != [_HEADER_MODULE, _HEADER_CLASS] or strings[2] != "dtype" or strings[5] != "shape":
         raise ValueError("unexpected header pickle layout")
-    return getattr(torch, strings[4]), tuple(ints), record[4 + hlen :]
+    return getattr(torch, strings[4]), tuple(ints), memoryview(record)[4 + hlen :]  # a view: no second copy
 
 
 def read_item(record: bytes, storage_offsets: Sequence[int], lengths: Sequence[int]) -> torch.Tensor:
@@ -211,7 +212,9 @@ def read_item(record: bytes, storage_offsets: Sequence[int], lengths: Sequence[i
     if len(payload) == 0:
         t = torch.empty(shape, dtype=dtype)
     else:
-        t = torch.frombuffer(bytearray(payload), dtype=dtype).reshape(shape)
+        with warnings.catch_warnings():  # frombuffer over read-only bytes, exactly as the reference does
+            warnings.simplefilter("ignore")
+            t = torch.frombuffer(payload, dtype=dtype).reshape(shape)
     for dim, (off, length) in enumerate(zip(storage_offsets, lengths)):
         if length < t.size(dim):
             t = t.narrow(dim, off, length)

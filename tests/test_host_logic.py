@@ -1,0 +1,192 @@
+"""Host-side duties of the saver/loader plug-ins and the small core types, on the CPU (no kernel is launched).
+
+Expectations are those of the reference's tests (tests/core/test_checkpoint_saver.py: markers :324-384, metadata
+:1760-1867, removal of older steps :2014-2155; tests/core/test_checkpoint_id_types.py; tests/core/test_checkpoint_loader.py
+discovery of complete steps), re-expressed against this package.
+"""
+
+import os
+import pickle
+import subprocess
+
+import pytest
+import torch
+from torch.distributed.checkpoint.metadata import Metadata
+
+from ml_flashpoint.checkpoint_object_manager.checkpoint_object_manager import CheckpointObjectManager
+from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId, CheckpointObjectId
+from ml_flashpoint.core.checkpoint_loader import DefaultMLFlashpointCheckpointLoader, MLFlashpointCheckpointLoader
+from ml_flashpoint.core.checkpoint_saver import (
+    DEFAULT_INITIAL_BUFFER_SIZE_BYTES,
+    DefaultMLFlashpointCheckpointSaver,
+    MLFlashpointCheckpointSaver,
+    ObjectWriteBucket,
+)
+from ml_flashpoint.core.defaults import CheckpointFormat, default_metadata_object_name
+from ml_flashpoint.core.hfid import generate_hfid
+from ml_flashpoint.core.tensor_header import TensorHeader
+
+
+def make_saver(local_rank=0, barrier=None, **kw):
+    calls = []
+    saver = DefaultMLFlashpointCheckpointSaver(
+        global_rank_getter=lambda: 3,
+        local_rank_getter=lambda: local_rank,
+        global_barrier_func=barrier or (lambda: calls.append("barrier")),
+        ckpt_obj_manager=CheckpointObjectManager(),
+        replication_manager=None,
+        **kw,
+    )
+    saver._test_calls = calls
+    return saver
+
+
+def test_plugin_classes_and_defaults():
+    assert DEFAULT_INITIAL_BUFFER_SIZE_BYTES == 16 * 1024**3
+    assert issubclass(DefaultMLFlashpointCheckpointSaver, MLFlashpointCheckpointSaver)
+    assert issubclass(DefaultMLFlashpointCheckpointLoader, MLFlashpointCheckpointLoader)
+    assert CheckpointFormat.MLF_FORMAT == b"MLF_TENS" and CheckpointFormat.TORCH_SAVE == b"TORCH___"
+    assert default_metadata_object_name() == ".metadata"
+    with pytest.raises(TypeError):
+        MLFlashpointCheckpointSaver()  # abstract
+
+
+@pytest.mark.parametrize("local_rank", [0, 5])
+def test_dirty_marker_lifecycle(tmp_path, local_rank):
+    saver = make_saver(local_rank)
+    cid = CheckpointContainerId(str(tmp_path / "job" / "step-7_ckpt"))
+    marker = f"{cid}__{local_rank}__unfinished"
+    saver.initialize_checkpoint(cid)
+    assert os.path.isfile(marker) and os.path.getsize(marker) == 0 and os.path.isdir(cid.data)
+    saver.initialize_checkpoint(cid)  # idempotent
+    assert CheckpointContainerId.get_dirty_version_checkpoint_container_pattern().match(os.path.basename(marker))
+    proc = saver.finalize_checkpoint(cid)
+    assert not os.path.exists(marker) and saver._test_calls == ["barrier"]
+    assert proc is None  # nothing older to delete (and only local rank 0 would)
+    saver.finalize_checkpoint(cid)  # marker already gone: a warning, not an error
+    assert saver._get_dirty_marker_file_path(CheckpointContainerId(cid.data + "/")) == marker
+
+
+def test_write_metadata_is_atomic_and_round_trips(tmp_path):
+    saver = make_saver()
+    cid = CheckpointContainerId(str(tmp_path / "step-1_ckpt"))
+    md = Metadata(state_dict_metadata={}, planner_data={"k": 1}, storage_data={"a": 2})
+    saver.write_metadata(cid, md)
+    assert sorted(os.listdir(cid.data)) == [".metadata"]  # the .tmp file was renamed away
+    loader = DefaultMLFlashpointCheckpointLoader(CheckpointObjectManager(), None)
+    back = loader.read_metadata(cid)
+    assert back.planner_data == {"k": 1} and back.storage_data == {"a": 2}
+    saver.write_metadata(cid, md, md_object_name="nested/custom.md")
+    assert pickle.load(open(os.path.join(cid.data, "nested", "custom.md"), "rb")).planner_data == {"k": 1}
+    with pytest.raises(FileNotFoundError):
+        loader.read_metadata(cid, object_name="absent")
+
+
+@pytest.mark.parametrize(
+    "older_than_step, steps, expected_deleted",
+    [
+        (3, [1, 2, 3, 4, 5], [1, 2]),
+        (10, [1, 5, 9, 10, 11], [1, 5, 9]),
+        (100, [1, 10, 99, 100, 101], [1, 10, 99]),
+        (1, [1, 2, 3], []),
+        (5, [1, 2, 3, 4], [1, 2, 3, 4]),
+        (10, [1, 5, 9, 10, 11, "invalid", "step-abc_ckpt", "step-10_ckpt_extra", "step--100_ckpt", "step-3.14_ckpt"], [1, 5, 9]),
+    ],
+)
+def test_finalize_removes_only_older_well_formed_steps(tmp_path, older_than_step, steps, expected_deleted):
+    base = tmp_path / "checkpoints"
+    created = []
+    for s in steps:
+        name = CheckpointContainerId.format_version_container(s) if isinstance(s, int) else s
+        os.makedirs(base / name)
+        created.append(str(base / name))
+    (base / "step-0_ckpt_file").write_text("a file, not a directory")
+    saver = make_saver(local_rank=0)
+    cid = CheckpointContainerId(str(base / CheckpointContainerId.format_version_container(older_than_step)))
+    os.makedirs(cid.data, exist_ok=True)
+    proc = saver.finalize_checkpoint(cid)
+    if expected_deleted:
+        assert isinstance(proc, subprocess.Popen)
+        proc.wait()
+    else:
+        assert proc is None
+    gone = {str(base / CheckpointContainerId.format_version_container(s)) for s in expected_deleted}
+    for d in created:
+        assert os.path.exists(d) != (d in gone), d
+    assert make_saver(local_rank=1).finalize_checkpoint(cid) is None  # only local rank 0 cleans up
+    assert saver._remove_older_checkpoints(CheckpointContainerId(str(base / "not-a-step"))) is None
+
+
+def test_latest_complete_checkpoint_skips_unfinished_steps(tmp_path):
+    loader = DefaultMLFlashpointCheckpointLoader(CheckpointObjectManager(), None)
+    base = CheckpointContainerId(str(tmp_path / "job"))
+    assert loader.get_latest_complete_checkpoint(base) is None
+    for step in (5, 10, 20, 30):
+        os.makedirs(os.path.join(base.data, f"step-{step}_ckpt"))
+    os.makedirs(os.path.join(base.data, "latest"))
+    open(os.path.join(base.data, "step-30_ckpt__0__unfinished"), "w").close()  # still being written
+    open(os.path.join(base.data, "step-20_ckpt__3__unfinished"), "w").close()  # another local rank's marker counts too
+    assert loader.get_latest_complete_checkpoint(base).data == os.path.join(base.data, "step-10_ckpt")
+    os.remove(os.path.join(base.data, "step-30_ckpt__0__unfinished"))
+    assert loader.get_latest_complete_checkpoint(base).data == os.path.join(base.data, "step-30_ckpt")
+
+
+def test_saver_crosses_process_boundaries_as_configuration_only(tmp_path):
+    saver = make_saver(initial_buffer_size_bytes=123, crc_chunk_bytes=1 << 20)
+    saver._barrier_func = None  # lambdas do not pickle; the reference's users pass module-level callables
+    saver._global_rank_getter = saver._local_rank_getter = None
+    saver._test_calls = None
+    clone = pickle.loads(pickle.dumps(saver))
+    assert clone._initial_buffer_size_bytes == 123 and clone._crc_chunk_bytes == 1 << 20
+    assert clone._replication_manager is None and clone._engine is None and clone.kernel_events == []
+
+
+# ---- ids, hfid, header type -------------------------------------------------------------------------------------
+def test_checkpoint_ids():
+    c = CheckpointContainerId("/a/b/step-12_ckpt///")
+    assert c.data == "/a/b/step-12_ckpt" and str(c) == c.data
+    assert CheckpointContainerId.parse_version_container_step("step-12_ckpt") == 12
+    for bad in ("step-12", "step-x_ckpt", "xstep-1_ckpt", "step-1_ckpt_", "step--1_ckpt"):
+        assert CheckpointContainerId.parse_version_container_step(bad) is None
+    assert CheckpointContainerId.format_version_container(7) == "step-7_ckpt"
+    assert c.get_parent().data == "/a/b" and c.get_parent(2).data == "/a" and c.get_parent(3) is None
+    with pytest.raises(ValueError, match="levels_up"):
+        c.get_parent(0)
+    for bad, msg in (("a/b", "must begin with '/'"), ("/a//b", "cannot be empty"), ("/a/b.", "cannot end with a '.'"), ("/", "root path")):
+        with pytest.raises(ValueError, match=msg):
+            CheckpointContainerId(bad)
+    with pytest.raises(ValueError, match="not a valid leaf ID"):
+        CheckpointObjectId("/")
+    o = CheckpointObjectId.from_container(c, " /data_0_src3.distcp/ ")
+    assert o.data == "/a/b/step-12_ckpt/data_0_src3.distcp" and o.get_parent() == c
+    with pytest.raises(ValueError, match="must not be empty"):
+        CheckpointObjectId.from_container(c, " // ")
+    with pytest.raises(TypeError):
+        CheckpointObjectId.from_container("/a", "x")
+    assert CheckpointContainerId.create_child(c, "/").data == c.data
+    assert CheckpointContainerId.create_child(c, "/sub/dir/").data == c.data + "/sub/dir"
+    assert c == "/a/b/step-12_ckpt" and hash(c) == hash(CheckpointContainerId("/a/b/step-12_ckpt"))  # dict keys
+
+
+def test_hfid():
+    a, b = generate_hfid("memwritersave"), generate_hfid("memwritersave")
+    assert a != b and a.startswith("memwritersave_") and len(a.split("_")[1]) == 32
+    for bad in ("", "Has_Upper", "with-dash", "sp ace"):
+        with pytest.raises(ValueError):
+            generate_hfid(bad)
+
+
+def test_tensor_header_round_trip_and_length_prefix():
+    h = TensorHeader(dtype=torch.bfloat16, shape=torch.Size([4, 0, 3]))
+    raw = h.to_bytes()
+    assert int.from_bytes(raw[:4], "little") == len(raw) - 4
+    back, used = TensorHeader.from_bytes(raw + b"trailing payload")
+    assert used == len(raw) and back == h and isinstance(back.shape, torch.Size)
+
+
+def test_bucket_dataclass_is_replaceable():
+    import dataclasses
+
+    b = ObjectWriteBucket(CheckpointObjectId("/x/y"), "y", [], [])
+    c = dataclasses.replace(b, tensor_data=[("item", "tensor")])
+    assert c.object_id == b.object_id and c.tensor_data and not b.tensor_data

@@ -107,32 +107,48 @@ def mixtral_expert_shard(device, seed=87, layers=32, experts=8, d=4096, ffn=1433
     return sd
 
 
-def strided_views(device, seed=5, count=2000, min_dim=1024, max_dim=16384) -> Tuple[Dict[str, torch.Tensor], list]:
-    """C5: transposed / every-other-column / 16-row-block views of bf16 / fp8-e4m3 / fp32 parents whose bytes are
-    uniform random.  Returns (state dict of views, list of parents kept alive)."""
+def strided_views(device, seed=5, count=2000, min_dim=1024, max_dim=16384, n_parents=None,
+                  mean_view_bytes=10 << 20) -> Tuple[Dict[str, torch.Tensor], list]:
+    """C5: ``count`` non-contiguous views - transposed blocks, every-other-column slices and 16-row blocks - of
+    bf16 / fp8-e4m3 / fp32 parents with 1k..16k rows and columns (multiples of 16) whose bytes are uniform random.
+    Views average ``mean_view_bytes`` of payload (2000 x 10 MB = 20 GB) and share ``n_parents`` parents
+    (default count // 32).  Returns (state dict of views, list of parents kept alive)."""
     cpu = torch.Generator().manual_seed(seed)
     g = _gen(device, seed)
     dtypes = [torch.bfloat16, torch.float8_e4m3fn, torch.float32]
-    sd, parents = {}, []
+    n_parents = n_parents or max(3, count // 32)
     span = (max_dim - min_dim) // 16
-    for i in range(count):
-        rows = min_dim + 16 * int(torch.randint(0, span + 1, (1,), generator=cpu))
-        cols = min_dim + 16 * int(torch.randint(0, span + 1, (1,), generator=cpu))
-        dtype = dtypes[i % 3]
+
+    def rnd(lo, hi):  # integer in [lo, hi]
+        return lo + int(torch.randint(0, max(hi - lo, 0) + 1, (1,), generator=cpu))
+
+    parents = []
+    for p in range(n_parents):
+        rows, cols = min_dim + 16 * rnd(0, span), min_dim + 16 * rnd(0, span)
+        dtype = dtypes[p % 3]
         esz = torch.empty((), dtype=dtype).element_size()
         raw = torch.randint(0, 256, (rows * cols * esz,), generator=g, device=device, dtype=torch.uint8)
-        parent = raw.view(dtype).reshape(rows, cols)
-        parents.append(parent)
-        kind = (i // 3) % 3
-        if kind == 0:
-            view = parent.t()
-        elif kind == 1:
-            view = parent[:, ::2]
-        else:
-            blocks = rows // 16
-            k = int(torch.randint(0, blocks, (1,), generator=cpu))
-            r = int(torch.randint(1, blocks - k + 1, (1,), generator=cpu))
-            view = parent[16 * k : 16 * k + 16 * r, :]
+        parents.append(raw.view(dtype).reshape(rows, cols))
+    sd = {}
+    for i in range(count):
+        parent = parents[i % n_parents]
+        rows, cols = parent.shape
+        esz = parent.element_size()
+        want = rnd(mean_view_bytes // 5, 2 * mean_view_bytes - mean_view_bytes // 5) // esz  # elements, mean = target
+        kind = (i // n_parents) % 3
+        if kind == 0:  # transposed block: h x w of the parent, seen as w x h
+            h = 16 * rnd(4, min(rows, 4096) // 16)
+            w = max(16, min(cols, (want // h) // 16 * 16))
+            r0, c0 = 16 * rnd(0, (rows - h) // 16), 16 * rnd(0, (cols - w) // 16)
+            view = parent[r0 : r0 + h, c0 : c0 + w].t()
+        elif kind == 1:  # every other column of a band of rows
+            h = max(1, min(rows, want // (cols // 2)))
+            r0 = rnd(0, rows - h)
+            view = parent[r0 : r0 + h, ::2]
+        else:  # block of 16-row groups (contiguous in memory, but a view with a storage offset)
+            r = max(1, min(rows // 16, want // (16 * cols)))
+            k = rnd(0, rows // 16 - r)
+            view = parent[16 * k : 16 * (k + r), :]
         sd[f"views.{i}"] = view
     return sd, parents
 
