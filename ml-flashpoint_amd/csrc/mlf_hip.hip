@@ -15,7 +15,10 @@
 //     this ordering is worth ~25 % over long-running workgroups that each stream a large private region.
 //     Tiles are not listed one by one: a table entry ("span") describes up to 128 (or 16, or 1) consecutive
 //     tiles of one contiguous item and the workgroups that share it derive their tile from blockIdx.
-//   * strided kernel: generic N-d index walk for non-contiguous sources/targets and sub-box restores.
+//   * transpose kernel: views whose contiguous dimension differs between tensor and image (e.g. `.t()`) go
+//     through an LDS tile so that both sides see whole consecutive runs.
+//   * strided kernel: generic, division-free N-d index walk for every other non-contiguous source/target and
+//     for sub-box restores.
 //   * crc kernel: per wavefront a 64 KiB segment is read as coalesced 1 KiB rows; every lane keeps four
 //     Horner accumulators advanced by x^8192 through LDS tables, then lanes are folded with GF(2) multiplies.
 #include "mlf_hip.h"
@@ -83,12 +86,38 @@ struct StridedDesc {
   int64_t shape[MLF_MAX_DIMS];
   int64_t tstride[MLF_MAX_DIMS];  // bytes
   int64_t istride[MLF_MAX_DIMS];  // bytes
+  int64_t step[MLF_MAX_DIMS];     // 256 written in the mixed radix of `shape`: what one loop trip adds to the index
 };
 
 struct StridedWork {  // one workgroup's work: elements [start, start+count) of descriptor `desc`
   uint64_t start;
   uint32_t count;
   uint32_t desc;
+};
+
+constexpr int kMaxBatchDims = MLF_MAX_DIMS - 2;
+constexpr uint32_t kTransTilesPerEntry = 256;
+
+// A 2-D transposition (plus outer "batch" dims): dim a is contiguous on the tensor side, dim b on the image side.
+struct TransDesc {
+  uint64_t tensor;  // device address of element 0
+  uint64_t image;   // byte offset of element 0 in the image
+  uint32_t esz;
+  uint32_t nbatch;
+  int64_t na, nb;   // extents of a and b
+  int64_t ld_t;     // tensor-side byte stride of dim b (dim a has byte stride esz there)
+  int64_t ld_i;     // image-side byte stride of dim a  (dim b has byte stride esz there)
+  uint32_t tiles_a, tiles_b;
+  uint64_t n_tiles;  // batch count * tiles_a * tiles_b
+  int64_t bshape[kMaxBatchDims];
+  int64_t bts[kMaxBatchDims];  // bytes
+  int64_t bis[kMaxBatchDims];  // bytes
+};
+
+struct TransWork {  // kTransTilesPerEntry consecutive tiles of descriptor `desc`, starting at `first_tile`
+  uint64_t first_tile;
+  uint32_t desc;
+  uint32_t pad;
 };
 
 
@@ -157,36 +186,161 @@ __device__ __forceinline__ void copy_elem(char* dst, const char* src) {
   *reinterpret_cast<unaligned_t*>(dst) = *reinterpret_cast<const unaligned_t*>(src);
 }
 
+// Generic N-d walk.  A thread decomposes its first element index once (divisions), then advances the multi-index
+// by the block size with one add-and-carry per dimension per trip: no division in the loop.
+template <bool PACK, typename T>
+__device__ __forceinline__ void strided_walk(const StridedDesc* __restrict__ d, const StridedWork& w,
+                                             char* __restrict__ image) {
+  const int ndim = (int)d->ndim;
+  char* tbase = reinterpret_cast<char*>(d->tensor);
+  char* ibase = image + d->image;
+  int64_t idx[MLF_MAX_DIMS];
+  {
+    uint64_t e = w.start + threadIdx.x;
+#pragma unroll
+    for (int dim = MLF_MAX_DIMS - 1; dim >= 0; --dim) {
+      idx[dim] = 0;
+      if (dim < ndim) {
+        const uint64_t extent = (uint64_t)d->shape[dim];
+        const uint64_t q = e / extent;
+        idx[dim] = (int64_t)(e - q * extent);
+        e = q;
+      }
+    }
+  }
+  for (uint32_t k = threadIdx.x; k < w.count; k += 256) {
+    int64_t toff = 0, ioff = 0;
+#pragma unroll
+    for (int dim = 0; dim < MLF_MAX_DIMS; ++dim) {
+      if (dim < ndim) {
+        toff += idx[dim] * d->tstride[dim];
+        ioff += idx[dim] * d->istride[dim];
+      }
+    }
+    copy_elem<T>(PACK ? ibase + ioff : tbase + toff, PACK ? tbase + toff : ibase + ioff);
+    int64_t carry = 0;
+#pragma unroll
+    for (int dim = MLF_MAX_DIMS - 1; dim >= 0; --dim) {
+      if (dim < ndim) {
+        int64_t v = idx[dim] + d->step[dim] + carry;
+        carry = 0;
+        if (v >= d->shape[dim]) {
+          v -= d->shape[dim];
+          carry = 1;
+        }
+        idx[dim] = v;
+      }
+    }
+  }
+}
+
 template <bool PACK>
 __global__ void __launch_bounds__(256) mlf_strided_kernel(const StridedDesc* __restrict__ descs,
                                                           const StridedWork* __restrict__ work,
                                                           char* __restrict__ image) {
   const StridedWork w = work[blockIdx.x];
   const StridedDesc* __restrict__ d = descs + w.desc;
-  const uint32_t esz = d->esz;
-  const int ndim = (int)d->ndim;
-  char* tbase = reinterpret_cast<char*>(d->tensor);
-  char* ibase = image + d->image;
-  for (uint32_t k = threadIdx.x; k < w.count; k += blockDim.x) {
-    uint64_t e = w.start + k;
-    int64_t toff = 0, ioff = 0;
-    for (int dim = ndim - 1; dim >= 0; --dim) {
-      const uint64_t extent = (uint64_t)d->shape[dim];
-      const uint64_t q = e / extent;
-      const int64_t idx = (int64_t)(e - q * extent);
-      e = q;
-      toff += idx * d->tstride[dim];
-      ioff += idx * d->istride[dim];
+  switch (d->esz) {
+    case 1: strided_walk<PACK, uint8_t>(d, w, image); break;
+    case 2: strided_walk<PACK, uint16_t>(d, w, image); break;
+    case 4: strided_walk<PACK, uint32_t>(d, w, image); break;
+    case 8: strided_walk<PACK, uint64_t>(d, w, image); break;
+    default: strided_walk<PACK, u32x4>(d, w, image); break;  // 16
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// transpose kernel (LDS-tiled)
+// ---------------------------------------------------------------------------------------------------------
+// One workgroup moves one T x T tile of a 2-D transposition through LDS so that both the read (along the source's
+// contiguous dimension) and the write (along the destination's) are made of whole, consecutive >= 128-byte runs.
+// Global accesses are max(4, esz)-byte vectors (hardware-unaligned where the view starts off a boundary); LDS is
+// addressed per element on the transposed side.  T = 128 / 64 / 64 / 32 / 16 elements for esz = 1 / 2 / 4 / 8 / 16;
+// rows of the LDS tile are padded by one vector so that a column walk does not stay in one bank.
+constexpr uint32_t kTransLdsBytes = 128 * (128 + 4);
+
+__host__ __device__ inline uint32_t trans_tile_dim(uint32_t esz) {
+  return esz == 1 ? 128u : esz <= 4 ? 64u : esz == 8 ? 32u : 16u;
+}
+
+template <bool PACK, typename E, typename V>
+__device__ __forceinline__ void trans_tile(const TransDesc* __restrict__ d, uint64_t tile, char* __restrict__ image,
+                                           char* __restrict__ lds) {
+  constexpr uint32_t ESZ = sizeof(E), VEC = sizeof(V), EPV = VEC / ESZ;
+  const uint32_t T = trans_tile_dim(ESZ);
+  const uint32_t pitch = T * ESZ + VEC;
+  typedef V vec_u __attribute__((aligned(1)));
+  typedef E elem_u __attribute__((aligned(1)));
+
+  // which tile: batch index, then tile row (a) and tile column (b); b runs fastest
+  const uint64_t per_batch = (uint64_t)d->tiles_a * d->tiles_b;
+  uint64_t batch = tile / per_batch;
+  const uint32_t rem = (uint32_t)(tile - batch * per_batch);
+  const uint32_t ta = rem / d->tiles_b, tb = rem - ta * d->tiles_b;
+  int64_t toff = 0, ioff = 0;
+  for (int k = (int)d->nbatch - 1; k >= 0; --k) {
+    const uint64_t extent = (uint64_t)d->bshape[k];
+    const uint64_t q = batch / extent;
+    const int64_t i = (int64_t)(batch - q * extent);
+    batch = q;
+    toff += i * d->bts[k];
+    ioff += i * d->bis[k];
+  }
+  const int64_t a0 = (int64_t)ta * T, b0 = (int64_t)tb * T;
+  // x: the source's contiguous dimension, y: the destination's
+  const int64_t nx = PACK ? d->na : d->nb, ny = PACK ? d->nb : d->na;
+  const int64_t x0 = PACK ? a0 : b0, y0 = PACK ? b0 : a0;
+  const int64_t ld_src = PACK ? d->ld_t : d->ld_i, ld_dst = PACK ? d->ld_i : d->ld_t;
+  const char* src = (PACK ? reinterpret_cast<const char*>(d->tensor) + toff : image + d->image + ioff) + x0 * ESZ + y0 * ld_src;
+  char* dst = (PACK ? image + d->image + ioff : reinterpret_cast<char*>(d->tensor) + toff) + x0 * ld_dst + y0 * ESZ;
+  const uint32_t xn = (uint32_t)(nx - x0 < (int64_t)T ? nx - x0 : T);  // valid extent of this tile
+  const uint32_t yn = (uint32_t)(ny - y0 < (int64_t)T ? ny - y0 : T);
+  const uint32_t vec_per_row = T / EPV, n_vec = T * vec_per_row;
+
+  for (uint32_t v = threadIdx.x; v < n_vec; v += 256) {
+    const uint32_t y = v / vec_per_row, x = (v - y * vec_per_row) * EPV;
+    if (y >= yn || x >= xn) continue;
+    const char* g = src + (int64_t)y * ld_src + (int64_t)x * ESZ;
+    char* l = lds + y * pitch + x * ESZ;
+    if (x + EPV <= xn) {
+      *reinterpret_cast<V*>(l) = *reinterpret_cast<const vec_u*>(g);
+    } else {
+      for (uint32_t k = 0; x + k < xn; ++k) reinterpret_cast<E*>(l)[k] = reinterpret_cast<const elem_u*>(g)[k];
     }
-    const char* s = PACK ? tbase + toff : ibase + ioff;
-    char* o = PACK ? ibase + ioff : tbase + toff;
-    switch (esz) {
-      case 1: *o = *s; break;
-      case 2: copy_elem<uint16_t>(o, s); break;
-      case 4: copy_elem<uint32_t>(o, s); break;
-      case 8: copy_elem<uint64_t>(o, s); break;
-      default: copy_elem<u32x4>(o, s); break;  // 16
+  }
+  __syncthreads();
+  for (uint32_t v = threadIdx.x; v < n_vec; v += 256) {
+    const uint32_t x = v / vec_per_row, y = (v - x * vec_per_row) * EPV;
+    if (x >= xn || y >= yn) continue;
+    char* g = dst + (int64_t)x * ld_dst + (int64_t)y * ESZ;
+    const char* l = lds + y * pitch + x * ESZ;
+    if (y + EPV <= yn) {
+      V out;
+      E* parts = reinterpret_cast<E*>(&out);
+#pragma unroll
+      for (uint32_t k = 0; k < EPV; ++k) parts[k] = *reinterpret_cast<const E*>(l + k * pitch);
+      *reinterpret_cast<vec_u*>(g) = out;
+    } else {
+      for (uint32_t k = 0; y + k < yn; ++k) reinterpret_cast<elem_u*>(g)[k] = *reinterpret_cast<const E*>(l + k * pitch);
     }
+  }
+}
+
+template <bool PACK>
+__global__ void __launch_bounds__(256) mlf_transpose_kernel(const TransDesc* __restrict__ descs,
+                                                            const TransWork* __restrict__ work,
+                                                            char* __restrict__ image) {
+  __shared__ __attribute__((aligned(16))) char lds[kTransLdsBytes];
+  const TransWork w = work[blockIdx.x / kTransTilesPerEntry];
+  const TransDesc* __restrict__ d = descs + w.desc;
+  const uint64_t tile = w.first_tile + (blockIdx.x % kTransTilesPerEntry);
+  if (tile >= d->n_tiles) return;  // uniform per workgroup: nobody reaches the barrier
+  switch (d->esz) {
+    case 1: trans_tile<PACK, uint8_t, uint32_t>(d, tile, image, lds); break;
+    case 2: trans_tile<PACK, uint16_t, uint32_t>(d, tile, image, lds); break;
+    case 4: trans_tile<PACK, uint32_t, uint32_t>(d, tile, image, lds); break;
+    case 8: trans_tile<PACK, uint64_t, uint64_t>(d, tile, image, lds); break;
+    default: trans_tile<PACK, u32x4, u32x4>(d, tile, image, lds); break;  // 16
   }
 }
 
@@ -469,6 +623,8 @@ struct mlf_plan {
   uint32_t tile_bytes = 4096;
   StridedDesc* d_descs = nullptr;
   StridedWork* d_work = nullptr;
+  TransDesc* d_tdescs = nullptr;
+  TransWork* d_twork = nullptr;
   char* d_blob = nullptr;
   uint32_t block_threads = 256;
   uint32_t unroll = 1;
@@ -599,6 +755,8 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
   SpanTables tiles;
   std::vector<StridedDesc> descs;
   std::vector<StridedWork> work;
+  std::vector<TransDesc> tdescs;
+  std::vector<TransWork> twork;
   mlf_plan_info& info = plan->info;
   info.n_items = n_items;
   info.image_bytes = image_bytes;
@@ -679,6 +837,41 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
       }
       continue;
     }
+    // a dimension other than the last that is contiguous on the tensor side while the last one is contiguous on
+    // the image side: a transposition.  Both extents must be worth a tile.
+    if (c.is[last] == 1 && c.ts[last] != 1 && c.shape[last] >= 16) {
+      int a = -1;
+      for (int d = 0; d < last; ++d)
+        if (c.ts[d] == 1 && c.shape[d] >= 16) a = d;
+      if (a >= 0) {
+        TransDesc td{};
+        td.tensor = it.ptr;
+        td.image = it.image_off;
+        td.esz = esz;
+        td.na = c.shape[a];
+        td.nb = c.shape[last];
+        td.ld_t = c.ts[last] * (int64_t)esz;
+        td.ld_i = c.is[a] * (int64_t)esz;
+        const uint32_t T = trans_tile_dim(esz);
+        td.tiles_a = (uint32_t)((td.na + T - 1) / T);
+        td.tiles_b = (uint32_t)((td.nb + T - 1) / T);
+        uint64_t batches = 1;
+        for (int d = 0; d < last; ++d) {
+          if (d == a) continue;
+          td.bshape[td.nbatch] = c.shape[d];
+          td.bts[td.nbatch] = c.ts[d] * (int64_t)esz;
+          td.bis[td.nbatch] = c.is[d] * (int64_t)esz;
+          ++td.nbatch;
+          batches *= (uint64_t)c.shape[d];
+        }
+        td.n_tiles = batches * td.tiles_a * td.tiles_b;
+        const uint32_t tdesc_idx = (uint32_t)tdescs.size();
+        tdescs.push_back(td);
+        for (uint64_t first = 0; first < td.n_tiles; first += kTransTilesPerEntry) twork.push_back(TransWork{first, tdesc_idx, 0});
+        ++info.n_transposed_items;
+        continue;
+      }
+    }
     StridedDesc sd{};
     sd.tensor = it.ptr;
     sd.image = it.image_off;
@@ -688,6 +881,13 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
       sd.shape[d] = c.shape[d];
       sd.tstride[d] = c.ts[d] * (int64_t)esz;
       sd.istride[d] = c.is[d] * (int64_t)esz;
+    }
+    {  // 256 in the mixed radix of the collapsed shape (least significant digit = last dimension)
+      uint64_t rest = 256;
+      for (int d = c.ndim - 1; d >= 0; --d) {
+        sd.step[d] = (int64_t)(rest % (uint64_t)c.shape[d]);
+        rest /= (uint64_t)c.shape[d];
+      }
     }
     const uint32_t desc_idx = (uint32_t)descs.size();
     descs.push_back(sd);
@@ -701,6 +901,8 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
   }
   if (rc == MLF_HIP_OK) rc = upload(descs, &plan->d_descs);
   if (rc == MLF_HIP_OK) rc = upload(work, &plan->d_work);
+  if (rc == MLF_HIP_OK) rc = upload(tdescs, &plan->d_tdescs);
+  if (rc == MLF_HIP_OK) rc = upload(twork, &plan->d_twork);
   if (rc != MLF_HIP_OK) {
     std::string keep = g_err;
     mlf_plan_destroy(plan.release());
@@ -708,7 +910,9 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
     return rc;
   }
   info.n_flat_tiles = 0;
-  info.table_bytes = descs.size() * sizeof(StridedDesc) + work.size() * sizeof(StridedWork) + blob_bytes;
+  info.table_bytes = descs.size() * sizeof(StridedDesc) + work.size() * sizeof(StridedWork) +
+                     tdescs.size() * sizeof(TransDesc) + twork.size() * sizeof(TransWork) + blob_bytes;
+  info.n_transposed_work = twork.size();
   for (int c = 0; c < kSpanClasses; ++c) {
     info.n_flat_tiles += plan->n_spans[c] << kSpanShift[c];
     info.table_bytes += plan->n_spans[c] * sizeof(Span);
@@ -723,6 +927,8 @@ int mlf_plan_destroy(mlf_plan* plan) {
   for (Span* t : plan->d_spans) (void)hipFree(t);
   (void)hipFree(plan->d_descs);
   (void)hipFree(plan->d_work);
+  (void)hipFree(plan->d_tdescs);
+  (void)hipFree(plan->d_twork);
   (void)hipFree(plan->d_blob);
   delete plan;
   return MLF_HIP_OK;
@@ -760,6 +966,12 @@ int launch_plan(const mlf_plan* plan, char* image, hipStream_t stream) {
       }
       HIP_TRY(hipGetLastError());
     }
+  }
+  for (uint64_t first = 0; first < plan->info.n_transposed_work; first += (1u << 15)) {
+    const uint64_t count = std::min<uint64_t>(1u << 15, plan->info.n_transposed_work - first);
+    hipLaunchKernelGGL((mlf_transpose_kernel<PACK>), dim3((uint32_t)(count * kTransTilesPerEntry)), dim3(256), 0, stream,
+                       plan->d_tdescs, plan->d_twork + first, image);
+    HIP_TRY(hipGetLastError());
   }
   for (uint64_t first = 0; first < plan->info.n_strided_work; first += (1u << 23)) {
     const uint64_t count = std::min<uint64_t>(1u << 23, plan->info.n_strided_work - first);

@@ -124,6 +124,91 @@ def test_pack_strided_views_match_bruteforce_oracle(dtype):
     assert plan.info.n_strided_items > 0
 
 
+TRANSPOSE_SHAPES = [(16, 16), (17, 130), (128, 128), (129, 257), (300, 31), (64, 1000), (5, 40, 70)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.bfloat16, torch.float32, torch.int64, torch.complex128])
+def test_transposed_views_pack_and_unpack_through_lds_tiles(dtype):
+    """`.t()`-like views (tensor-contiguous dimension != image-contiguous dimension), tile-multiple and ragged
+    extents, with and without batch dimensions and storage offsets; both directions."""
+    from ml_flashpoint.hip import plan as P
+
+    gen = torch.Generator().manual_seed(31)
+    cpu_views, dev_views = [], []
+    for shape in TRANSPOSE_SHAPES:
+        parent = _rand_tensor(gen, tuple(d + 3 for d in shape), dtype)
+        dev_parent = parent.to(DEV)
+        sl = tuple(slice(1, 1 + d) for d in shape)
+        cpu_views.append(parent[sl].transpose(-1, -2))
+        dev_views.append(dev_parent[sl].transpose(-1, -2))
+    layout, plan, image, got = _pack_image(dev_views)
+    assert plan.info.n_transposed_items == len(TRANSPOSE_SHAPES) and plan.info.n_strided_items == 0
+    want, spans = oracle_fmt.data_section(cpu_views)
+    assert got == want
+    assert got == b"".join(
+        oracle_fmt.header_bytes(oracle_fmt.dtype_name(t.dtype), tuple(t.shape)) + oracle_fmt.payload_bytes_bruteforce(t)
+        for t in cpu_views[:3]
+    ) + want[spans[3][0] :]
+    # restore the image into transposed targets embedded in larger zeroed parents
+    table = P.ItemTable()
+    parents, targets = [], []
+    for view, (off, length) in zip(cpu_views, spans):
+        tshape = tuple(view.shape[:-2]) + (view.shape[-1] + 2, view.shape[-2] + 5)
+        parent = torch.zeros(tshape, dtype=torch.uint8 if dtype == torch.float8_e4m3fn else dtype, device=DEV)
+        parent = parent.view(dtype) if dtype == torch.float8_e4m3fn else parent
+        target = parent[..., 2:, 5:].transpose(-1, -2)
+        assert target.shape == view.shape
+        nbytes = view.numel() * view.element_size()
+        table.add_device(target.data_ptr(), off + length - nbytes, view.element_size(), tuple(view.shape), tuple(target.stride()))
+        parents.append(parent)
+        targets.append(target)
+    uplan = P.Plan(table.to_array(), b"", layout.image_bytes, align_to_tensor=True)
+    assert uplan.info.n_transposed_items == len(TRANSPOSE_SHAPES)
+    uplan.unpack(image)
+    torch.cuda.synchronize()
+    for view, target, parent in zip(cpu_views, targets, parents):
+        assert torch.equal(target.cpu().contiguous().reshape(-1).view(torch.uint8), view.contiguous().reshape(-1).view(torch.uint8))
+        p8 = parent.cpu().reshape(-1).view(torch.uint8)
+        assert int(p8.count_nonzero()) <= view.numel() * view.element_size()  # nothing outside the target was touched
+        assert int(parent[..., :2, :].cpu().reshape(-1).view(torch.uint8).count_nonzero()) == 0
+        assert int(parent[..., :, :5].cpu().reshape(-1).view(torch.uint8).count_nonzero()) == 0
+
+
+def test_strided_walk_many_shapes_against_bruteforce():
+    """The division-free index walk: inner extents smaller and larger than the block, up to 5 dims, both directions."""
+    from ml_flashpoint.hip import plan as P
+
+    gen = torch.Generator().manual_seed(32)
+    base = _rand_tensor(gen, (7, 6, 5, 9, 11), torch.int16)
+    dev = base.to(DEV)
+    pick = lambda t: [  # noqa: E731
+        t[::2, :, ::2, :, ::3],
+        t[:, 1:4, :, ::4, 2:9:2],
+        t.permute(4, 2, 0, 1, 3)[::2],
+        t[3, :, :, :, ::5],
+        t[..., ::7],
+        t[:, :, :, 1, 1],
+        t.flatten()[3::13],
+    ]
+    cpu_views, dev_views = pick(base), pick(dev)
+    layout, plan, image, got = _pack_image(dev_views)
+    assert plan.info.n_strided_items == len(cpu_views)
+    want = b"".join(
+        oracle_fmt.header_bytes("int16", tuple(t.shape)) + oracle_fmt.payload_bytes_bruteforce(t) for t in cpu_views
+    )
+    assert got == want
+    back = torch.zeros_like(dev)
+    table = P.ItemTable()
+    for src, tgt, (off, length) in zip(cpu_views, pick(back), layout.spans):
+        table.add_device(tgt.data_ptr(), off + length - src.numel() * 2, 2, tuple(src.shape), tuple(tgt.stride()))
+    P.Plan(table.to_array(), b"", layout.image_bytes, align_to_tensor=True).unpack(image)
+    torch.cuda.synchronize()
+    mask = torch.zeros_like(base, dtype=torch.bool)
+    for m in pick(mask):
+        m.fill_(True)
+    assert torch.equal(back.cpu()[mask], base[mask]) and int(back.cpu()[~mask].abs().sum()) == 0
+
+
 def test_pack_large_rows_go_through_flat_kernel():
     gen = torch.Generator().manual_seed(15)
     base_cpu = _rand_tensor(gen, (64, 8192), torch.bfloat16)
