@@ -76,6 +76,7 @@ typedef struct mlf_plan_info {
   uint64_t blob_bytes;        /* bytes that come from the host blob                                            */
   uint64_t image_bytes;
   uint64_t table_bytes;       /* device memory held by the plan's tables + blob                                */
+  uint64_t n_small_items;     /* pieces of at most 1 KiB that are copied one per wavefront                     */
 } mlf_plan_info;
 
 typedef struct mlf_plan mlf_plan;
@@ -140,6 +141,14 @@ int mlf_engine_destroy(mlf_engine* engine);
  * copy_ into the mapping.  Safe to call from a thread other than the one that launched the pack. */
 int mlf_engine_d2h(mlf_engine* engine, const void* src_dev, void* dst_host, uint64_t nbytes,
                    void* producer_stream, mlf_xfer_stats* stats);
+
+/* mlf_engine_d2h that also checksums what it sends: CRC-32C of every `crc_chunk_bytes` piece of the source
+ * (same definition and constraints as mlf_crc32c_device), computed on a third stream while the copies run, so
+ * the check costs no blocking time and no transfer time.  `crc_out_host` receives ceil(nbytes/crc_chunk_bytes)
+ * values before the call returns.  No reference counterpart (the reference has no checksum). */
+int mlf_engine_d2h_crc(mlf_engine* engine, const void* src_dev, void* dst_host, uint64_t nbytes,
+                       void* producer_stream, uint64_t crc_chunk_bytes, uint32_t* crc_out_host,
+                       uint64_t n_crc_out, mlf_xfer_stats* stats);
 
 /* Host -> device.  Copies `nbytes` from `src_host` (pageable, e.g. the read-only mapping) to `dst_dev`
  * and makes `consumer_stream` wait for the last chunk, so an unpack launched on it afterwards sees the data.

@@ -177,6 +177,36 @@ __global__ void __launch_bounds__(1024) mlf_flat_kernel(const Span* __restrict__
   }
 }
 
+// Items of at most 1 KiB (record headers, scalars, step counters, the tails of small tensors): one wavefront per
+// item, four items per workgroup, so that thousands of tiny items do not each occupy a workgroup of their own.
+constexpr uint32_t kSmallItemBytes = 1024;
+
+template <bool PACK>
+__global__ void __launch_bounds__(256) mlf_small_kernel(const Span* __restrict__ spans, uint32_t n_spans,
+                                                        char* __restrict__ image) {
+  const uint32_t item = blockIdx.x * 4u + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  if (item >= n_spans) return;
+  const uint32_t lane = threadIdx.x & 63u;
+  const Span sp = spans[item];
+  const char* src = PACK ? reinterpret_cast<const char*>(sp.tensor) : image + sp.image;
+  char* dst = PACK ? image + sp.image : reinterpret_cast<char*>(sp.tensor);
+  uint32_t n = sp.n;
+  uint32_t head = (16u - (uint32_t)(reinterpret_cast<uintptr_t>(dst) & 15u)) & 15u;
+  head = head < n ? head : n;
+  if (lane < head) dst[lane] = src[lane];
+  src += head;
+  dst += head;
+  n -= head;
+  const uint32_t nvec = n >> 4;  // <= 64: one vector per lane
+  if (lane < nvec)
+    reinterpret_cast<u32x4*>(dst)[lane] = *reinterpret_cast<const u32x4_u*>(src + (size_t)lane * 16);
+  const uint32_t tail = n & 15u;
+  if (lane < tail) {
+    const uint32_t o = (nvec << 4) + lane;
+    dst[o] = src[o];
+  }
+}
+
 // ---------------------------------------------------------------------------------------------------------
 // strided kernel (generic)
 // ---------------------------------------------------------------------------------------------------------
@@ -464,6 +494,75 @@ void crc_init_host() {
   g_crc_host.xseg = x_pow_bytes(kCrcSegBytes);
 }
 
+// A CRC pass in flight: scratch on the device, results in a pinned host array, all ordered on `stream`.
+struct CrcJob {
+  CrcConsts* d_consts = nullptr;
+  uint32_t* d_seg = nullptr;
+  uint32_t* d_out = nullptr;
+  uint32_t* h_out = nullptr;  // pinned
+  uint64_t n_chunks = 0;
+  hipStream_t stream = nullptr;
+};
+
+void crc_release(CrcJob* job) {
+  (void)hipFree(job->d_consts);
+  (void)hipFree(job->d_seg);
+  (void)hipFree(job->d_out);
+  if (job->h_out) (void)hipHostFree(job->h_out);
+  *job = CrcJob();
+}
+
+// Enqueues the two CRC kernels and the copy of the per-chunk values on `stream`; does not wait.
+int crc_enqueue(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint64_t n_out, hipStream_t stream,
+                CrcJob* job) {
+  if (!dev_ptr) return fail(MLF_HIP_BAD_ARG, "null pointer");
+  if (reinterpret_cast<uintptr_t>(dev_ptr) & 15) return fail(MLF_HIP_BAD_ARG, "device buffer must be 16-byte aligned");
+  if (chunk_bytes == 0 || chunk_bytes % kCrcSegBytes)
+    return fail(MLF_HIP_BAD_ARG, "chunk_bytes must be a positive multiple of 65536");
+  const uint64_t n_chunks = (nbytes + chunk_bytes - 1) / chunk_bytes;
+  const uint64_t n_segs = (nbytes + kCrcSegBytes - 1) / kCrcSegBytes;
+  if (n_out < n_chunks) return fail(MLF_HIP_BAD_ARG, "output array too small");
+  if (n_segs > 0xFFFFFFF0ull) return fail(MLF_HIP_BAD_ARG, "buffer too large for one CRC call");
+  std::call_once(g_crc_once, crc_init_host);
+  job->n_chunks = n_chunks;
+  job->stream = stream;
+#define CRC_TRY(expr)                                                                             \
+  do {                                                                                            \
+    hipError_t e__ = (expr);                                                                      \
+    if (e__ != hipSuccess) {                                                                      \
+      crc_release(job);                                                                           \
+      return fail(MLF_HIP_RUNTIME, std::string(#expr) + " failed: " + hipGetErrorString(e__));    \
+    }                                                                                             \
+  } while (0)
+  CRC_TRY(hipMalloc(reinterpret_cast<void**>(&job->d_consts), sizeof(CrcConsts)));
+  CRC_TRY(hipMalloc(reinterpret_cast<void**>(&job->d_seg), n_segs * sizeof(uint32_t)));
+  CRC_TRY(hipMalloc(reinterpret_cast<void**>(&job->d_out), n_chunks * sizeof(uint32_t)));
+  CRC_TRY(hipHostMalloc(reinterpret_cast<void**>(&job->h_out), n_chunks * sizeof(uint32_t), hipHostMallocDefault));
+  CRC_TRY(hipMemcpyAsync(job->d_consts, &g_crc_host, sizeof(CrcConsts), hipMemcpyHostToDevice, stream));
+  const uint32_t grid = (uint32_t)((n_segs + 3) / 4);
+  hipLaunchKernelGGL(mlf_crc_segments_kernel, dim3(grid), dim3(256), 0, stream, static_cast<const char*>(dev_ptr),
+                     nbytes, job->d_consts, job->d_seg, (uint32_t)n_segs);
+  CRC_TRY(hipGetLastError());
+  const uint64_t last_seg_len = nbytes - (n_segs - 1) * kCrcSegBytes;
+  hipLaunchKernelGGL(mlf_crc_chunks_kernel, dim3((uint32_t)((n_chunks + 63) / 64)), dim3(64), 0, stream, job->d_seg,
+                     (uint32_t)(chunk_bytes / kCrcSegBytes), (uint32_t)n_segs, g_crc_host.xseg,
+                     x_pow_bytes(last_seg_len), job->d_out, (uint32_t)n_chunks);
+  CRC_TRY(hipGetLastError());
+  CRC_TRY(hipMemcpyAsync(job->h_out, job->d_out, n_chunks * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+#undef CRC_TRY
+  return MLF_HIP_OK;
+}
+
+// Waits for the job, hands the values out and frees the scratch.
+int crc_finish(CrcJob* job, uint32_t* out_host) {
+  hipError_t e = hipStreamSynchronize(job->stream);
+  if (e == hipSuccess && out_host) memcpy(out_host, job->h_out, job->n_chunks * sizeof(uint32_t));
+  crc_release(job);
+  if (e != hipSuccess) return fail(MLF_HIP_RUNTIME, std::string("hipStreamSynchronize failed: ") + hipGetErrorString(e));
+  if (!out_host) return fail(MLF_HIP_BAD_ARG, "null pointer");
+  return MLF_HIP_OK;
+}
+
 // ---------------------------------------------------------------------------------------------------------
 // host thread pool: run(n, fn) executes fn(0..n-1) on the pool's threads plus the caller
 // ---------------------------------------------------------------------------------------------------------
@@ -613,13 +712,14 @@ int pool_host_copy(WorkerPool& pool, const HostEnd& host, uint64_t host_off, cha
 // ---------------------------------------------------------------------------------------------------------
 // plan
 // ---------------------------------------------------------------------------------------------------------
-constexpr int kSpanClasses = 3;
-constexpr uint32_t kSpanShift[kSpanClasses] = {7, 4, 0};  // 128, 16 or 1 tiles per table entry
+constexpr int kSpanClasses = 4;
+constexpr int kSmallClass = 3;  // items <= kSmallItemBytes: served per wavefront by mlf_small_kernel
+constexpr uint32_t kSpanShift[kSpanClasses] = {7, 4, 0, 0};  // 128, 16 or 1 tiles per table entry
 
 struct mlf_plan {
   int device = 0;
-  Span* d_spans[kSpanClasses] = {nullptr, nullptr, nullptr};
-  uint64_t n_spans[kSpanClasses] = {0, 0, 0};
+  Span* d_spans[kSpanClasses] = {nullptr, nullptr, nullptr, nullptr};
+  uint64_t n_spans[kSpanClasses] = {0, 0, 0, 0};
   uint32_t tile_bytes = 4096;
   StridedDesc* d_descs = nullptr;
   StridedWork* d_work = nullptr;
@@ -641,7 +741,7 @@ struct SpanTables {
 };
 
 // Covers [0, n) of one contiguous item with spans: as many 128-tile entries as fit, then 16-tile entries, then
-// single tiles.  Every entry is self-contained (the kernel derives tile cuts from the entry's own first
+// single tiles; a rest of at most 1 KiB goes to the per-wavefront table.  Every entry is self-contained (the kernel derives tile cuts from the entry's own first
 // destination address), so pieces may start anywhere.
 void cut_spans(SpanTables& out, uint64_t tensor_addr, uint64_t image_off, uint64_t n, uint32_t tile,
                bool align_to_tensor) {
@@ -650,8 +750,12 @@ void cut_spans(SpanTables& out, uint64_t tensor_addr, uint64_t image_off, uint64
     const uint64_t dst_addr = (align_to_tensor ? tensor_addr : image_off) + done;  // image base is 256-byte aligned
     const uint64_t head = (16 - (dst_addr & 15)) & 15;
     const uint64_t left = n - done;
-    int c = kSpanClasses - 1;
-    for (int k = 0; k < kSpanClasses; ++k) {
+    if (left <= kSmallItemBytes) {
+      out.cls[kSmallClass].push_back(Span{tensor_addr + done, image_off + done, (uint32_t)left, 0});
+      break;
+    }
+    int c = kSmallClass - 1;
+    for (int k = 0; k < kSmallClass; ++k) {
       if (left >= ((uint64_t)tile << kSpanShift[k])) {
         c = k;
         break;
@@ -660,7 +764,7 @@ void cut_spans(SpanTables& out, uint64_t tensor_addr, uint64_t image_off, uint64
     // a full entry of class c holds (tile << shift) bytes; the single-tile class also takes the short rest,
     // and its first tile may carry the head bytes on top
     uint64_t len = (uint64_t)tile << kSpanShift[c];
-    if (c == kSpanClasses - 1) len = std::min<uint64_t>(left, tile + head);
+    if (c == kSmallClass - 1) len = std::min<uint64_t>(left, tile + head);
     len = std::min(len, left);
     out.cls[c].push_back(Span{tensor_addr + done, image_off + done, (uint32_t)len, 0});
     done += len;
@@ -914,9 +1018,10 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
                      tdescs.size() * sizeof(TransDesc) + twork.size() * sizeof(TransWork) + blob_bytes;
   info.n_transposed_work = twork.size();
   for (int c = 0; c < kSpanClasses; ++c) {
-    info.n_flat_tiles += plan->n_spans[c] << kSpanShift[c];
+    if (c != kSmallClass) info.n_flat_tiles += plan->n_spans[c] << kSpanShift[c];
     info.table_bytes += plan->n_spans[c] * sizeof(Span);
   }
+  info.n_small_items = plan->n_spans[kSmallClass];
   info.n_strided_work = work.size();
   *out = plan.release();
   return MLF_HIP_OK;
@@ -951,7 +1056,7 @@ int launch_plan(const mlf_plan* plan, char* image, hipStream_t stream) {
   if (reinterpret_cast<uintptr_t>(image) & 255) return fail(MLF_HIP_BAD_ARG, "image must be 256-byte aligned");
   // a launch may not exceed 2^32 - 1 threads in total, so large tables go out in several launches
   const uint64_t max_blocks = 0xFFFFFFFFull / plan->block_threads;
-  for (int c = 0; c < kSpanClasses; ++c) {
+  for (int c = 0; c < kSmallClass; ++c) {
     const uint32_t shift = kSpanShift[c], tile = plan->tile_bytes;
     const uint64_t per_launch = std::max<uint64_t>(1, max_blocks >> shift);
     for (uint64_t first = 0; first < plan->n_spans[c]; first += per_launch) {
@@ -966,6 +1071,12 @@ int launch_plan(const mlf_plan* plan, char* image, hipStream_t stream) {
       }
       HIP_TRY(hipGetLastError());
     }
+  }
+  for (uint64_t first = 0; first < plan->n_spans[kSmallClass]; first += (1u << 24)) {
+    const uint32_t count = (uint32_t)std::min<uint64_t>(1u << 24, plan->n_spans[kSmallClass] - first);
+    hipLaunchKernelGGL((mlf_small_kernel<PACK>), dim3((count + 3) / 4), dim3(256), 0, stream,
+                       plan->d_spans[kSmallClass] + first, count, image);
+    HIP_TRY(hipGetLastError());
   }
   for (uint64_t first = 0; first < plan->info.n_transposed_work; first += (1u << 15)) {
     const uint64_t count = std::min<uint64_t>(1u << 15, plan->info.n_transposed_work - first);
@@ -1020,52 +1131,10 @@ uint32_t mlf_crc32c_combine(uint32_t crc_a, uint32_t crc_b, uint64_t len_b) {
 
 int mlf_crc32c_device(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint32_t* out_host,
                       uint64_t n_out, void* stream_) {
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
   if (nbytes == 0) return MLF_HIP_OK;
-  if (!dev_ptr || !out_host) return fail(MLF_HIP_BAD_ARG, "null pointer");
-  if (reinterpret_cast<uintptr_t>(dev_ptr) & 15) return fail(MLF_HIP_BAD_ARG, "device buffer must be 16-byte aligned");
-  if (chunk_bytes == 0 || chunk_bytes % kCrcSegBytes)
-    return fail(MLF_HIP_BAD_ARG, "chunk_bytes must be a positive multiple of 65536");
-  const uint64_t n_chunks = (nbytes + chunk_bytes - 1) / chunk_bytes;
-  const uint64_t n_segs = (nbytes + kCrcSegBytes - 1) / kCrcSegBytes;
-  if (n_out < n_chunks) return fail(MLF_HIP_BAD_ARG, "output array too small");
-  if (n_segs > 0xFFFFFFF0ull) return fail(MLF_HIP_BAD_ARG, "buffer too large for one CRC call");
-  std::call_once(g_crc_once, crc_init_host);
-
-  CrcConsts* d_consts = nullptr;
-  uint32_t* d_seg = nullptr;
-  uint32_t* d_out = nullptr;
-  auto cleanup = [&] {
-    (void)hipFree(d_consts);
-    (void)hipFree(d_seg);
-    (void)hipFree(d_out);
-  };
-#define CRC_TRY(expr)                                                                             \
-  do {                                                                                            \
-    hipError_t e__ = (expr);                                                                      \
-    if (e__ != hipSuccess) {                                                                      \
-      cleanup();                                                                                  \
-      return fail(MLF_HIP_RUNTIME, std::string(#expr) + " failed: " + hipGetErrorString(e__));    \
-    }                                                                                             \
-  } while (0)
-  CRC_TRY(hipMalloc(reinterpret_cast<void**>(&d_consts), sizeof(CrcConsts)));
-  CRC_TRY(hipMalloc(reinterpret_cast<void**>(&d_seg), n_segs * sizeof(uint32_t)));
-  CRC_TRY(hipMalloc(reinterpret_cast<void**>(&d_out), n_chunks * sizeof(uint32_t)));
-  CRC_TRY(hipMemcpyAsync(d_consts, &g_crc_host, sizeof(CrcConsts), hipMemcpyHostToDevice, stream));
-  const uint32_t grid = (uint32_t)((n_segs + 3) / 4);
-  hipLaunchKernelGGL(mlf_crc_segments_kernel, dim3(grid), dim3(256), 0, stream, static_cast<const char*>(dev_ptr),
-                     nbytes, d_consts, d_seg, (uint32_t)n_segs);
-  CRC_TRY(hipGetLastError());
-  const uint64_t last_seg_len = nbytes - (n_segs - 1) * kCrcSegBytes;
-  hipLaunchKernelGGL(mlf_crc_chunks_kernel, dim3((uint32_t)((n_chunks + 63) / 64)), dim3(64), 0, stream, d_seg,
-                     (uint32_t)(chunk_bytes / kCrcSegBytes), (uint32_t)n_segs, g_crc_host.xseg,
-                     x_pow_bytes(last_seg_len), d_out, (uint32_t)n_chunks);
-  CRC_TRY(hipGetLastError());
-  CRC_TRY(hipMemcpyAsync(out_host, d_out, n_chunks * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
-  CRC_TRY(hipStreamSynchronize(stream));
-#undef CRC_TRY
-  cleanup();
-  return MLF_HIP_OK;
+  CrcJob job;
+  if (int rc = crc_enqueue(dev_ptr, nbytes, chunk_bytes, n_out, static_cast<hipStream_t>(stream_), &job)) return rc;
+  return crc_finish(&job, out_host);
 }
 
 }  // extern "C"
@@ -1079,6 +1148,7 @@ struct mlf_engine {
   std::vector<char*> slots;
   std::vector<hipEvent_t> slot_done;
   hipStream_t streams[2] = {nullptr, nullptr};
+  hipStream_t crc_stream = nullptr;  // checksum kernels run beside the copies, not before them
   hipEvent_t gate = nullptr;
   std::unique_ptr<WorkerPool> pool;
   std::mutex busy;  // one transfer at a time per engine
@@ -1093,6 +1163,7 @@ int mlf_engine_destroy(mlf_engine* e) {
   if (e->gate) (void)hipEventDestroy(e->gate);
   for (hipStream_t s : e->streams)
     if (s) (void)hipStreamDestroy(s);
+  if (e->crc_stream) (void)hipStreamDestroy(e->crc_stream);
   delete e;
   return MLF_HIP_OK;
 }
@@ -1112,6 +1183,7 @@ int mlf_engine_create(uint64_t slot_bytes, uint32_t n_slots, uint32_t n_threads,
   check(hipGetDevice(&e->device), "hipGetDevice");
   for (int i = 0; i < 2 && rc == MLF_HIP_OK; ++i)
     check(hipStreamCreateWithFlags(&e->streams[i], hipStreamNonBlocking), "hipStreamCreateWithFlags");
+  if (rc == MLF_HIP_OK) check(hipStreamCreateWithFlags(&e->crc_stream, hipStreamNonBlocking), "hipStreamCreateWithFlags");
   if (rc == MLF_HIP_OK) check(hipEventCreateWithFlags(&e->gate, hipEventDisableTiming), "hipEventCreateWithFlags");
   for (uint32_t i = 0; i < n_slots && rc == MLF_HIP_OK; ++i) {
     char* p = nullptr;
@@ -1138,8 +1210,14 @@ int mlf_engine_create(uint64_t slot_bytes, uint32_t n_slots, uint32_t n_threads,
 
 namespace {
 
+struct CrcRequest {
+  uint64_t chunk_bytes = 0;  // 0: no checksum
+  uint32_t* out_host = nullptr;
+  uint64_t n_out = 0;
+};
+
 int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t nbytes, void* producer_stream,
-               mlf_xfer_stats* stats) {
+               mlf_xfer_stats* stats, const CrcRequest& crc = CrcRequest()) {
   if (!e) return fail(MLF_HIP_BAD_ARG, "null engine");
   if (nbytes && (!src_dev || (host.fd < 0 && !host.ptr))) return fail(MLF_HIP_BAD_ARG, "null pointer");
   std::lock_guard<std::mutex> g(e->busy);
@@ -1149,6 +1227,24 @@ int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t
   HIP_TRY(hipEventRecord(e->gate, static_cast<hipStream_t>(producer_stream)));
   for (hipStream_t s : e->streams) HIP_TRY(hipStreamWaitEvent(s, e->gate, 0));
   const char* src = static_cast<const char*>(src_dev);
+  CrcJob crc_job;
+  const bool want_crc = crc.chunk_bytes != 0 && nbytes != 0;
+  if (want_crc) {
+    // the image is complete once the gate has passed and is not modified afterwards, so its checksum can be
+    // computed while the link-bound copies run: it costs neither blocking time nor transfer time
+    HIP_TRY(hipStreamWaitEvent(e->crc_stream, e->gate, 0));
+    if (int rc = crc_enqueue(src_dev, nbytes, crc.chunk_bytes, crc.n_out, e->crc_stream, &crc_job)) return rc;
+  }
+  struct CrcGuard {  // scratch is released on every exit path, after the kernels that use it have finished
+    CrcJob* job;
+    bool armed;
+    ~CrcGuard() {
+      if (armed) {
+        (void)hipStreamSynchronize(job->stream);
+        crc_release(job);
+      }
+    }
+  } crc_guard{&crc_job, want_crc};
   const uint64_t slot = e->slot_bytes;
   const uint64_t n_chunks = (nbytes + slot - 1) / slot;
   const uint64_t n_slots = e->slots.size();
@@ -1178,6 +1274,10 @@ int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t
     }
     if (c + n_slots < n_chunks)
       if (int rc = issue(c + n_slots)) return rc;
+  }
+  if (want_crc) {
+    crc_guard.armed = false;
+    if (int rc = crc_finish(&crc_job, crc.out_host)) return rc;
   }
   if (stats) {
     stats->seconds = now_s() - t0;
@@ -1242,6 +1342,18 @@ int mlf_engine_h2d(mlf_engine* e, const void* src_host, void* dst_dev, uint64_t 
   HostEnd host;
   host.ptr = const_cast<char*>(static_cast<const char*>(src_host));
   return engine_h2d(e, host, dst_dev, nbytes, consumer_stream, stats);
+}
+
+int mlf_engine_d2h_crc(mlf_engine* e, const void* src_dev, void* dst_host, uint64_t nbytes, void* producer_stream,
+                       uint64_t crc_chunk_bytes, uint32_t* crc_out_host, uint64_t n_crc_out, mlf_xfer_stats* stats) {
+  if (crc_chunk_bytes && !crc_out_host) return fail(MLF_HIP_BAD_ARG, "null checksum output");
+  HostEnd host;
+  host.ptr = static_cast<char*>(dst_host);
+  CrcRequest crc;
+  crc.chunk_bytes = crc_chunk_bytes;
+  crc.out_host = crc_out_host;
+  crc.n_out = n_crc_out;
+  return engine_d2h(e, src_dev, host, nbytes, producer_stream, stats, crc);
 }
 
 int mlf_engine_d2h_fd(mlf_engine* e, const void* src_dev, int fd, uint64_t file_offset, uint64_t nbytes,

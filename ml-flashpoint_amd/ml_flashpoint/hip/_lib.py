@@ -55,6 +55,7 @@ class PlanInfo(ctypes.Structure):
             "blob_bytes",
             "image_bytes",
             "table_bytes",
+            "n_small_items",
         )
     ]
 
@@ -90,6 +91,7 @@ _SIGNATURES = {
     "mlf_engine_destroy": (_INT, [_VP]),
     "mlf_engine_d2h": (_INT, [_VP, _VP, _VP, _U64, _VP, ctypes.POINTER(XferStats)]),
     "mlf_engine_h2d": (_INT, [_VP, _VP, _VP, _U64, _VP, ctypes.POINTER(XferStats)]),
+    "mlf_engine_d2h_crc": (_INT, [_VP, _VP, _VP, _U64, _VP, _U64, _VP, _U64, ctypes.POINTER(XferStats)]),
     "mlf_engine_d2h_fd": (_INT, [_VP, _VP, _INT, _U64, _U64, _VP, ctypes.POINTER(XferStats)]),
     "mlf_engine_h2d_fd": (_INT, [_VP, _INT, _U64, _VP, _U64, _VP, ctypes.POINTER(XferStats)]),
 }

@@ -381,17 +381,20 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                     ensure(nbytes)  # pooled buffers grow once, to the exact total
                 with torch.cuda.device(staged.device_index):
                     _lib.check(_lib.load().mlf_hip_set_device(staged.device_index), "mlf_hip_set_device")
-                    if self._crc_chunk_bytes:
-                        t0 = time.perf_counter()
-                        crcs = hip_plan.crc32c_device(staged.image, nbytes, self._crc_chunk_bytes, staged.stream)
-                        xfer["crc_s"] += time.perf_counter() - t0
                     start = writer.tell()
                     writer.next_buffer_slice(nbytes).release()  # bounds check + position/high-water mark
                     fd = writer.fileno() if self._use_file_io else -1
+                    engine = self._get_engine()
                     if fd >= 0:
-                        st = self._get_engine().d2h_fd(staged.image.data_ptr(), fd, METADATA_SIZE + start, nbytes, staged.stream)
+                        if self._crc_chunk_bytes:
+                            crcs = hip_plan.crc32c_device(staged.image, nbytes, self._crc_chunk_bytes, staged.stream)
+                        st = engine.d2h_fd(staged.image.data_ptr(), fd, METADATA_SIZE + start, nbytes, staged.stream)
+                    elif self._crc_chunk_bytes:
+                        # checksum kernels run on the engine's third stream while the chunks cross the link
+                        st, crcs = engine.d2h_crc(staged.image.data_ptr(), writer.data_address(start), nbytes,
+                                                  staged.stream, self._crc_chunk_bytes)
                     else:
-                        st = self._get_engine().d2h(staged.image.data_ptr(), writer.data_address(start), nbytes, staged.stream)
+                        st = engine.d2h(staged.image.data_ptr(), writer.data_address(start), nbytes, staged.stream)
                     xfer["d2h_s"] += st.seconds
                     xfer["d2h_wait_s"] += st.wait_seconds
                     xfer["d2h_bytes"] += nbytes

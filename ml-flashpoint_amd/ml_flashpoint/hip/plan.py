@@ -241,6 +241,19 @@ class CopyEngine:
         )
         return stats
 
+    def d2h_crc(self, src_dev_ptr: int, dst_host_ptr: int, nbytes: int, producer_stream: int, crc_chunk_bytes: int):
+        """``d2h`` plus a CRC-32C per ``crc_chunk_bytes`` piece of the source, computed beside the copies.
+        Returns (stats, uint32 array of chunk checksums)."""
+        stats = _lib.XferStats()
+        n_chunks = (nbytes + crc_chunk_bytes - 1) // crc_chunk_bytes
+        crcs = np.zeros(max(n_chunks, 1), dtype=np.uint32)
+        _lib.check(
+            _lib.load().mlf_engine_d2h_crc(self._handle, src_dev_ptr, dst_host_ptr, nbytes, producer_stream, crc_chunk_bytes,
+                                           crcs.ctypes.data, len(crcs), ctypes.byref(stats)),
+            "mlf_engine_d2h_crc",
+        )
+        return stats, crcs[:n_chunks]
+
     def h2d(self, src_host_ptr: int, dst_dev_ptr: int, nbytes: int, consumer_stream: int = 0) -> _lib.XferStats:
         stats = _lib.XferStats()
         _lib.check(

@@ -245,6 +245,26 @@ def test_pack_and_unpack_tables_larger_than_one_launch():
     assert torch.equal(back, src)
 
 
+def test_tiny_items_are_copied_one_per_wavefront():
+    """Thousands of items of 1..1024 bytes at every alignment: headers and payloads all go through the small-item
+    kernel (four items per workgroup); the bytes still match the oracle."""
+    gen = torch.Generator().manual_seed(41)
+    base = _rand_tensor(gen, (300_000,), torch.uint8)
+    dev_base = base.to(DEV)
+    cpu, dev, pos = [], [], 0
+    for i in range(1500):
+        n = 1 + (i * 7) % 1024
+        cpu.append(base[pos + (i % 5) : pos + (i % 5) + n])
+        dev.append(dev_base[pos + (i % 5) : pos + (i % 5) + n])
+        pos += 190
+    cpu += [_rand_tensor(gen, (), torch.float64), _rand_tensor(gen, (3,), torch.int64)]
+    dev += [t.to(DEV) for t in cpu[-2:]]
+    layout, plan, _, got = _pack_image(dev)
+    assert got == oracle_fmt.data_section(cpu)[0]
+    info = plan.info
+    assert info.n_small_items == 2 * len(cpu) and info.n_flat_tiles == 0
+
+
 def test_pack_host_resident_tensors_travel_in_blob():
     gen = torch.Generator().manual_seed(16)
     cpu = [_rand_tensor(gen, (33, 3), torch.float32), _rand_tensor(gen, (5000,), torch.int64).t(), _rand_tensor(gen, (), torch.int64)]
@@ -351,7 +371,7 @@ def test_crc32c_known_vectors_on_device(oracle_c):
 
 
 @pytest.mark.parametrize("nbytes", [1, 4097, (1 << 20) + 5, (9 << 20) + 12345])
-def test_copy_engine_round_trip(nbytes, shm_dir):
+def test_copy_engine_round_trip(nbytes, shm_dir, oracle_c):
     """Device -> mapped tmpfs file -> device through the pinned ring, several chunks, ragged tail."""
     from ml_flashpoint.checkpoint_object_manager.buffer_object.buffer_object_ext import BufferObject
     from ml_flashpoint.hip import plan as P
@@ -369,6 +389,14 @@ def test_copy_engine_round_trip(nbytes, shm_dir):
     engine.h2d(bo.get_data_ptr() + 4096, back.data_ptr(), nbytes, stream)
     torch.cuda.synchronize()
     assert torch.equal(back[:nbytes].cpu(), host) and int(back[nbytes:].sum()) == 0
+    # device -> host with the checksum computed beside the copies: same bytes, CRCs equal to the oracle's
+    if nbytes >= 65536:
+        memoryview(bo)[4096:] = bytes(nbytes)
+        stats, crcs = engine.d2h_crc(dev.data_ptr(), bo.get_data_ptr() + 4096, nbytes, stream, 1 << 20)
+        assert bytes(memoryview(bo)[4096:]) == host.numpy().tobytes()
+        want = np.zeros(len(crcs), dtype=np.uint32)
+        oracle_c.oracle_crc32c_chunks(host.numpy().tobytes(), nbytes, 1 << 20, want.ctypes.data)
+        assert crcs.tolist() == want.tolist()
     # the same two transfers through the file descriptor (pwrite / pread), at an odd file offset
     memoryview(bo)[:] = bytes(4096 + nbytes)
     bo2 = BufferObject(f"{shm_dir}/obj2.bin", 4096 + 7 + nbytes, True)
