@@ -44,6 +44,16 @@ _LOGGER = get_logger(__name__)
 
 _MAX_HEADER_LEN = 1024 * 1024  # a larger "length" means the record is not in the MLF_TENS format
 _UPLOAD_ALIGN = 4096
+_U32 = struct.Struct("<I")
+_HEADER_CACHE: dict = {}  # header pickle bytes -> (dtype, shape, stored payload bytes)
+_ESZ_CACHE: dict = {}
+
+
+def _element_size(dtype: torch.dtype) -> int:
+    esz = _ESZ_CACHE.get(dtype)
+    if esz is None:
+        esz = _ESZ_CACHE[dtype] = torch.empty((), dtype=dtype).element_size()
+    return esz
 
 
 class HipMLFlashpointCheckpointLoader(MLFlashpointCheckpointLoader):
@@ -132,15 +142,22 @@ class HipMLFlashpointCheckpointLoader(MLFlashpointCheckpointLoader):
 
     @staticmethod
     def _parse_header(view: memoryview, offset: int, length: int):
-        """(dtype, shape, payload offset) of the record at data-section ``offset``; None if it is not MLF_TENS."""
+        """(dtype, shape, payload offset) of the record at data-section ``offset``; None if it is not MLF_TENS.
+        Identical header bytes (same dtype and shape) are unpickled once."""
         base = METADATA_SIZE + offset
         if length < 4:
             return None
-        (header_len,) = struct.unpack_from("<I", view, base)
+        (header_len,) = _U32.unpack_from(view, base)
         if header_len >= _MAX_HEADER_LEN or 4 + header_len > length:
             return None
-        header = pickle.loads(view[base + 4 : base + 4 + header_len])
-        return header.dtype, header.shape, offset + 4 + header_len
+        raw = bytes(view[base + 4 : base + 4 + header_len])
+        parsed = _HEADER_CACHE.get(raw)
+        if parsed is None:
+            header = pickle.loads(raw)
+            parsed = (header.dtype, header.shape, header.shape.numel() * _element_size(header.dtype))
+            if len(_HEADER_CACHE) < 1 << 16:
+                _HEADER_CACHE[raw] = parsed
+        return parsed[0], parsed[1], offset + 4 + header_len, parsed[2]
 
     # ---- read_data ------------------------------------------------------------------------------------
     @override
@@ -160,7 +177,8 @@ class HipMLFlashpointCheckpointLoader(MLFlashpointCheckpointLoader):
         stats = {"h2d_s": 0.0, "h2d_bytes": 0, "device_payload_bytes": 0, "host_items": 0, "device_items": 0}
         with self._checkpoint_object_manager.get_buffer(checkpoint_object_id) as stream:
             optimized = stream.format_signature == CheckpointFormat.MLF_FORMAT
-            device_reqs = []  # (req, target, dtype, shape, payload_off)
+            device_reqs = []  # (req, target, dtype, shape, payload_off, stored payload bytes)
+            whole = stream.raw_view()
             for req in read_items:
                 item_md = storage_data[req.storage_index]
                 if req.type == LoadItemType.BYTE_IO:
@@ -170,7 +188,7 @@ class HipMLFlashpointCheckpointLoader(MLFlashpointCheckpointLoader):
                     planner.load_bytes(req, data)
                     continue
                 target = planner.resolve_tensor(req).detach()
-                parsed = self._parse_header(stream.raw_view(), item_md.offset, item_md.length) if optimized else None
+                parsed = self._parse_header(whole, item_md.offset, item_md.length) if optimized else None
                 if parsed is None or target.device.type == "cpu":
                     view = cast(IO[bytes], _create_file_view(stream, item_md.offset, item_md.length))
                     tensor = self.read_tensor(view, req, use_optimized_loader=optimized)
@@ -195,31 +213,53 @@ class HipMLFlashpointCheckpointLoader(MLFlashpointCheckpointLoader):
         written = stream.len_written_data
         sidecar = integrity.read_sidecar(object_id.data) if self._verify_crc else None
 
-        # box of the stored tensor each request wants, as offsets/strides over the stored C-contiguous payload
-        boxes = []
+        # Every request becomes one table row whose image offset is, for now, absolute in the data section.  A request
+        # for a whole stored tensor into a contiguous target (the common case) is one run of bytes; anything else
+        # is described as a box over the stored C-contiguous payload (offsets/strides) and the target's strides.
+        table = hip_plan.ItemTable()
         lo, hi = None, 0
-        for req, target, dtype, shape, payload_off in device_reqs:
-            esz = torch.empty((), dtype=dtype).element_size()
-            stored_strides = hip_plan._contiguous_strides(tuple(shape))
-            # a dimension is narrowed only where the requested length is smaller than the stored size
-            lengths = [l if l < s else s for l, s in zip(req.lengths, shape)]
-            offsets = [o if l < s else 0 for o, l, s in zip(req.storage_offsets, req.lengths, shape)]
-            lengths += list(shape[len(lengths):])
-            offsets += [0] * (len(shape) - len(offsets))
-            box_shape = torch.Size(lengths)
-            assert target.size() == box_shape, f"req {req.storage_index} mismatch sizes {target.size()} vs {box_shape}"
+        for req, target, dtype, shape, payload_off, stored_bytes in device_reqs:
             if target.dtype != dtype:
                 raise TypeError(f"req {req.storage_index}: stored dtype {dtype} differs from target dtype {target.dtype}")
-            numel = box_shape.numel()
-            nbytes_stored = torch.Size(shape).numel() * esz
-            if payload_off + nbytes_stored > written:
+            if payload_off + stored_bytes > written:
                 raise ValueError(f"req {req.storage_index}: record reaches past the written data of '{object_id.data}'")
-            if numel:
-                first = payload_off + sum(o * s for o, s in zip(offsets, stored_strides)) * esz
-                last = first + (sum((l - 1) * s for l, s in zip(lengths, stored_strides)) + 1) * esz
-                lo = first if lo is None else min(lo, first)
-                hi = max(hi, last)
-            boxes.append((target, esz, lengths, stored_strides, payload_off, offsets, numel))
+            esz = _element_size(dtype)
+            ndim = len(shape)
+            req_lengths = req.lengths
+            # a dimension is narrowed only where the requested length is smaller than the stored size
+            narrowed = any(l < sz for l, sz in zip(req_lengths, shape))
+            if not narrowed:
+                assert target.size() == shape, f"req {req.storage_index} mismatch sizes {target.size()} vs {shape}"
+                if stored_bytes == 0:
+                    continue
+                first, last = payload_off, payload_off + stored_bytes
+                if target.is_contiguous():
+                    table.add_contiguous(target.data_ptr(), first, esz, stored_bytes)
+                elif ndim <= _lib.MAX_DIMS:
+                    table.add_device(target.data_ptr(), first, esz, tuple(shape), tuple(target.stride()))
+                else:
+                    raise NotImplementedError(f"rank > {_lib.MAX_DIMS} targets must be contiguous")
+            else:
+                stored_strides = hip_plan._contiguous_strides(tuple(shape))
+                lengths = [l if l < sz else sz for l, sz in zip(req_lengths, shape)]
+                offsets = [o if l < sz else 0 for o, l, sz in zip(req.storage_offsets, req_lengths, shape)]
+                lengths += list(shape[len(lengths):])
+                offsets += [0] * (ndim - len(offsets))
+                box_shape = torch.Size(lengths)
+                assert target.size() == box_shape, f"req {req.storage_index} mismatch sizes {target.size()} vs {box_shape}"
+                numel = box_shape.numel()
+                if numel == 0:
+                    continue
+                if ndim > _lib.MAX_DIMS:
+                    raise NotImplementedError(f"sub-box reads of rank > {_lib.MAX_DIMS} tensors are not supported")
+                first = payload_off + sum(o * st for o, st in zip(offsets, stored_strides)) * esz
+                last = first + (sum((l - 1) * st for l, st in zip(lengths, stored_strides)) + 1) * esz
+                table.add_device(target.data_ptr(), first, esz, tuple(lengths), tuple(target.stride()),
+                                 image_stride=tuple(stored_strides))
+                stored_bytes = numel * esz
+            stats["device_payload_bytes"] += stored_bytes
+            lo = first if lo is None else min(lo, first)
+            hi = max(hi, last)
         if lo is None:
             for req, target, *_ in device_reqs:
                 planner.commit_tensor(req, target)
@@ -228,20 +268,8 @@ class HipMLFlashpointCheckpointLoader(MLFlashpointCheckpointLoader):
             lo, hi = 0, written  # checksums cover the whole data section
         lo = lo // _UPLOAD_ALIGN * _UPLOAD_ALIGN
         span = hi - lo
-
-        table = hip_plan.ItemTable()
-        for target, esz, lengths, stored_strides, payload_off, offsets, numel in boxes:
-            if not numel:
-                continue
-            first = payload_off + sum(o * s for o, s in zip(offsets, stored_strides)) * esz
-            shape, tstride, istride = tuple(lengths), tuple(target.stride()), tuple(stored_strides)
-            if len(shape) > _lib.MAX_DIMS:
-                if not (target.is_contiguous() and all(o == 0 for o in offsets) and istride == tuple(
-                        hip_plan._contiguous_strides(shape))):
-                    raise NotImplementedError(f"rank > {_lib.MAX_DIMS} targets must be contiguous full tensors")
-                shape, tstride, istride = (numel,), (1,), (1,)
-            table.add_device(target.data_ptr(), first - lo, esz, shape, tstride, image_stride=istride)
-            stats["device_payload_bytes"] += numel * esz
+        items = table.to_array()
+        items["image_off"] -= lo  # offsets relative to the uploaded range
         with torch.cuda.device(device):
             _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
             image = torch.empty(span, dtype=torch.uint8, device=device)
@@ -264,7 +292,7 @@ class HipMLFlashpointCheckpointLoader(MLFlashpointCheckpointLoader):
                     raise integrity.ChecksumMismatchError(
                         f"'{object_id.data}': CRC-32C mismatch in chunk(s) {bad[:8]} of {len(want)} "
                         f"(chunk size {chunk_bytes})")
-            plan = hip_plan.Plan(table.to_array(), b"", span, tile_bytes=self._tile_bytes,
+            plan = hip_plan.Plan(items, b"", span, tile_bytes=self._tile_bytes,
                                  block_threads=self._block_threads, align_to_tensor=True)
             if self.record_kernel_events:
                 begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

@@ -39,16 +39,36 @@ def _contiguous_strides(shape: Sequence[int]) -> List[int]:
 
 
 class ItemTable:
-    """Column-wise builder of an ``mlf_item`` array (filled per column at the end: cheaper than per-row numpy)."""
+    """Column-wise builder of an ``mlf_item`` array.
+
+    Scalar columns are plain Python lists turned into numpy columns in one go; contiguous device items are stored
+    as 1-D (numel,) with unit strides, so only genuinely strided items carry per-dimension rows."""
 
     def __init__(self):
-        self._rows: List[tuple] = []
+        self.ptr: List[int] = []
+        self.image_off: List[int] = []
+        self.nbytes: List[int] = []
+        self.kind: List[int] = []
+        self.elem_size: List[int] = []
+        self._strided: List[tuple] = []  # (row, shape, stride, image_stride)
 
     def __len__(self):
-        return len(self._rows)
+        return len(self.ptr)
 
     def add_blob(self, blob_off: int, image_off: int, nbytes: int) -> None:
-        self._rows.append((blob_off, image_off, nbytes, ITEM_BLOB, 1, 0, (), (), ()))
+        self.ptr.append(blob_off)
+        self.image_off.append(image_off)
+        self.nbytes.append(nbytes)
+        self.kind.append(ITEM_BLOB)
+        self.elem_size.append(1)
+
+    def add_contiguous(self, ptr: int, image_off: int, elem_size: int, nbytes: int) -> None:
+        """Device item that is one run of bytes on both sides."""
+        self.ptr.append(ptr)
+        self.image_off.append(image_off)
+        self.nbytes.append(nbytes)
+        self.kind.append(ITEM_DEVICE)
+        self.elem_size.append(elem_size)
 
     def add_device(
         self,
@@ -66,26 +86,37 @@ class ItemTable:
             numel *= s
         if image_stride is None:
             image_stride = _contiguous_strides(shape)
-        self._rows.append(
-            (ptr, image_off, numel * elem_size, ITEM_DEVICE, elem_size, len(shape), tuple(shape), tuple(stride), tuple(image_stride))
-        )
+        self._strided.append((len(self.ptr), tuple(shape), tuple(stride), tuple(image_stride)))
+        self.add_contiguous(ptr, image_off, elem_size, numel * elem_size)
 
     def to_array(self) -> np.ndarray:
-        n = len(self._rows)
+        n = len(self.ptr)
         arr = np.zeros(n, dtype=ITEM_DTYPE)
         if n == 0:
             return arr
-        cols = list(zip(*self._rows))
-        arr["ptr"] = cols[0]
-        arr["image_off"] = cols[1]
-        arr["nbytes"] = cols[2]
-        arr["kind"] = cols[3]
-        arr["elem_size"] = cols[4]
-        arr["ndim"] = cols[5]
-        pad = (0,) * MAX_DIMS
-        arr["shape"] = [(s + pad)[:MAX_DIMS] for s in cols[6]]
-        arr["stride"] = [(s + pad)[:MAX_DIMS] for s in cols[7]]
-        arr["image_stride"] = [(s + pad)[:MAX_DIMS] for s in cols[8]]
+        arr["ptr"] = self.ptr
+        arr["image_off"] = self.image_off
+        nbytes = np.array(self.nbytes, dtype=np.uint64)
+        arr["nbytes"] = nbytes
+        arr["kind"] = self.kind
+        esz = np.array(self.elem_size, dtype=np.uint32)
+        arr["elem_size"] = esz
+        # default description of every item: one dimension of numel elements, unit strides
+        arr["ndim"] = 1
+        arr["shape"][:, 0] = nbytes // esz
+        arr["stride"][:, 0] = 1
+        arr["image_stride"][:, 0] = 1
+        for row, shape, stride, image_stride in self._strided:
+            k = len(shape)
+            item = arr[row]
+            item["ndim"] = k
+            item["shape"][:k] = shape
+            item["stride"][:k] = stride
+            item["image_stride"][:k] = image_stride
+            if k == 0:
+                item["shape"][0] = 0
+                item["stride"][0] = 0
+                item["image_stride"][0] = 0
         return arr
 
 
@@ -127,12 +158,10 @@ def build_save_layout(tensors: Sequence[torch.Tensor], blobs: Sequence[bytes] = 
                 table.add_blob(len(blob), pos, nbytes)
                 blob += flat.numpy().tobytes()
             else:
-                shape, stride = tuple(t.shape), tuple(t.stride())
-                if len(shape) > MAX_DIMS:
-                    if not t.is_contiguous():
-                        raise NotImplementedError(f"non-contiguous tensor of rank {len(shape)} > {MAX_DIMS}")
-                    shape, stride = (t.numel(),), (1,)
-                table.add_device(t.data_ptr(), pos, t.element_size(), shape, stride)
+                if t.is_contiguous():
+                    table.add_contiguous(t.data_ptr(), pos, t.element_size(), nbytes)
+                else:
+                    table.add_device(t.data_ptr(), pos, t.element_size(), tuple(t.shape), tuple(t.stride()))
                 keep.append(t)
                 device_bytes += nbytes
             pos += nbytes
