@@ -21,8 +21,10 @@ import logging
 import os
 import pickle
 import subprocess
+import tempfile
 import threading
 import time
+import uuid
 from typing import Callable, Optional, Union
 
 import torch
@@ -63,7 +65,12 @@ class EngineConfig:
 
 
 class StagedObject:
-    """Image of one checkpoint object in HBM, with the layout that produced it."""
+    """Image of one checkpoint object in HBM, with the layout that produced it.
+
+    With a background writer (``background_write=True``) the transfer into the buffer object starts as soon as the
+    pack is enqueued and ``future`` resolves to the object's WriteResults.  Such an object may cross a process
+    boundary: what arrives on the other side is a ``RemoteStagedObject`` that only waits for the transfer - the HIP
+    context, the image and the buffer stay with the process that owns the GPU."""
 
     def __init__(self, layout: hip_plan.SaveLayout, plan: Optional[hip_plan.Plan], image: Optional[torch.Tensor],
                  device_index: int, stream: int, items: list):
@@ -74,6 +81,48 @@ class StagedObject:
         self.stream = stream
         self.items = items  # WriteItems in span order: tensors, then byte blobs
         self.consumed = False
+        self.future: Optional[concurrent.futures.Future] = None
+        self.done_marker: Optional[str] = None
+        self.collected = False
+
+    def __reduce__(self):
+        if self.future is None or self.done_marker is None:
+            raise pickle.PicklingError(
+                "a packed checkpoint image lives in this process's GPU memory and cannot be sent to another process; "
+                "construct the saver with background_write=True so that this process writes it and the other one "
+                "only waits for the result"
+            )
+        return (RemoteStagedObject, (self.done_marker,))
+
+
+class RemoteStagedObject:
+    """What a ``StagedObject`` becomes in another process: the path of the marker file through which the owning
+    process reports the outcome (the pickled WriteResults, or the error text)."""
+
+    def __init__(self, done_marker: str):
+        self.done_marker = done_marker
+        self.consumed = False
+
+    def wait(self, timeout_s: float) -> list:
+        deadline = time.monotonic() + timeout_s
+        delay = 0.0005
+        while not os.path.exists(self.done_marker):
+            if time.monotonic() > deadline:
+                raise RuntimeError(
+                    f"timed out after {timeout_s:.0f} s waiting for the GPU-owning process to finish writing "
+                    f"(marker '{self.done_marker}' never appeared)"
+                )
+            time.sleep(delay)
+            delay = min(delay * 2, 0.01)
+        with open(self.done_marker, "rb") as f:
+            ok, payload = pickle.load(f)
+        try:
+            os.remove(self.done_marker)
+        except OSError:
+            pass
+        if not ok:
+            raise RuntimeError(f"writing the checkpoint object failed in the GPU-owning process: {payload}")
+        return payload
 
 
 class StagedTensorRef:
@@ -119,6 +168,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         block_threads: int = 0,
         crc_chunk_bytes: int = 0,
         use_file_io: bool = False,
+        background_write: bool = False,
+        remote_wait_timeout_s: float = 1800.0,
     ):
         """Same positional arguments as the reference's default saver (checkpoint_saver.py:290-321).
 
@@ -126,7 +177,10 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         split, 0 = library default), ``crc_chunk_bytes`` (> 0: compute a CRC-32C per chunk of every object on the
         GPU and keep it beside the object), ``use_file_io`` (False, the default: the host threads memcpy the
         pinned slots into the mapping, whose page-table entries a pooled buffer keeps from save to save; True: they
-        pwrite() through the file descriptor, which tmpfs serialises on the inode lock - measured 5x slower).
+        pwrite() through the file descriptor, which tmpfs serialises on the inode lock - measured 5x slower),
+        ``background_write`` (True: ``prepare_write_data`` also starts the transfer into the buffer object on a
+        background thread of this process; ``write_data`` - here or in a worker process that received the buckets -
+        then only waits for it, for at most ``remote_wait_timeout_s`` across processes).
         """
         if not use_optimized_save:
             raise ValueError(
@@ -146,6 +200,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         self._block_threads = block_threads
         self._crc_chunk_bytes = crc_chunk_bytes
         self._use_file_io = use_file_io
+        self._background_write = background_write
+        self._remote_wait_timeout_s = remote_wait_timeout_s
         self._init_runtime_state()
 
     def _init_runtime_state(self):
@@ -280,9 +336,11 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             refs = [
                 (item, StagedTensorRef(staged, i, t.dtype, t.shape)) for i, (item, t) in enumerate(tensor_data)
             ]
-            write_buckets.append(
-                ObjectWriteBucket(object_id=object_id, object_name=object_name, bytesio_data=bytes_data, tensor_data=refs)
-            )
+            bucket_out = ObjectWriteBucket(object_id=object_id, object_name=object_name, bytesio_data=bytes_data,
+                                           tensor_data=refs)
+            write_buckets.append(bucket_out)
+            if self._background_write and refs:
+                self._start_background_write(staged, bucket_out)
         stats["prepare_s"] = time.perf_counter() - t_start
         self.last_save_stats = stats
         return write_buckets
@@ -354,11 +412,12 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             raise errors[0]
         return all_results
 
-    def _staged_of(self, bucket: ObjectWriteBucket) -> StagedObject:
+    def _staged_of(self, bucket: ObjectWriteBucket):
         refs = [t for _, t in bucket.tensor_data]
         if refs and all(isinstance(r, StagedTensorRef) for r in refs):
             staged = refs[0].staged
-            if all(r.staged is staged for r in refs) and not staged.consumed:
+            in_flight = isinstance(staged, RemoteStagedObject) or staged.future is not None
+            if all(r.staged is staged for r in refs) and (in_flight or not staged.consumed):
                 return staged
             raise ValueError(f"bucket for '{bucket.object_id}' refers to a staged image that was already written")
         if any(isinstance(r, StagedTensorRef) for r in refs):
@@ -366,8 +425,58 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         return self._stage_object(bucket.tensor_data, bucket.bytesio_data, {"plan_build_s": 0.0, "objects": 0,
                                                                             "device_payload_bytes": 0, "image_bytes": 0})
 
+    def _start_background_write(self, staged: StagedObject, bucket: ObjectWriteBucket) -> None:
+        """Runs the transfer of ``bucket`` on a thread of this process and publishes the outcome twice: through
+        ``staged.future`` (same process) and through a marker file (for a process that received the bucket)."""
+        staged.future = concurrent.futures.Future()
+        staged.done_marker = os.path.join(tempfile.gettempdir(), f"mlf_write_{os.getpid()}_{uuid.uuid4().hex}.done")
+
+        def run():
+            try:
+                results = self._transfer_bucket(staged, bucket, {"d2h_s": 0.0, "d2h_wait_s": 0.0, "d2h_bytes": 0})
+                outcome = (True, results)
+            except BaseException as e:  # reported to whoever waits; the thread itself must not die silently
+                _LOGGER.exception("Background write of '%s' failed", bucket.object_id)
+                outcome = (False, f"{type(e).__name__}: {e}")
+            try:
+                tmp = staged.done_marker + ".tmp"
+                with open(tmp, "wb") as f:
+                    pickle.dump(outcome, f)
+                os.rename(tmp, staged.done_marker)
+            finally:
+                if outcome[0]:
+                    staged.future.set_result(outcome[1])
+                else:
+                    staged.future.set_exception(RuntimeError(outcome[1]))
+
+        threading.Thread(target=run, name=f"mlf-write-{bucket.object_name}", daemon=True).start()
+
     def _write_bucket(self, bucket: ObjectWriteBucket, replicate_after_write: bool, xfer: dict) -> list[WriteResult]:
         staged = self._staged_of(bucket)
+        if isinstance(staged, RemoteStagedObject):
+            # this process only received the bucket: the process that owns the GPU is writing it
+            if staged.consumed:
+                raise ValueError(f"bucket for '{bucket.object_id}' was already written")
+            staged.consumed = True
+            return staged.wait(self._remote_wait_timeout_s)
+        if staged.future is not None:
+            if staged.collected:
+                raise ValueError(f"bucket for '{bucket.object_id}' was already written")
+            staged.collected = True
+            results = staged.future.result()
+            try:
+                os.remove(staged.done_marker)
+            except OSError:
+                pass
+        else:
+            results = self._transfer_bucket(staged, bucket, xfer)
+        if replicate_after_write and self._replication_manager is not None:
+            # without a replication manager (single node, or this package used on its own) there is no peer to
+            # send to; an explicit async_replicate_object() call still raises
+            self.async_replicate_object(bucket.object_id)
+        return results
+
+    def _transfer_bucket(self, staged: StagedObject, bucket: ObjectWriteBucket, xfer: dict) -> list[WriteResult]:
         layout = staged.layout
         nbytes = layout.image_bytes
         crcs = None
@@ -412,10 +521,6 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             )
             for item, (offset, length) in zip(staged.items, layout.spans)
         ]
-        if replicate_after_write and self._replication_manager is not None:
-            # without a replication manager (single node, or this package used on its own) there is no peer to
-            # send to; an explicit async_replicate_object() call still raises
-            self.async_replicate_object(bucket.object_id)
         return results
 
     # ---- replication hand-off, metadata, finalize (host logic kept as in the reference) -------------------
