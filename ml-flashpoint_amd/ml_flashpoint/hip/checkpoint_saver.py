@@ -170,6 +170,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         use_file_io: bool = False,
         background_write: bool = False,
         remote_wait_timeout_s: float = 1800.0,
+        max_image_bytes: Optional[int] = None,
     ):
         """Same positional arguments as the reference's default saver (checkpoint_saver.py:290-321).
 
@@ -180,7 +181,9 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         pwrite() through the file descriptor, which tmpfs serialises on the inode lock - measured 5x slower),
         ``background_write`` (True: ``prepare_write_data`` also starts the transfer into the buffer object on a
         background thread of this process; ``write_data`` - here or in a worker process that received the buckets -
-        then only waits for it, for at most ``remote_wait_timeout_s`` across processes).
+        then only waits for it, for at most ``remote_wait_timeout_s`` across processes), ``max_image_bytes`` (largest
+        image to hold in HBM at once; default: what is free on the device.  A larger object is packed and sent window
+        by window inside ``prepare_write_data``, which then blocks for the whole transfer).
         """
         if not use_optimized_save:
             raise ValueError(
@@ -202,6 +205,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         self._use_file_io = use_file_io
         self._background_write = background_write
         self._remote_wait_timeout_s = remote_wait_timeout_s
+        self._max_image_bytes = max_image_bytes
         self._init_runtime_state()
 
     def _init_runtime_state(self):
@@ -332,20 +336,29 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                 continue
             object_name = f"{object_name_prefix}_{len(write_buckets)}_src{rank}{_DEFAULT_OBJ_NAME_SUFFIX}"
             object_id = CheckpointObjectId.from_container(checkpoint_id, object_name)
-            staged = self._stage_object(tensor_data, bytes_data, stats)
+            staged = self._stage_object(tensor_data, bytes_data, stats, object_id, object_name)
             refs = [
                 (item, StagedTensorRef(staged, i, t.dtype, t.shape)) for i, (item, t) in enumerate(tensor_data)
             ]
             bucket_out = ObjectWriteBucket(object_id=object_id, object_name=object_name, bytesio_data=bytes_data,
                                            tensor_data=refs)
             write_buckets.append(bucket_out)
-            if self._background_write and refs:
+            if self._background_write and refs and staged.future is None:
                 self._start_background_write(staged, bucket_out)
         stats["prepare_s"] = time.perf_counter() - t_start
         self.last_save_stats = stats
         return write_buckets
 
-    def _stage_object(self, tensor_data, bytes_data, stats: dict) -> StagedObject:
+    def _image_limit(self, device: torch.device) -> int:
+        """Bytes of HBM an image may take: the explicit limit, or what the device and torch's allocator have free
+        (minus a margin for the tables and for whatever the training step allocates next)."""
+        if self._max_image_bytes is not None:
+            return self._max_image_bytes
+        free, _ = torch.cuda.mem_get_info(device)
+        cached = torch.cuda.memory_reserved(device) - torch.cuda.memory_allocated(device)
+        return max(free + cached - (2 << 30), 64 << 20)
+
+    def _stage_object(self, tensor_data, bytes_data, stats: dict, object_id=None, object_name=None) -> StagedObject:
         blobs = []
         for _, data in bytes_data:
             data.seek(0)
@@ -361,6 +374,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         items = [item for item, _ in tensor_data] + [item for item, _ in bytes_data]
         plan = image = None
         stream = 0
+        if layout.image_bytes and object_id is not None and layout.image_bytes > self._image_limit(device):
+            return self._stage_windowed(layout, items, object_id, object_name, device, stats)
         if layout.image_bytes:
             with torch.cuda.device(device):
                 _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
@@ -381,6 +396,75 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         stats["device_payload_bytes"] += layout.device_payload_bytes
         stats["image_bytes"] += layout.image_bytes
         return StagedObject(layout, plan, image, device.index or 0, stream, items)
+
+    def _stage_windowed(self, layout, items, object_id, object_name, device, stats: dict) -> StagedObject:
+        """Fallback for an object whose image does not fit in HBM beside the live state: consecutive records are
+        grouped into windows of at most the image limit (a single larger record gets a window of its own), and each
+        window is packed into one reusable device buffer and sent before the next is packed.  The live tensors are
+        read until the last window, so this runs to completion here, inside the blocking part of the save."""
+        _LOGGER.warning("checkpoint image of %d bytes exceeds the HBM limit; saving '%s' window by window (blocking)",
+                        layout.image_bytes, object_id)
+        arr = layout.items
+        ends = (arr["image_off"] + arr["nbytes"]).tolist()
+        starts = arr["image_off"].tolist()
+        limit = max(self._image_limit(device), 1)
+        windows, r0, n = [], 0, len(arr)
+        while r0 < n:
+            r1 = r0 + 1
+            while r1 < n and ends[r1] - starts[r0] <= limit:
+                r1 += 1
+            windows.append((r0, r1, starts[r0], ends[r1 - 1]))
+            r0 = r1
+        nbytes = layout.image_bytes
+        xfer = {"d2h_s": 0.0, "d2h_wait_s": 0.0, "d2h_bytes": 0}
+        with self._chkpt_obj_manager.acquire_buffer(object_id, max(self._initial_buffer_size_bytes, nbytes)) as writer:
+            writer.set_format_signature(CheckpointFormat.MLF_FORMAT)
+            ensure = getattr(writer, "ensure_capacity", None)
+            if ensure is not None:
+                ensure(nbytes)
+            with torch.cuda.device(device):
+                _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
+                start = writer.tell()
+                writer.next_buffer_slice(nbytes).release()
+                stream = torch.cuda.current_stream(device).cuda_stream
+                buf = torch.empty(max(e - b for _, _, b, e in windows), dtype=torch.uint8, device=device)
+                engine = self._get_engine()
+                for r0, r1, begin, end in windows:
+                    sub = arr[r0:r1].copy()
+                    sub["image_off"] -= begin
+                    plan = hip_plan.Plan(sub, layout.blob, end - begin, tile_bytes=self._tile_bytes,
+                                         block_threads=self._block_threads)
+                    plan.pack(buf, stream)
+                    st = engine.d2h(buf.data_ptr(), writer.data_address(start + begin), end - begin, stream)
+                    plan.destroy()
+                    xfer["d2h_s"] += st.seconds
+                    xfer["d2h_bytes"] += end - begin
+        if self._crc_chunk_bytes:
+            _LOGGER.warning("no CRC sidecar is written for '%s': it was saved window by window", object_id)
+        stats["objects"] += 1
+        stats["windows"] = stats.get("windows", 0) + len(windows)
+        stats["device_payload_bytes"] += layout.device_payload_bytes
+        stats["image_bytes"] += nbytes
+        stats.update({k: stats.get(k, 0) + v for k, v in xfer.items()})
+        staged = StagedObject(layout, None, None, device.index or 0, 0, items)
+        staged.consumed = True
+        staged.future = concurrent.futures.Future()
+        staged.future.set_result(self._results_of(staged, object_name))
+        staged.done_marker = os.path.join(tempfile.gettempdir(), f"mlf_write_{os.getpid()}_{uuid.uuid4().hex}.done")
+        with open(staged.done_marker, "wb") as f:
+            pickle.dump((True, staged.future.result()), f)
+        return staged
+
+    @staticmethod
+    def _results_of(staged: StagedObject, object_name: str) -> list[WriteResult]:
+        return [
+            WriteResult(
+                index=item.index,
+                size_in_bytes=length,
+                storage_data=_StorageInfo(relative_path=object_name, offset=offset, length=length),
+            )
+            for item, (offset, length) in zip(staged.items, staged.layout.spans)
+        ]
 
     # ---- write_data -----------------------------------------------------------------------------
     @override
@@ -513,15 +597,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             staged.plan.destroy()
         if crcs is not None:
             integrity.write_sidecar(str(bucket.object_id), self._crc_chunk_bytes, nbytes, crcs)
-        results = [
-            WriteResult(
-                index=item.index,
-                size_in_bytes=length,
-                storage_data=_StorageInfo(relative_path=bucket.object_name, offset=offset, length=length),
-            )
-            for item, (offset, length) in zip(staged.items, layout.spans)
-        ]
-        return results
+        return self._results_of(staged, bucket.object_name)
 
     # ---- replication hand-off, metadata, finalize (host logic kept as in the reference) -------------------
     @log_execution_time(logger=_LOGGER, name="async_replicate_object")

@@ -361,6 +361,22 @@ def test_multiple_buckets_and_overwrite_of_existing_object(shm_dir):
     assert raw == fmt.file_image([torch.ones(3)])[0]
 
 
+def test_object_larger_than_the_hbm_limit_is_saved_window_by_window(shm_dir, manager_future):
+    """With ``max_image_bytes`` far below the object size the saver packs and sends windows of records through
+    one small device buffer; the file is the same."""
+    sd_cpu = {k: v for k, v in _mixed_state_dict().items()}
+    sd_cpu["big"] = torch.arange(200_000, dtype=torch.float32)  # one record larger than the limit
+    sd_dev = _to_dev(sd_cpu, keep_on_host=("w.i64",))
+    ckpt = os.path.join(shm_dir, "step-8_ckpt")
+    saver = _saver(max_image_bytes=64 << 10)
+    dcp.save(sd_dev, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(saver, manager_future), no_dist=True)
+    assert saver.last_save_stats["windows"] >= 4
+    raw = open(os.path.join(ckpt, "__0__0_src0.distcp"), "rb").read()
+    metadata = pickle.load(open(os.path.join(ckpt, ".metadata"), "rb"))
+    image, spans, got_spans = _expected_file(sd_cpu, metadata, raw)
+    assert raw == image and got_spans == spans
+
+
 def test_legacy_torch_save_objects_are_still_readable(shm_dir):
     """An object whose signature is TORCH___ holds torch.save records; the loader reads it on the host."""
     from ml_flashpoint.core.defaults import CheckpointFormat
