@@ -287,7 +287,9 @@ __global__ void __launch_bounds__(256) mlf_strided_kernel(const StridedDesc* __r
 // Global accesses are max(4, esz)-byte vectors (hardware-unaligned where the view starts off a boundary); LDS is
 // addressed per element on the transposed side.  T = 128 / 64 / 64 / 32 / 16 elements for esz = 1 / 2 / 4 / 8 / 16;
 // rows of the LDS tile are padded by one vector so that a column walk does not stay in one bank.
-constexpr uint32_t kTransLdsBytes = 128 * (128 + 4);
+constexpr uint32_t kTransThreads = 256;
+constexpr uint32_t kTransBand = 8;  // tile-rows per band of the visiting order (measured: 8 beats 1 by 10-40 %)
+constexpr uint32_t kTransLdsBytes = 128 * (128 + 16);
 
 __host__ __device__ inline uint32_t trans_tile_dim(uint32_t esz) {
   return esz == 1 ? 128u : esz <= 4 ? 64u : esz == 8 ? 32u : 16u;
@@ -306,7 +308,13 @@ __device__ __forceinline__ void trans_tile(const TransDesc* __restrict__ d, uint
   const uint64_t per_batch = (uint64_t)d->tiles_a * d->tiles_b;
   uint64_t batch = tile / per_batch;
   const uint32_t rem = (uint32_t)(tile - batch * per_batch);
-  const uint32_t ta = rem / d->tiles_b, tb = rem - ta * d->tiles_b;
+  // tiles are visited in bands of kTransBand tile-rows, a fastest inside a band: eight consecutive workgroups read
+  // eight neighbouring runs of the same source rows, and the next eight write next to them in the same
+  // destination rows, so both sides keep hitting DRAM pages that are already open
+  const uint32_t band = rem / (kTransBand * d->tiles_b);
+  const uint32_t in_band = rem - band * (kTransBand * d->tiles_b);
+  const uint32_t band_rows = d->tiles_a - band * kTransBand < kTransBand ? d->tiles_a - band * kTransBand : kTransBand;
+  const uint32_t tb = in_band / band_rows, ta = band * kTransBand + (in_band - tb * band_rows);
   int64_t toff = 0, ioff = 0;
   for (int k = (int)d->nbatch - 1; k >= 0; --k) {
     const uint64_t extent = (uint64_t)d->bshape[k];
@@ -327,7 +335,7 @@ __device__ __forceinline__ void trans_tile(const TransDesc* __restrict__ d, uint
   const uint32_t yn = (uint32_t)(ny - y0 < (int64_t)T ? ny - y0 : T);
   const uint32_t vec_per_row = T / EPV, n_vec = T * vec_per_row;
 
-  for (uint32_t v = threadIdx.x; v < n_vec; v += 256) {
+  for (uint32_t v = threadIdx.x; v < n_vec; v += kTransThreads) {
     const uint32_t y = v / vec_per_row, x = (v - y * vec_per_row) * EPV;
     if (y >= yn || x >= xn) continue;
     const char* g = src + (int64_t)y * ld_src + (int64_t)x * ESZ;
@@ -339,7 +347,7 @@ __device__ __forceinline__ void trans_tile(const TransDesc* __restrict__ d, uint
     }
   }
   __syncthreads();
-  for (uint32_t v = threadIdx.x; v < n_vec; v += 256) {
+  for (uint32_t v = threadIdx.x; v < n_vec; v += kTransThreads) {
     const uint32_t x = v / vec_per_row, y = (v - x * vec_per_row) * EPV;
     if (x >= xn || y >= yn) continue;
     char* g = dst + (int64_t)x * ld_dst + (int64_t)y * ESZ;
@@ -357,7 +365,7 @@ __device__ __forceinline__ void trans_tile(const TransDesc* __restrict__ d, uint
 }
 
 template <bool PACK>
-__global__ void __launch_bounds__(256) mlf_transpose_kernel(const TransDesc* __restrict__ descs,
+__global__ void __launch_bounds__(kTransThreads) mlf_transpose_kernel(const TransDesc* __restrict__ descs,
                                                             const TransWork* __restrict__ work,
                                                             char* __restrict__ image) {
   __shared__ __attribute__((aligned(16))) char lds[kTransLdsBytes];
@@ -1078,9 +1086,10 @@ int launch_plan(const mlf_plan* plan, char* image, hipStream_t stream) {
                        plan->d_spans[kSmallClass] + first, count, image);
     HIP_TRY(hipGetLastError());
   }
-  for (uint64_t first = 0; first < plan->info.n_transposed_work; first += (1u << 15)) {
-    const uint64_t count = std::min<uint64_t>(1u << 15, plan->info.n_transposed_work - first);
-    hipLaunchKernelGGL((mlf_transpose_kernel<PACK>), dim3((uint32_t)(count * kTransTilesPerEntry)), dim3(256), 0, stream,
+  const uint64_t trans_per_launch = std::max<uint64_t>(1, 0xFFFFFFFFull / ((uint64_t)kTransTilesPerEntry * kTransThreads));
+  for (uint64_t first = 0; first < plan->info.n_transposed_work; first += trans_per_launch) {
+    const uint64_t count = std::min<uint64_t>(trans_per_launch, plan->info.n_transposed_work - first);
+    hipLaunchKernelGGL((mlf_transpose_kernel<PACK>), dim3((uint32_t)(count * kTransTilesPerEntry)), dim3(kTransThreads), 0, stream,
                        plan->d_tdescs, plan->d_twork + first, image);
     HIP_TRY(hipGetLastError());
   }
