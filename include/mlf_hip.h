@@ -119,6 +119,12 @@ int mlf_crc32c_device(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes
 /* Same function on host memory (SSE4.2), and the combine law crc(A||B) from crc(A), crc(B), len(B). */
 uint32_t mlf_crc32c_host(const void* data, uint64_t nbytes);
 uint32_t mlf_crc32c_combine(uint32_t crc_a, uint32_t crc_b, uint64_t len_b);
+/* Host-only: CRC-32C of every `chunk_bytes` piece of the byte range [file_offset, file_offset + nbytes) of an
+ * open file, read with pread() by `threads` threads (no mapping is built, no GPU is touched).  Writes
+ * ceil(nbytes/chunk_bytes) values.  Lets recovery discovery check an object against the values recorded when it
+ * was saved before choosing it (the reference's discovery, checkpoint_loader.py:340-424, checks presence only). */
+int mlf_crc32c_file(int fd, uint64_t file_offset, uint64_t nbytes, uint64_t chunk_bytes, uint32_t* out_host,
+                    uint64_t n_out, uint32_t threads);
 
 /* Copy engine: a ring of pinned host slots, two copy streams and a pool of host threads that move data
  * between device memory and pageable host memory (the MAP_SHARED buffer file) at link speed. */

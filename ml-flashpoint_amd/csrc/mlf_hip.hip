@@ -1138,6 +1138,45 @@ uint32_t mlf_crc32c_combine(uint32_t crc_a, uint32_t crc_b, uint64_t len_b) {
   return gf_mul(x_pow_bytes(len_b), crc_a) ^ crc_b;
 }
 
+int mlf_crc32c_file(int fd, uint64_t file_offset, uint64_t nbytes, uint64_t chunk_bytes, uint32_t* out_host,
+                    uint64_t n_out, uint32_t threads) {
+  if (fd < 0) return fail(MLF_HIP_BAD_ARG, "bad file descriptor");
+  if (nbytes == 0) return MLF_HIP_OK;
+  if (chunk_bytes == 0 || !out_host) return fail(MLF_HIP_BAD_ARG, "chunk_bytes must be positive and out_host non-null");
+  const uint64_t n_chunks = (nbytes + chunk_bytes - 1) / chunk_bytes;
+  if (n_out < n_chunks) return fail(MLF_HIP_BAD_ARG, "checksum output too small");
+  if (threads < 1 || threads > 256) return fail(MLF_HIP_BAD_ARG, "threads must be in [1, 256]");
+  const size_t piece = (size_t)std::min<uint64_t>(chunk_bytes, (uint64_t)4 << 20);  // read granularity per thread
+  std::atomic<uint64_t> next{0};
+  std::atomic<int> err{0};
+  auto work = [&] {
+    std::vector<char> buf(piece);
+    for (;;) {
+      const uint64_t c = next.fetch_add(1);
+      if (c >= n_chunks || err.load()) return;
+      const uint64_t begin = c * chunk_bytes, len = std::min(chunk_bytes, nbytes - begin);
+      uint32_t crc = 0;
+      for (uint64_t done = 0; done < len; done += piece) {
+        const size_t n = (size_t)std::min<uint64_t>(piece, len - done);
+        if (int e = full_pread(fd, buf.data(), n, file_offset + begin + done)) {
+          err.store(e);
+          return;
+        }
+        const uint32_t part = mlf_crc32c_host(buf.data(), n);
+        crc = done == 0 ? part : mlf_crc32c_combine(crc, part, n);
+      }
+      out_host[c] = crc;
+    }
+  };
+  std::vector<std::thread> pool;
+  const unsigned width = (unsigned)std::min<uint64_t>(threads, n_chunks);
+  for (unsigned i = 1; i < width; ++i) pool.emplace_back(work);
+  work();
+  for (auto& t : pool) t.join();
+  if (int e = err.load()) return fail(MLF_HIP_RUNTIME, std::string("pread() failed: ") + strerror(e));
+  return MLF_HIP_OK;
+}
+
 int mlf_crc32c_device(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint32_t* out_host,
                       uint64_t n_out, void* stream_) {
   if (nbytes == 0) return MLF_HIP_OK;

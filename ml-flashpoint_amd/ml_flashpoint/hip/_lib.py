@@ -87,6 +87,7 @@ _SIGNATURES = {
     "mlf_crc32c_device": (_INT, [_VP, _U64, _U64, _VP, _U64, _VP]),
     "mlf_crc32c_host": (_U32, [_VP, _U64]),
     "mlf_crc32c_combine": (_U32, [_U32, _U32, _U64]),
+    "mlf_crc32c_file": (_INT, [_INT, _U64, _U64, _U64, _VP, _U64, _U32]),
     "mlf_engine_create": (_INT, [_U64, _U32, _U32, ctypes.POINTER(_VP)]),
     "mlf_engine_destroy": (_INT, [_VP]),
     "mlf_engine_d2h": (_INT, [_VP, _VP, _VP, _U64, _VP, ctypes.POINTER(XferStats)]),

@@ -17,6 +17,7 @@ import logging
 import os
 import pickle
 import struct
+import threading
 import time
 from pathlib import Path
 from typing import IO, Callable, List, Optional, cast
@@ -32,8 +33,9 @@ from typing_extensions import override
 from ml_flashpoint.checkpoint_object_manager.buffer_metadata import METADATA_SIZE
 from ml_flashpoint.checkpoint_object_manager.checkpoint_object_manager import CheckpointObjectManager
 from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId, CheckpointObjectId
+from ml_flashpoint.core.checkpoint_discovery import CheckpointDiscoveryMixin
 from ml_flashpoint.core.checkpoint_loader import MLFlashpointCheckpointLoader
-from ml_flashpoint.core.defaults import DIRTY_MARKER_SUFFIX, CheckpointFormat, default_metadata_object_name
+from ml_flashpoint.core.defaults import CheckpointFormat, default_metadata_object_name
 from ml_flashpoint.core.mlf_logging import get_logger
 from ml_flashpoint.core.utils import log_execution_time
 from ml_flashpoint.hip import _lib, integrity
@@ -56,7 +58,7 @@ def _element_size(dtype: torch.dtype) -> int:
     return esz
 
 
-class HipMLFlashpointCheckpointLoader(MLFlashpointCheckpointLoader):
+class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointCheckpointLoader):
     def __init__(
         self,
         checkpoint_object_manager: CheckpointObjectManager,
@@ -72,9 +74,12 @@ class HipMLFlashpointCheckpointLoader(MLFlashpointCheckpointLoader):
         block_threads: int = 0,
         verify_crc: bool = True,
         use_file_io: bool = True,
+        verify_on_discovery: bool = False,
     ):
         """Arguments as the reference's default loader (checkpoint_loader.py:126-158), plus the copy-engine and
-        kernel work-split knobs and ``verify_crc`` (check the CRC-32C sidecar of an object, when it has one)."""
+        kernel work-split knobs, ``verify_crc`` (check the CRC-32C sidecar of an object, when it has one, while
+        restoring it) and ``verify_on_discovery`` (also check it, on the host, while choosing the checkpoint to
+        recover from, so that a corrupted copy counts as missing)."""
         _lib.load()
         self._checkpoint_object_manager = checkpoint_object_manager
         self._replication_manager = replication_manager
@@ -90,17 +95,21 @@ class HipMLFlashpointCheckpointLoader(MLFlashpointCheckpointLoader):
         # pread() the buffer file into the pinned slots instead of reading through the (fresh, read-only) mapping:
         # reads of tmpfs run in parallel, and no page-table entry per 4 KiB has to be built and torn down
         self._use_file_io = use_file_io
+        self.verify_on_discovery = verify_on_discovery
         self._engine: Optional[hip_plan.CopyEngine] = None
+        self._engine_lock = threading.Lock()
+        self._init_discovery()
         self.last_load_stats: dict = {}
         # set to True to bracket every unpack launch with timing events; see the saver's attribute of the same name
         self.record_kernel_events = False
         self.kernel_events: list = []
 
     def _get_engine(self) -> hip_plan.CopyEngine:
-        if self._engine is None:
-            cfg = self._engine_config
-            self._engine = hip_plan.CopyEngine(cfg.slot_bytes, cfg.n_slots, cfg.copy_threads)
-        return self._engine
+        with self._engine_lock:  # read_data runs on one executor thread per object
+            if self._engine is None:
+                cfg = self._engine_config
+                self._engine = hip_plan.CopyEngine(cfg.slot_bytes, cfg.n_slots, cfg.copy_threads)
+            return self._engine
 
     @override
     @log_execution_time(logger=_LOGGER, name="read_metadata")
@@ -169,7 +178,7 @@ class HipMLFlashpointCheckpointLoader(MLFlashpointCheckpointLoader):
         planner: LoadPlanner,
         storage_data: dict[int, _StorageInfo],
     ) -> None:
-        if not os.path.exists(checkpoint_object_id.data):
+        if not os.path.exists(checkpoint_object_id.data) and not self._try_retrieve_object_if_missing(checkpoint_object_id):
             msg = f"Checkpoint object '{checkpoint_object_id.data}' does not exist on any node in the cluster"
             _LOGGER.error(msg)
             raise FileNotFoundError(msg)
@@ -308,34 +317,24 @@ class HipMLFlashpointCheckpointLoader(MLFlashpointCheckpointLoader):
             planner.commit_tensor(req, target)
         stats["device_items"] += len(device_reqs)
 
-    # ---- discovery --------------------------------------------------------------------------------------
-    @override
-    def get_latest_complete_checkpoint(
-        self, checkpoint_base_container: CheckpointContainerId
-    ) -> Optional[CheckpointContainerId]:
-        """Single-node form of the reference's discovery (checkpoint_loader.py:507-577): the highest
-        ``step-N_ckpt`` directory under the base that has no ``*unfinished`` marker beside it.  Agreement across
-        nodes and retrieval of missing objects from peers belong to the replication layer, which this package
-        does not implement."""
-        base = checkpoint_base_container.data
-        if not os.path.isdir(base):
-            return None
-        names = os.listdir(base)
-        dirty_pattern = CheckpointContainerId.get_dirty_version_checkpoint_container_pattern()
-        dirty_steps = set()
-        for name in names:
-            m = dirty_pattern.match(name)
-            if m and name.endswith(DIRTY_MARKER_SUFFIX):
-                dirty_steps.add(int(m.group(1)))
-        best = None
-        for name in names:
-            step = CheckpointContainerId.parse_version_container_step(name)
-            if step is None or step in dirty_steps or not os.path.isdir(os.path.join(base, name)):
-                continue
-            if best is None or step > best:
-                best = step
-        if best is None:
-            return None
-        return CheckpointContainerId.create_child(
-            checkpoint_base_container, CheckpointContainerId.format_version_container(best)
-        )
+    # ---- discovery (core/checkpoint_discovery.py) ----------------------------------------------------------
+    def _object_is_intact(self, path: str) -> bool:
+        """False when the object has a CRC-32C sidecar and its data section no longer matches it (host-side
+        check: pread + SSE4.2, no GPU).  Objects without a sidecar, and the sidecars themselves, pass."""
+        sidecar = integrity.read_sidecar(path)
+        if sidecar is None:
+            return True
+        chunk_bytes, data_bytes, want = sidecar
+        try:
+            fd = os.open(path, os.O_RDONLY)
+        except OSError:
+            return False
+        try:
+            if os.fstat(fd).st_size != METADATA_SIZE + data_bytes:
+                return False
+            got = hip_plan.crc32c_file(fd, METADATA_SIZE, data_bytes, chunk_bytes, self._engine_config.copy_threads)
+        except _lib.HipError:
+            return False
+        finally:
+            os.close(fd)
+        return bool((got == want).all())

@@ -342,3 +342,13 @@ def crc32c_host(ptr: int, nbytes: int) -> int:
 
 def crc32c_combine(crc_a: int, crc_b: int, len_b: int) -> int:
     return int(_lib.load().mlf_crc32c_combine(crc_a, crc_b, len_b))
+
+
+def crc32c_file(fd: int, file_offset: int, nbytes: int, chunk_bytes: int, threads: int = 8) -> np.ndarray:
+    """CRC-32C of each ``chunk_bytes`` piece of a byte range of an open file, computed on the host."""
+    n_chunks = (nbytes + chunk_bytes - 1) // chunk_bytes if nbytes else 0
+    out = np.zeros(n_chunks, dtype=np.uint32)
+    if n_chunks:
+        _lib.check(_lib.load().mlf_crc32c_file(fd, file_offset, nbytes, chunk_bytes, out.ctypes.data, n_chunks, threads),
+                   "mlf_crc32c_file")
+    return out

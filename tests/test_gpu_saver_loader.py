@@ -205,6 +205,7 @@ def test_megatron_style_sequence_with_pool_and_finalize(shm_dir, manager_future)
         results = writer.write_staged_data_buckets(cid, staged, replicate_after_write=False).wait()
         assert writer.get_write_results(cid) is not None
         writer.finish_checkpoint(cid, metadata, [results])
+        open(os.path.join(cid.data, "common.pt"), "wb").write(b"common state, written by the strategy")
         proc = saver.finalize_checkpoint(cid)
         assert not os.path.exists(marker)
         if proc is not None:

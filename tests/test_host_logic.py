@@ -117,20 +117,6 @@ def test_finalize_removes_only_older_well_formed_steps(tmp_path, older_than_step
     assert saver._remove_older_checkpoints(CheckpointContainerId(str(base / "not-a-step"))) is None
 
 
-def test_latest_complete_checkpoint_skips_unfinished_steps(tmp_path):
-    loader = DefaultMLFlashpointCheckpointLoader(CheckpointObjectManager(), None)
-    base = CheckpointContainerId(str(tmp_path / "job"))
-    assert loader.get_latest_complete_checkpoint(base) is None
-    for step in (5, 10, 20, 30):
-        os.makedirs(os.path.join(base.data, f"step-{step}_ckpt"))
-    os.makedirs(os.path.join(base.data, "latest"))
-    open(os.path.join(base.data, "step-30_ckpt__0__unfinished"), "w").close()  # still being written
-    open(os.path.join(base.data, "step-20_ckpt__3__unfinished"), "w").close()  # another local rank's marker counts too
-    assert loader.get_latest_complete_checkpoint(base).data == os.path.join(base.data, "step-10_ckpt")
-    os.remove(os.path.join(base.data, "step-30_ckpt__0__unfinished"))
-    assert loader.get_latest_complete_checkpoint(base).data == os.path.join(base.data, "step-30_ckpt")
-
-
 def test_saver_crosses_process_boundaries_as_configuration_only(tmp_path):
     saver = make_saver(initial_buffer_size_bytes=123, crc_chunk_bytes=1 << 20)
     saver._barrier_func = None  # lambdas do not pickle; the reference's users pass module-level callables
