@@ -18,7 +18,7 @@ from ml_flashpoint.adapter.pytorch.memory_storage_writer import MemoryStorageWri
 from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId
 from ml_flashpoint.core.checkpoint_saver import ObjectWriteBucket
 from ml_flashpoint.core.mlf_logging import get_logger
-from ml_flashpoint.core.utils import log_execution_time
+from ml_flashpoint.core.utils import gc_paused, log_execution_time
 
 _LOGGER = get_logger(__name__)
 
@@ -39,6 +39,11 @@ def generate_plan(
     saves compares equal, ``validated_cache_reuse`` turns True and later saves skip ``create_local_plan``, the plan
     reduce-scatter and the metadata broadcast (``global_metadata`` is then None: the caller reuses the one it has).
     """
+    with gc_paused():  # planning allocates ~10 small objects per tensor; see gc_paused
+        return _generate_plan(checkpoint_id, state_dict, storage_writer, planner, world_dist_wrapper, cached_ckpt_structure)
+
+
+def _generate_plan(checkpoint_id, state_dict, storage_writer, planner, world_dist_wrapper, cached_ckpt_structure):
     cached_central_plan, cached_local_plan, validated = cached_ckpt_structure or (None, None, False)
     global_metadata: torchdistsaver.Metadata | None = None
 

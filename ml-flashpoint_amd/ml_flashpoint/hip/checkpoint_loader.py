@@ -37,7 +37,7 @@ from ml_flashpoint.core.checkpoint_discovery import CheckpointDiscoveryMixin
 from ml_flashpoint.core.checkpoint_loader import MLFlashpointCheckpointLoader
 from ml_flashpoint.core.defaults import CheckpointFormat, default_metadata_object_name
 from ml_flashpoint.core.mlf_logging import get_logger
-from ml_flashpoint.core.utils import log_execution_time
+from ml_flashpoint.core.utils import gc_paused, log_execution_time
 from ml_flashpoint.hip import _lib, integrity
 from ml_flashpoint.hip import plan as hip_plan
 from ml_flashpoint.hip.checkpoint_saver import EngineConfig
@@ -120,7 +120,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
     ) -> Metadata:
         path = Path(checkpoint_id.data) / object_name
         try:
-            with open(path, "rb") as f:
+            with open(path, "rb") as f, gc_paused():  # unpickling creates ~5 objects per item and no cycles
                 return pickle.load(f)
         except Exception:
             _LOGGER.exception("Error reading metadata from '%s'", path)
@@ -184,7 +184,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
             raise FileNotFoundError(msg)
         t_start = time.perf_counter()
         stats = {"h2d_s": 0.0, "h2d_bytes": 0, "device_payload_bytes": 0, "host_items": 0, "device_items": 0}
-        with self._checkpoint_object_manager.get_buffer(checkpoint_object_id) as stream:
+        with gc_paused(), self._checkpoint_object_manager.get_buffer(checkpoint_object_id) as stream:
             optimized = stream.format_signature == CheckpointFormat.MLF_FORMAT
             device_reqs = []  # (req, target, dtype, shape, payload_off, stored payload bytes)
             whole = stream.raw_view()

@@ -46,7 +46,7 @@ from ml_flashpoint.core.checkpoint_saver import (
 )
 from ml_flashpoint.core.defaults import DIRTY_MARKER_SUFFIX, CheckpointFormat, default_metadata_object_name
 from ml_flashpoint.core.mlf_logging import get_logger
-from ml_flashpoint.core.utils import log_execution_time
+from ml_flashpoint.core.utils import gc_paused, log_execution_time
 from ml_flashpoint.hip import _lib, integrity
 from ml_flashpoint.hip import plan as hip_plan
 
@@ -318,6 +318,10 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         """Groups the items exactly as the reference does (same bucketing routine, same object names) and, per
         object, enqueues the pack of its image on the current stream.  The returned buckets carry
         ``StagedTensorRef`` placeholders; ``write_data`` finds the image through them."""
+        with gc_paused():
+            return self._prepare_write_data(checkpoint_id, write_items, write_item_resolver, object_name_prefix, bucket_count)
+
+    def _prepare_write_data(self, checkpoint_id, write_items, write_item_resolver, object_name_prefix, bucket_count):
         t_start = time.perf_counter()
         bucket_count = max(bucket_count, 1)
         rank = self._global_rank_getter()
@@ -487,7 +491,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         xfer = {"d2h_s": 0.0, "d2h_wait_s": 0.0, "d2h_bytes": 0, "crc_s": 0.0}
         for bucket in write_buckets:
             try:
-                all_results.extend(self._write_bucket(bucket, replicate_after_write, xfer))
+                with gc_paused():
+                    all_results.extend(self._write_bucket(bucket, replicate_after_write, xfer))
             except Exception as e:  # collected, first one re-raised: same contract as the reference's workers
                 _LOGGER.exception("Error writing object '%s'", bucket.object_id)
                 errors.append(e)
@@ -617,7 +622,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         final_path = os.path.join(checkpoint_id.data, md_object_name)
         tmp_path = final_path + ".tmp"
         os.makedirs(os.path.dirname(final_path), exist_ok=True)
-        with open(tmp_path, "wb") as f:
+        with open(tmp_path, "wb") as f, gc_paused():
             pickle.dump(metadata, f)
         os.rename(tmp_path, final_path)
 
