@@ -50,7 +50,7 @@ def parse_args():
     ap.add_argument("--block-threads", type=int, default=0)
     ap.add_argument("--slot-mib", type=int, default=32)
     ap.add_argument("--slots", type=int, default=4)
-    ap.add_argument("--copy-threads", type=int, default=8)
+    ap.add_argument("--copy-threads", type=int, default=0, help="0 = the engine's default (CPUs available, at most 16)")
     ap.add_argument("--crc-chunk-mib", type=int, default=0, help="> 0: CRC-32C per chunk on save, verified on restore")
     ap.add_argument("--cpu-baseline-gb", type=float, default=12.0, help="size of the CPU baseline's sample (0 = skip)")
     ap.add_argument("--plan-cache", action="store_true",
@@ -375,7 +375,7 @@ def main():
             "data": "synthetic",
             "config": {"workload": f"{args.workload}: {label}", "tensors": len(sd), "payload_bytes": payload,
                        "file_bytes": file_bytes, "scale": args.scale, "tile_bytes": args.tile_bytes or 4096,
-                       "engine": {"slot_mib": args.slot_mib, "slots": args.slots, "copy_threads": args.copy_threads},
+                       "engine": {"slot_mib": args.slot_mib, "slots": args.slots, "copy_threads": engine_cfg.resolved_copy_threads()},
                        "crc_chunk_mib": args.crc_chunk_mib, "plan_cache": args.plan_cache, "save_io": args.save_io, "restore_io": args.restore_io},
             "save_GBps": round(gb / mean(rec["save"]), 3),
             "restore_GBps": round(gb / mean(rec["restore"]), 3),

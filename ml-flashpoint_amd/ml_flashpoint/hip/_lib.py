@@ -38,6 +38,8 @@ class PlanOpts(ctypes.Structure):
         ("block_threads", ctypes.c_uint32),
         ("align_to_tensor", ctypes.c_uint32),
         ("unroll", ctypes.c_uint32),
+        ("grid_x_log2", ctypes.c_uint32),
+        ("reserved", ctypes.c_uint32),
     ]
 
 

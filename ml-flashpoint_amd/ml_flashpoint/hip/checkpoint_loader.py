@@ -108,7 +108,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         with self._engine_lock:  # read_data runs on one executor thread per object
             if self._engine is None:
                 cfg = self._engine_config
-                self._engine = hip_plan.CopyEngine(cfg.slot_bytes, cfg.n_slots, cfg.copy_threads)
+                self._engine = hip_plan.CopyEngine(cfg.slot_bytes, cfg.n_slots, cfg.resolved_copy_threads())
             return self._engine
 
     @override
@@ -332,7 +332,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         try:
             if os.fstat(fd).st_size != METADATA_SIZE + data_bytes:
                 return False
-            got = hip_plan.crc32c_file(fd, METADATA_SIZE, data_bytes, chunk_bytes, self._engine_config.copy_threads)
+            got = hip_plan.crc32c_file(fd, METADATA_SIZE, data_bytes, chunk_bytes, self._engine_config.resolved_copy_threads())
         except _lib.HipError:
             return False
         finally:

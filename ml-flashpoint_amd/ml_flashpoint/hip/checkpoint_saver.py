@@ -61,7 +61,18 @@ class EngineConfig:
 
     slot_bytes: int = 32 << 20
     n_slots: int = 4
-    copy_threads: int = 8
+    # host threads that move a slot to/from the buffer file; 0 = the CPUs this process may run on, at most 16
+    # (reading a tmpfs file back at link speed takes ~12 of them, writing the mapping ~6)
+    copy_threads: int = 0
+
+    def resolved_copy_threads(self) -> int:
+        if self.copy_threads > 0:
+            return self.copy_threads
+        try:
+            cpus = len(os.sched_getaffinity(0))
+        except (AttributeError, OSError):
+            cpus = os.cpu_count() or 1
+        return max(1, min(16, cpus))
 
 
 class StagedObject:
@@ -233,7 +244,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         with self._engine_lock:
             if self._engine is None:
                 cfg = self._engine_config
-                self._engine = hip_plan.CopyEngine(cfg.slot_bytes, cfg.n_slots, cfg.copy_threads)
+                self._engine = hip_plan.CopyEngine(cfg.slot_bytes, cfg.n_slots, cfg.resolved_copy_threads())
             return self._engine
 
     # ---- dirty marker / directory ----------------------------------------------------------------------

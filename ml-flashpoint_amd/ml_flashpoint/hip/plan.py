@@ -195,10 +195,11 @@ class Plan:
         block_threads: int = 0,
         align_to_tensor: bool = False,
         unroll: int = 0,
+        grid_x_log2: int = 0,
     ):
         lib = _lib.load()
         assert items.dtype == ITEM_DTYPE and items.flags["C_CONTIGUOUS"]
-        opts = _lib.PlanOpts(tile_bytes, block_threads, 1 if align_to_tensor else 0, unroll)
+        opts = _lib.PlanOpts(tile_bytes, block_threads, 1 if align_to_tensor else 0, unroll, grid_x_log2, 0)
         handle = ctypes.c_void_p()
         blob_buf = (ctypes.c_char * len(blob)).from_buffer_copy(blob) if blob else None
         _lib.check(

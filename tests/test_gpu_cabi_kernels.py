@@ -79,6 +79,30 @@ def test_pack_tile_and_block_shapes(tile_bytes, threads):
     assert got == oracle_fmt.data_section(cpu)[0]
 
 
+@pytest.mark.parametrize("grid_x_log2", [1, 3, 8, 11])
+def test_flat_kernel_grid_rows(grid_x_log2):
+    """All three span classes (entries shared by 128, 16 and 1 workgroups) go out in one launch whose workgroups are
+    numbered row by row over a 2-D grid; with rows of 1, 4, 128 and 1024 workgroups, class boundaries and the padding of the last row fall
+    everywhere.  Pack is compared with the oracle, unpack must restore the tensors."""
+    from ml_flashpoint.hip import plan as P
+
+    gen = torch.Generator().manual_seed(14)
+    shapes = [((3 << 20) + 5,), ((1 << 19) + 1,), (70001,), (4097,), (1500,), (9,)]  # 1 KiB tiles: 128-, 16-, 1-tile spans
+    cpu = [_rand_tensor(gen, s, torch.uint8) for s in shapes]
+    dev = [t.to(DEV) for t in cpu]
+    layout, plan, image, got = _pack_image(dev, tile_bytes=1024, block_threads=64, grid_x_log2=grid_x_log2)
+    assert plan.info.n_flat_tiles > 3000
+    assert got == oracle_fmt.data_section(cpu)[0]
+    targets = [torch.zeros_like(t) for t in dev]
+    table = P.ItemTable()
+    for t, (off, length) in zip(targets, layout.spans):
+        table.add_device(t.data_ptr(), off + length - t.numel(), 1, tuple(t.shape), (1,))
+    P.Plan(table.to_array(), b"", layout.image_bytes, tile_bytes=1024, block_threads=64, align_to_tensor=True,
+           grid_x_log2=grid_x_log2).unpack(image)
+    torch.cuda.synchronize()
+    assert all(torch.equal(a, b) for a, b in zip(targets, dev))
+
+
 def test_pack_misaligned_sources():
     """Views that start at odd element offsets: the source address is not 16-byte aligned."""
     gen = torch.Generator().manual_seed(13)
@@ -219,9 +243,8 @@ def test_pack_large_rows_go_through_flat_kernel():
     assert plan.info.n_strided_items == 0 and plan.info.n_flat_tiles >= 64
 
 
-def test_pack_and_unpack_tables_larger_than_one_launch():
-    """5 GiB through 1 KiB tiles of 1024 threads needs more than 2^32 threads: the work goes out in several
-    launches.  Checked on the device (payload region of the image == source; round trip restores the source)."""
+def test_pack_and_unpack_grids_of_more_than_2_to_32_threads():
+    """5 GiB through 1 KiB tiles of 1024 threads needs more than 2^32 threads: the grid gets a second dimension.  Checked on the device (payload region of the image == source; round trip restores the source)."""
     from ml_flashpoint.hip import plan as P
 
     n = 5 * (1 << 30) + 12345
