@@ -3,8 +3,10 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload llama3-8b-shard] [--scale S]
 
 A *step* is one full save of the workload's state dict (resident in HBM) into a pooled tmpfs buffer object, followed
-by one full restore of that object into the (zeroed) live tensors, both driven through the PyTorch DCP adapters
-(``MemoryStorageWriter`` / ``MemoryStorageReader``) with the gfx950 saver/loader plugged in.  Prints ONE JSON line:
+by one full restore of that object into the (zeroed) live tensors.  The save is the reference's three-call sequence
+(``generate_plan`` -> stage -> ``write_data`` -> ``finish_write``, then ``finalize_checkpoint``) over
+``MemoryStorageWriter``; the restore is ``dcp.load`` over ``MemoryStorageReader``; the gfx950 saver/loader are plugged
+in, CRC-32C per 32 MiB chunk is computed on save and verified on restore.  Prints ONE JSON line:
 
 * ``value``          GB/s moved through the path per step: (bytes saved + bytes restored) / step time
 * ``save_GBps`` / ``restore_GBps`` / ``blocking_save_ms`` (save entry -> training stream may continue) and the
@@ -51,7 +53,9 @@ def parse_args():
     ap.add_argument("--slot-mib", type=int, default=32)
     ap.add_argument("--slots", type=int, default=4)
     ap.add_argument("--copy-threads", type=int, default=0, help="0 = the engine's default (CPUs available, at most 16)")
-    ap.add_argument("--crc-chunk-mib", type=int, default=0, help="> 0: CRC-32C per chunk on save, verified on restore")
+    ap.add_argument("--crc-chunk-mib", type=int, default=32,
+                    help="CRC-32C per chunk of this size, computed on the GPU during the save and verified on the GPU during "
+                         "the restore (0 = off)")
     ap.add_argument("--cpu-baseline-gb", type=float, default=12.0, help="size of the CPU baseline's sample (0 = skip)")
     ap.add_argument("--plan-cache", action="store_true",
                     help="reuse the save plan across steps once two consecutive plans compared equal, as the reference's "
