@@ -124,9 +124,10 @@ struct TransWork {  // kTransTilesPerEntry consecutive tiles of descriptor `desc
 // ---------------------------------------------------------------------------------------------------------
 // flat kernel
 // ---------------------------------------------------------------------------------------------------------
-// Workgroup b of a class serves tile (b & mask) of span (b >> shift).  Tile boundaries inside a span sit at 16-byte
-// boundaries of the destination: tile 0 is [0, head + T), tile j is [head + j*T, head + (j+1)*T), the last one
-// is cut at the span's end, where head = bytes from the span's first destination byte to the next boundary.
+// Workgroup b of a class serves tile (b & mask) of span (b >> shift).  Tile boundaries inside a span sit on a grid
+// of the destination (image offsets when packing, tensor addresses when unpacking; up to 4 KiB, so that full tiles
+// write whole, aligned lines): tile 0 is [0, head + T), tile j is [head + j*T, head + (j+1)*T), the last one
+// is cut at the span's end, where head = bytes from the span's first destination byte to the next grid line.
 // Threads interleave at 16-byte granularity, so a wavefront moves 1 KiB of consecutive bytes per access.
 constexpr int kFlatClasses = 3;  // span tables whose entries are shared by 128, 16 and 1 workgroups
 
@@ -145,6 +146,7 @@ __global__ void __launch_bounds__(1024) mlf_flat_kernel(const Span* __restrict__
                                                         const Span* __restrict__ spans2, uint32_t first1,
                                                         uint32_t first2, uint32_t total, uint32_t grid_x_log2,
                                                         uint32_t tile_bytes, uint32_t block_threads,
+                                                        uint32_t cut_mask, uint32_t cut_on_tensor,
                                                         char* __restrict__ image) {
   uint32_t wg = (blockIdx.y << grid_x_log2) + blockIdx.x;
   const bool live = wg < total;
@@ -157,7 +159,9 @@ __global__ void __launch_bounds__(1024) mlf_flat_kernel(const Span* __restrict__
   const uint32_t span_n = live ? sp.n : 0u;
   const char* src0 = PACK ? reinterpret_cast<const char*>(sp.tensor) : image + sp.image;
   char* dst0 = PACK ? image + sp.image : reinterpret_cast<char*>(sp.tensor);
-  uint32_t head0 = (16u - (uint32_t)(reinterpret_cast<uintptr_t>(dst0) & 15u)) & 15u;
+  // tile cuts sit on the plan's grid: multiples of (cut_mask + 1) bytes of the image offset or of the tensor address
+  const uint32_t cut_pos = (uint32_t)(cut_on_tensor ? sp.tensor : sp.image);
+  uint32_t head0 = (0u - cut_pos) & cut_mask;
   head0 = head0 < span_n ? head0 : span_n;
   uint32_t start = sub ? head0 + sub * tile_bytes : 0u;
   start = start < span_n ? start : span_n;  // unused slot of a partly filled span: nothing left
@@ -169,7 +173,9 @@ __global__ void __launch_bounds__(1024) mlf_flat_kernel(const Span* __restrict__
   uint32_t n = end - start;
   const uint32_t tid = threadIdx.x;
   const uint32_t bd = block_threads;
-  uint32_t head = sub ? 0u : head0;  // only a span's first tile starts off a boundary
+  // bytes up to the destination's next 16-byte boundary (none when the cuts are on the destination's side, except
+  // in a span's first tile)
+  uint32_t head = (0u - (uint32_t)reinterpret_cast<uintptr_t>(dst)) & 15u;
   head = head < n ? head : n;
   if (tid < head) dst[tid] = src[tid];
   src += head;
@@ -799,6 +805,8 @@ struct mlf_plan {
   char* d_blob = nullptr;
   uint32_t block_threads = 256;
   uint32_t unroll = 1;
+  uint32_t cut_mask = 15;     // tile cuts sit on multiples of cut_mask + 1 bytes ...
+  uint32_t cut_on_tensor = 0;  // ... of the tensor address (1) or of the image offset (0)
   uint32_t grid_x_log2 = 20;  // log2 of the workgroups per grid row of the flat kernel's launch
   uint32_t flat_first[kFlatClasses] = {0, 0, 0};  // first workgroup of each span class in that launch
   uint32_t flat_total = 0;
@@ -818,28 +826,26 @@ struct SpanTables {
 // single tiles; a rest of at most 1 KiB goes to the per-wavefront table.  Every entry is self-contained (the kernel derives tile cuts from the entry's own first
 // destination address), so pieces may start anywhere.
 void cut_spans(SpanTables& out, uint64_t tensor_addr, uint64_t image_off, uint64_t n, uint32_t tile,
-               bool align_to_tensor) {
+               bool align_to_tensor, uint32_t cut_mask) {
   uint64_t done = 0;
   while (done < n) {
-    const uint64_t dst_addr = (align_to_tensor ? tensor_addr : image_off) + done;  // image base is 256-byte aligned
-    const uint64_t head = (16 - (dst_addr & 15)) & 15;
+    const uint64_t cut_pos = (align_to_tensor ? tensor_addr : image_off) + done;
+    const uint64_t head = (0 - cut_pos) & cut_mask;  // bytes to the next grid line; 0 after an item's first span
     const uint64_t left = n - done;
     if (left <= kSmallItemBytes) {
       out.cls[kSmallClass].push_back(Span{tensor_addr + done, image_off + done, (uint32_t)left, 0});
       break;
     }
+    // an entry of class c holds head + (tile << shift) bytes: its first tile carries the head on top, so every
+    // later tile, and every later span of the item, starts on the grid; the single-tile class also takes a short rest
     int c = kSmallClass - 1;
     for (int k = 0; k < kSmallClass; ++k) {
-      if (left >= ((uint64_t)tile << kSpanShift[k])) {
+      if (left >= head + ((uint64_t)tile << kSpanShift[k])) {
         c = k;
         break;
       }
     }
-    // a full entry of class c holds (tile << shift) bytes; the single-tile class also takes the short rest,
-    // and its first tile may carry the head bytes on top
-    uint64_t len = (uint64_t)tile << kSpanShift[c];
-    if (c == kSmallClass - 1) len = std::min<uint64_t>(left, tile + head);
-    len = std::min(len, left);
+    const uint64_t len = std::min<uint64_t>(left, head + ((uint64_t)tile << kSpanShift[c]));
     out.cls[c].push_back(Span{tensor_addr + done, image_off + done, (uint32_t)len, 0});
     done += len;
   }
@@ -922,6 +928,9 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
   plan->block_threads = threads;
   plan->tile_bytes = tile;
   plan->unroll = opts && opts->unroll ? opts->unroll : 1;
+  // cuts on the largest power of two that divides the tile size, at most 4 KiB: full tiles then write whole lines
+  plan->cut_mask = std::min<uint32_t>(tile & (0u - tile), 4096u) - 1u;
+  plan->cut_on_tensor = align_to_tensor ? 1u : 0u;
   // gridDim.x * blockDim.x must stay below 2^32.  Rows of 2^16 workgroups measured fastest on the 112 GB shard
   // (36.5 ms per pack; rows of 2^20: 36.9 ms, of 2^23: 39.2 ms)
   uint32_t widest = 0;
@@ -957,7 +966,7 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
         rc = fail(MLF_HIP_BAD_ARG, "blob item " + std::to_string(k) + " lies outside the host blob");
         break;
       }
-      cut_spans(tiles, blob_base + it.ptr, it.image_off, it.nbytes, tile, false);
+      cut_spans(tiles, blob_base + it.ptr, it.image_off, it.nbytes, tile, align_to_tensor, plan->cut_mask);
       info.blob_bytes += it.nbytes;
       continue;
     }
@@ -997,7 +1006,7 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
     info.device_bytes += it.nbytes;
     const Collapsed c = collapse_dims(it);
     if (c.ndim == 0 || (c.ndim == 1 && c.ts[0] == 1 && c.is[0] == 1)) {
-      cut_spans(tiles, it.ptr, it.image_off, it.nbytes, tile, align_to_tensor);
+      cut_spans(tiles, it.ptr, it.image_off, it.nbytes, tile, align_to_tensor, plan->cut_mask);
       continue;
     }
     // rows that are contiguous on both sides and long enough go through the flat kernel, one row at a time
@@ -1013,7 +1022,7 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
           ioff += idx[d] * c.is[d];
         }
         cut_spans(tiles, it.ptr + (uint64_t)(toff * (int64_t)esz), it.image_off + (uint64_t)(ioff * (int64_t)esz),
-                  row_bytes, tile, align_to_tensor);
+                  row_bytes, tile, align_to_tensor, plan->cut_mask);
         for (int d = last - 1; d >= 0; --d) {
           if (++idx[d] < c.shape[d]) break;
           idx[d] = 0;
@@ -1153,7 +1162,7 @@ int launch_plan(const mlf_plan* plan, char* image, hipStream_t stream) {
 #define MLF_FLAT_LAUNCH(U)                                                                                     \
   hipLaunchKernelGGL((mlf_flat_kernel<PACK, U>), grid, block, 0, stream, plan->d_spans[0], plan->d_spans[1],     \
                      plan->d_spans[2], plan->flat_first[1], plan->flat_first[2], total, row_log2,              \
-                     plan->tile_bytes, plan->block_threads, image)
+                     plan->tile_bytes, plan->block_threads, plan->cut_mask, plan->cut_on_tensor, image)
     switch (plan->unroll) {
       case 2: MLF_FLAT_LAUNCH(2); break;
       case 4: MLF_FLAT_LAUNCH(4); break;
