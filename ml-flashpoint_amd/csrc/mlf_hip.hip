@@ -71,6 +71,19 @@ double now_s() {
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef u32x4 u32x4_u __attribute__((aligned(1)));  // dwordx4 access at any byte address
 
+// Tensor addresses arrive as integers, which the compiler can only treat as generic ("flat") pointers: flat accesses
+// count against both memory counters and are kept in order with LDS traffic.  Everything this library touches is
+// global memory, so the hot accesses say so.
+#define MLF_GLOBAL __attribute__((address_space(1)))
+template <typename T>
+__device__ __forceinline__ const MLF_GLOBAL T* gload(const void* p) {
+  return (const MLF_GLOBAL T*)p;
+}
+template <typename T>
+__device__ __forceinline__ MLF_GLOBAL T* gstore(void* p) {
+  return (MLF_GLOBAL T*)p;
+}
+
 struct Span {       // n bytes of one contiguous item, copied by the (1 << shift) workgroups that share the entry
   uint64_t tensor;  // absolute device address on the tensor (or blob) side
   uint64_t image;   // byte offset in the image
@@ -190,9 +203,9 @@ __global__ void __launch_bounds__(1024) mlf_flat_kernel(const Span* __restrict__
       u32x4 v[U];
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_u*>(src + (size_t)(i + u * bd) * 16));
+        v[u] = __builtin_nontemporal_load(gload<u32x4_u>(src + (size_t)(i + u * bd) * 16));
 #pragma unroll
-      for (int u = 0; u < U; ++u) __builtin_nontemporal_store(v[u], &d[i + u * bd]);
+      for (int u = 0; u < U; ++u) __builtin_nontemporal_store(v[u], gstore<u32x4>(&d[i + u * bd]));
     }
   }
   const uint32_t delta = (uint32_t)(reinterpret_cast<uintptr_t>(src) & 15u);  // uniform over the workgroup
@@ -200,8 +213,8 @@ __global__ void __launch_bounds__(1024) mlf_flat_kernel(const Span* __restrict__
     // dwordx4 loads need dword alignment only: a source that is off the 16-byte grid by 4, 8 or 12 bytes is read
     // directly (measured faster than the exchange below: 6.44 vs 6.29 TB/s at delta = 8)
     for (; i < nvec; i += bd) {
-      u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_u*>(src + (size_t)i * 16));
-      __builtin_nontemporal_store(v, &d[i]);
+      u32x4 v = __builtin_nontemporal_load(gload<u32x4_u>(src + (size_t)i * 16));
+      __builtin_nontemporal_store(v, gstore<u32x4>(&d[i]));
     }
   } else {
     // The source is off the destination's grid by a number of bytes that is not a multiple of 4.  Instead of
@@ -214,8 +227,8 @@ __global__ void __launch_bounds__(1024) mlf_flat_kernel(const Span* __restrict__
     for (; (i & ~63u) < nvec; i += bd) {  // whole wavefronts stay in the loop: the lane exchange needs them
       u32x4 lo = {0u, 0u, 0u, 0u}, far = {0u, 0u, 0u, 0u}, hi;
       const bool edge = lane == 63u && i < nvec;  // this lane's neighbour is in another wavefront
-      if (i <= nvec) lo = __builtin_nontemporal_load(a + i);
-      if (edge) far = __builtin_nontemporal_load(a + i + 1);  // issued with the load above, not after the exchange
+      if (i <= nvec) lo = __builtin_nontemporal_load(gload<u32x4>(a + i));
+      if (edge) far = __builtin_nontemporal_load(gload<u32x4>(a + i + 1));  // issued with the load above, not after the exchange
       hi.x = (uint32_t)__shfl_down((int)lo.x, 1);
       hi.y = (uint32_t)__shfl_down((int)lo.y, 1);
       hi.z = (uint32_t)__shfl_down((int)lo.z, 1);
@@ -234,7 +247,7 @@ __global__ void __launch_bounds__(1024) mlf_flat_kernel(const Span* __restrict__
         v.y = __builtin_amdgcn_alignbyte(w2, w1, r);
         v.z = __builtin_amdgcn_alignbyte(w3, w2, r);
         v.w = __builtin_amdgcn_alignbyte(w4, w3, r);
-        __builtin_nontemporal_store(v, &d[i]);
+        __builtin_nontemporal_store(v, gstore<u32x4>(&d[i]));
       }
     }
   }
@@ -281,7 +294,7 @@ __global__ void __launch_bounds__(256) mlf_small_kernel(const Span* __restrict__
 template <typename T>
 __device__ __forceinline__ void copy_elem(char* dst, const char* src) {
   typedef T unaligned_t __attribute__((aligned(1)));
-  *reinterpret_cast<unaligned_t*>(dst) = *reinterpret_cast<const unaligned_t*>(src);
+  *gstore<unaligned_t>(dst) = *gload<unaligned_t>(src);
 }
 
 // Generic N-d walk.  A thread decomposes its first element index once (divisions), then advances the multi-index
@@ -1084,8 +1097,8 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
     }
     const uint32_t desc_idx = (uint32_t)descs.size();
     descs.push_back(sd);
-    for (uint64_t s = 0; s < numel; s += kStridedElemsPerBlock)
-      work.push_back(StridedWork{s, (uint32_t)std::min<uint64_t>(kStridedElemsPerBlock, numel - s), desc_idx});
+    for (uint64_t s0 = 0; s0 < numel; s0 += kStridedElemsPerBlock)
+      work.push_back(StridedWork{s0, (uint32_t)std::min<uint64_t>(kStridedElemsPerBlock, numel - s0), desc_idx});
     ++info.n_strided_items;
   }
   for (int c = 0; c < kSpanClasses && rc == MLF_HIP_OK; ++c) {

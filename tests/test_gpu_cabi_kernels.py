@@ -233,6 +233,49 @@ def test_strided_walk_many_shapes_against_bruteforce():
     assert torch.equal(back.cpu()[mask], base[mask]) and int(back.cpu()[~mask].abs().sum()) == 0
 
 
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.bfloat16, torch.float32, torch.int64, torch.complex128])
+def test_strided_views_with_long_rows(dtype):
+    """Strided views with rows of hundreds to tens of thousands of elements (a workgroup's share of 32 Ki elements
+    then covers many rows, or less than one), both directions, against the oracle."""
+    from ml_flashpoint.hip import plan as P
+
+    gen = torch.Generator().manual_seed(33)
+    base = _rand_tensor(gen, (3, 7, 2100), dtype)
+    wide = _rand_tensor(gen, (2, 70001), dtype)
+    esz = base.element_size()
+    pick = lambda t, w: [  # noqa: E731
+        t[:, :, ::2],                      # 1050 per row, 21 rows
+        t[:, :, 1::3],
+        t[:, ::2, 5:1500:1][:, :, ::1][..., 3:],  # contiguous rows of 1492, too short for the flat kernel at 1 byte
+        t[1, :, :997:1][:, ::1][:, 1::2],
+        t.permute(1, 0, 2)[:, :, 2:2000:2],
+        t[:, :, 40:700],                   # 660 per row
+        w[:, ::2],                         # 35001 per row: more than one workgroup's share
+        w[1:, 5::1][:, ::3],
+    ]
+    dev, wide_dev = base.to(DEV), wide.to(DEV)
+    cpu_views, dev_views = pick(base, wide), pick(dev, wide_dev)
+    layout, plan, image, got = _pack_image(dev_views)
+    name = oracle_fmt.dtype_name(dtype)
+    want = b"".join(oracle_fmt.header_bytes(name, tuple(t.shape)) + oracle_fmt.payload_bytes(t) for t in cpu_views)
+    assert got == want
+    small = cpu_views[1]
+    assert oracle_fmt.payload_bytes(small) == oracle_fmt.payload_bytes_bruteforce(small)
+    back, wide_back = torch.zeros_like(dev), torch.zeros_like(wide_dev)
+    table = P.ItemTable()
+    for src, tgt, (off, length) in zip(cpu_views, pick(back, wide_back), layout.spans):
+        table.add_device(tgt.data_ptr(), off + length - src.numel() * esz, esz, tuple(src.shape), tuple(tgt.stride()))
+    P.Plan(table.to_array(), b"", layout.image_bytes, align_to_tensor=True).unpack(image)
+    torch.cuda.synchronize()
+    mask_base, mask_wide = torch.zeros(base.shape, dtype=torch.bool), torch.zeros(wide.shape, dtype=torch.bool)
+    for m in pick(mask_base, mask_wide):
+        m.fill_(True)
+    for ref, got_dev, mask in ((base, back, mask_base), (wide, wide_back, mask_wide)):
+        got_b = got_dev.cpu().contiguous().view(torch.uint8).reshape(*ref.shape, esz)
+        want_b = ref.contiguous().view(torch.uint8).reshape(*ref.shape, esz)
+        assert torch.equal(got_b[mask], want_b[mask]) and int(got_b[~mask].count_nonzero()) == 0
+
+
 def test_pack_large_rows_go_through_flat_kernel():
     gen = torch.Generator().manual_seed(15)
     base_cpu = _rand_tensor(gen, (64, 8192), torch.bfloat16)
