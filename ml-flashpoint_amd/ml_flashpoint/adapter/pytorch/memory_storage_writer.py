@@ -26,7 +26,7 @@ from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId, Checkp
 from ml_flashpoint.core.checkpoint_saver import MLFlashpointCheckpointSaver, ObjectWriteBucket
 from ml_flashpoint.core.hfid import generate_hfid
 from ml_flashpoint.core.mlf_logging import get_logger
-from ml_flashpoint.core.utils import log_execution_time
+from ml_flashpoint.core.utils import gc_paused, log_execution_time
 
 _LOGGER = get_logger(__name__)
 
@@ -132,6 +132,7 @@ class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
 
     @staticmethod
     @log_execution_time(logger=_LOGGER, name="stage_write_data_buckets", level=logging.INFO)
+    @gc_paused()
     def stage_write_data_buckets(
         _: CheckpointContainerId, write_buckets: list[ObjectWriteBucket], non_blocking: bool = True
     ):
@@ -149,6 +150,7 @@ class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
         return staged
 
     @log_execution_time(logger=_LOGGER, name="write_staged_write_buckets", level=logging.INFO)
+    @gc_paused()
     def write_staged_data_buckets(
         self,
         checkpoint_id: CheckpointContainerId,
@@ -218,6 +220,7 @@ class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
         self.finish_checkpoint(self.current_checkpoint_id, metadata, results)
 
     @log_execution_time(logger=_LOGGER, name="finish_checkpoint", level=logging.INFO)
+    @gc_paused()
     def finish_checkpoint(
         self, checkpoint_id: CheckpointContainerId, metadata: Metadata, results: list[list[WriteResult]]
     ) -> None:
