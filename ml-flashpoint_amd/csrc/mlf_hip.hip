@@ -438,9 +438,9 @@ __global__ void __launch_bounds__(256) mlf_strided_kernel(const StridedDesc* __r
 // ---------------------------------------------------------------------------------------------------------
 // One workgroup moves one T x T tile of a 2-D transposition through LDS so that both the read (along the source's
 // contiguous dimension) and the write (along the destination's) are made of whole, consecutive >= 128-byte runs.
-// Global accesses are max(4, esz)-byte vectors (hardware-unaligned where the view starts off a boundary); LDS is
-// addressed per element on the transposed side.  T = 128 / 64 / 64 / 32 / 16 elements for esz = 1 / 2 / 4 / 8 / 16;
-// rows of the LDS tile are padded by one vector so that a column walk does not stay in one bank.
+// Global accesses are 16-byte vectors on both sides (hardware-unaligned where the view starts off a boundary; narrower
+// accesses are bound by the number of lane accesses, not by bytes); LDS is addressed per element on the transposed side.  T = 128 / 64 / 64 / 32 / 16 elements for esz = 1 / 2 / 4 / 8 / 16;
+// rows of the LDS tile are padded so that a column walk does not stay in one bank.
 constexpr uint32_t kTransThreads = 256;
 constexpr uint32_t kTransBand = 8;  // tile-rows per band of the visiting order (measured: 8 beats 1 by 10-40 %)
 constexpr uint32_t kTransLdsBytes = 128 * (128 + 16);
@@ -454,8 +454,11 @@ __device__ __forceinline__ void trans_tile(const TransDesc* __restrict__ d, uint
                                            char* __restrict__ lds) {
   constexpr uint32_t ESZ = sizeof(E), VEC = sizeof(V), EPV = VEC / ESZ;
   const uint32_t T = trans_tile_dim(ESZ);
-  const uint32_t pitch = T * ESZ + VEC;
+  // LDS rows are padded by one dword (two for 8-byte elements): a column walk of one vector per lane then spreads
+  // over the banks (lane stride EPV * pitch = 8, 16, 4, 4 banks modulo 64 for 2-, 1-, 4-, 8-byte elements)
+  const uint32_t pitch = T * ESZ + (ESZ == 16 ? 16u : ESZ == 8 ? 8u : 4u);
   typedef V vec_u __attribute__((aligned(1)));
+  typedef V vec_lds __attribute__((aligned(ESZ < 4 ? 4 : ESZ)));  // as aligned as an LDS row start is
   typedef E elem_u __attribute__((aligned(1)));
 
   // which tile: batch index, then tile row (a) and tile column (b); b runs fastest
@@ -495,7 +498,7 @@ __device__ __forceinline__ void trans_tile(const TransDesc* __restrict__ d, uint
     const char* g = src + (int64_t)y * ld_src + (int64_t)x * ESZ;
     char* l = lds + y * pitch + x * ESZ;
     if (x + EPV <= xn) {
-      *reinterpret_cast<V*>(l) = *reinterpret_cast<const vec_u*>(g);
+      *reinterpret_cast<vec_lds*>(l) = *gload<vec_u>(g);
     } else {
       for (uint32_t k = 0; x + k < xn; ++k) reinterpret_cast<E*>(l)[k] = reinterpret_cast<const elem_u*>(g)[k];
     }
@@ -511,7 +514,7 @@ __device__ __forceinline__ void trans_tile(const TransDesc* __restrict__ d, uint
       E* parts = reinterpret_cast<E*>(&out);
 #pragma unroll
       for (uint32_t k = 0; k < EPV; ++k) parts[k] = *reinterpret_cast<const E*>(l + k * pitch);
-      *reinterpret_cast<vec_u*>(g) = out;
+      *gstore<vec_u>(g) = out;
     } else {
       for (uint32_t k = 0; y + k < yn; ++k) reinterpret_cast<elem_u*>(g)[k] = *reinterpret_cast<const E*>(l + k * pitch);
     }
@@ -528,10 +531,10 @@ __global__ void __launch_bounds__(kTransThreads) mlf_transpose_kernel(const Tran
   const uint64_t tile = w.first_tile + (blockIdx.x % kTransTilesPerEntry);
   if (tile >= d->n_tiles) return;  // uniform per workgroup: nobody reaches the barrier
   switch (d->esz) {
-    case 1: trans_tile<PACK, uint8_t, uint32_t>(d, tile, image, lds); break;
-    case 2: trans_tile<PACK, uint16_t, uint32_t>(d, tile, image, lds); break;
-    case 4: trans_tile<PACK, uint32_t, uint32_t>(d, tile, image, lds); break;
-    case 8: trans_tile<PACK, uint64_t, uint64_t>(d, tile, image, lds); break;
+    case 1: trans_tile<PACK, uint8_t, u32x4>(d, tile, image, lds); break;
+    case 2: trans_tile<PACK, uint16_t, u32x4>(d, tile, image, lds); break;
+    case 4: trans_tile<PACK, uint32_t, u32x4>(d, tile, image, lds); break;
+    case 8: trans_tile<PACK, uint64_t, u32x4>(d, tile, image, lds); break;
     default: trans_tile<PACK, u32x4, u32x4>(d, tile, image, lds); break;  // 16
   }
 }
