@@ -37,7 +37,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, vendor figure
 # with `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`, each scaled against a torch.add kernel of known size
 # (summary: profiles/pmc_traffic_mlf_flat_kernel_llama3-8b-shard.md).  Hardware counters cannot be read from
 # inside this script, so the ratio is applied to the live algorithmic byte count of the same workload only.
-PACK_TRAFFIC_RATIO_LLAMA3_8B = 1.0205
+PACK_TRAFFIC_RATIO_LLAMA3_8B = 1.0160
 
 
 def parse_args():
