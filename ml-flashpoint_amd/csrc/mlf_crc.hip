@@ -1,0 +1,284 @@
+// CRC-32C (Castagnoli) of a checkpoint image: per-chunk values computed on the GPU, the same function on host
+// memory and on a byte range of a file, and the combine law.  Part of the library behind include/mlf_hip.h.
+//
+// Device side: per wavefront a 64 KiB segment is read as coalesced 1 KiB rows; every lane keeps four Horner
+// accumulators advanced by x^8192 through LDS tables, then lanes are folded with GF(2) multiplies; a second, tiny
+// kernel chains the segment values of every chunk.
+#include "mlf_internal.h"
+
+#include <nmmintrin.h>
+
+#include <algorithm>
+#include <atomic>
+#include <mutex>
+#include <string>
+#include <thread>
+#include <vector>
+
+namespace mlf {
+
+struct CrcConsts {
+  uint32_t row_tab[4][256];  // state advanced by one 1 KiB row, sliced by state byte
+  uint32_t x4, x16, x32, x64, x128, x256, x512;  // x^(8*n) for the fold steps
+  uint32_t xseg;             // x^(8*kCrcSegBytes)
+};
+
+}  // namespace mlf
+
+using namespace mlf;
+
+namespace {
+
+// ---------------------------------------------------------------------------------------------------------
+// CRC-32C
+// ---------------------------------------------------------------------------------------------------------
+constexpr uint32_t kPolyReflected = 0x82F63B78u;
+constexpr uint32_t kCrcSegBytes = 64 * 1024;  // bytes per wavefront
+constexpr uint32_t kCrcRowBytes = 1024;       // one coalesced wavefront row: 64 lanes x 16 bytes
+
+// a(x) * b(x) mod P in the reflected representation (bit 31 is x^0).
+__host__ __device__ inline uint32_t gf_mul(uint32_t a, uint32_t b) {
+  uint32_t p = 0;
+  for (int i = 31; i >= 0; --i) {
+    p ^= ((a >> i) & 1u) ? b : 0u;
+    b = (b >> 1) ^ ((b & 1u) ? kPolyReflected : 0u);
+  }
+  return p;
+}
+
+// x^(8*nbytes) mod P.
+uint32_t x_pow_bytes(uint64_t nbytes) {
+  uint32_t result = 0x80000000u;      // x^0
+  uint32_t sq = gf_mul(0x40000000u, 0x40000000u);  // x^2
+  sq = gf_mul(sq, sq);                // x^4
+  sq = gf_mul(sq, sq);                // x^8 : one byte
+  while (nbytes) {
+    if (nbytes & 1) result = gf_mul(result, sq);
+    sq = gf_mul(sq, sq);
+    nbytes >>= 1;
+  }
+  return result;
+}
+
+__device__ __forceinline__ uint32_t crc_byte_step(uint32_t s, uint8_t b) {
+  s ^= b;
+  for (int k = 0; k < 8; ++k) s = (s >> 1) ^ ((s & 1u) ? kPolyReflected : 0u);
+  return s;
+}
+
+// One wavefront per segment: raw remainder (zero initial state, no final xor) of the segment's bytes.
+__global__ void __launch_bounds__(256) mlf_crc_segments_kernel(const char* __restrict__ data, uint64_t nbytes,
+                                                               const CrcConsts* __restrict__ consts,
+                                                               uint32_t* __restrict__ seg_crc, uint32_t n_segs) {
+  __shared__ uint32_t tab[4][256];
+  for (uint32_t i = threadIdx.x; i < 1024; i += blockDim.x) tab[i >> 8][i & 255] = consts->row_tab[i >> 8][i & 255];
+  __syncthreads();
+  const uint32_t seg = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (seg >= n_segs) return;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint64_t seg_off = (uint64_t)seg * kCrcSegBytes;
+  const uint64_t remaining = nbytes - seg_off;
+  const uint32_t seg_len = remaining < kCrcSegBytes ? (uint32_t)remaining : kCrcSegBytes;
+  const uint32_t rows = seg_len / kCrcRowBytes;
+  const u32x4* p = reinterpret_cast<const u32x4*>(data + seg_off) + lane;
+  uint32_t a0 = 0, a1 = 0, a2 = 0, a3 = 0;
+#define MLF_ROW_ADV(a) (tab[0][(a) & 255] ^ tab[1][((a) >> 8) & 255] ^ tab[2][((a) >> 16) & 255] ^ tab[3][(a) >> 24])
+  for (uint32_t r = 0; r < rows; ++r) {
+    const u32x4 v = __builtin_nontemporal_load(p + (size_t)r * 64);
+    a0 = MLF_ROW_ADV(a0) ^ v.x;
+    a1 = MLF_ROW_ADV(a1) ^ v.y;
+    a2 = MLF_ROW_ADV(a2) ^ v.z;
+    a3 = MLF_ROW_ADV(a3) ^ v.w;
+  }
+#undef MLF_ROW_ADV
+  // fold the four columns of this lane: x^128*a0 + x^96*a1 + x^64*a2 + x^32*a3
+  const uint32_t x4 = consts->x4;
+  uint32_t acc = gf_mul(x4, a0) ^ a1;
+  acc = gf_mul(x4, acc) ^ a2;
+  acc = gf_mul(x4, acc) ^ a3;
+  acc = gf_mul(x4, acc);
+  // fold lanes pairwise: lower lane is earlier in the message, so it is the one that gets shifted
+  const uint32_t xs[6] = {consts->x16, consts->x32, consts->x64, consts->x128, consts->x256, consts->x512};
+#pragma unroll
+  for (int s = 0; s < 6; ++s) {
+    const uint32_t other = __shfl_down(acc, 1u << s, 64);
+    acc = gf_mul(xs[s], acc) ^ other;
+  }
+  if (lane == 0) {
+    // bytes of a short last segment that do not fill a row
+    uint32_t state = rows ? acc : 0u;
+    const char* tailp = data + seg_off + (uint64_t)rows * kCrcRowBytes;
+    for (uint32_t i = 0, n = seg_len - rows * kCrcRowBytes; i < n; ++i) state = crc_byte_step(state, (uint8_t)tailp[i]);
+    seg_crc[seg] = state;
+  }
+}
+
+// One thread per chunk: chain the segment remainders, apply init and final xor.
+__global__ void mlf_crc_chunks_kernel(const uint32_t* __restrict__ seg_crc, uint32_t segs_per_chunk, uint32_t n_segs,
+                                      uint32_t xseg, uint32_t x_last_seg, uint32_t* __restrict__ out,
+                                      uint32_t n_chunks) {
+  const uint32_t c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= n_chunks) return;
+  uint32_t s = 0xFFFFFFFFu;
+  const uint32_t first = c * segs_per_chunk;
+  const uint32_t last = first + segs_per_chunk < n_segs ? first + segs_per_chunk : n_segs;
+  for (uint32_t i = first; i < last; ++i) s = gf_mul(i == n_segs - 1 ? x_last_seg : xseg, s) ^ seg_crc[i];
+  out[c] = s ^ 0xFFFFFFFFu;
+}
+
+std::once_flag g_crc_once;
+CrcConsts g_crc_host;
+
+void crc_init_host() {
+  const uint32_t xrow = x_pow_bytes(kCrcRowBytes);
+  for (int b = 0; b < 4; ++b)
+    for (uint32_t v = 0; v < 256; ++v) g_crc_host.row_tab[b][v] = gf_mul(xrow, v << (8 * b));
+  g_crc_host.x4 = x_pow_bytes(4);
+  g_crc_host.x16 = x_pow_bytes(16);
+  g_crc_host.x32 = x_pow_bytes(32);
+  g_crc_host.x64 = x_pow_bytes(64);
+  g_crc_host.x128 = x_pow_bytes(128);
+  g_crc_host.x256 = x_pow_bytes(256);
+  g_crc_host.x512 = x_pow_bytes(512);
+  g_crc_host.xseg = x_pow_bytes(kCrcSegBytes);
+}
+
+}  // namespace
+
+namespace mlf {
+
+
+void crc_release(CrcJob* job) {
+  (void)hipFree(job->d_consts);
+  (void)hipFree(job->d_seg);
+  (void)hipFree(job->d_out);
+  if (job->h_out) (void)hipHostFree(job->h_out);
+  *job = CrcJob();
+}
+
+// Enqueues the two CRC kernels and the copy of the per-chunk values on `stream`; does not wait.
+int crc_enqueue(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint64_t n_out, hipStream_t stream,
+                CrcJob* job) {
+  if (!dev_ptr) return fail(MLF_HIP_BAD_ARG, "null pointer");
+  if (reinterpret_cast<uintptr_t>(dev_ptr) & 15) return fail(MLF_HIP_BAD_ARG, "device buffer must be 16-byte aligned");
+  if (chunk_bytes == 0 || chunk_bytes % kCrcSegBytes)
+    return fail(MLF_HIP_BAD_ARG, "chunk_bytes must be a positive multiple of 65536");
+  const uint64_t n_chunks = (nbytes + chunk_bytes - 1) / chunk_bytes;
+  const uint64_t n_segs = (nbytes + kCrcSegBytes - 1) / kCrcSegBytes;
+  if (n_out < n_chunks) return fail(MLF_HIP_BAD_ARG, "output array too small");
+  if (n_segs > 0xFFFFFFF0ull) return fail(MLF_HIP_BAD_ARG, "buffer too large for one CRC call");
+  std::call_once(g_crc_once, crc_init_host);
+  job->n_chunks = n_chunks;
+  job->stream = stream;
+#define CRC_TRY(expr)                                                                             \
+  do {                                                                                            \
+    hipError_t e__ = (expr);                                                                      \
+    if (e__ != hipSuccess) {                                                                      \
+      crc_release(job);                                                                           \
+      return fail(MLF_HIP_RUNTIME, std::string(#expr) + " failed: " + hipGetErrorString(e__));    \
+    }                                                                                             \
+  } while (0)
+  CRC_TRY(hipMalloc(reinterpret_cast<void**>(&job->d_consts), sizeof(CrcConsts)));
+  CRC_TRY(hipMalloc(reinterpret_cast<void**>(&job->d_seg), n_segs * sizeof(uint32_t)));
+  CRC_TRY(hipMalloc(reinterpret_cast<void**>(&job->d_out), n_chunks * sizeof(uint32_t)));
+  CRC_TRY(hipHostMalloc(reinterpret_cast<void**>(&job->h_out), n_chunks * sizeof(uint32_t), hipHostMallocDefault));
+  CRC_TRY(hipMemcpyAsync(job->d_consts, &g_crc_host, sizeof(CrcConsts), hipMemcpyHostToDevice, stream));
+  const uint32_t grid = (uint32_t)((n_segs + 3) / 4);
+  hipLaunchKernelGGL(mlf_crc_segments_kernel, dim3(grid), dim3(256), 0, stream, static_cast<const char*>(dev_ptr),
+                     nbytes, job->d_consts, job->d_seg, (uint32_t)n_segs);
+  CRC_TRY(hipGetLastError());
+  const uint64_t last_seg_len = nbytes - (n_segs - 1) * kCrcSegBytes;
+  hipLaunchKernelGGL(mlf_crc_chunks_kernel, dim3((uint32_t)((n_chunks + 63) / 64)), dim3(64), 0, stream, job->d_seg,
+                     (uint32_t)(chunk_bytes / kCrcSegBytes), (uint32_t)n_segs, g_crc_host.xseg,
+                     x_pow_bytes(last_seg_len), job->d_out, (uint32_t)n_chunks);
+  CRC_TRY(hipGetLastError());
+  CRC_TRY(hipMemcpyAsync(job->h_out, job->d_out, n_chunks * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+#undef CRC_TRY
+  return MLF_HIP_OK;
+}
+
+// Waits for the job, hands the values out and frees the scratch.
+int crc_finish(CrcJob* job, uint32_t* out_host) {
+  hipError_t e = hipStreamSynchronize(job->stream);
+  if (e == hipSuccess && out_host) memcpy(out_host, job->h_out, job->n_chunks * sizeof(uint32_t));
+  crc_release(job);
+  if (e != hipSuccess) return fail(MLF_HIP_RUNTIME, std::string("hipStreamSynchronize failed: ") + hipGetErrorString(e));
+  if (!out_host) return fail(MLF_HIP_BAD_ARG, "null pointer");
+  return MLF_HIP_OK;
+}
+
+}  // namespace mlf
+
+extern "C" {
+
+// ---------------------------------------------------------------------------------------------------------
+// CRC entry points
+// ---------------------------------------------------------------------------------------------------------
+uint32_t mlf_crc32c_host(const void* data, uint64_t nbytes) {
+  const unsigned char* p = static_cast<const unsigned char*>(data);
+  uint64_t s = 0xFFFFFFFFu;
+  while (nbytes && (reinterpret_cast<uintptr_t>(p) & 7)) {
+    s = _mm_crc32_u8((uint32_t)s, *p++);
+    --nbytes;
+  }
+  for (; nbytes >= 8; nbytes -= 8, p += 8) {
+    uint64_t w;
+    memcpy(&w, p, 8);
+    s = _mm_crc32_u64(s, w);
+  }
+  while (nbytes--) s = _mm_crc32_u8((uint32_t)s, *p++);
+  return (uint32_t)s ^ 0xFFFFFFFFu;
+}
+
+uint32_t mlf_crc32c_combine(uint32_t crc_a, uint32_t crc_b, uint64_t len_b) {
+  return gf_mul(x_pow_bytes(len_b), crc_a) ^ crc_b;
+}
+
+int mlf_crc32c_file(int fd, uint64_t file_offset, uint64_t nbytes, uint64_t chunk_bytes, uint32_t* out_host,
+                    uint64_t n_out, uint32_t threads) {
+  if (fd < 0) return fail(MLF_HIP_BAD_ARG, "bad file descriptor");
+  if (nbytes == 0) return MLF_HIP_OK;
+  if (chunk_bytes == 0 || !out_host) return fail(MLF_HIP_BAD_ARG, "chunk_bytes must be positive and out_host non-null");
+  const uint64_t n_chunks = (nbytes + chunk_bytes - 1) / chunk_bytes;
+  if (n_out < n_chunks) return fail(MLF_HIP_BAD_ARG, "checksum output too small");
+  if (threads < 1 || threads > 256) return fail(MLF_HIP_BAD_ARG, "threads must be in [1, 256]");
+  const size_t piece = (size_t)std::min<uint64_t>(chunk_bytes, (uint64_t)4 << 20);  // read granularity per thread
+  std::atomic<uint64_t> next{0};
+  std::atomic<int> err{0};
+  auto work = [&] {
+    std::vector<char> buf(piece);
+    for (;;) {
+      const uint64_t c = next.fetch_add(1);
+      if (c >= n_chunks || err.load()) return;
+      const uint64_t begin = c * chunk_bytes, len = std::min(chunk_bytes, nbytes - begin);
+      uint32_t crc = 0;
+      for (uint64_t done = 0; done < len; done += piece) {
+        const size_t n = (size_t)std::min<uint64_t>(piece, len - done);
+        if (int e = full_pread(fd, buf.data(), n, file_offset + begin + done)) {
+          err.store(e);
+          return;
+        }
+        const uint32_t part = mlf_crc32c_host(buf.data(), n);
+        crc = done == 0 ? part : mlf_crc32c_combine(crc, part, n);
+      }
+      out_host[c] = crc;
+    }
+  };
+  std::vector<std::thread> pool;
+  const unsigned width = (unsigned)std::min<uint64_t>(threads, n_chunks);
+  for (unsigned i = 1; i < width; ++i) pool.emplace_back(work);
+  work();
+  for (auto& t : pool) t.join();
+  if (int e = err.load()) return fail(MLF_HIP_RUNTIME, std::string("pread() failed: ") + strerror(e));
+  return MLF_HIP_OK;
+}
+
+int mlf_crc32c_device(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint32_t* out_host,
+                      uint64_t n_out, void* stream_) {
+  if (nbytes == 0) return MLF_HIP_OK;
+  CrcJob job;
+  if (int rc = crc_enqueue(dev_ptr, nbytes, chunk_bytes, n_out, static_cast<hipStream_t>(stream_), &job)) return rc;
+  return crc_finish(&job, out_host);
+}
+
+}  // extern "C"

@@ -1,0 +1,372 @@
+// Copy engine between HBM and pageable host memory (a tmpfs mapping or file): a ring of pinned slots, two copy
+// streams plus a checksum stream, and a persistent pool of host threads.  Part of the library behind
+// include/mlf_hip.h.
+#include "mlf_internal.h"
+
+#include <algorithm>
+#include <atomic>
+#include <condition_variable>
+#include <functional>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <thread>
+#include <vector>
+
+using namespace mlf;
+
+namespace {
+
+// ---------------------------------------------------------------------------------------------------------
+// host thread pool: run(n, fn) executes fn(0..n-1) on the pool's threads plus the caller
+// ---------------------------------------------------------------------------------------------------------
+class WorkerPool {
+ public:
+  explicit WorkerPool(unsigned extra_threads) {
+    for (unsigned i = 0; i < extra_threads; ++i) threads_.emplace_back([this] { loop(); });
+  }
+  ~WorkerPool() {
+    {
+      std::lock_guard<std::mutex> g(m_);
+      stop_ = true;
+    }
+    cv_.notify_all();
+    for (auto& t : threads_) t.join();
+  }
+  unsigned width() const { return (unsigned)threads_.size() + 1; }
+
+  void run(unsigned n, const std::function<void(unsigned)>& fn) {
+    if (n == 0) return;
+    {
+      std::lock_guard<std::mutex> g(m_);
+      fn_ = &fn;
+      total_ = n;
+      next_ = 0;
+      pending_ = n;
+      ++generation_;
+    }
+    cv_.notify_all();
+    drain();
+    std::unique_lock<std::mutex> l(m_);
+    done_cv_.wait(l, [this] { return pending_ == 0; });
+    fn_ = nullptr;
+  }
+
+ private:
+  void drain() {
+    for (;;) {
+      unsigned idx;
+      const std::function<void(unsigned)>* fn;
+      {
+        std::lock_guard<std::mutex> g(m_);
+        if (!fn_ || next_ >= total_) return;
+        idx = next_++;
+        fn = fn_;
+      }
+      (*fn)(idx);
+      {
+        std::lock_guard<std::mutex> g(m_);
+        if (--pending_ == 0) done_cv_.notify_all();
+      }
+    }
+  }
+  void loop() {
+    uint64_t seen = 0;
+    for (;;) {
+      {
+        std::unique_lock<std::mutex> l(m_);
+        cv_.wait(l, [&] { return stop_ || generation_ != seen; });
+        if (stop_) return;
+        seen = generation_;
+      }
+      drain();
+    }
+  }
+  std::vector<std::thread> threads_;
+  std::mutex m_;
+  std::condition_variable cv_, done_cv_;
+  const std::function<void(unsigned)>* fn_ = nullptr;
+  unsigned total_ = 0, next_ = 0, pending_ = 0;
+  uint64_t generation_ = 0;
+  bool stop_ = false;
+};
+
+void pool_memcpy(WorkerPool& pool, char* dst, const char* src, size_t n) {
+  const unsigned parts = std::max<unsigned>(1, std::min<size_t>(pool.width(), n / ((size_t)1 << 20)));
+  size_t per = (n + parts - 1) / parts;
+  per = (per + 4095) & ~(size_t)4095;
+  pool.run(parts, [&](unsigned i) {
+    const size_t off = (size_t)i * per;
+    if (off < n) memcpy(dst + off, src + off, std::min(per, n - off));
+  });
+}
+
+// The pageable end of a transfer: a plain pointer, or a byte range of an open file (pread/pwrite).  Going
+// through the file descriptor moves the same page-cache pages as a MAP_SHARED mapping would, without building
+// (and later tearing down) one page-table entry per 4 KiB of a buffer that can be 100+ GB.
+struct HostEnd {
+  char* ptr = nullptr;
+  int fd = -1;
+  uint64_t file_off = 0;
+};
+
+// slot -> host end (to_host) or host end -> slot, split over the pool; returns 0 or an errno value
+int pool_host_copy(WorkerPool& pool, const HostEnd& host, uint64_t host_off, char* slot, size_t n, bool to_host) {
+  if (host.fd < 0) {
+    if (to_host) pool_memcpy(pool, host.ptr + host_off, slot, n);
+    else pool_memcpy(pool, slot, host.ptr + host_off, n);
+    return 0;
+  }
+  const unsigned parts = std::max<unsigned>(1, std::min<size_t>(pool.width(), n / ((size_t)1 << 20)));
+  size_t per = (n + parts - 1) / parts;
+  per = (per + 4095) & ~(size_t)4095;
+  std::atomic<int> err{0};
+  pool.run(parts, [&](unsigned i) {
+    const size_t off = (size_t)i * per;
+    if (off >= n) return;
+    const size_t len = std::min(per, n - off);
+    const int e = to_host ? full_pwrite(host.fd, slot + off, len, host.file_off + host_off + off)
+                          : full_pread(host.fd, slot + off, len, host.file_off + host_off + off);
+    if (e) err.store(e);
+  });
+  return err.load();
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------------------
+// copy engine
+// ---------------------------------------------------------------------------------------------------------
+struct mlf_engine {
+  int device = 0;
+  uint64_t slot_bytes = 0;
+  std::vector<char*> slots;
+  std::vector<hipEvent_t> slot_done;
+  hipStream_t streams[2] = {nullptr, nullptr};
+  hipStream_t crc_stream = nullptr;  // checksum kernels run beside the copies, not before them
+  hipEvent_t gate = nullptr;
+  std::unique_ptr<WorkerPool> pool;
+  std::mutex busy;  // one transfer at a time per engine
+};
+
+extern "C" {
+
+int mlf_engine_destroy(mlf_engine* e) {
+  if (!e) return MLF_HIP_OK;
+  for (char* s : e->slots) (void)hipHostFree(s);
+  for (hipEvent_t ev : e->slot_done) (void)hipEventDestroy(ev);
+  if (e->gate) (void)hipEventDestroy(e->gate);
+  for (hipStream_t s : e->streams)
+    if (s) (void)hipStreamDestroy(s);
+  if (e->crc_stream) (void)hipStreamDestroy(e->crc_stream);
+  delete e;
+  return MLF_HIP_OK;
+}
+
+int mlf_engine_create(uint64_t slot_bytes, uint32_t n_slots, uint32_t n_threads, mlf_engine** out) {
+  if (!out) return fail(MLF_HIP_BAD_ARG, "null out");
+  *out = nullptr;
+  if (slot_bytes < (1u << 20) || slot_bytes % 4096) return fail(MLF_HIP_BAD_ARG, "slot_bytes must be a multiple of 4096, at least 1 MiB");
+  if (n_slots < 2 || n_slots > 64) return fail(MLF_HIP_BAD_ARG, "n_slots must be in [2, 64]");
+  if (n_threads < 1 || n_threads > 256) return fail(MLF_HIP_BAD_ARG, "n_threads must be in [1, 256]");
+  std::unique_ptr<mlf_engine> e(new mlf_engine());
+  e->slot_bytes = slot_bytes;
+  int rc = MLF_HIP_OK;
+  auto check = [&](hipError_t err, const char* what) {
+    if (err != hipSuccess && rc == MLF_HIP_OK) rc = fail(MLF_HIP_RUNTIME, std::string(what) + " failed: " + hipGetErrorString(err));
+  };
+  check(hipGetDevice(&e->device), "hipGetDevice");
+  for (int i = 0; i < 2 && rc == MLF_HIP_OK; ++i)
+    check(hipStreamCreateWithFlags(&e->streams[i], hipStreamNonBlocking), "hipStreamCreateWithFlags");
+  if (rc == MLF_HIP_OK) check(hipStreamCreateWithFlags(&e->crc_stream, hipStreamNonBlocking), "hipStreamCreateWithFlags");
+  if (rc == MLF_HIP_OK) check(hipEventCreateWithFlags(&e->gate, hipEventDisableTiming), "hipEventCreateWithFlags");
+  for (uint32_t i = 0; i < n_slots && rc == MLF_HIP_OK; ++i) {
+    char* p = nullptr;
+    check(hipHostMalloc(reinterpret_cast<void**>(&p), slot_bytes, hipHostMallocDefault), "hipHostMalloc");
+    if (rc != MLF_HIP_OK) break;
+    memset(p, 0, slot_bytes);  // touch the pages once, outside any timed transfer
+    e->slots.push_back(p);
+    hipEvent_t ev = nullptr;
+    check(hipEventCreateWithFlags(&ev, hipEventDisableTiming), "hipEventCreateWithFlags");
+    if (rc == MLF_HIP_OK) e->slot_done.push_back(ev);
+  }
+  if (rc != MLF_HIP_OK) {
+    const std::string keep = last_error();
+    mlf_engine_destroy(e.release());
+    last_error() = keep;
+    return rc;
+  }
+  e->pool.reset(new WorkerPool(n_threads - 1));
+  *out = e.release();
+  return MLF_HIP_OK;
+}
+
+}  // extern "C"
+
+namespace {
+
+struct CrcRequest {
+  uint64_t chunk_bytes = 0;  // 0: no checksum
+  uint32_t* out_host = nullptr;
+  uint64_t n_out = 0;
+};
+
+int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t nbytes, void* producer_stream,
+               mlf_xfer_stats* stats, const CrcRequest& crc = CrcRequest()) {
+  if (!e) return fail(MLF_HIP_BAD_ARG, "null engine");
+  if (nbytes && (!src_dev || (host.fd < 0 && !host.ptr))) return fail(MLF_HIP_BAD_ARG, "null pointer");
+  std::lock_guard<std::mutex> g(e->busy);
+  HIP_TRY(hipSetDevice(e->device));
+  const double t0 = now_s();
+  // the copy streams start after whatever the producer has enqueued so far (the pack)
+  HIP_TRY(hipEventRecord(e->gate, static_cast<hipStream_t>(producer_stream)));
+  for (hipStream_t s : e->streams) HIP_TRY(hipStreamWaitEvent(s, e->gate, 0));
+  const char* src = static_cast<const char*>(src_dev);
+  CrcJob crc_job;
+  const bool want_crc = crc.chunk_bytes != 0 && nbytes != 0;
+  if (want_crc) {
+    // the image is complete once the gate has passed and is not modified afterwards, so its checksum can be
+    // computed while the link-bound copies run: it costs neither blocking time nor transfer time
+    HIP_TRY(hipStreamWaitEvent(e->crc_stream, e->gate, 0));
+    if (int rc = crc_enqueue(src_dev, nbytes, crc.chunk_bytes, crc.n_out, e->crc_stream, &crc_job)) return rc;
+  }
+  struct CrcGuard {  // scratch is released on every exit path, after the kernels that use it have finished
+    CrcJob* job;
+    bool armed;
+    ~CrcGuard() {
+      if (armed) {
+        (void)hipStreamSynchronize(job->stream);
+        crc_release(job);
+      }
+    }
+  } crc_guard{&crc_job, want_crc};
+  const uint64_t slot = e->slot_bytes;
+  const uint64_t n_chunks = (nbytes + slot - 1) / slot;
+  const uint64_t n_slots = e->slots.size();
+  auto issue = [&](uint64_t c) -> int {
+    const uint64_t off = c * slot, len = std::min(slot, nbytes - off);
+    const uint64_t s = c % n_slots;
+    hipStream_t st = e->streams[c & 1];
+    HIP_TRY(hipMemcpyAsync(e->slots[s], src + off, len, hipMemcpyDeviceToHost, st));
+    HIP_TRY(hipEventRecord(e->slot_done[s], st));
+    return MLF_HIP_OK;
+  };
+  auto drain_streams = [&] {
+    for (hipStream_t s : e->streams) (void)hipStreamSynchronize(s);
+  };
+  for (uint64_t c = 0; c < std::min(n_chunks, n_slots); ++c)
+    if (int rc = issue(c)) return rc;
+  double wait = 0;
+  for (uint64_t c = 0; c < n_chunks; ++c) {
+    const uint64_t off = c * slot, len = std::min(slot, nbytes - off);
+    const uint64_t s = c % n_slots;
+    const double w0 = now_s();
+    HIP_TRY(hipEventSynchronize(e->slot_done[s]));
+    if (c == 0) wait = now_s() - w0;
+    if (int err = pool_host_copy(*e->pool, host, off, e->slots[s], len, true)) {
+      drain_streams();  // copies still in flight target the slots: let them land before anyone reuses them
+      return fail(MLF_HIP_RUNTIME, std::string("pwrite() to the buffer file failed: ") + strerror(err));
+    }
+    if (c + n_slots < n_chunks)
+      if (int rc = issue(c + n_slots)) return rc;
+  }
+  if (want_crc) {
+    crc_guard.armed = false;
+    if (int rc = crc_finish(&crc_job, crc.out_host)) return rc;
+  }
+  if (stats) {
+    stats->seconds = now_s() - t0;
+    stats->wait_seconds = wait;
+    stats->bytes = nbytes;
+    stats->chunks = n_chunks;
+  }
+  return MLF_HIP_OK;
+}
+
+int engine_h2d(mlf_engine* e, const HostEnd& host, void* dst_dev, uint64_t nbytes, void* consumer_stream,
+               mlf_xfer_stats* stats) {
+  if (!e) return fail(MLF_HIP_BAD_ARG, "null engine");
+  if (nbytes && (!dst_dev || (host.fd < 0 && !host.ptr))) return fail(MLF_HIP_BAD_ARG, "null pointer");
+  std::lock_guard<std::mutex> g(e->busy);
+  HIP_TRY(hipSetDevice(e->device));
+  const double t0 = now_s();
+  char* dst = static_cast<char*>(dst_dev);
+  const uint64_t slot = e->slot_bytes;
+  const uint64_t n_chunks = (nbytes + slot - 1) / slot;
+  const uint64_t n_slots = e->slots.size();
+  for (uint64_t c = 0; c < n_chunks; ++c) {
+    const uint64_t off = c * slot, len = std::min(slot, nbytes - off);
+    const uint64_t s = c % n_slots;
+    if (c >= n_slots) HIP_TRY(hipEventSynchronize(e->slot_done[s]));  // the slot's previous upload has left it
+    if (int err = pool_host_copy(*e->pool, host, off, e->slots[s], len, false)) {
+      for (hipStream_t st : e->streams) (void)hipStreamSynchronize(st);
+      return fail(MLF_HIP_RUNTIME, std::string("pread() from the buffer file failed: ") + strerror(err));
+    }
+    hipStream_t st = e->streams[c & 1];
+    HIP_TRY(hipMemcpyAsync(dst + off, e->slots[s], len, hipMemcpyHostToDevice, st));
+    HIP_TRY(hipEventRecord(e->slot_done[s], st));
+  }
+  // the consumer (unpack) waits for both copy streams; the host waits too, so the slots are reusable
+  for (hipStream_t s : e->streams) {
+    HIP_TRY(hipEventRecord(e->gate, s));
+    HIP_TRY(hipStreamWaitEvent(static_cast<hipStream_t>(consumer_stream), e->gate, 0));
+    HIP_TRY(hipStreamSynchronize(s));
+  }
+  if (stats) {
+    stats->seconds = now_s() - t0;
+    stats->wait_seconds = 0;
+    stats->bytes = nbytes;
+    stats->chunks = n_chunks;
+  }
+  return MLF_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mlf_engine_d2h(mlf_engine* e, const void* src_dev, void* dst_host, uint64_t nbytes, void* producer_stream,
+                   mlf_xfer_stats* stats) {
+  HostEnd host;
+  host.ptr = static_cast<char*>(dst_host);
+  return engine_d2h(e, src_dev, host, nbytes, producer_stream, stats);
+}
+
+int mlf_engine_h2d(mlf_engine* e, const void* src_host, void* dst_dev, uint64_t nbytes, void* consumer_stream,
+                   mlf_xfer_stats* stats) {
+  HostEnd host;
+  host.ptr = const_cast<char*>(static_cast<const char*>(src_host));
+  return engine_h2d(e, host, dst_dev, nbytes, consumer_stream, stats);
+}
+
+int mlf_engine_d2h_crc(mlf_engine* e, const void* src_dev, void* dst_host, uint64_t nbytes, void* producer_stream,
+                       uint64_t crc_chunk_bytes, uint32_t* crc_out_host, uint64_t n_crc_out, mlf_xfer_stats* stats) {
+  if (crc_chunk_bytes && !crc_out_host) return fail(MLF_HIP_BAD_ARG, "null checksum output");
+  HostEnd host;
+  host.ptr = static_cast<char*>(dst_host);
+  CrcRequest crc;
+  crc.chunk_bytes = crc_chunk_bytes;
+  crc.out_host = crc_out_host;
+  crc.n_out = n_crc_out;
+  return engine_d2h(e, src_dev, host, nbytes, producer_stream, stats, crc);
+}
+
+int mlf_engine_d2h_fd(mlf_engine* e, const void* src_dev, int fd, uint64_t file_offset, uint64_t nbytes,
+                      void* producer_stream, mlf_xfer_stats* stats) {
+  if (fd < 0) return fail(MLF_HIP_BAD_ARG, "bad file descriptor");
+  HostEnd host;
+  host.fd = fd;
+  host.file_off = file_offset;
+  return engine_d2h(e, src_dev, host, nbytes, producer_stream, stats);
+}
+
+int mlf_engine_h2d_fd(mlf_engine* e, int fd, uint64_t file_offset, void* dst_dev, uint64_t nbytes,
+                      void* consumer_stream, mlf_xfer_stats* stats) {
+  if (fd < 0) return fail(MLF_HIP_BAD_ARG, "bad file descriptor");
+  HostEnd host;
+  host.fd = fd;
+  host.file_off = file_offset;
+  return engine_h2d(e, host, dst_dev, nbytes, consumer_stream, stats);
+}
+
+}  // extern "C"

@@ -1,0 +1,91 @@
+// Internal to the translation units behind include/mlf_hip.h: error reporting, small host helpers, and the
+// interface between the checksum code (mlf_crc.hip) and the copy engine (mlf_engine.hip).
+#ifndef MLF_INTERNAL_H_
+#define MLF_INTERNAL_H_
+
+#include "mlf_hip.h"
+
+#include <hip/hip_runtime.h>
+#include <errno.h>
+#include <stdint.h>
+#include <string.h>
+#include <unistd.h>
+
+#include <chrono>
+#include <string>
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef u32x4 u32x4_u __attribute__((aligned(1)));  // dwordx4 access at any byte address
+
+namespace mlf {
+
+enum { MLF_HIP_OK = 0, MLF_HIP_BAD_ARG = 1, MLF_HIP_RUNTIME = 2 };
+
+// Message of the calling thread's last failure (what mlf_hip_last_error returns).
+std::string& last_error();
+// Records `msg` for the calling thread and returns `code`.
+int fail(int code, const std::string& msg);
+
+#define HIP_TRY(expr)                                                                                   \
+  do {                                                                                                  \
+    hipError_t e__ = (expr);                                                                            \
+    if (e__ != hipSuccess)                                                                              \
+      return ::mlf::fail(::mlf::MLF_HIP_RUNTIME, std::string(#expr) + " failed: " + hipGetErrorString(e__)); \
+  } while (0)
+
+inline double now_s() {
+  return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+
+// pread / pwrite of a whole range; return 0 or an errno value
+inline int full_pwrite(int fd, const char* buf, size_t len, uint64_t off) {
+  while (len) {
+    ssize_t w = pwrite(fd, buf, len, (off_t)off);
+    if (w < 0) {
+      if (errno == EINTR) continue;
+      return errno;
+    }
+    buf += w;
+    off += (uint64_t)w;
+    len -= (size_t)w;
+  }
+  return 0;
+}
+
+inline int full_pread(int fd, char* buf, size_t len, uint64_t off) {
+  while (len) {
+    ssize_t r = pread(fd, buf, len, (off_t)off);
+    if (r < 0) {
+      if (errno == EINTR) continue;
+      return errno;
+    }
+    if (r == 0) return ENODATA;  // file shorter than the requested range
+    buf += r;
+    off += (uint64_t)r;
+    len -= (size_t)r;
+  }
+  return 0;
+}
+
+// A CRC pass in flight: scratch on the device, results in a pinned host array, all ordered on `stream`.
+struct CrcConsts;
+struct CrcJob {
+  CrcConsts* d_consts = nullptr;
+  uint32_t* d_seg = nullptr;
+  uint32_t* d_out = nullptr;
+  uint32_t* h_out = nullptr;  // pinned
+  uint64_t n_chunks = 0;
+  hipStream_t stream = nullptr;
+};
+
+// Enqueues the two CRC kernels and the copy of the per-chunk values on `stream`; does not wait.
+int crc_enqueue(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint64_t n_out, hipStream_t stream,
+                CrcJob* job);
+// Waits for the job, hands the values out and frees the scratch.
+int crc_finish(CrcJob* job, uint32_t* out_host);
+// Frees the scratch of a job that is not going to be finished (its stream must be idle).
+void crc_release(CrcJob* job);
+
+}  // namespace mlf
+
+#endif  // MLF_INTERNAL_H_

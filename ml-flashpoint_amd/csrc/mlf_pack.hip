@@ -1,4 +1,5 @@
-// MI355X (gfx950) save/restore data path behind the C-ABI in include/mlf_hip.h.
+// MI355X (gfx950) save/restore data path behind the C-ABI in include/mlf_hip.h.  This file: plans and the pack /
+// unpack kernels.  mlf_crc.hip holds the checksum, mlf_engine.hip the copy engine between HBM and host memory.
 //
 //   pack    live tensors (+ host blob of headers)  -> byte-exact image of a checkpoint object, in HBM
 //   unpack  image in HBM                           -> live tensors
@@ -21,55 +22,34 @@
 //     for sub-box restores.
 //   * crc kernel: per wavefront a 64 KiB segment is read as coalesced 1 KiB rows; every lane keeps four
 //     Horner accumulators advanced by x^8192 through LDS tables, then lanes are folded with GF(2) multiplies.
-#include "mlf_hip.h"
-
-#include <hip/hip_runtime.h>
-#include <errno.h>
-#include <nmmintrin.h>
-#include <string.h>
-#include <unistd.h>
+#include "mlf_internal.h"
 
 #include <algorithm>
-#include <atomic>
-#include <chrono>
-#include <condition_variable>
-#include <functional>
 #include <memory>
-#include <mutex>
 #include <string>
-#include <thread>
 #include <vector>
 
-// ---------------------------------------------------------------------------------------------------------
-// errors
-// ---------------------------------------------------------------------------------------------------------
-namespace {
+using namespace mlf;
 
-thread_local std::string g_err;
+namespace mlf {
+
+std::string& last_error() {
+  thread_local std::string message;
+  return message;
+}
 
 int fail(int code, const std::string& msg) {
-  g_err = msg;
+  last_error() = msg;
   return code;
 }
 
-enum { MLF_HIP_OK = 0, MLF_HIP_BAD_ARG = 1, MLF_HIP_RUNTIME = 2 };
+}  // namespace mlf
 
-#define HIP_TRY(expr)                                                                                   \
-  do {                                                                                                  \
-    hipError_t e__ = (expr);                                                                            \
-    if (e__ != hipSuccess)                                                                              \
-      return fail(MLF_HIP_RUNTIME, std::string(#expr) + " failed: " + hipGetErrorString(e__));          \
-  } while (0)
-
-double now_s() {
-  return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
-}
+namespace {
 
 // ---------------------------------------------------------------------------------------------------------
 // device-side tables
 // ---------------------------------------------------------------------------------------------------------
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-typedef u32x4 u32x4_u __attribute__((aligned(1)));  // dwordx4 access at any byte address
 
 // Tensor addresses arrive as integers, which the compiler can only treat as generic ("flat") pointers: flat accesses
 // count against both memory counters and are kept in order with LDS traffic.  Everything this library touches is
@@ -539,339 +519,6 @@ __global__ void __launch_bounds__(kTransThreads) mlf_transpose_kernel(const Tran
   }
 }
 
-// ---------------------------------------------------------------------------------------------------------
-// CRC-32C
-// ---------------------------------------------------------------------------------------------------------
-constexpr uint32_t kPolyReflected = 0x82F63B78u;
-constexpr uint32_t kCrcSegBytes = 64 * 1024;  // bytes per wavefront
-constexpr uint32_t kCrcRowBytes = 1024;       // one coalesced wavefront row: 64 lanes x 16 bytes
-
-// a(x) * b(x) mod P in the reflected representation (bit 31 is x^0).
-__host__ __device__ inline uint32_t gf_mul(uint32_t a, uint32_t b) {
-  uint32_t p = 0;
-  for (int i = 31; i >= 0; --i) {
-    p ^= ((a >> i) & 1u) ? b : 0u;
-    b = (b >> 1) ^ ((b & 1u) ? kPolyReflected : 0u);
-  }
-  return p;
-}
-
-// x^(8*nbytes) mod P.
-uint32_t x_pow_bytes(uint64_t nbytes) {
-  uint32_t result = 0x80000000u;      // x^0
-  uint32_t sq = gf_mul(0x40000000u, 0x40000000u);  // x^2
-  sq = gf_mul(sq, sq);                // x^4
-  sq = gf_mul(sq, sq);                // x^8 : one byte
-  while (nbytes) {
-    if (nbytes & 1) result = gf_mul(result, sq);
-    sq = gf_mul(sq, sq);
-    nbytes >>= 1;
-  }
-  return result;
-}
-
-struct CrcConsts {
-  uint32_t row_tab[4][256];  // state advanced by one 1 KiB row, sliced by state byte
-  uint32_t x4, x16, x32, x64, x128, x256, x512;  // x^(8*n) for the fold steps
-  uint32_t xseg;             // x^(8*kCrcSegBytes)
-};
-
-__device__ __forceinline__ uint32_t crc_byte_step(uint32_t s, uint8_t b) {
-  s ^= b;
-  for (int k = 0; k < 8; ++k) s = (s >> 1) ^ ((s & 1u) ? kPolyReflected : 0u);
-  return s;
-}
-
-// One wavefront per segment: raw remainder (zero initial state, no final xor) of the segment's bytes.
-__global__ void __launch_bounds__(256) mlf_crc_segments_kernel(const char* __restrict__ data, uint64_t nbytes,
-                                                               const CrcConsts* __restrict__ consts,
-                                                               uint32_t* __restrict__ seg_crc, uint32_t n_segs) {
-  __shared__ uint32_t tab[4][256];
-  for (uint32_t i = threadIdx.x; i < 1024; i += blockDim.x) tab[i >> 8][i & 255] = consts->row_tab[i >> 8][i & 255];
-  __syncthreads();
-  const uint32_t seg = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  if (seg >= n_segs) return;
-  const uint32_t lane = threadIdx.x & 63;
-  const uint64_t seg_off = (uint64_t)seg * kCrcSegBytes;
-  const uint64_t remaining = nbytes - seg_off;
-  const uint32_t seg_len = remaining < kCrcSegBytes ? (uint32_t)remaining : kCrcSegBytes;
-  const uint32_t rows = seg_len / kCrcRowBytes;
-  const u32x4* p = reinterpret_cast<const u32x4*>(data + seg_off) + lane;
-  uint32_t a0 = 0, a1 = 0, a2 = 0, a3 = 0;
-#define MLF_ROW_ADV(a) (tab[0][(a) & 255] ^ tab[1][((a) >> 8) & 255] ^ tab[2][((a) >> 16) & 255] ^ tab[3][(a) >> 24])
-  for (uint32_t r = 0; r < rows; ++r) {
-    const u32x4 v = __builtin_nontemporal_load(p + (size_t)r * 64);
-    a0 = MLF_ROW_ADV(a0) ^ v.x;
-    a1 = MLF_ROW_ADV(a1) ^ v.y;
-    a2 = MLF_ROW_ADV(a2) ^ v.z;
-    a3 = MLF_ROW_ADV(a3) ^ v.w;
-  }
-#undef MLF_ROW_ADV
-  // fold the four columns of this lane: x^128*a0 + x^96*a1 + x^64*a2 + x^32*a3
-  const uint32_t x4 = consts->x4;
-  uint32_t acc = gf_mul(x4, a0) ^ a1;
-  acc = gf_mul(x4, acc) ^ a2;
-  acc = gf_mul(x4, acc) ^ a3;
-  acc = gf_mul(x4, acc);
-  // fold lanes pairwise: lower lane is earlier in the message, so it is the one that gets shifted
-  const uint32_t xs[6] = {consts->x16, consts->x32, consts->x64, consts->x128, consts->x256, consts->x512};
-#pragma unroll
-  for (int s = 0; s < 6; ++s) {
-    const uint32_t other = __shfl_down(acc, 1u << s, 64);
-    acc = gf_mul(xs[s], acc) ^ other;
-  }
-  if (lane == 0) {
-    // bytes of a short last segment that do not fill a row
-    uint32_t state = rows ? acc : 0u;
-    const char* tailp = data + seg_off + (uint64_t)rows * kCrcRowBytes;
-    for (uint32_t i = 0, n = seg_len - rows * kCrcRowBytes; i < n; ++i) state = crc_byte_step(state, (uint8_t)tailp[i]);
-    seg_crc[seg] = state;
-  }
-}
-
-// One thread per chunk: chain the segment remainders, apply init and final xor.
-__global__ void mlf_crc_chunks_kernel(const uint32_t* __restrict__ seg_crc, uint32_t segs_per_chunk, uint32_t n_segs,
-                                      uint32_t xseg, uint32_t x_last_seg, uint32_t* __restrict__ out,
-                                      uint32_t n_chunks) {
-  const uint32_t c = blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= n_chunks) return;
-  uint32_t s = 0xFFFFFFFFu;
-  const uint32_t first = c * segs_per_chunk;
-  const uint32_t last = first + segs_per_chunk < n_segs ? first + segs_per_chunk : n_segs;
-  for (uint32_t i = first; i < last; ++i) s = gf_mul(i == n_segs - 1 ? x_last_seg : xseg, s) ^ seg_crc[i];
-  out[c] = s ^ 0xFFFFFFFFu;
-}
-
-std::once_flag g_crc_once;
-CrcConsts g_crc_host;
-
-void crc_init_host() {
-  const uint32_t xrow = x_pow_bytes(kCrcRowBytes);
-  for (int b = 0; b < 4; ++b)
-    for (uint32_t v = 0; v < 256; ++v) g_crc_host.row_tab[b][v] = gf_mul(xrow, v << (8 * b));
-  g_crc_host.x4 = x_pow_bytes(4);
-  g_crc_host.x16 = x_pow_bytes(16);
-  g_crc_host.x32 = x_pow_bytes(32);
-  g_crc_host.x64 = x_pow_bytes(64);
-  g_crc_host.x128 = x_pow_bytes(128);
-  g_crc_host.x256 = x_pow_bytes(256);
-  g_crc_host.x512 = x_pow_bytes(512);
-  g_crc_host.xseg = x_pow_bytes(kCrcSegBytes);
-}
-
-// A CRC pass in flight: scratch on the device, results in a pinned host array, all ordered on `stream`.
-struct CrcJob {
-  CrcConsts* d_consts = nullptr;
-  uint32_t* d_seg = nullptr;
-  uint32_t* d_out = nullptr;
-  uint32_t* h_out = nullptr;  // pinned
-  uint64_t n_chunks = 0;
-  hipStream_t stream = nullptr;
-};
-
-void crc_release(CrcJob* job) {
-  (void)hipFree(job->d_consts);
-  (void)hipFree(job->d_seg);
-  (void)hipFree(job->d_out);
-  if (job->h_out) (void)hipHostFree(job->h_out);
-  *job = CrcJob();
-}
-
-// Enqueues the two CRC kernels and the copy of the per-chunk values on `stream`; does not wait.
-int crc_enqueue(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint64_t n_out, hipStream_t stream,
-                CrcJob* job) {
-  if (!dev_ptr) return fail(MLF_HIP_BAD_ARG, "null pointer");
-  if (reinterpret_cast<uintptr_t>(dev_ptr) & 15) return fail(MLF_HIP_BAD_ARG, "device buffer must be 16-byte aligned");
-  if (chunk_bytes == 0 || chunk_bytes % kCrcSegBytes)
-    return fail(MLF_HIP_BAD_ARG, "chunk_bytes must be a positive multiple of 65536");
-  const uint64_t n_chunks = (nbytes + chunk_bytes - 1) / chunk_bytes;
-  const uint64_t n_segs = (nbytes + kCrcSegBytes - 1) / kCrcSegBytes;
-  if (n_out < n_chunks) return fail(MLF_HIP_BAD_ARG, "output array too small");
-  if (n_segs > 0xFFFFFFF0ull) return fail(MLF_HIP_BAD_ARG, "buffer too large for one CRC call");
-  std::call_once(g_crc_once, crc_init_host);
-  job->n_chunks = n_chunks;
-  job->stream = stream;
-#define CRC_TRY(expr)                                                                             \
-  do {                                                                                            \
-    hipError_t e__ = (expr);                                                                      \
-    if (e__ != hipSuccess) {                                                                      \
-      crc_release(job);                                                                           \
-      return fail(MLF_HIP_RUNTIME, std::string(#expr) + " failed: " + hipGetErrorString(e__));    \
-    }                                                                                             \
-  } while (0)
-  CRC_TRY(hipMalloc(reinterpret_cast<void**>(&job->d_consts), sizeof(CrcConsts)));
-  CRC_TRY(hipMalloc(reinterpret_cast<void**>(&job->d_seg), n_segs * sizeof(uint32_t)));
-  CRC_TRY(hipMalloc(reinterpret_cast<void**>(&job->d_out), n_chunks * sizeof(uint32_t)));
-  CRC_TRY(hipHostMalloc(reinterpret_cast<void**>(&job->h_out), n_chunks * sizeof(uint32_t), hipHostMallocDefault));
-  CRC_TRY(hipMemcpyAsync(job->d_consts, &g_crc_host, sizeof(CrcConsts), hipMemcpyHostToDevice, stream));
-  const uint32_t grid = (uint32_t)((n_segs + 3) / 4);
-  hipLaunchKernelGGL(mlf_crc_segments_kernel, dim3(grid), dim3(256), 0, stream, static_cast<const char*>(dev_ptr),
-                     nbytes, job->d_consts, job->d_seg, (uint32_t)n_segs);
-  CRC_TRY(hipGetLastError());
-  const uint64_t last_seg_len = nbytes - (n_segs - 1) * kCrcSegBytes;
-  hipLaunchKernelGGL(mlf_crc_chunks_kernel, dim3((uint32_t)((n_chunks + 63) / 64)), dim3(64), 0, stream, job->d_seg,
-                     (uint32_t)(chunk_bytes / kCrcSegBytes), (uint32_t)n_segs, g_crc_host.xseg,
-                     x_pow_bytes(last_seg_len), job->d_out, (uint32_t)n_chunks);
-  CRC_TRY(hipGetLastError());
-  CRC_TRY(hipMemcpyAsync(job->h_out, job->d_out, n_chunks * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
-#undef CRC_TRY
-  return MLF_HIP_OK;
-}
-
-// Waits for the job, hands the values out and frees the scratch.
-int crc_finish(CrcJob* job, uint32_t* out_host) {
-  hipError_t e = hipStreamSynchronize(job->stream);
-  if (e == hipSuccess && out_host) memcpy(out_host, job->h_out, job->n_chunks * sizeof(uint32_t));
-  crc_release(job);
-  if (e != hipSuccess) return fail(MLF_HIP_RUNTIME, std::string("hipStreamSynchronize failed: ") + hipGetErrorString(e));
-  if (!out_host) return fail(MLF_HIP_BAD_ARG, "null pointer");
-  return MLF_HIP_OK;
-}
-
-// ---------------------------------------------------------------------------------------------------------
-// host thread pool: run(n, fn) executes fn(0..n-1) on the pool's threads plus the caller
-// ---------------------------------------------------------------------------------------------------------
-class WorkerPool {
- public:
-  explicit WorkerPool(unsigned extra_threads) {
-    for (unsigned i = 0; i < extra_threads; ++i) threads_.emplace_back([this] { loop(); });
-  }
-  ~WorkerPool() {
-    {
-      std::lock_guard<std::mutex> g(m_);
-      stop_ = true;
-    }
-    cv_.notify_all();
-    for (auto& t : threads_) t.join();
-  }
-  unsigned width() const { return (unsigned)threads_.size() + 1; }
-
-  void run(unsigned n, const std::function<void(unsigned)>& fn) {
-    if (n == 0) return;
-    {
-      std::lock_guard<std::mutex> g(m_);
-      fn_ = &fn;
-      total_ = n;
-      next_ = 0;
-      pending_ = n;
-      ++generation_;
-    }
-    cv_.notify_all();
-    drain();
-    std::unique_lock<std::mutex> l(m_);
-    done_cv_.wait(l, [this] { return pending_ == 0; });
-    fn_ = nullptr;
-  }
-
- private:
-  void drain() {
-    for (;;) {
-      unsigned idx;
-      const std::function<void(unsigned)>* fn;
-      {
-        std::lock_guard<std::mutex> g(m_);
-        if (!fn_ || next_ >= total_) return;
-        idx = next_++;
-        fn = fn_;
-      }
-      (*fn)(idx);
-      {
-        std::lock_guard<std::mutex> g(m_);
-        if (--pending_ == 0) done_cv_.notify_all();
-      }
-    }
-  }
-  void loop() {
-    uint64_t seen = 0;
-    for (;;) {
-      {
-        std::unique_lock<std::mutex> l(m_);
-        cv_.wait(l, [&] { return stop_ || generation_ != seen; });
-        if (stop_) return;
-        seen = generation_;
-      }
-      drain();
-    }
-  }
-  std::vector<std::thread> threads_;
-  std::mutex m_;
-  std::condition_variable cv_, done_cv_;
-  const std::function<void(unsigned)>* fn_ = nullptr;
-  unsigned total_ = 0, next_ = 0, pending_ = 0;
-  uint64_t generation_ = 0;
-  bool stop_ = false;
-};
-
-void pool_memcpy(WorkerPool& pool, char* dst, const char* src, size_t n) {
-  const unsigned parts = std::max<unsigned>(1, std::min<size_t>(pool.width(), n / ((size_t)1 << 20)));
-  size_t per = (n + parts - 1) / parts;
-  per = (per + 4095) & ~(size_t)4095;
-  pool.run(parts, [&](unsigned i) {
-    const size_t off = (size_t)i * per;
-    if (off < n) memcpy(dst + off, src + off, std::min(per, n - off));
-  });
-}
-
-// The pageable end of a transfer: a plain pointer, or a byte range of an open file (pread/pwrite).  Going
-// through the file descriptor moves the same page-cache pages as a MAP_SHARED mapping would, without building
-// (and later tearing down) one page-table entry per 4 KiB of a buffer that can be 100+ GB.
-struct HostEnd {
-  char* ptr = nullptr;
-  int fd = -1;
-  uint64_t file_off = 0;
-};
-
-int full_pwrite(int fd, const char* buf, size_t len, uint64_t off) {
-  while (len) {
-    ssize_t w = pwrite(fd, buf, len, (off_t)off);
-    if (w < 0) {
-      if (errno == EINTR) continue;
-      return errno;
-    }
-    buf += w;
-    off += (uint64_t)w;
-    len -= (size_t)w;
-  }
-  return 0;
-}
-
-int full_pread(int fd, char* buf, size_t len, uint64_t off) {
-  while (len) {
-    ssize_t r = pread(fd, buf, len, (off_t)off);
-    if (r < 0) {
-      if (errno == EINTR) continue;
-      return errno;
-    }
-    if (r == 0) return ENODATA;  // file shorter than the requested range
-    buf += r;
-    off += (uint64_t)r;
-    len -= (size_t)r;
-  }
-  return 0;
-}
-
-// slot -> host end (to_host) or host end -> slot, split over the pool; returns 0 or an errno value
-int pool_host_copy(WorkerPool& pool, const HostEnd& host, uint64_t host_off, char* slot, size_t n, bool to_host) {
-  if (host.fd < 0) {
-    if (to_host) pool_memcpy(pool, host.ptr + host_off, slot, n);
-    else pool_memcpy(pool, slot, host.ptr + host_off, n);
-    return 0;
-  }
-  const unsigned parts = std::max<unsigned>(1, std::min<size_t>(pool.width(), n / ((size_t)1 << 20)));
-  size_t per = (n + parts - 1) / parts;
-  per = (per + 4095) & ~(size_t)4095;
-  std::atomic<int> err{0};
-  pool.run(parts, [&](unsigned i) {
-    const size_t off = (size_t)i * per;
-    if (off >= n) return;
-    const size_t len = std::min(per, n - off);
-    const int e = to_host ? full_pwrite(host.fd, slot + off, len, host.file_off + host_off + off)
-                          : full_pread(host.fd, slot + off, len, host.file_off + host_off + off);
-    if (e) err.store(e);
-  });
-  return err.load();
-}
-
 }  // namespace
 
 // ---------------------------------------------------------------------------------------------------------
@@ -981,7 +628,7 @@ int upload(const std::vector<T>& host, T** dev) {
 
 extern "C" {
 
-const char* mlf_hip_last_error(void) { return g_err.c_str(); }
+const char* mlf_hip_last_error(void) { return last_error().c_str(); }
 
 int mlf_hip_device_count(int* out) {
   if (!out) return fail(MLF_HIP_BAD_ARG, "null out");
@@ -1204,9 +851,9 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
   if (rc == MLF_HIP_OK) rc = upload(tdescs, &plan->d_tdescs);
   if (rc == MLF_HIP_OK) rc = upload(twork, &plan->d_twork);
   if (rc != MLF_HIP_OK) {
-    std::string keep = g_err;
+    const std::string keep = last_error();
     mlf_plan_destroy(plan.release());
-    g_err = keep;
+    last_error() = keep;
     return rc;
   }
   info.n_flat_tiles = 0;
@@ -1312,313 +959,6 @@ int mlf_pack_launch(const mlf_plan* plan, void* image_dev, void* stream) {
 int mlf_unpack_launch(const mlf_plan* plan, const void* image_dev, void* stream) {
   return launch_plan<false>(plan, const_cast<char*>(static_cast<const char*>(image_dev)),
                             static_cast<hipStream_t>(stream));
-}
-
-// ---------------------------------------------------------------------------------------------------------
-// CRC entry points
-// ---------------------------------------------------------------------------------------------------------
-uint32_t mlf_crc32c_host(const void* data, uint64_t nbytes) {
-  const unsigned char* p = static_cast<const unsigned char*>(data);
-  uint64_t s = 0xFFFFFFFFu;
-  while (nbytes && (reinterpret_cast<uintptr_t>(p) & 7)) {
-    s = _mm_crc32_u8((uint32_t)s, *p++);
-    --nbytes;
-  }
-  for (; nbytes >= 8; nbytes -= 8, p += 8) {
-    uint64_t w;
-    memcpy(&w, p, 8);
-    s = _mm_crc32_u64(s, w);
-  }
-  while (nbytes--) s = _mm_crc32_u8((uint32_t)s, *p++);
-  return (uint32_t)s ^ 0xFFFFFFFFu;
-}
-
-uint32_t mlf_crc32c_combine(uint32_t crc_a, uint32_t crc_b, uint64_t len_b) {
-  return gf_mul(x_pow_bytes(len_b), crc_a) ^ crc_b;
-}
-
-int mlf_crc32c_file(int fd, uint64_t file_offset, uint64_t nbytes, uint64_t chunk_bytes, uint32_t* out_host,
-                    uint64_t n_out, uint32_t threads) {
-  if (fd < 0) return fail(MLF_HIP_BAD_ARG, "bad file descriptor");
-  if (nbytes == 0) return MLF_HIP_OK;
-  if (chunk_bytes == 0 || !out_host) return fail(MLF_HIP_BAD_ARG, "chunk_bytes must be positive and out_host non-null");
-  const uint64_t n_chunks = (nbytes + chunk_bytes - 1) / chunk_bytes;
-  if (n_out < n_chunks) return fail(MLF_HIP_BAD_ARG, "checksum output too small");
-  if (threads < 1 || threads > 256) return fail(MLF_HIP_BAD_ARG, "threads must be in [1, 256]");
-  const size_t piece = (size_t)std::min<uint64_t>(chunk_bytes, (uint64_t)4 << 20);  // read granularity per thread
-  std::atomic<uint64_t> next{0};
-  std::atomic<int> err{0};
-  auto work = [&] {
-    std::vector<char> buf(piece);
-    for (;;) {
-      const uint64_t c = next.fetch_add(1);
-      if (c >= n_chunks || err.load()) return;
-      const uint64_t begin = c * chunk_bytes, len = std::min(chunk_bytes, nbytes - begin);
-      uint32_t crc = 0;
-      for (uint64_t done = 0; done < len; done += piece) {
-        const size_t n = (size_t)std::min<uint64_t>(piece, len - done);
-        if (int e = full_pread(fd, buf.data(), n, file_offset + begin + done)) {
-          err.store(e);
-          return;
-        }
-        const uint32_t part = mlf_crc32c_host(buf.data(), n);
-        crc = done == 0 ? part : mlf_crc32c_combine(crc, part, n);
-      }
-      out_host[c] = crc;
-    }
-  };
-  std::vector<std::thread> pool;
-  const unsigned width = (unsigned)std::min<uint64_t>(threads, n_chunks);
-  for (unsigned i = 1; i < width; ++i) pool.emplace_back(work);
-  work();
-  for (auto& t : pool) t.join();
-  if (int e = err.load()) return fail(MLF_HIP_RUNTIME, std::string("pread() failed: ") + strerror(e));
-  return MLF_HIP_OK;
-}
-
-int mlf_crc32c_device(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint32_t* out_host,
-                      uint64_t n_out, void* stream_) {
-  if (nbytes == 0) return MLF_HIP_OK;
-  CrcJob job;
-  if (int rc = crc_enqueue(dev_ptr, nbytes, chunk_bytes, n_out, static_cast<hipStream_t>(stream_), &job)) return rc;
-  return crc_finish(&job, out_host);
-}
-
-}  // extern "C"
-
-// ---------------------------------------------------------------------------------------------------------
-// copy engine
-// ---------------------------------------------------------------------------------------------------------
-struct mlf_engine {
-  int device = 0;
-  uint64_t slot_bytes = 0;
-  std::vector<char*> slots;
-  std::vector<hipEvent_t> slot_done;
-  hipStream_t streams[2] = {nullptr, nullptr};
-  hipStream_t crc_stream = nullptr;  // checksum kernels run beside the copies, not before them
-  hipEvent_t gate = nullptr;
-  std::unique_ptr<WorkerPool> pool;
-  std::mutex busy;  // one transfer at a time per engine
-};
-
-extern "C" {
-
-int mlf_engine_destroy(mlf_engine* e) {
-  if (!e) return MLF_HIP_OK;
-  for (char* s : e->slots) (void)hipHostFree(s);
-  for (hipEvent_t ev : e->slot_done) (void)hipEventDestroy(ev);
-  if (e->gate) (void)hipEventDestroy(e->gate);
-  for (hipStream_t s : e->streams)
-    if (s) (void)hipStreamDestroy(s);
-  if (e->crc_stream) (void)hipStreamDestroy(e->crc_stream);
-  delete e;
-  return MLF_HIP_OK;
-}
-
-int mlf_engine_create(uint64_t slot_bytes, uint32_t n_slots, uint32_t n_threads, mlf_engine** out) {
-  if (!out) return fail(MLF_HIP_BAD_ARG, "null out");
-  *out = nullptr;
-  if (slot_bytes < (1u << 20) || slot_bytes % 4096) return fail(MLF_HIP_BAD_ARG, "slot_bytes must be a multiple of 4096, at least 1 MiB");
-  if (n_slots < 2 || n_slots > 64) return fail(MLF_HIP_BAD_ARG, "n_slots must be in [2, 64]");
-  if (n_threads < 1 || n_threads > 256) return fail(MLF_HIP_BAD_ARG, "n_threads must be in [1, 256]");
-  std::unique_ptr<mlf_engine> e(new mlf_engine());
-  e->slot_bytes = slot_bytes;
-  int rc = MLF_HIP_OK;
-  auto check = [&](hipError_t err, const char* what) {
-    if (err != hipSuccess && rc == MLF_HIP_OK) rc = fail(MLF_HIP_RUNTIME, std::string(what) + " failed: " + hipGetErrorString(err));
-  };
-  check(hipGetDevice(&e->device), "hipGetDevice");
-  for (int i = 0; i < 2 && rc == MLF_HIP_OK; ++i)
-    check(hipStreamCreateWithFlags(&e->streams[i], hipStreamNonBlocking), "hipStreamCreateWithFlags");
-  if (rc == MLF_HIP_OK) check(hipStreamCreateWithFlags(&e->crc_stream, hipStreamNonBlocking), "hipStreamCreateWithFlags");
-  if (rc == MLF_HIP_OK) check(hipEventCreateWithFlags(&e->gate, hipEventDisableTiming), "hipEventCreateWithFlags");
-  for (uint32_t i = 0; i < n_slots && rc == MLF_HIP_OK; ++i) {
-    char* p = nullptr;
-    check(hipHostMalloc(reinterpret_cast<void**>(&p), slot_bytes, hipHostMallocDefault), "hipHostMalloc");
-    if (rc != MLF_HIP_OK) break;
-    memset(p, 0, slot_bytes);  // touch the pages once, outside any timed transfer
-    e->slots.push_back(p);
-    hipEvent_t ev = nullptr;
-    check(hipEventCreateWithFlags(&ev, hipEventDisableTiming), "hipEventCreateWithFlags");
-    if (rc == MLF_HIP_OK) e->slot_done.push_back(ev);
-  }
-  if (rc != MLF_HIP_OK) {
-    std::string keep = g_err;
-    mlf_engine_destroy(e.release());
-    g_err = keep;
-    return rc;
-  }
-  e->pool.reset(new WorkerPool(n_threads - 1));
-  *out = e.release();
-  return MLF_HIP_OK;
-}
-
-}  // extern "C"
-
-namespace {
-
-struct CrcRequest {
-  uint64_t chunk_bytes = 0;  // 0: no checksum
-  uint32_t* out_host = nullptr;
-  uint64_t n_out = 0;
-};
-
-int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t nbytes, void* producer_stream,
-               mlf_xfer_stats* stats, const CrcRequest& crc = CrcRequest()) {
-  if (!e) return fail(MLF_HIP_BAD_ARG, "null engine");
-  if (nbytes && (!src_dev || (host.fd < 0 && !host.ptr))) return fail(MLF_HIP_BAD_ARG, "null pointer");
-  std::lock_guard<std::mutex> g(e->busy);
-  HIP_TRY(hipSetDevice(e->device));
-  const double t0 = now_s();
-  // the copy streams start after whatever the producer has enqueued so far (the pack)
-  HIP_TRY(hipEventRecord(e->gate, static_cast<hipStream_t>(producer_stream)));
-  for (hipStream_t s : e->streams) HIP_TRY(hipStreamWaitEvent(s, e->gate, 0));
-  const char* src = static_cast<const char*>(src_dev);
-  CrcJob crc_job;
-  const bool want_crc = crc.chunk_bytes != 0 && nbytes != 0;
-  if (want_crc) {
-    // the image is complete once the gate has passed and is not modified afterwards, so its checksum can be
-    // computed while the link-bound copies run: it costs neither blocking time nor transfer time
-    HIP_TRY(hipStreamWaitEvent(e->crc_stream, e->gate, 0));
-    if (int rc = crc_enqueue(src_dev, nbytes, crc.chunk_bytes, crc.n_out, e->crc_stream, &crc_job)) return rc;
-  }
-  struct CrcGuard {  // scratch is released on every exit path, after the kernels that use it have finished
-    CrcJob* job;
-    bool armed;
-    ~CrcGuard() {
-      if (armed) {
-        (void)hipStreamSynchronize(job->stream);
-        crc_release(job);
-      }
-    }
-  } crc_guard{&crc_job, want_crc};
-  const uint64_t slot = e->slot_bytes;
-  const uint64_t n_chunks = (nbytes + slot - 1) / slot;
-  const uint64_t n_slots = e->slots.size();
-  auto issue = [&](uint64_t c) -> int {
-    const uint64_t off = c * slot, len = std::min(slot, nbytes - off);
-    const uint64_t s = c % n_slots;
-    hipStream_t st = e->streams[c & 1];
-    HIP_TRY(hipMemcpyAsync(e->slots[s], src + off, len, hipMemcpyDeviceToHost, st));
-    HIP_TRY(hipEventRecord(e->slot_done[s], st));
-    return MLF_HIP_OK;
-  };
-  auto drain_streams = [&] {
-    for (hipStream_t s : e->streams) (void)hipStreamSynchronize(s);
-  };
-  for (uint64_t c = 0; c < std::min(n_chunks, n_slots); ++c)
-    if (int rc = issue(c)) return rc;
-  double wait = 0;
-  for (uint64_t c = 0; c < n_chunks; ++c) {
-    const uint64_t off = c * slot, len = std::min(slot, nbytes - off);
-    const uint64_t s = c % n_slots;
-    const double w0 = now_s();
-    HIP_TRY(hipEventSynchronize(e->slot_done[s]));
-    if (c == 0) wait = now_s() - w0;
-    if (int err = pool_host_copy(*e->pool, host, off, e->slots[s], len, true)) {
-      drain_streams();  // copies still in flight target the slots: let them land before anyone reuses them
-      return fail(MLF_HIP_RUNTIME, std::string("pwrite() to the buffer file failed: ") + strerror(err));
-    }
-    if (c + n_slots < n_chunks)
-      if (int rc = issue(c + n_slots)) return rc;
-  }
-  if (want_crc) {
-    crc_guard.armed = false;
-    if (int rc = crc_finish(&crc_job, crc.out_host)) return rc;
-  }
-  if (stats) {
-    stats->seconds = now_s() - t0;
-    stats->wait_seconds = wait;
-    stats->bytes = nbytes;
-    stats->chunks = n_chunks;
-  }
-  return MLF_HIP_OK;
-}
-
-int engine_h2d(mlf_engine* e, const HostEnd& host, void* dst_dev, uint64_t nbytes, void* consumer_stream,
-               mlf_xfer_stats* stats) {
-  if (!e) return fail(MLF_HIP_BAD_ARG, "null engine");
-  if (nbytes && (!dst_dev || (host.fd < 0 && !host.ptr))) return fail(MLF_HIP_BAD_ARG, "null pointer");
-  std::lock_guard<std::mutex> g(e->busy);
-  HIP_TRY(hipSetDevice(e->device));
-  const double t0 = now_s();
-  char* dst = static_cast<char*>(dst_dev);
-  const uint64_t slot = e->slot_bytes;
-  const uint64_t n_chunks = (nbytes + slot - 1) / slot;
-  const uint64_t n_slots = e->slots.size();
-  for (uint64_t c = 0; c < n_chunks; ++c) {
-    const uint64_t off = c * slot, len = std::min(slot, nbytes - off);
-    const uint64_t s = c % n_slots;
-    if (c >= n_slots) HIP_TRY(hipEventSynchronize(e->slot_done[s]));  // the slot's previous upload has left it
-    if (int err = pool_host_copy(*e->pool, host, off, e->slots[s], len, false)) {
-      for (hipStream_t st : e->streams) (void)hipStreamSynchronize(st);
-      return fail(MLF_HIP_RUNTIME, std::string("pread() from the buffer file failed: ") + strerror(err));
-    }
-    hipStream_t st = e->streams[c & 1];
-    HIP_TRY(hipMemcpyAsync(dst + off, e->slots[s], len, hipMemcpyHostToDevice, st));
-    HIP_TRY(hipEventRecord(e->slot_done[s], st));
-  }
-  // the consumer (unpack) waits for both copy streams; the host waits too, so the slots are reusable
-  for (hipStream_t s : e->streams) {
-    HIP_TRY(hipEventRecord(e->gate, s));
-    HIP_TRY(hipStreamWaitEvent(static_cast<hipStream_t>(consumer_stream), e->gate, 0));
-    HIP_TRY(hipStreamSynchronize(s));
-  }
-  if (stats) {
-    stats->seconds = now_s() - t0;
-    stats->wait_seconds = 0;
-    stats->bytes = nbytes;
-    stats->chunks = n_chunks;
-  }
-  return MLF_HIP_OK;
-}
-
-}  // namespace
-
-extern "C" {
-
-int mlf_engine_d2h(mlf_engine* e, const void* src_dev, void* dst_host, uint64_t nbytes, void* producer_stream,
-                   mlf_xfer_stats* stats) {
-  HostEnd host;
-  host.ptr = static_cast<char*>(dst_host);
-  return engine_d2h(e, src_dev, host, nbytes, producer_stream, stats);
-}
-
-int mlf_engine_h2d(mlf_engine* e, const void* src_host, void* dst_dev, uint64_t nbytes, void* consumer_stream,
-                   mlf_xfer_stats* stats) {
-  HostEnd host;
-  host.ptr = const_cast<char*>(static_cast<const char*>(src_host));
-  return engine_h2d(e, host, dst_dev, nbytes, consumer_stream, stats);
-}
-
-int mlf_engine_d2h_crc(mlf_engine* e, const void* src_dev, void* dst_host, uint64_t nbytes, void* producer_stream,
-                       uint64_t crc_chunk_bytes, uint32_t* crc_out_host, uint64_t n_crc_out, mlf_xfer_stats* stats) {
-  if (crc_chunk_bytes && !crc_out_host) return fail(MLF_HIP_BAD_ARG, "null checksum output");
-  HostEnd host;
-  host.ptr = static_cast<char*>(dst_host);
-  CrcRequest crc;
-  crc.chunk_bytes = crc_chunk_bytes;
-  crc.out_host = crc_out_host;
-  crc.n_out = n_crc_out;
-  return engine_d2h(e, src_dev, host, nbytes, producer_stream, stats, crc);
-}
-
-int mlf_engine_d2h_fd(mlf_engine* e, const void* src_dev, int fd, uint64_t file_offset, uint64_t nbytes,
-                      void* producer_stream, mlf_xfer_stats* stats) {
-  if (fd < 0) return fail(MLF_HIP_BAD_ARG, "bad file descriptor");
-  HostEnd host;
-  host.fd = fd;
-  host.file_off = file_offset;
-  return engine_d2h(e, src_dev, host, nbytes, producer_stream, stats);
-}
-
-int mlf_engine_h2d_fd(mlf_engine* e, int fd, uint64_t file_offset, void* dst_dev, uint64_t nbytes,
-                      void* consumer_stream, mlf_xfer_stats* stats) {
-  if (fd < 0) return fail(MLF_HIP_BAD_ARG, "bad file descriptor");
-  HostEnd host;
-  host.fd = fd;
-  host.file_off = file_offset;
-  return engine_h2d(e, host, dst_dev, nbytes, consumer_stream, stats);
 }
 
 }  // extern "C"
