@@ -547,6 +547,17 @@ struct mlf_plan {
   uint32_t flat_first[kFlatClasses] = {0, 0, 0};  // first workgroup of each span class in that launch
   uint32_t flat_total = 0;
   mlf_plan_info info{};
+  mlf_plan() = default;
+  mlf_plan(const mlf_plan&) = delete;
+  mlf_plan& operator=(const mlf_plan&) = delete;
+  ~mlf_plan() {  // every exit path of mlf_plan_create, and mlf_plan_destroy
+    for (Span* t : d_spans) (void)hipFree(t);
+    (void)hipFree(d_descs);
+    (void)hipFree(d_work);
+    (void)hipFree(d_tdescs);
+    (void)hipFree(d_twork);
+    (void)hipFree(d_blob);
+  }
 };
 
 namespace {
@@ -883,14 +894,7 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
 }
 
 int mlf_plan_destroy(mlf_plan* plan) {
-  if (!plan) return MLF_HIP_OK;
-  for (Span* t : plan->d_spans) (void)hipFree(t);
-  (void)hipFree(plan->d_descs);
-  (void)hipFree(plan->d_work);
-  (void)hipFree(plan->d_tdescs);
-  (void)hipFree(plan->d_twork);
-  (void)hipFree(plan->d_blob);
-  delete plan;
+  delete plan;  // the destructor frees the device tables
   return MLF_HIP_OK;
 }
 

@@ -176,3 +176,54 @@ def test_bucket_dataclass_is_replaceable():
     b = ObjectWriteBucket(CheckpointObjectId("/x/y"), "y", [], [])
     c = dataclasses.replace(b, tensor_data=[("item", "tensor")])
     assert c.object_id == b.object_id and c.tensor_data and not b.tensor_data
+
+
+def test_gc_pause_is_reentrant_and_restores_the_previous_state():
+    import gc
+    import threading
+
+    from ml_flashpoint.core.utils import gc_paused
+
+    assert gc.isenabled()
+    with gc_paused():
+        assert not gc.isenabled()
+        with gc_paused():  # nested
+            assert not gc.isenabled()
+        assert not gc.isenabled()
+
+        def other_thread():  # another thread entering and leaving while the outer pause lasts does not end it
+            with gc_paused():
+                pass
+
+        t = threading.Thread(target=other_thread)
+        t.start()
+        t.join()
+        assert not gc.isenabled()
+    assert gc.isenabled()
+    with pytest.raises(ValueError):
+        with gc_paused():
+            raise ValueError("the collector comes back on after an exception")
+    assert gc.isenabled()
+
+    @gc_paused()
+    def decorated():
+        return gc.isenabled()
+
+    assert decorated() is False and decorated() is False and gc.isenabled()
+    gc.disable()  # a caller who runs with the collector off keeps it off
+    try:
+        with gc_paused():
+            pass
+        assert not gc.isenabled()
+    finally:
+        gc.enable()
+
+
+def test_copy_threads_default_follows_the_cpus_available(monkeypatch):
+    from ml_flashpoint.hip.checkpoint_saver import EngineConfig
+
+    assert EngineConfig(copy_threads=5).resolved_copy_threads() == 5
+    monkeypatch.setattr(os, "sched_getaffinity", lambda pid: set(range(64)))
+    assert EngineConfig().resolved_copy_threads() == 16
+    monkeypatch.setattr(os, "sched_getaffinity", lambda pid: {0, 1, 2})
+    assert EngineConfig().resolved_copy_threads() == 3
