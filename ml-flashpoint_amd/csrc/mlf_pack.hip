@@ -127,6 +127,7 @@ struct TransWork {  // kTransTilesPerEntry consecutive tiles of descriptor `desc
 // is cut at the span's end, where head = bytes from the span's first destination byte to the next grid line.
 // Threads interleave at 16-byte granularity, so a wavefront moves 1 KiB of consecutive bytes per access.
 constexpr int kFlatClasses = 3;  // span tables whose entries are shared by 128, 16 and 1 workgroups
+constexpr uint32_t kXcdRun = 64;  // consecutive tiles handed to one XCD (see mlf_flat_kernel)
 
 __host__ __device__ constexpr uint32_t flat_shift(int cls) { return cls == 0 ? 7u : cls == 1 ? 4u : 0u; }
 
@@ -150,7 +151,23 @@ __global__ void __launch_bounds__(1024) mlf_flat_kernel(const Span* __restrict__
   wg = live ? wg : 0u;
   const Span* __restrict__ table = wg >= first2 ? spans2 : wg >= first1 ? spans1 : spans0;
   const uint32_t shift = wg >= first2 ? flat_shift(2) : wg >= first1 ? flat_shift(1) : flat_shift(0);
-  const uint32_t local = wg - (wg >= first2 ? first2 : wg >= first1 ? first1 : 0u);
+  const uint32_t cls_first = wg >= first2 ? first2 : wg >= first1 ? first1 : 0u;
+  const uint32_t cls_end = wg >= first2 ? total : wg >= first1 ? first2 : first1;
+  uint32_t local = wg - cls_first;
+  {
+    // Workgroups go to the eight XCDs round-robin, so neighbouring tiles would land in eight different L2s and a
+    // source line that straddles a tile cut would be fetched from HBM by both.  Within every full group of
+    // 8 * kXcdRun workgroups the tiles are dealt out so that each XCD gets kXcdRun consecutive ones (256 KiB).
+    // Measured on the 112 GB shard: runs of 1 / 16 / 64 / 256 tiles -> 35.7 / 34.8 / 34.2 / 37.5 ms per pack.
+    constexpr uint32_t G = 8u * kXcdRun;
+    const uint32_t g0 = local / G * G;
+    if (cls_first + g0 + G <= cls_end) {
+      const uint32_t c0 = cls_first & 7u;        // XCD of the class's first workgroup
+      const uint32_t rp = (local - g0) + c0;     // position in the group, counted from XCD 0's slot
+      const uint32_t xcd = rp & 7u;
+      local = g0 + xcd * kXcdRun + (rp >> 3) - (xcd < c0 ? 1u : 0u);
+    }
+  }
   const Span sp = table[local >> shift];
   const uint32_t sub = local & ((1u << shift) - 1u);
   const uint32_t span_n = live ? sp.n : 0u;
