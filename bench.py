@@ -37,7 +37,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, vendor figure
 # with `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`, each scaled against a torch.add kernel of known size
 # (summary: profiles/pmc_traffic_mlf_flat_kernel_llama3-8b-shard.md).  Hardware counters cannot be read from
 # inside this script, so the ratio is applied to the live algorithmic byte count of the same workload only.
-PACK_TRAFFIC_RATIO_LLAMA3_8B = 1.0160
+PACK_TRAFFIC_RATIO_LLAMA3_8B = 1.0008
 
 
 def parse_args():
@@ -387,6 +387,8 @@ def main():
             "blocking_breakdown_ms": {"dcp_plan": round(mean(rec["plan"]) * 1e3, 2),
                                       "layout_and_pack_launch": round(mean(rec["pack_launch"]) * 1e3, 2),
                                       "pack_kernel": round(pack_s * 1e3, 3)},
+            # host work in the blocking window per tensor: planning + layout + launch, without the kernel itself
+            "blocking_host_us_per_tensor": round((mean(rec["blocking"]) - pack_s) * 1e6 / max(len(sd), 1), 2),
             "pack_GBps": round(pack_gbps, 1),
             "unpack_GBps": round(2 * mean(rec["unpack_bytes"]) / 1e9 / unpack_s, 1) if unpack_s > 0 else None,
             "d2h_GBps": round(gb / mean(rec["d2h"]), 2) if mean(rec["d2h"]) > 0 else None,
