@@ -61,7 +61,7 @@ typedef struct mlf_item {
 typedef struct mlf_plan_opts {
   uint32_t tile_bytes;       /* bytes one workgroup copies per work item (multiple of 1024; 0 = default)       */
   uint32_t block_threads;    /* threads per workgroup for the copy kernels (multiple of 64; 0 = default)       */
-  uint32_t align_to_tensor;  /* 0: cut tiles at 16-byte boundaries of the image (pack); 1: of the tensor (unpack) */
+  uint32_t align_to_tensor;  /* tile cuts sit on a 4 KiB grid of: 0 = image offsets (pack), 1 = tensor addresses (unpack) */
   uint32_t unroll;           /* 16-byte vectors in flight per thread in the copy loop: 1, 2, 4, 8 (0 = default) */
   uint32_t grid_x_log2;      /* 0 = default; k > 0: rows of 2^(k-1) workgroups in the copy kernel's grid (a row may
                                 not exceed 2^32 - 1 threads),
