@@ -121,6 +121,8 @@ def payload_bytes(t: torch.Tensor) -> bytes:
     if t.numel() == 0:
         return b""
     flat = t.detach().to("cpu").contiguous().reshape(-1)
+    if flat.stride(0) != 1:  # a one-element tensor keeps whatever stride its view had
+        flat = torch.empty(flat.shape, dtype=flat.dtype, device=flat.device).copy_(flat)
     return flat.view(torch.uint8).numpy().tobytes()
 
 

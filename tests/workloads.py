@@ -160,7 +160,10 @@ def payload_bytes(sd) -> int:
 def fingerprint(t: torch.Tensor) -> Tuple[int, int]:
     """Order-sensitive 2x63-bit checksum of a tensor's bytes, computed on its device (bit patterns, not values).
     Used to compare restored tensors with the originals at sizes where a second copy does not fit."""
-    flat = t.detach().contiguous().reshape(-1).view(torch.uint8)
+    flat = t.detach().contiguous().reshape(-1)
+    if flat.numel() and flat.stride(0) != 1:  # a one-element tensor keeps whatever stride its view had
+        flat = torch.empty(flat.shape, dtype=flat.dtype, device=flat.device).copy_(flat)
+    flat = flat.view(torch.uint8)
     n = flat.numel()
     pad = (-n) % 8
     if pad:
