@@ -3,25 +3,23 @@
 //
 //   pack    live tensors (+ host blob of headers)  -> byte-exact image of a checkpoint object, in HBM
 //   unpack  image in HBM                           -> live tensors
-//   crc     CRC-32C per chunk of an image
-//   engine  image <-> pageable host memory through a ring of pinned slots and a host thread pool
 //
-// Everything on this path is integer byte movement, so the bound is HBM bandwidth (pack/unpack/crc) or the
-// host link (engine).  Kernels are written for 64-wide wavefronts and 16-byte accesses:
-//   * flat kernel: one small workgroup per tile (default 256 threads x one 16-byte vector = 4 KiB).  The
-//     destination is peeled to a 16-byte boundary, the body is non-temporal dwordx4 stores fed by dwordx4
-//     loads from a possibly misaligned source (gfx950 runs in unaligned-access mode), the tail is bytes.
-//     No LDS, no barriers.  Workgroups are short-lived and consecutive workgroups copy consecutive tiles, so
-//     the set of tiles in flight at any moment is a compact, sequential window of HBM; measured on MI355X
-//     this ordering is worth ~25 % over long-running workgroups that each stream a large private region.
+// Everything here is integer byte movement, so the bound is HBM bandwidth.  Kernels are written for 64-wide
+// wavefronts, 16-byte accesses and the eight XCDs (each with its own L2) that workgroups reach round-robin:
+//   * flat kernel: one small workgroup per tile (default 256 threads x one 16-byte vector = 4 KiB).  Tiles are cut
+//     on a 4 KiB grid of the destination, so full tiles write whole lines with non-temporal dwordx4 stores; the
+//     source is read with dwordx4 loads, or, where it is byte-misaligned relative to the destination, as aligned
+//     granules that are realigned across lanes.  No LDS, no barriers.  Workgroups are short-lived and follow the
+//     tiles in address order, so the set of tiles in flight is a compact, sequential window of HBM (worth ~25 %
+//     over long-running workgroups that each stream a private region); within groups of 512 the tiles are dealt
+//     out so that every XCD gets 64 consecutive ones and lines that straddle a cut stay in one L2.
 //     Tiles are not listed one by one: a table entry ("span") describes up to 128 (or 16, or 1) consecutive
-//     tiles of one contiguous item and the workgroups that share it derive their tile from blockIdx.
+//     tiles of one contiguous item and the workgroups that share it derive their tile from their number.
+//   * small kernel: pieces of at most 1 KiB (record headers, scalars, tails), one per wavefront.
 //   * transpose kernel: views whose contiguous dimension differs between tensor and image (e.g. `.t()`) go
-//     through an LDS tile so that both sides see whole consecutive runs.
+//     through an LDS tile so that both sides move whole 16-byte vectors along their contiguous dimension.
 //   * strided kernel: generic, division-free N-d index walk for every other non-contiguous source/target and
-//     for sub-box restores.
-//   * crc kernel: per wavefront a 64 KiB segment is read as coalesced 1 KiB rows; every lane keeps four
-//     Horner accumulators advanced by x^8192 through LDS tables, then lanes are folded with GF(2) multiplies.
+//     for sub-box restores, plus a vector gather for packing `[..., ::k]` out of long rows.
 #include "mlf_internal.h"
 
 #include <algorithm>
@@ -439,7 +437,8 @@ __global__ void __launch_bounds__(256) mlf_strided_kernel(const StridedDesc* __r
 // accesses are bound by the number of lane accesses, not by bytes); LDS is addressed per element on the transposed side.  T = 128 / 64 / 64 / 32 / 16 elements for esz = 1 / 2 / 4 / 8 / 16;
 // rows of the LDS tile are padded so that a column walk does not stay in one bank.
 constexpr uint32_t kTransThreads = 256;
-constexpr uint32_t kTransBand = 8;  // tile-rows per band of the visiting order (measured: 8 beats 1 by 10-40 %)
+constexpr uint32_t kTransBand = 8;   // tile-rows per band of the visiting order (measured: 8 beats 1 by 10-40 %)
+constexpr uint32_t kTransPatch = 8;  // neighbouring tile-rows per XCD where 64 tile-rows are left
 constexpr uint32_t kTransLdsBytes = 128 * (128 + 16);
 
 __host__ __device__ inline uint32_t trans_tile_dim(uint32_t esz) {
@@ -462,13 +461,32 @@ __device__ __forceinline__ void trans_tile(const TransDesc* __restrict__ d, uint
   const uint64_t per_batch = (uint64_t)d->tiles_a * d->tiles_b;
   uint64_t batch = tile / per_batch;
   const uint32_t rem = (uint32_t)(tile - batch * per_batch);
-  // tiles are visited in bands of kTransBand tile-rows, a fastest inside a band: eight consecutive workgroups read
-  // eight neighbouring runs of the same source rows, and the next eight write next to them in the same
-  // destination rows, so both sides keep hitting DRAM pages that are already open
-  const uint32_t band = rem / (kTransBand * d->tiles_b);
-  const uint32_t in_band = rem - band * (kTransBand * d->tiles_b);
-  const uint32_t band_rows = d->tiles_a - band * kTransBand < kTransBand ? d->tiles_a - band * kTransBand : kTransBand;
-  const uint32_t tb = in_band / band_rows, ta = band * kTransBand + (in_band - tb * band_rows);
+  // Visiting order.  Workgroups reach the eight XCDs round-robin, and every XCD has its own L2, so the order decides
+  // which L2 sees which lines.  Tile-rows are taken in bands; within a band the tile-column advances slowly and
+  // eight consecutive workgroups take eight different tile-rows, so that the tiles next to each other along b (they
+  // share destination lines when packing) are always eight workgroups apart: same XCD.  Where 8 * kTransPatch
+  // tile-rows are left, XCD k takes the kTransPatch neighbouring tile-rows [k * kTransPatch, (k + 1) * kTransPatch)
+  // of the band, so that tiles next to each other along a (they share source lines) are on one XCD too; the last
+  // rows use bands of eight.  (Full 8192 x 16384 transposes, TB/s: bands of 8: 2.9-3.9; patches of 8: 3.8-5.2.)
+  const uint32_t patch_rows = d->tiles_a / (8u * kTransPatch) * (8u * kTransPatch);
+  const uint32_t patch_tiles = patch_rows * d->tiles_b;
+  uint32_t ta, tb;
+  if (rem < patch_tiles) {
+    constexpr uint32_t kBand = 8u * kTransPatch;
+    const uint32_t band = rem / (kBand * d->tiles_b);
+    const uint32_t in_band = rem - band * (kBand * d->tiles_b);
+    tb = in_band / kBand;
+    const uint32_t j = in_band - tb * kBand;
+    ta = band * kBand + (j & 7u) * kTransPatch + (j >> 3);
+  } else {
+    const uint32_t left = rem - patch_tiles;
+    const uint32_t band = left / (kTransBand * d->tiles_b);
+    const uint32_t in_band = left - band * (kTransBand * d->tiles_b);
+    const uint32_t rows_here = d->tiles_a - patch_rows - band * kTransBand;
+    const uint32_t band_rows = rows_here < kTransBand ? rows_here : kTransBand;
+    tb = in_band / band_rows;
+    ta = patch_rows + band * kTransBand + (in_band - tb * band_rows);
+  }
   int64_t toff = 0, ioff = 0;
   for (int k = (int)d->nbatch - 1; k >= 0; --k) {
     const uint64_t extent = (uint64_t)d->bshape[k];
