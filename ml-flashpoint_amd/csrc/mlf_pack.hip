@@ -438,7 +438,7 @@ __global__ void __launch_bounds__(256) mlf_strided_kernel(const StridedDesc* __r
 // rows of the LDS tile are padded so that a column walk does not stay in one bank.
 constexpr uint32_t kTransThreads = 256;
 constexpr uint32_t kTransBand = 8;   // tile-rows per band of the visiting order (measured: 8 beats 1 by 10-40 %)
-constexpr uint32_t kTransPatch = 8;  // neighbouring tile-rows per XCD where 64 tile-rows are left
+constexpr uint32_t kTransPatch = 8;  // neighbouring tile-rows per XCD where 64 tile-rows are left (then 4, 2, 1)
 constexpr uint32_t kTransLdsBytes = 128 * (128 + 16);
 
 __host__ __device__ inline uint32_t trans_tile_dim(uint32_t esz) {
@@ -466,26 +466,28 @@ __device__ __forceinline__ void trans_tile(const TransDesc* __restrict__ d, uint
   // eight consecutive workgroups take eight different tile-rows, so that the tiles next to each other along b (they
   // share destination lines when packing) are always eight workgroups apart: same XCD.  Where 8 * kTransPatch
   // tile-rows are left, XCD k takes the kTransPatch neighbouring tile-rows [k * kTransPatch, (k + 1) * kTransPatch)
-  // of the band, so that tiles next to each other along a (they share source lines) are on one XCD too; the last
-  // rows use bands of eight.  (Full 8192 x 16384 transposes, TB/s: bands of 8: 2.9-3.9; patches of 8: 3.8-5.2.)
-  const uint32_t patch_rows = d->tiles_a / (8u * kTransPatch) * (8u * kTransPatch);
-  const uint32_t patch_tiles = patch_rows * d->tiles_b;
-  uint32_t ta, tb;
-  if (rem < patch_tiles) {
-    constexpr uint32_t kBand = 8u * kTransPatch;
-    const uint32_t band = rem / (kBand * d->tiles_b);
-    const uint32_t in_band = rem - band * (kBand * d->tiles_b);
-    tb = in_band / kBand;
-    const uint32_t j = in_band - tb * kBand;
-    ta = band * kBand + (j & 7u) * kTransPatch + (j >> 3);
-  } else {
-    const uint32_t left = rem - patch_tiles;
-    const uint32_t band = left / (kTransBand * d->tiles_b);
-    const uint32_t in_band = left - band * (kTransBand * d->tiles_b);
-    const uint32_t rows_here = d->tiles_a - patch_rows - band * kTransBand;
-    const uint32_t band_rows = rows_here < kTransBand ? rows_here : kTransBand;
-    tb = in_band / band_rows;
-    ta = patch_rows + band * kTransBand + (in_band - tb * band_rows);
+  // of the band, so that tiles next to each other along a (they share source lines) are on one XCD too; fewer rows
+  // are covered with patches of 4, then 2, then plain bands of eight.  (Full 8192 x 16384 transposes, TB/s: bands of
+  // 8: 2.9-3.9; patches of 8: 3.8-5.2.)
+  uint32_t ta = 0, tb = 0, row0 = 0, left = rem;
+#pragma unroll
+  for (uint32_t patch = kTransPatch; patch >= 1; patch >>= 1) {
+    // rows [row0, row0 + rows) are visited in bands of 8 * patch tile-rows; the last pass (patch == 1) takes all
+    // that is left, its last band possibly short of eight rows
+    const uint32_t band_h = 8u * patch;
+    const uint32_t rows = patch > 1 ? (d->tiles_a - row0) / band_h * band_h : d->tiles_a - row0;
+    const uint32_t tiles = rows * d->tiles_b;
+    if (left < tiles) {
+      const uint32_t band = left / (band_h * d->tiles_b);
+      const uint32_t in_band = left - band * (band_h * d->tiles_b);
+      const uint32_t rows_here = rows - band * band_h < band_h ? rows - band * band_h : band_h;
+      tb = in_band / rows_here;
+      const uint32_t j = in_band - tb * rows_here;
+      ta = row0 + band * band_h + (rows_here == band_h ? (j & 7u) * patch + (j >> 3) : j);
+      break;
+    }
+    left -= tiles;
+    row0 += rows;
   }
   int64_t toff = 0, ioff = 0;
   for (int k = (int)d->nbatch - 1; k >= 0; --k) {
