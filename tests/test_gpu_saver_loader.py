@@ -254,6 +254,33 @@ def test_crc_sidecar_written_and_corruption_detected(shm_dir, manager_future):
     dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, _loader(verify_crc=False)), no_dist=True)
 
 
+@pytest.mark.parametrize("save_file_io,load_file_io", [(False, False), (False, True), (True, False), (True, True)])
+def test_mapping_and_file_descriptor_io_write_and_read_the_same_object(shm_dir, manager_future, save_file_io, load_file_io):
+    """The host end of a transfer is either the MAP_SHARED mapping (memcpy) or the file descriptor (pwrite / pread);
+    every combination produces the oracle's bytes, a valid checksum sidecar, and a bit-exact restore."""
+    from ml_flashpoint.hip import integrity
+
+    sd_cpu = _mixed_state_dict()
+    sd_cpu["w.big"] = torch.randn(3_000_001, generator=torch.Generator().manual_seed(3))
+    sd_dev = _to_dev(sd_cpu)
+    ckpt = os.path.join(shm_dir, "step-3_ckpt")
+    saver = _saver(use_file_io=save_file_io, crc_chunk_bytes=1 << 20)
+    dcp.save(sd_dev, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(saver, manager_future), no_dist=True)
+    obj = os.path.join(ckpt, "__0__0_src0.distcp")
+    raw = open(obj, "rb").read()
+    metadata = pickle.load(open(os.path.join(ckpt, ".metadata"), "rb"))
+    image, spans, got_spans = _expected_file(sd_cpu, metadata, raw)
+    assert raw == image and got_spans == spans
+    chunk, nbytes, crcs = integrity.read_sidecar(obj)
+    assert nbytes == len(raw) - METADATA_SIZE and len(crcs) == -(-nbytes // chunk)
+    target = {k: (torch.zeros_like(v) if isinstance(v, torch.Tensor) else None) for k, v in sd_dev.items()}
+    loader = _loader(use_file_io=load_file_io)
+    dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), no_dist=True)
+    for k, v in sd_cpu.items():
+        if isinstance(v, torch.Tensor):
+            assert torch.equal(_bits(target[k]), _bits(v)), k
+
+
 def test_stage_data_returns_host_copies(shm_dir):
     sd_cpu = _mixed_state_dict()
     sd_dev = _to_dev(sd_cpu, keep_on_host=("w.i64",))
