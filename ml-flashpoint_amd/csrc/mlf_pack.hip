@@ -394,6 +394,49 @@ __device__ __forceinline__ void strided_gather(const StridedDesc* __restrict__ d
   if (j < w.count) *gstore<elem_u>(dp + (size_t)j * sizeof(T)) = *gload<elem_u>(sp + (size_t)j * (K * sizeof(T)));
 }
 
+// The way back, unpacking into `x[..., ::k]`: the gaps must not be written, so the stores stay element-sized, but
+// the image side is read as whole vectors and handed out through LDS so that neighbouring lanes store neighbouring
+// elements.  That removes almost half of the element-sized accesses (all the loads).
+template <typename T>
+__device__ __forceinline__ void strided_scatter(const StridedDesc* __restrict__ d, const StridedWork& w,
+                                                char* __restrict__ image, u32x4* __restrict__ lds) {
+  typedef T elem_u __attribute__((aligned(1)));
+  constexpr uint32_t EPV = 16 / (uint32_t)sizeof(T);
+  const int last = (int)d->ndim - 1;
+  const uint64_t len = (uint64_t)d->shape[last];
+  uint64_t row = w.start / len;  // uniform over the workgroup: scalar arithmetic
+  const uint64_t j0 = w.start - row * len;
+  const int64_t ts = d->tstride[last];
+  int64_t toff = (int64_t)j0 * ts, ioff = (int64_t)j0 * d->istride[last];
+#pragma unroll
+  for (int dim = MLF_MAX_DIMS - 2; dim >= 0; --dim) {
+    if (dim < last) {
+      const uint64_t extent = (uint64_t)d->shape[dim];
+      const uint64_t q = row / extent;
+      const int64_t at = (int64_t)(row - q * extent);
+      toff += at * d->tstride[dim];
+      ioff += at * d->istride[dim];
+      row = q;
+    }
+  }
+  const char* sp = image + d->image + ioff;
+  char* dp = reinterpret_cast<char*>(d->tensor) + toff;
+  const uint32_t n_units = w.count / EPV;
+  const T* __restrict__ lds_elems = reinterpret_cast<const T*>(lds);
+  for (uint32_t base = 0; base < n_units; base += 256) {  // uniform trip count: every thread reaches the barriers
+    const uint32_t u = base + threadIdx.x;
+    if (u < n_units) lds[threadIdx.x] = __builtin_nontemporal_load(gload<u32x4_u>(sp + (size_t)u * 16));
+    __syncthreads();
+    const uint32_t here = (n_units - base < 256u ? n_units - base : 256u) * EPV;
+#pragma unroll 4
+    for (uint32_t e = threadIdx.x; e < here; e += 256)
+      *gstore<elem_u>(dp + (int64_t)(base * EPV + e) * ts) = lds_elems[e];
+    __syncthreads();
+  }
+  const uint32_t j = n_units * EPV + threadIdx.x;  // fewer than EPV elements are left
+  if (j < w.count) *gstore<elem_u>(dp + (int64_t)j * ts) = *gload<elem_u>(sp + (size_t)j * sizeof(T));
+}
+
 template <typename T>
 __device__ __forceinline__ void strided_gather_k(const StridedDesc* __restrict__ d, const StridedWork& w,
                                                  char* __restrict__ image) {
@@ -416,6 +459,16 @@ __global__ void __launch_bounds__(256) mlf_strided_kernel(const StridedDesc* __r
       case 2: strided_gather_k<uint16_t>(d, w, image); break;
       case 4: strided_gather_k<uint32_t>(d, w, image); break;
       default: strided_gather_k<uint64_t>(d, w, image); break;
+    }
+    return;
+  }
+  if (!PACK && d->gather_k) {
+    __shared__ u32x4 lds[256];
+    switch (d->esz) {
+      case 1: strided_scatter<uint8_t>(d, w, image, lds); break;
+      case 2: strided_scatter<uint16_t>(d, w, image, lds); break;
+      case 4: strided_scatter<uint32_t>(d, w, image, lds); break;
+      default: strided_scatter<uint64_t>(d, w, image, lds); break;
     }
     return;
   }
