@@ -365,7 +365,7 @@ def main():
         unpack_s = mean(rec["unpack_ms"]) * 1e-3
         pack_gbps = 2 * mean(rec["pack_bytes"]) / 1e9 / pack_s if pack_s > 0 else 0.0
         result = {
-            "metric": "save+restore GB/s through the shm buffer path (with blocking save ms), 1 MI355X",
+            "metric": "save/restore GB/s + blocking save ms, 8B bf16+fp32-Adam shard, 1 MI355X",
             "value": round(2 * gb / step_s, 3),
             "unit": "GB/s",
             "n_gpus": 1,
