@@ -99,7 +99,9 @@ class MemoryStorageReader(StorageReader):
                     len(per_file),
                 )
         else:
-            _LOGGER.info("Rank %d: No files to read for plan in '%s'", torch.distributed.get_rank(), self._path)
+            # a single-process load has no process group to ask; the line is informational either way
+            rank = torch.distributed.get_rank() if torch.distributed.is_initialized() else 0
+            _LOGGER.info("Rank %d: No files to read for plan in '%s'", rank, self._path)
         done: Future = Future()
         done.set_result(None)
         return done
