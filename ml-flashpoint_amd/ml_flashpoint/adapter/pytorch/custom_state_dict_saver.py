@@ -8,6 +8,7 @@ With the gfx950 saver the blocking work of a save ends inside ``generate_plan``:
 
 import logging
 
+import torch
 from torch import distributed as torchdist
 from torch.distributed.checkpoint import state_dict_saver as torchdistsaver
 from torch.distributed.checkpoint.planner import SavePlan
@@ -15,6 +16,7 @@ from torch.distributed.checkpoint.storage import WriteResult
 from torch.distributed.checkpoint.utils import _DistWrapper
 
 from ml_flashpoint.adapter.pytorch.memory_storage_writer import MemoryStorageWriter
+from ml_flashpoint.core import utils
 from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId
 from ml_flashpoint.core.checkpoint_saver import ObjectWriteBucket
 from ml_flashpoint.core.mlf_logging import get_logger
@@ -102,3 +104,10 @@ def finish_write(
         all_results = world_dist_wrapper.broadcast_object(all_results)
     if torchdist.get_node_local_rank(fallback_rank=0) == 0:
         storage_writer.finish_checkpoint(checkpoint_id=checkpoint_id, metadata=global_metadata, results=all_results)
+
+
+def _get_local_rank_0_global_ranks() -> list[int]:
+    """Global ranks that are rank 0 of their node, assuming every node runs one rank per visible GPU
+    (reference: custom_state_dict_saver.py:218-227; nothing calls it there either)."""
+    per_node = torch.cuda.device_count()
+    return [node * per_node for node in range(utils.get_num_of_nodes())]
