@@ -1,17 +1,22 @@
-"""DCP's ``save()`` cut into three calls - plan, write, finish - so that an async framework can run the write in a
-worker while the training process goes on (interface and semantics of the reference's
-src/ml_flashpoint/adapter/pytorch/custom_state_dict_saver.py:42-215, itself derived from torch's state_dict_saver).
+"""A DCP save cut into three calls - ``generate_plan``, ``write_data``, ``finish_write`` - so that an async framework
+can run the middle one in a worker while the training process goes on.  Names, arguments and results are those of the
+reference's module (src/ml_flashpoint/adapter/pytorch/custom_state_dict_saver.py:42-227), which the Megatron/NeMo
+strategies call.
 
 With the gfx950 saver the blocking work of a save ends inside ``generate_plan``: its last step,
-``prepare_write_data_buckets``, enqueues the pack of the checkpoint image on the training stream.
+``storage_writer.prepare_write_data_buckets``, lays the object out and enqueues the pack of its image on the
+training stream.
 """
 
+from __future__ import annotations
+
 import logging
+from typing import NamedTuple
 
 import torch
-from torch import distributed as torchdist
-from torch.distributed.checkpoint import state_dict_saver as torchdistsaver
-from torch.distributed.checkpoint.planner import SavePlan
+import torch.distributed as torchdist
+from torch.distributed.checkpoint.metadata import STATE_DICT_TYPE, Metadata
+from torch.distributed.checkpoint.planner import SavePlan, SavePlanner
 from torch.distributed.checkpoint.storage import WriteResult
 from torch.distributed.checkpoint.utils import _DistWrapper
 
@@ -20,90 +25,94 @@ from ml_flashpoint.core import utils
 from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId
 from ml_flashpoint.core.checkpoint_saver import ObjectWriteBucket
 from ml_flashpoint.core.mlf_logging import get_logger
-from ml_flashpoint.core.utils import gc_paused, log_execution_time
 
 _LOGGER = get_logger(__name__)
 
 
-@log_execution_time(logger=_LOGGER, name="generate_plan", level=logging.INFO)
+class _CachedStructure(NamedTuple):
+    """What a caller keeps from one save for the next (``cached_ckpt_structure``)."""
+
+    central_plan: SavePlan | None = None  # this rank's share of the global plan
+    local_plan: SavePlan | None = None    # this rank's own plan, before the global step
+    validated: bool = False               # two consecutive saves produced the same central plan
+
+
+@utils.log_execution_time(logger=_LOGGER, name="generate_plan", level=logging.INFO)
 def generate_plan(
     checkpoint_id: CheckpointContainerId,
-    state_dict: torchdistsaver.STATE_DICT_TYPE,
+    state_dict: STATE_DICT_TYPE,
     storage_writer: MemoryStorageWriter,
-    planner: torchdistsaver.SavePlanner,
+    planner: SavePlanner,
     world_dist_wrapper: _DistWrapper,
     cached_ckpt_structure: tuple[SavePlan, SavePlan, bool] | None = None,
-) -> tuple[list[ObjectWriteBucket], torchdistsaver.Metadata | None, SavePlan, SavePlan, bool]:
-    """Planning phase of a save.
+) -> tuple[list[ObjectWriteBucket], Metadata | None, SavePlan, SavePlan, bool]:
+    """Planning phase: ``(write_buckets, global_metadata, central_plan, local_plan, validated_cache_reuse)``.
 
-    Returns ``(write_buckets, global_metadata, central_plan, local_plan, validated_cache_reuse)``.  The last three are
-    what the caller keeps as ``cached_ckpt_structure`` for the next save: once the central plan of two consecutive
-    saves compares equal, ``validated_cache_reuse`` turns True and later saves skip ``create_local_plan``, the plan
-    reduce-scatter and the metadata broadcast (``global_metadata`` is then None: the caller reuses the one it has).
+    The last three are the next save's ``cached_ckpt_structure``.  As long as the cache is not validated every save
+    plans from scratch (local plan, reduce-scatter through the coordinator's global plan, metadata broadcast) and
+    compares its central plan with the cached one; once they were equal, later saves skip all three steps and
+    ``global_metadata`` comes back as None - the caller already holds the metadata that goes with the cached plan.
     """
-    with gc_paused():  # planning allocates ~10 small objects per tensor; see gc_paused
-        return _generate_plan(checkpoint_id, state_dict, storage_writer, planner, world_dist_wrapper, cached_ckpt_structure)
+    with utils.gc_paused():  # planning allocates ~10 small objects per tensor, none of them cyclic
+        cache = _CachedStructure(*cached_ckpt_structure) if cached_ckpt_structure else _CachedStructure()
+        coordinator = world_dist_wrapper.is_coordinator
+        planner.set_up_planner(state_dict=state_dict, storage_meta=storage_writer.storage_meta(), is_coordinator=coordinator)
+        storage_writer.set_up_storage_writer(coordinator)
+        if cache.validated and cache.central_plan:
+            local_plan = storage_writer.prepare_local_plan(cache.local_plan or planner.create_local_plan())
+            central_plan, global_metadata = cache.central_plan, None
+        else:
+            local_plan = storage_writer.prepare_local_plan(planner.create_local_plan())
+            central_plan, global_metadata = _agree_on_plan(local_plan, storage_writer, planner, world_dist_wrapper)
+        buckets = storage_writer.prepare_write_data_buckets(checkpoint_id, planner.finish_plan(central_plan), planner)
+        return buckets, global_metadata, central_plan, local_plan, cache.central_plan == central_plan
 
 
-def _generate_plan(checkpoint_id, state_dict, storage_writer, planner, world_dist_wrapper, cached_ckpt_structure):
-    cached_central_plan, cached_local_plan, validated = cached_ckpt_structure or (None, None, False)
-    global_metadata: torchdistsaver.Metadata | None = None
+def _agree_on_plan(local_plan, storage_writer, planner, dist: _DistWrapper):
+    """Every rank's plan goes to the coordinator, which merges them, lets the writer number them and hands each rank
+    its share back; the metadata that the merge produced exists on the coordinator only and is broadcast."""
+    merged_metadata = None
 
-    def local_step() -> SavePlan:
-        planner.set_up_planner(
-            state_dict=state_dict,
-            storage_meta=storage_writer.storage_meta(),
-            is_coordinator=world_dist_wrapper.is_coordinator,
-        )
-        storage_writer.set_up_storage_writer(world_dist_wrapper.is_coordinator)
-        plan = cached_local_plan if (cached_local_plan and validated) else planner.create_local_plan()
-        return storage_writer.prepare_local_plan(plan)
-
-    def global_step(all_local_plans: list[SavePlan]) -> list[SavePlan]:
-        nonlocal global_metadata
-        all_local_plans, global_metadata = planner.create_global_plan(all_local_plans)
+    def merge(all_local_plans: list[SavePlan]) -> list[SavePlan]:
+        nonlocal merged_metadata
+        all_local_plans, merged_metadata = planner.create_global_plan(all_local_plans)
         return storage_writer.prepare_global_plan(all_local_plans)
 
-    if validated and cached_central_plan:
-        local_plan = local_step()
-        central_plan = cached_central_plan
-    else:
-        with log_execution_time(logger=_LOGGER, name="generate_plan__reduce_scatter_plan"):
-            local_plan = local_step()
-            central_plan = world_dist_wrapper.reduce_scatter("plan", lambda: local_plan, global_step)
-        with log_execution_time(logger=_LOGGER, name="generate_plan__broadcast_metadata"):
-            global_metadata = world_dist_wrapper.broadcast_object(global_metadata)
-
-    final_local_plan = planner.finish_plan(central_plan)
-    write_buckets = storage_writer.prepare_write_data_buckets(checkpoint_id, final_local_plan, planner)
-    return write_buckets, global_metadata, central_plan, local_plan, cached_central_plan == central_plan
+    with utils.log_execution_time(logger=_LOGGER, name="generate_plan__reduce_scatter_plan"):
+        central_plan = dist.reduce_scatter("plan", lambda: local_plan, merge)
+    with utils.log_execution_time(logger=_LOGGER, name="generate_plan__broadcast_metadata"):
+        return central_plan, dist.broadcast_object(merged_metadata)
 
 
-@log_execution_time(logger=_LOGGER, name="write_data", level=logging.INFO)
+@utils.log_execution_time(logger=_LOGGER, name="write_data", level=logging.INFO)
 def write_data(
     checkpoint_id: CheckpointContainerId,
     storage_writer: MemoryStorageWriter,
     staged_write_buckets: list[ObjectWriteBucket],
     replicate_after_write: bool,
 ) -> list[WriteResult]:
-    """Write phase; synchronous.  This is the call an async framework runs in its worker."""
-    return storage_writer.write_staged_data_buckets(checkpoint_id, staged_write_buckets, replicate_after_write).wait()
+    """Write phase, synchronous: the call an async framework runs in its worker."""
+    pending = storage_writer.write_staged_data_buckets(checkpoint_id, staged_write_buckets, replicate_after_write)
+    return pending.wait()
 
 
-@log_execution_time(logger=_LOGGER, name="finish_write", level=logging.INFO)
+@utils.log_execution_time(logger=_LOGGER, name="finish_write", level=logging.INFO)
 def finish_write(
     checkpoint_id: CheckpointContainerId,
     storage_writer: MemoryStorageWriter,
-    global_metadata: torchdistsaver.Metadata,
+    global_metadata: Metadata,
     world_dist_wrapper: _DistWrapper,
 ) -> None:
-    """Gathers every rank's write results on the coordinator, broadcasts them, and writes the ``.metadata`` object
-    once per node (on node-local rank 0).  Call only after the write of ``checkpoint_id`` is known to be complete."""
-    all_results = world_dist_wrapper.gather_object(storage_writer.get_write_results(checkpoint_id))
-    with log_execution_time(logger=_LOGGER, name="finish_write__broadcast_results"):
-        all_results = world_dist_wrapper.broadcast_object(all_results)
-    if torchdist.get_node_local_rank(fallback_rank=0) == 0:
-        storage_writer.finish_checkpoint(checkpoint_id=checkpoint_id, metadata=global_metadata, results=all_results)
+    """Completion phase, to be called once the write of ``checkpoint_id`` is known to be done on this rank: the
+    ranks' write results are gathered on the coordinator and broadcast back, and the first rank of every node
+    writes the checkpoint's metadata object."""
+    own = storage_writer.get_write_results(checkpoint_id)
+    everyones = world_dist_wrapper.gather_object(own)
+    with utils.log_execution_time(logger=_LOGGER, name="finish_write__broadcast_results"):
+        everyones = world_dist_wrapper.broadcast_object(everyones)
+    if torchdist.get_node_local_rank(fallback_rank=0) != 0:
+        return
+    storage_writer.finish_checkpoint(checkpoint_id=checkpoint_id, metadata=global_metadata, results=everyones)
 
 
 def _get_local_rank_0_global_ranks() -> list[int]:

@@ -1,41 +1,87 @@
-"""PyTorch DCP ``StorageWriter`` that saves into in-memory buffer objects through a checkpoint saver plug-in.
+"""DCP ``StorageWriter`` whose storage is a set of checkpoint buffer objects filled by a saver plug-in.
 
-Interface and behaviour follow the reference (src/ml_flashpoint/adapter/pytorch/memory_storage_writer.py:53-401):
-two ways to drive it - the classic DCP ``write_data(plan, planner)``, or the split
-``prepare_write_data_buckets -> stage_write_data_buckets -> write_staged_data_buckets`` used by async frameworks -
-and write results are handed across processes through ``torch.multiprocessing.Manager`` proxies.
+The public surface is the one the reference's adapter has (src/ml_flashpoint/adapter/pytorch/memory_storage_writer.py
+:53-401), because DCP, the three-call saver (``custom_state_dict_saver``) and async frameworks call it:
+
+* classic DCP:  ``reset -> prepare_local_plan -> prepare_global_plan -> write_data -> finish``
+* split form:   ``prepare_write_data_buckets`` (training process; with the gfx950 saver this is where the image is
+                packed) -> ``stage_write_data_buckets`` (static; ends the blocking part) ->
+                ``write_staged_data_buckets`` (possibly another process) -> ``get_write_results`` ->
+                ``finish_checkpoint``
+
+What crosses the process boundary in the split form is kept in one place, ``_WriteLedger``: per checkpoint id a
+completion event and the list of write results, both held by a ``torch.multiprocessing`` manager.
 """
+
+from __future__ import annotations
 
 import concurrent.futures
 import dataclasses
 import logging
 import os
 import time
-from typing import Optional, Union
 
 import torch
-import torch.multiprocessing as torch_mp
-from torch.distributed.checkpoint import Metadata, SavePlan, SavePlanner, StorageWriter, staging
-from torch.distributed.checkpoint.filesystem import _StorageInfo
-from torch.distributed.checkpoint.metadata import STATE_DICT_TYPE, MetadataIndex, StorageMeta
-from torch.distributed.checkpoint.storage import WriteResult
+from torch.distributed.checkpoint import staging
+from torch.distributed.checkpoint.metadata import STATE_DICT_TYPE, Metadata, StorageMeta
+from torch.distributed.checkpoint.planner import SavePlan, SavePlanner
+from torch.distributed.checkpoint.storage import StorageWriter, WriteResult
 from torch.futures import Future as TorchFuture
 from typing_extensions import override
 
+from ml_flashpoint.core import utils
 from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId, CheckpointObjectId
 from ml_flashpoint.core.checkpoint_saver import MLFlashpointCheckpointSaver, ObjectWriteBucket
 from ml_flashpoint.core.hfid import generate_hfid
 from ml_flashpoint.core.mlf_logging import get_logger
-from ml_flashpoint.core.utils import gc_paused, log_execution_time
 
 _LOGGER = get_logger(__name__)
+_timed = utils.log_execution_time
+
+_NOT_RESET = "MemoryStorageWriter has not been reset. Call reset() before using this method."
+_BAD_PLAN = (
+    "SavePlan.storage_data is not a valid _StorageDataContext or prefix is empty. "
+    "This is likely because prepare_global_plan was not called on this SavePlan."
+)
+_NEVER_SIGNALLED = (
+    "Event was never set for checkpoint_id '%s', meaning we cannot confirm that the write "
+    "has completed, and its results are available."
+)
+_MISSING_RANK_RESULTS = (
+    "finish: write results[%d] is None! This suggests an error in producing or gathering "
+    "the write_results list from that local rank (%d)."
+)
 
 
 @dataclasses.dataclass
 class _StorageDataContext:
-    """Per-plan context set by ``prepare_global_plan``: the object-name prefix of that rank's plan."""
+    """What ``prepare_global_plan`` attaches to each rank's plan: the prefix of that plan's object names."""
 
     prefix: str
+
+
+class _WriteLedger:
+    """Completion events and write results per checkpoint id, shared between the process that prepares a save and
+    the one that writes it.  Empty until ``open`` is given a manager; a ledger that travelled to another process
+    keeps working through its proxies but cannot create new events there."""
+
+    def __init__(self):
+        self.events = None   # manager dict: CheckpointContainerId -> manager Event
+        self.results = None  # manager dict: CheckpointContainerId -> list[WriteResult]
+
+    def open(self, manager) -> None:
+        self.events, self.results = manager.dict(), manager.dict()
+
+    def expect(self, checkpoint_id: CheckpointContainerId, manager_future) -> None:
+        if checkpoint_id not in self.events:
+            self.events[checkpoint_id] = manager_future.result().Event()
+
+    def publish(self, checkpoint_id: CheckpointContainerId, results: list[WriteResult]) -> None:
+        self.results[checkpoint_id] = results
+        self.events[checkpoint_id].set()
+
+    def wait(self, checkpoint_id: CheckpointContainerId, timeout_s: float) -> bool:
+        return self.events[checkpoint_id].wait(timeout=timeout_s)
 
 
 class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
@@ -45,208 +91,212 @@ class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
         mp_manager_future: concurrent.futures.Future,
         thread_count: int = 1,
     ):
-        """``mp_manager_future`` resolves to a ``torch.multiprocessing.Manager`` (ideally created with the 'spawn'
-        context); it backs the per-checkpoint result dict and completion events shared with worker processes."""
+        """``mp_manager_future`` resolves to a ``torch.multiprocessing`` manager (best created with the 'spawn'
+        context) of the main process; it is consulted lazily and never pickled.  ``thread_count`` is both the
+        number of objects a save is split into and the saver's writer-thread count; values below 1 mean 1."""
         super().__init__()
-        self._current_checkpoint_id: CheckpointContainerId | None = None
-        self._current_save_id: str | None = None
-        self._checkpoint_saver = checkpoint_saver
         if thread_count < 1:
             _LOGGER.warning("thread_count must be >= 1, but was %d. Setting to 1.", thread_count)
-            thread_count = 1
-        self._thread_count = thread_count
-        self._main_process_torchmp_manager_future = mp_manager_future  # main process only: not picklable
-        self._write_events_per_checkpoint_id: Optional[dict[CheckpointContainerId, torch_mp.Event]] = None
-        self._write_results_per_checkpoint_id: Optional[dict[CheckpointContainerId, list[WriteResult]]] = None
+        self._thread_count = max(thread_count, 1)
+        self._checkpoint_saver = checkpoint_saver
+        self._main_process_torchmp_manager_future = mp_manager_future
+        self._ledger = _WriteLedger()
+        self._current_checkpoint_id: CheckpointContainerId | None = None
+        self._current_save_id: str | None = None
 
-    def __getstate__(self):
-        state = self.__dict__.copy()
-        state.pop("_main_process_torchmp_manager_future", None)
-        return state
+    # the ledger's two dicts under the names other code (and the reference's tests) know them by
+    @property
+    def _write_events_per_checkpoint_id(self):
+        return self._ledger.events
 
-    def __setstate__(self, state):
-        self.__dict__.update(state)
-        self._main_process_torchmp_manager_future = None
-
-    def _check_checkpoint_id(self) -> None:
-        if self._current_checkpoint_id is None:
-            raise ValueError("MemoryStorageWriter has not been reset. Call reset() before using this method.")
+    @_write_events_per_checkpoint_id.setter
+    def _write_events_per_checkpoint_id(self, value):
+        self._ledger.events = value
 
     @property
-    def current_checkpoint_id(self) -> Optional[CheckpointContainerId]:
+    def _write_results_per_checkpoint_id(self):
+        return self._ledger.results
+
+    @_write_results_per_checkpoint_id.setter
+    def _write_results_per_checkpoint_id(self, value):
+        self._ledger.results = value
+
+    def __getstate__(self):
+        return {k: v for k, v in self.__dict__.items() if k != "_main_process_torchmp_manager_future"}
+
+    def __setstate__(self, state):
+        self.__dict__.update(state, _main_process_torchmp_manager_future=None)
+
+    # ---- identity of the save in progress ------------------------------------------------------------------------
+    def _require_reset(self) -> CheckpointContainerId:
+        if self._current_checkpoint_id is None:
+            raise ValueError(_NOT_RESET)
+        return self._current_checkpoint_id
+
+    _check_checkpoint_id = _require_reset
+
+    @property
+    def current_checkpoint_id(self) -> CheckpointContainerId | None:
         return self._current_checkpoint_id
 
     @property
-    def path(self) -> Optional[str]:
-        return None if self._current_checkpoint_id is None else self._current_checkpoint_id.data
+    def path(self) -> str | None:
+        current = self._current_checkpoint_id
+        return current.data if current is not None else None
 
     @property
     def checkpoint_saver(self) -> MLFlashpointCheckpointSaver:
         return self._checkpoint_saver
 
     @override
-    def reset(self, checkpoint_id: Union[str, os.PathLike, None] = None) -> None:
+    def reset(self, checkpoint_id: str | os.PathLike | None = None) -> None:
+        """Starts a save: new id, new save id.  Entries of earlier ids stay in the ledger."""
         self._current_checkpoint_id = CheckpointContainerId(checkpoint_id)
         self._current_save_id = generate_hfid("memwritersave")
-        if self._write_events_per_checkpoint_id is None and self._main_process_torchmp_manager_future is not None:
-            manager = self._main_process_torchmp_manager_future.result()
-            self._write_events_per_checkpoint_id = manager.dict()
-            self._write_results_per_checkpoint_id = manager.dict()
+        have_manager = self._main_process_torchmp_manager_future is not None
+        if self._ledger.events is None and have_manager:
+            self._ledger.open(self._main_process_torchmp_manager_future.result())
 
-    def storage_meta(self) -> Optional[StorageMeta]:
-        self._check_checkpoint_id()
-        return StorageMeta(checkpoint_id=self._current_checkpoint_id.data, save_id=self._current_save_id)
+    def storage_meta(self) -> StorageMeta | None:
+        return StorageMeta(checkpoint_id=self._require_reset().data, save_id=self._current_save_id)
 
+    @classmethod
+    @override
+    def validate_checkpoint_id(cls, checkpoint_id: str | os.PathLike) -> bool:
+        try:
+            CheckpointContainerId(checkpoint_id)
+        except Exception as e:
+            _LOGGER.warning("Unable to validate checkpoint_id: %s, %s", checkpoint_id, e)
+            return False
+        return True
+
+    # ---- planning hooks --------------------------------------------------------------------------------------------
     @override
     def set_up_storage_writer(self, is_coordinator: bool) -> None:
-        pass
+        """Nothing to set up: objects are created when they are written."""
 
     @override
-    @log_execution_time(logger=_LOGGER, name="prepare_local_plan")
+    @_timed(logger=_LOGGER, name="prepare_local_plan")
     def prepare_local_plan(self, plan: SavePlan) -> SavePlan:
-        self._check_checkpoint_id()
-        self._checkpoint_saver.initialize_checkpoint(self._current_checkpoint_id)
+        self._checkpoint_saver.initialize_checkpoint(self._require_reset())  # marks the checkpoint as unfinished
         return plan
 
     @override
-    @log_execution_time(logger=_LOGGER, name="prepare_global_plan")
+    @_timed(logger=_LOGGER, name="prepare_global_plan")
     def prepare_global_plan(self, plans: list[SavePlan]) -> list[SavePlan]:
-        return [dataclasses.replace(p, storage_data=_StorageDataContext(f"__{i}_")) for i, p in enumerate(plans)]
+        numbered = []
+        for rank_position, plan in enumerate(plans):
+            context = _StorageDataContext(prefix=f"__{rank_position}_")
+            numbered.append(dataclasses.replace(plan, storage_data=context))
+        return numbered
 
+    # ---- the write, whole or in three parts ----------------------------------------------------------------------
     @override
-    @log_execution_time(logger=_LOGGER, name="stage", level=logging.INFO)
+    @_timed(logger=_LOGGER, name="stage", level=logging.INFO)
     def stage(self, state_dict: STATE_DICT_TYPE) -> STATE_DICT_TYPE:
         return super().stage(state_dict)
 
-    @log_execution_time(logger=_LOGGER, name="prepare_write_data_buckets")
+    @override
+    @_timed(logger=_LOGGER, name="write_data", level=logging.INFO)
+    def write_data(self, plan: SavePlan, planner: SavePlanner) -> TorchFuture[list[WriteResult]]:
+        checkpoint_id = self._require_reset()
+        context = plan.storage_data
+        if not (isinstance(context, _StorageDataContext) and context.prefix):
+            raise ValueError(_BAD_PLAN)
+        write_buckets = self.prepare_write_data_buckets(checkpoint_id, plan, planner)
+        return self.write_staged_data_buckets(checkpoint_id, write_buckets, replicate_after_write=True)
+
+    @_timed(logger=_LOGGER, name="prepare_write_data_buckets")
     def prepare_write_data_buckets(
         self, checkpoint_id: CheckpointContainerId, plan: SavePlan, planner: SavePlanner
     ) -> list[ObjectWriteBucket]:
-        if checkpoint_id not in self._write_events_per_checkpoint_id:
-            self._write_events_per_checkpoint_id[checkpoint_id] = (
-                self._main_process_torchmp_manager_future.result().Event()
-            )
-        return self.checkpoint_saver.prepare_write_data(
+        """Registers the completion event of ``checkpoint_id`` (only the main process can create one) and lets the
+        saver turn the plan into one bucket per object."""
+        self._ledger.expect(checkpoint_id, self._main_process_torchmp_manager_future)
+        return self._checkpoint_saver.prepare_write_data(
             checkpoint_id, plan.items, planner, plan.storage_data.prefix, bucket_count=self._thread_count
         )
 
     @staticmethod
-    @log_execution_time(logger=_LOGGER, name="stage_write_data_buckets", level=logging.INFO)
-    @gc_paused()
+    @_timed(logger=_LOGGER, name="stage_write_data_buckets", level=logging.INFO)
+    @utils.gc_paused()
     def stage_write_data_buckets(
         _: CheckpointContainerId, write_buckets: list[ObjectWriteBucket], non_blocking: bool = True
     ):
-        """Makes the buckets independent of live training tensors.  Entries that a GPU-native saver already packed
-        are placeholders whose ``.to()`` returns themselves, so for them this only runs the device synchronize
-        that ends the blocking part of a save."""
-        staged = [
-            dataclasses.replace(
-                b, tensor_data=[(item, t.to(device="cpu", non_blocking=non_blocking)) for item, t in b.tensor_data]
-            )
-            for b in write_buckets
-        ]
+        """Returns buckets that no longer depend on live training tensors.  Static, because async frameworks call
+        it on the class.  A bucket prepared by the gfx950 saver holds placeholders for an image that is already
+        being packed in HBM: their ``.to()`` is the identity, and the device synchronize below is then the moment
+        the training stream may overwrite its tensors again."""
+
+        def on_host(pairs):
+            return [(item, tensor.to(device="cpu", non_blocking=non_blocking)) for item, tensor in pairs]
+
+        staged = [dataclasses.replace(bucket, tensor_data=on_host(bucket.tensor_data)) for bucket in write_buckets]
         if non_blocking and torch.cuda.is_available():
             torch.cuda.synchronize()
         return staged
 
-    @log_execution_time(logger=_LOGGER, name="write_staged_write_buckets", level=logging.INFO)
-    @gc_paused()
+    @_timed(logger=_LOGGER, name="write_staged_write_buckets", level=logging.INFO)
+    @utils.gc_paused()
     def write_staged_data_buckets(
         self,
         checkpoint_id: CheckpointContainerId,
         staged_write_buckets: list[ObjectWriteBucket],
         replicate_after_write: bool,
     ) -> TorchFuture[list[WriteResult]]:
-        start = time.perf_counter()
-        write_results = self._checkpoint_saver.write_data(
+        """Synchronous write of prepared buckets; publishes the results for ``get_write_results`` (in whichever
+        process that is called) and also returns them in a completed future.  A failing write publishes nothing."""
+        began = time.perf_counter()
+        outcome = self._checkpoint_saver.write_data(
             checkpoint_id,
             write_buckets=staged_write_buckets,
             thread_count=self._thread_count,
             replicate_after_write=replicate_after_write,
         )
-        duration = time.perf_counter() - start
-        total = sum(r.size_in_bytes for r in write_results)
-        if duration > 0:
-            _LOGGER.info(
-                "Written %d bytes in %.4f s (%.2f GB/s) from %d buckets",
-                total,
-                duration,
-                (total / 1e9) / duration,
-                len(staged_write_buckets),
-            )
-        self._write_results_per_checkpoint_id[checkpoint_id] = write_results
-        self._write_events_per_checkpoint_id[checkpoint_id].set()
-        fut: TorchFuture = TorchFuture()
-        fut.set_result(write_results)
-        return fut
+        utils.log_rate(_LOGGER, "Written", sum(r.size_in_bytes for r in outcome), time.perf_counter() - began,
+                       len(staged_write_buckets), "buckets")
+        self._ledger.publish(checkpoint_id, outcome)
+        done: TorchFuture = TorchFuture()
+        done.set_result(outcome)
+        return done
 
-    @override
-    @log_execution_time(logger=_LOGGER, name="write_data", level=logging.INFO)
-    def write_data(self, plan: SavePlan, planner: SavePlanner) -> TorchFuture[list[WriteResult]]:
-        self._check_checkpoint_id()
-        if not isinstance(plan.storage_data, _StorageDataContext) or not plan.storage_data.prefix:
-            raise ValueError(
-                "SavePlan.storage_data is not a valid _StorageDataContext or prefix is empty. "
-                "This is likely because prepare_global_plan was not called on this SavePlan."
-            )
-        buckets = self.prepare_write_data_buckets(self.current_checkpoint_id, plan, planner)
-        return self.write_staged_data_buckets(self.current_checkpoint_id, buckets, replicate_after_write=True)
-
-    def replicate_written_objects(self, object_ids: set[CheckpointObjectId]) -> list[concurrent.futures.Future]:
-        futures = []
-        for object_id in object_ids:
-            futures.extend(self._checkpoint_saver.async_replicate_object(object_id))
-        return futures
-
-    @log_execution_time(logger=_LOGGER, name="get_write_results")
+    @_timed(logger=_LOGGER, name="get_write_results")
     def get_write_results(
         self, checkpoint_id: CheckpointContainerId, wait_timeout_sec: float = 15.0
     ) -> list[WriteResult]:
-        """Waits (up to ``wait_timeout_sec``) for the write of ``checkpoint_id`` to be signalled, then returns its
-        results.  KeyError if no write was prepared for the id, RuntimeError on timeout."""
-        if not self._write_events_per_checkpoint_id[checkpoint_id].wait(timeout=wait_timeout_sec):
-            msg = (
-                "Event was never set for checkpoint_id '%s', meaning we cannot confirm that the write "
-                "has completed, and its results are available." % checkpoint_id
-            )
-            _LOGGER.error(msg)
-            raise RuntimeError(msg)
-        return self._write_results_per_checkpoint_id.get(checkpoint_id)
+        """Results of the write of ``checkpoint_id`` once it has been signalled: ``KeyError`` when no write was ever
+        prepared for that id, ``RuntimeError`` when the signal does not come within ``wait_timeout_sec``."""
+        if self._ledger.wait(checkpoint_id, wait_timeout_sec):
+            return self._ledger.results.get(checkpoint_id)
+        complaint = _NEVER_SIGNALLED % checkpoint_id
+        _LOGGER.error(complaint)
+        raise RuntimeError(complaint)
 
+    def replicate_written_objects(self, object_ids: set[CheckpointObjectId]) -> list[concurrent.futures.Future]:
+        replicate = self._checkpoint_saver.async_replicate_object
+        return [future for object_id in object_ids for future in replicate(object_id)]
+
+    # ---- completion --------------------------------------------------------------------------------------------------
     @override
-    @log_execution_time(logger=_LOGGER, name="finish")
+    @_timed(logger=_LOGGER, name="finish")
     def finish(self, metadata: Metadata, results: list[list[WriteResult]]) -> None:
-        self._check_checkpoint_id()
-        self.finish_checkpoint(self.current_checkpoint_id, metadata, results)
+        self.finish_checkpoint(self._require_reset(), metadata, results)
 
-    @log_execution_time(logger=_LOGGER, name="finish_checkpoint", level=logging.INFO)
-    @gc_paused()
+    @_timed(logger=_LOGGER, name="finish_checkpoint", level=logging.INFO)
+    @utils.gc_paused()
     def finish_checkpoint(
         self, checkpoint_id: CheckpointContainerId, metadata: Metadata, results: list[list[WriteResult]]
     ) -> None:
-        """``finish`` with an explicit id, safe when saves of several ids overlap."""
-        storage_data: dict[MetadataIndex, _StorageInfo] = {}
-        for idx, per_rank in enumerate(results):
-            if per_rank is None:
-                msg = (
-                    "finish: write results[%d] is None! This suggests an error in producing or gathering "
-                    "the write_results list from that local rank (%d)." % (idx, idx)
-                )
-                _LOGGER.error(msg)
-                raise RuntimeError(msg)
-            for wr in per_rank:
-                storage_data[wr.index] = wr.storage_data
-        metadata.storage_data = storage_data
-        metadata.storage_meta = self.storage_meta()
+        """``finish`` for an explicit id (saves of several ids may overlap): records where every item went, writes
+        the metadata object, then forgets the stored results of that id.  Nothing is forgotten on failure."""
+        where = {}
+        for position, rank_results in enumerate(results):
+            if rank_results is None:
+                complaint = _MISSING_RANK_RESULTS % (position, position)
+                _LOGGER.error(complaint)
+                raise RuntimeError(complaint)
+            where.update((result.index, result.storage_data) for result in rank_results)  # a repeated index: last wins
+        metadata.storage_data, metadata.storage_meta = where, self.storage_meta()
         self._checkpoint_saver.write_metadata(checkpoint_id, metadata)
-        self._write_results_per_checkpoint_id.pop(checkpoint_id, None)
-
-    @classmethod
-    @override
-    def validate_checkpoint_id(cls, checkpoint_id: Union[str, os.PathLike]) -> bool:
-        try:
-            CheckpointContainerId(checkpoint_id)
-            return True
-        except Exception as e:
-            _LOGGER.warning("Unable to validate checkpoint_id: %s, %s", checkpoint_id, e)
-            return False
+        if self._ledger.results is not None:
+            self._ledger.results.pop(checkpoint_id, None)

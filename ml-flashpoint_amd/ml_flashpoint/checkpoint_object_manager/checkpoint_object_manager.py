@@ -1,14 +1,18 @@
-"""Entry point for creating, opening, closing and deleting checkpoint buffers.
+"""Where checkpoint buffers come from and go to: create (``acquire_buffer``), open read-only (``get_buffer``), close,
+delete.  One instance per saver/loader; the buffer pool behind it is one per process.
 
-Follows the reference (src/ml_flashpoint/checkpoint_object_manager/checkpoint_object_manager.py:30-284):
-``acquire_buffer`` prefers the process-wide ``BufferPool`` and falls back to a standalone file; ``get_buffer``
-opens read-only and returns ``None`` on failure.
+Behaviour, names and messages are the reference's (src/ml_flashpoint/checkpoint_object_manager/
+checkpoint_object_manager.py:30-284).  What matters for the MI355X path: an acquired buffer is preferably a pooled one
+(a symlink to a file whose mapping and pages outlive the checkpoint, see ``core/buffer_pool.py``), and only if the
+pool has none left a file of its own, whose pages are then faulted in while the image arrives.
 """
+
+from __future__ import annotations
 
 import os
 import shutil
 import threading
-from typing import ClassVar, Optional
+from typing import ClassVar
 
 from ml_flashpoint.checkpoint_object_manager.buffer_io import BufferIO
 from ml_flashpoint.checkpoint_object_manager.buffer_metadata import METADATA_SIZE
@@ -21,49 +25,50 @@ _LOGGER = get_logger(__name__)
 
 
 class CheckpointObjectManager:
-    # one pool per process, shared by every manager instance in it
-    _worker_pool: ClassVar[Optional[BufferPool]] = None
+    # The pool belongs to the process, not to a manager: managers are pickled into worker processes (where the first
+    # acquire creates that process's pool from the configuration) and several of them may coexist.
+    _worker_pool: ClassVar[BufferPool | None] = None
     _worker_pool_lock: ClassVar[threading.Lock] = threading.Lock()
 
-    def __init__(self, pool_config: Optional[BufferPoolConfig] = None):
+    def __init__(self, pool_config: BufferPoolConfig | None = None):
         self._pool_config = pool_config
 
-    def _get_or_create_buffer_pool(self) -> Optional[BufferPool]:
-        cls = CheckpointObjectManager
-        if cls._worker_pool:
-            return cls._worker_pool
-        if not self._pool_config:
-            return None
-        with cls._worker_pool_lock:
-            if cls._worker_pool is None:
+    # ---- the process-wide pool ----------------------------------------------------------------------------------
+    def _get_or_create_buffer_pool(self) -> BufferPool | None:
+        """This process's pool; created on first use if this manager has a configuration.  None without one, and
+        None (with the failure logged) if creating it fails - callers then fall back to stand-alone files."""
+        owner = CheckpointObjectManager
+        if owner._worker_pool or not self._pool_config:
+            return owner._worker_pool or None
+        with owner._worker_pool_lock:
+            if owner._worker_pool is None:
                 try:
-                    cfg = self._pool_config
-                    cls._worker_pool = BufferPool(
-                        pool_dir_path=cfg.pool_dir_path,
-                        rank=cfg.rank,
-                        num_buffers=cfg.num_buffers,
-                        buffer_size=cfg.buffer_size,
-                    )
+                    wanted = self._pool_config
+                    owner._worker_pool = BufferPool(pool_dir_path=wanted.pool_dir_path, rank=wanted.rank,
+                                                    num_buffers=wanted.num_buffers, buffer_size=wanted.buffer_size)
                 except Exception:
                     _LOGGER.exception("Failed to initialize BufferPool")
-        return cls._worker_pool
+            return owner._worker_pool
 
     def teardown_pool(self):
-        cls = CheckpointObjectManager
-        with cls._worker_pool_lock:
-            pool, cls._worker_pool = cls._worker_pool, None
-        if pool:
-            try:
-                pool.teardown()
-            except Exception as e:
-                _LOGGER.debug("Failed to teardown BufferPool: %s", e)
+        owner = CheckpointObjectManager
+        with owner._worker_pool_lock:
+            pool, owner._worker_pool = owner._worker_pool, None
+        if pool is None:
+            return
+        try:
+            pool.teardown()
+        except Exception as e:
+            _LOGGER.debug("Failed to teardown BufferPool: %s", e)
 
+    # ---- buffers ------------------------------------------------------------------------------------------------
     def acquire_buffer(self, object_id: CheckpointObjectId, buffer_size: int, overwrite: bool = True) -> "BufferIO":
-        """Returns a writable stream for ``object_id`` with room for ``buffer_size`` data bytes (the metadata
-        block is added on top).  A pooled buffer may start smaller and grows while written."""
+        """A writable stream for a new object with room for ``buffer_size`` bytes of data (the 4096-byte metadata
+        block comes on top; a pooled buffer may be smaller and grows as it is written).  An existing object is
+        replaced, or ``FileExistsError`` with ``overwrite=False``; any other failure to create the buffer is a
+        ``RuntimeError`` that names the object."""
         if buffer_size <= 0:
             raise ValueError("Buffer size must be a positive integer.")
-        buffer_size += METADATA_SIZE
         path = str(object_id)
         try:
             os.makedirs(os.path.dirname(path), exist_ok=True)
@@ -74,45 +79,50 @@ class CheckpointObjectManager:
             pool = self._get_or_create_buffer_pool()
             if pool:
                 return pool.acquire(associated_symlink=path)
-        except RuntimeError:
+        except RuntimeError:  # every pooled buffer is taken
             _LOGGER.debug("BufferPool exhausted. Falling back to standalone buffer creation.")
         try:
-            return BufferIO(BufferObject(path, buffer_size, overwrite))
+            return BufferIO(BufferObject(path, METADATA_SIZE + buffer_size, overwrite))
         except Exception as e:
             _LOGGER.exception("Failed to create buffer for object_id='%s'", object_id)
             raise RuntimeError(f"Failed to create buffer for '{object_id}'") from e
 
-    def get_buffer(self, object_id: CheckpointObjectId) -> Optional["BufferIO"]:
+    def get_buffer(self, object_id: CheckpointObjectId) -> "BufferIO | None":
+        """A read-only stream over an existing object, or None if it cannot be opened as one (missing, a directory,
+        shorter than a metadata block, ...)."""
         try:
             return BufferIO(BufferObject(str(object_id)))
         except (OSError, ValueError, RuntimeError):
             _LOGGER.exception("Could not open buffer '%s'. Returning None.", object_id)
-            return None
+        return None
 
     def close_buffer(self, buffer_io: BufferIO, skip_close_if_symlink: bool = False, truncate: bool = True) -> None:
+        """Closes an open ``BufferIO`` (anything else is ignored with a warning).  ``skip_close_if_symlink`` leaves a
+        stream whose object is a symlink - a pooled buffer - open for its owner."""
         if not isinstance(buffer_io, BufferIO) or buffer_io.closed:
             _LOGGER.warning("Attempted to close an invalid or already-closed buffer. Ignoring.")
+        elif not (skip_close_if_symlink and os.path.islink(buffer_io.buffer_obj.get_id())):
+            buffer_io.close(truncate=truncate)
+
+    # ---- deletion -------------------------------------------------------------------------------------------------
+    def delete_object(self, object_id: CheckpointObjectId) -> None:
+        """Removes the object's file or symlink (a dangling symlink too); a missing one is only worth a warning."""
+        path = str(object_id)
+        if not os.path.lexists(path):
+            _LOGGER.warning("Object '%s' does not exist. Nothing to delete.", path)
             return
-        object_id = buffer_io.buffer_obj.get_id()
-        if skip_close_if_symlink and os.path.islink(object_id):
-            return
-        buffer_io.close(truncate=truncate)
+        os.remove(path)
 
     def delete_container(self, container_id: CheckpointContainerId) -> None:
+        """Removes a container directory with everything in it.  Files that vanish while it runs (another rank is
+        deleting the same tree) are passed over; a path that is not a directory is left alone."""
         path = str(container_id)
+        if not os.path.isdir(path):
+            _LOGGER.warning("Container '%s' is not a directory or does not exist. Nothing to delete from disk.", path)
+            return
 
-        def _ignore_missing(func, p, exc_info):
+        def unless_already_gone(function, failed_path, exc_info):
             if not isinstance(exc_info[1], FileNotFoundError):
                 raise exc_info[1]
 
-        if os.path.isdir(path):
-            shutil.rmtree(path, onerror=_ignore_missing)
-        else:
-            _LOGGER.warning("Container '%s' is not a directory or does not exist. Nothing to delete from disk.", path)
-
-    def delete_object(self, object_id: CheckpointObjectId) -> None:
-        path = str(object_id)
-        if os.path.lexists(path):
-            os.remove(path)
-        else:
-            _LOGGER.warning("Object '%s' does not exist. Nothing to delete.", path)
+        shutil.rmtree(path, onerror=unless_already_gone)

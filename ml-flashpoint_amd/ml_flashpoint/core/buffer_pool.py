@@ -1,59 +1,49 @@
-"""Per-rank pool of persistent, pre-allocated buffer files.
+"""A rank's pool of long-lived buffer files, and the stream type it hands out.
 
-A checkpoint object acquired through the pool is a *symlink* to one of ``num_buffers`` files named
-``buffer_<rank>_<idx>.dist``.  The mapping of a pool file stays open across checkpoints, so its pages stay
-resident: after the first save a buffer is written without page faults.  A buffer returns to the free list
-when its symlink no longer resolves.  Semantics follow the reference (src/ml_flashpoint/core/buffer_pool.py:35-342).
+Why a pool: a checkpoint object written into a fresh tmpfs file pays for page allocation (4-9 GB/s on the MI355X
+host, against 57 GB/s for the link), a file whose mapping stays open from save to save does not.  So the pool
+creates ``num_buffers`` files ``buffer_<rank>_<idx>.dist`` once, keeps them mapped, and a checkpoint object
+"acquired" from it is only a symlink to one of them.  Deleting the object (the symlink) is what gives the file
+back: the pool notices on its next ``acquire``.
+
+Behaviour, names and messages are the reference's (src/ml_flashpoint/core/buffer_pool.py:35-342); ``ensure_capacity``
+is an addition for writers that know the total size up front.
 """
 
+from __future__ import annotations
+
+import dataclasses
 import logging
 import os
 import threading
-from dataclasses import dataclass
-from typing import Dict, List, Optional
+from typing import NamedTuple
 
 from ml_flashpoint.checkpoint_object_manager.buffer_io import BufferIO
 from ml_flashpoint.checkpoint_object_manager.buffer_metadata import METADATA_SIZE
 from ml_flashpoint.checkpoint_object_manager.buffer_object.buffer_object_ext import BufferObject
+from ml_flashpoint.core import utils
 from ml_flashpoint.core.mlf_logging import get_logger
-from ml_flashpoint.core.utils import log_execution_time
 
 _LOGGER = get_logger(__name__)
 
-PADDING_SIZE = 1024 * 1024
+# growth rule of a pooled stream that runs out of room: at least 10 % more, and at least 1 MiB beyond what is needed
 RESIZE_FACTOR = 1.1
+PADDING_SIZE = 1 << 20
 
 
 class PooledBufferIO:
-    """Proxy handed to writers: ``close()`` releases the proxy but keeps the pool's mapping alive, and writes
-    grow the file on demand instead of failing."""
+    """A ``BufferIO`` on loan from the pool.  Everything not defined here goes straight to the underlying stream.
+    Two things differ: writing past the end grows the file instead of failing, and ``close`` ends the loan without
+    unmapping - it only cuts the file to what was written, so readers of the symlink see an object of exact size."""
 
     def __init__(self, buffer_io: BufferIO):
         self._buffer_io = buffer_io
         self._closed = False
 
-    def __getattr__(self, name):
+    def __getattr__(self, name):  # only reached for names this class does not define
         if self._closed:
             _LOGGER.warning("PooledBufferIO: Accessing closed buffer")
         return getattr(self._buffer_io, name)
-
-    @log_execution_time(logger=_LOGGER, name="close", level=logging.INFO)
-    def close(self, truncate: bool = True):
-        if self._closed:
-            return
-        self._closed = True
-        if not truncate or self._buffer_io.is_readonly:
-            return
-        try:
-            wanted = METADATA_SIZE + self._buffer_io._metadata.len_written_data
-            if wanted != len(self._buffer_io._mv):
-                self._buffer_io.resize(wanted)
-        except Exception:
-            _LOGGER.warning("PooledBufferIO: Failed to truncate buffer during close.", exc_info=True)
-
-    @property
-    def closed(self) -> bool:
-        return self._closed or self._buffer_io.closed
 
     def __enter__(self):
         return self
@@ -61,16 +51,36 @@ class PooledBufferIO:
     def __exit__(self, exc_type, exc_value, traceback):
         self.close()
 
+    @property
+    def closed(self) -> bool:
+        return self._closed or self._buffer_io.closed
+
+    @utils.log_execution_time(logger=_LOGGER, name="close", level=logging.INFO)
+    def close(self, truncate: bool = True):
+        already, self._closed = self._closed, True
+        if already or not truncate or self._buffer_io.is_readonly:
+            return
+        try:
+            exact = METADATA_SIZE + self._buffer_io._metadata.len_written_data
+            if len(self._buffer_io._mv) != exact:
+                self._buffer_io.resize(exact)
+        except Exception:
+            _LOGGER.warning("PooledBufferIO: Failed to truncate buffer during close.", exc_info=True)
+
+    # ---- growing ----------------------------------------------------------------------------------------------------
+    def _missing_room(self, more_bytes: int) -> bool:
+        stream = self._buffer_io
+        return METADATA_SIZE + stream.tell() + more_bytes > stream.buffer_obj.get_capacity()
+
     def _auto_resize(self, required_bytes: int):
-        """Grows the file so that ``required_bytes`` more fit at the current position: the larger of +10 % and
-        exact need + 1 MiB."""
-        capacity = self._buffer_io.buffer_obj.get_capacity()
-        needed = METADATA_SIZE + self._buffer_io.tell() + required_bytes
-        self._buffer_io.resize(int(max(capacity * RESIZE_FACTOR, needed + PADDING_SIZE)))
+        stream = self._buffer_io
+        by_factor = stream.buffer_obj.get_capacity() * RESIZE_FACTOR
+        by_need = METADATA_SIZE + stream.tell() + required_bytes + PADDING_SIZE
+        stream.resize(int(max(by_factor, by_need)))
 
     def ensure_capacity(self, required_bytes: int) -> None:
-        """Grows the file once, up front, when the total to be written from the current position is known."""
-        if METADATA_SIZE + self._buffer_io.tell() + required_bytes > self._buffer_io.buffer_obj.get_capacity():
+        """Makes room for ``required_bytes`` at the current position in one step (one remap instead of several)."""
+        if self._missing_room(required_bytes):
             self._auto_resize(required_bytes)
 
     def write(self, data: bytes) -> int:
@@ -82,8 +92,10 @@ class PooledBufferIO:
         return self._buffer_io.next_buffer_slice(size)
 
 
-@dataclass
+@dataclasses.dataclass
 class BufferPoolConfig:
+    """Picklable description of a pool; the pool itself is created lazily in the process that writes."""
+
     pool_dir_path: str
     rank: int
     num_buffers: int
@@ -92,10 +104,15 @@ class BufferPoolConfig:
     def __post_init__(self):
         if not self.pool_dir_path:
             raise ValueError("pool_dir_path must be provided in BufferPoolConfig")
-        for field in ("rank", "num_buffers", "buffer_size"):
-            value = getattr(self, field)
-            if not isinstance(value, int) or value < 0:
-                raise ValueError(f"{field} must be a non-negative integer in BufferPoolConfig")
+        for name in ("rank", "num_buffers", "buffer_size"):
+            given = getattr(self, name)
+            if not (isinstance(given, int) and given >= 0):
+                raise ValueError(f"{name} must be a non-negative integer in BufferPoolConfig")
+
+
+class _Loan(NamedTuple):
+    stream: BufferIO
+    symlink: str | None  # None while the borrower has not named its object yet: never reclaimed
 
 
 class BufferPool:
@@ -106,62 +123,63 @@ class BufferPool:
             raise ValueError(f"Buffer size must be positive. Got {buffer_size}.")
         if not pool_dir_path:
             raise ValueError("Pool directory path must be provided.")
-        self.pool_dir = pool_dir_path
-        self.rank = rank
-        self.num_buffers = num_buffers
-        self.buffer_size = buffer_size
-        self.free_buffers: List[BufferIO] = []
-        self.active_buffers: Dict[str, tuple[BufferIO, str]] = {}  # pool file path -> (stream, symlink path)
+        self.pool_dir, self.rank, self.num_buffers, self.buffer_size = pool_dir_path, rank, num_buffers, buffer_size
         self._lock = threading.Lock()
-        os.makedirs(self.pool_dir, exist_ok=True)
-        self._preallocate_buffers()
+        self.active_buffers: dict[str, _Loan] = {}  # pool file path -> who has it
+        os.makedirs(pool_dir_path, exist_ok=True)
+        self.free_buffers: list[BufferIO] = [self._create(index) for index in range(num_buffers)]
+
+    def _create(self, index: int) -> BufferIO:
+        path = os.path.join(self.pool_dir, f"buffer_{self.rank}_{index}.dist")
+        return BufferIO(BufferObject(path, self.buffer_size, overwrite=True))
 
     def _preallocate_buffers(self) -> None:
-        for idx in range(self.num_buffers):
-            path = os.path.join(self.pool_dir, f"buffer_{self.rank}_{idx}.dist")
-            self.free_buffers.append(BufferIO(BufferObject(path, self.buffer_size, overwrite=True)))
+        """(Re)creates the pool files; all of them must be free."""
+        self.free_buffers = [self._create(index) for index in range(self.num_buffers)]
 
-    @log_execution_time(logger=_LOGGER, name="acquire", level=logging.INFO)
-    def acquire(self, associated_symlink: Optional[str] = None) -> PooledBufferIO:
-        """Hands out a free pool buffer and links ``associated_symlink`` to it; raises RuntimeError when all
-        buffers are in use."""
+    @utils.log_execution_time(logger=_LOGGER, name="acquire", level=logging.INFO)
+    def acquire(self, associated_symlink: str | None = None) -> PooledBufferIO:
+        """Lends out a free buffer, rewound and empty, and creates ``associated_symlink`` pointing at its file.
+        ``RuntimeError`` when every buffer is on loan; if the link cannot be created the buffer stays free and the
+        ``OSError`` is the caller's."""
         with self._lock:
             self._gc()
             if not self.free_buffers:
                 raise RuntimeError(f"BufferPool exhausted. All {self.num_buffers} buffers are in use.")
-            candidate = self.free_buffers.pop()
+            stream = self.free_buffers.pop()
             try:
-                return PooledBufferIO(self._reuse_buffer(candidate, associated_symlink))
+                self._reuse_buffer(stream, associated_symlink)
             except Exception:
-                self.active_buffers.pop(candidate.buffer_obj.get_id(), None)
-                self.free_buffers.append(candidate)
+                self.active_buffers.pop(stream.buffer_obj.get_id(), None)
+                self.free_buffers.append(stream)
                 raise
+            return PooledBufferIO(stream)
 
-    def _gc(self) -> None:
-        """Frees buffers whose symlink is gone or dangling (``exists`` follows the link on purpose)."""
-        stale = [path for path, (_, link) in self.active_buffers.items() if link and not os.path.exists(link)]
-        for path in stale:
-            stream, _ = self.active_buffers.pop(path)
-            self.free_buffers.append(stream)
-
-    @log_execution_time(logger=_LOGGER, name="_reuse_buffer", level=logging.INFO)
-    def _reuse_buffer(self, buffer_io: BufferIO, symlink: Optional[str]) -> BufferIO:
+    @utils.log_execution_time(logger=_LOGGER, name="_reuse_buffer", level=logging.INFO)
+    def _reuse_buffer(self, buffer_io: BufferIO, symlink: str | None) -> BufferIO:
         buffer_io.seek(0)
         buffer_io._metadata.len_written_data = 0
-        path = buffer_io.buffer_obj.get_id()
-        self.active_buffers[path] = (buffer_io, symlink)
+        pool_file = buffer_io.buffer_obj.get_id()
+        self.active_buffers[pool_file] = _Loan(buffer_io, symlink)
         if symlink:
-            os.symlink(path, symlink)
+            os.symlink(pool_file, symlink)
         return buffer_io
 
+    def _gc(self) -> None:
+        """Takes back every buffer whose symlink no longer leads anywhere (``os.path.exists`` follows links, so a
+        deleted link and a dangling one count alike)."""
+        for pool_file, loan in list(self.active_buffers.items()):
+            if loan.symlink and not os.path.exists(loan.symlink):
+                del self.active_buffers[pool_file]
+                self.free_buffers.append(loan.stream)
+
     def teardown(self) -> None:
-        """Closes every mapping; the files stay on disk."""
+        """Unmaps everything, on loan or not; the files stay where they are."""
         with self._lock:
-            streams = list(self.free_buffers) + [s for s, _ in self.active_buffers.values()]
-            self.free_buffers.clear()
-            self.active_buffers.clear()
-            for stream in streams:
-                try:
-                    stream.close(truncate=True)
-                except Exception:
-                    _LOGGER.warning("PooledBufferIO: Failed to close buffer during teardown.", exc_info=True)
+            streams = self.free_buffers + [loan.stream for loan in self.active_buffers.values()]
+            self.free_buffers, self.active_buffers = [], {}
+        for stream in streams:
+            try:
+                stream.close(truncate=True)
+            except Exception:
+                _LOGGER.warning("PooledBufferIO: Failed to close buffer during teardown.", exc_info=True)

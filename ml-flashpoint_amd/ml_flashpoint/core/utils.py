@@ -67,6 +67,12 @@ def log_execution_time(logger: logging.Logger, name: str, level: int = logging.D
             logger.log(level, "%s took %.4fs", name, time.perf_counter() - start)
 
 
+def log_rate(logger: logging.Logger, verb: str, nbytes: int, seconds: float, count: int, what: str) -> None:
+    """One INFO line ``"<verb> N bytes in S s (R GB/s) from C <what>"`` for a finished transfer."""
+    if seconds > 0:
+        logger.info("%s %d bytes in %.4f s (%.2f GB/s) from %d %s", verb, nbytes, seconds, nbytes / 1e9 / seconds, count, what)
+
+
 _gc_pause_lock = threading.Lock()
 _gc_pause_depth = 0
 _gc_was_enabled = False
