@@ -75,11 +75,14 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         verify_crc: bool = True,
         use_file_io: bool = True,
         verify_on_discovery: bool = False,
+        max_image_bytes: Optional[int] = None,
     ):
         """Arguments as the reference's default loader (checkpoint_loader.py:126-158), plus the copy-engine and
         kernel work-split knobs, ``verify_crc`` (check the CRC-32C sidecar of an object, when it has one, while
         restoring it) and ``verify_on_discovery`` (also check it, on the host, while choosing the checkpoint to
-        recover from, so that a corrupted copy counts as missing)."""
+        recover from, so that a corrupted copy counts as missing) and ``max_image_bytes`` (largest range of an
+        object that is uploaded to HBM in one piece; default: what the device has free minus 2 GiB.  A larger
+        range is restored window by window through one buffer of that size)."""
         _lib.load()
         self._checkpoint_object_manager = checkpoint_object_manager
         self._replication_manager = replication_manager
@@ -96,6 +99,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         # reads of tmpfs run in parallel, and no page-table entry per 4 KiB has to be built and torn down
         self._use_file_io = use_file_io
         self.verify_on_discovery = verify_on_discovery
+        self._max_image_bytes = max_image_bytes
         self._engine: Optional[hip_plan.CopyEngine] = None
         self._engine_lock = threading.Lock()
         self._init_discovery()
@@ -214,6 +218,15 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         stats["read_s"] = time.perf_counter() - t_start
         self.last_load_stats = stats
 
+    def _image_limit(self, device: torch.device) -> int:
+        """Bytes of HBM one uploaded range may take: the explicit limit, or what the device and torch's allocator
+        have free minus a margin for the tables and for whatever else allocates while the restore runs."""
+        if self._max_image_bytes is not None:
+            return max(self._max_image_bytes, 1)
+        free, _ = torch.cuda.mem_get_info(device)
+        cached = torch.cuda.memory_reserved(device) - torch.cuda.memory_allocated(device)
+        return max(free + cached - (2 << 30), 64 << 20)
+
     def _read_device_items(self, object_id, stream, device_reqs, planner, stats) -> None:
         devices = {t.device for _, t, *_ in device_reqs}
         if len(devices) != 1:
@@ -221,12 +234,15 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         device = devices.pop()
         written = stream.len_written_data
         sidecar = integrity.read_sidecar(object_id.data) if self._verify_crc else None
+        if sidecar is not None and sidecar[1] != written:
+            raise integrity.ChecksumMismatchError(
+                f"'{object_id.data}': sidecar covers {sidecar[1]} bytes, object holds {written}")
 
-        # Every request becomes one table row whose image offset is, for now, absolute in the data section.  A request
-        # for a whole stored tensor into a contiguous target (the common case) is one run of bytes; anything else
-        # is described as a box over the stored C-contiguous payload (offsets/strides) and the target's strides.
-        table = hip_plan.ItemTable()
-        lo, hi = None, 0
+        # Every request becomes one row: where its bytes lie in the data section ([first, last), absolute for now)
+        # and how to add it to a descriptor table once the offset of the uploaded range is known.  A request for a
+        # whole stored tensor into a contiguous target (the common case) is one run of bytes; anything else is a box
+        # over the stored C-contiguous payload (offsets/strides) with the target's strides on the other side.
+        rows = []  # (first, last, contiguous?, table arguments)
         for req, target, dtype, shape, payload_off, stored_bytes in device_reqs:
             if target.dtype != dtype:
                 raise TypeError(f"req {req.storage_index}: stored dtype {dtype} differs from target dtype {target.dtype}")
@@ -243,9 +259,9 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                     continue
                 first, last = payload_off, payload_off + stored_bytes
                 if target.is_contiguous():
-                    table.add_contiguous(target.data_ptr(), first, esz, stored_bytes)
+                    rows.append((first, last, True, (target.data_ptr(), esz)))
                 elif ndim <= _lib.MAX_DIMS:
-                    table.add_device(target.data_ptr(), first, esz, tuple(shape), tuple(target.stride()))
+                    rows.append((first, last, False, (target.data_ptr(), esz, tuple(shape), tuple(target.stride()), None)))
                 else:
                     raise NotImplementedError(f"rank > {_lib.MAX_DIMS} targets must be contiguous")
             else:
@@ -263,59 +279,140 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                     raise NotImplementedError(f"sub-box reads of rank > {_lib.MAX_DIMS} tensors are not supported")
                 first = payload_off + sum(o * st for o, st in zip(offsets, stored_strides)) * esz
                 last = first + (sum((l - 1) * st for l, st in zip(lengths, stored_strides)) + 1) * esz
-                table.add_device(target.data_ptr(), first, esz, tuple(lengths), tuple(target.stride()),
-                                 image_stride=tuple(stored_strides))
+                rows.append((first, last, False,
+                             (target.data_ptr(), esz, tuple(lengths), tuple(target.stride()), tuple(stored_strides))))
                 stored_bytes = numel * esz
             stats["device_payload_bytes"] += stored_bytes
-            lo = first if lo is None else min(lo, first)
-            hi = max(hi, last)
-        if lo is None:
-            for req, target, *_ in device_reqs:
-                planner.commit_tensor(req, target)
-            return
-        if sidecar is not None:
-            lo, hi = 0, written  # checksums cover the whole data section
-        lo = lo // _UPLOAD_ALIGN * _UPLOAD_ALIGN
-        span = hi - lo
-        items = table.to_array()
-        items["image_off"] -= lo  # offsets relative to the uploaded range
-        with torch.cuda.device(device):
-            _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
-            image = torch.empty(span, dtype=torch.uint8, device=device)
-            cur = torch.cuda.current_stream(device)
-            fd = stream.fileno() if self._use_file_io else -1
-            if fd >= 0:
-                st = self._get_engine().h2d_fd(fd, METADATA_SIZE + lo, image.data_ptr(), span, cur.cuda_stream)
-            else:
-                st = self._get_engine().h2d(stream.data_address(lo), image.data_ptr(), span, cur.cuda_stream)
-            stats["h2d_s"] += st.seconds
-            stats["h2d_bytes"] += span
+        if rows:
+            lo = min(r[0] for r in rows)
+            hi = max(r[1] for r in rows)
             if sidecar is not None:
-                chunk_bytes, data_bytes, want = sidecar
-                if data_bytes != written:
-                    raise integrity.ChecksumMismatchError(
-                        f"'{object_id.data}': sidecar covers {data_bytes} bytes, object holds {written}")
-                got = hip_plan.crc32c_device(image, written, chunk_bytes, cur.cuda_stream)
-                bad = [int(i) for i in (got != want).nonzero()[0]]
-                if bad:
-                    raise integrity.ChecksumMismatchError(
-                        f"'{object_id.data}': CRC-32C mismatch in chunk(s) {bad[:8]} of {len(want)} "
-                        f"(chunk size {chunk_bytes})")
-            plan = hip_plan.Plan(items, b"", span, tile_bytes=self._tile_bytes,
-                                 block_threads=self._block_threads, align_to_tensor=True)
+                lo, hi = 0, written  # checksums cover the whole data section
+            lo = lo // _UPLOAD_ALIGN * _UPLOAD_ALIGN
+            with torch.cuda.device(device):
+                _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
+                limit = self._image_limit(device)
+                if hi - lo <= limit:
+                    self._restore_range(object_id, stream, device, rows, lo, hi, sidecar, stats)
+                else:
+                    self._restore_windowed(object_id, stream, device, rows, limit, sidecar, stats)
+        for req, target, *_ in device_reqs:
+            planner.commit_tensor(req, target)
+        stats["device_items"] += len(device_reqs)
+
+    @staticmethod
+    def _table_of(rows, lo: int):
+        """Descriptor table of ``rows`` for a buffer that holds the data section from byte ``lo`` on."""
+        table = hip_plan.ItemTable()
+        for first, last, contiguous, args in rows:
+            if contiguous:
+                ptr, esz = args
+                table.add_contiguous(ptr, first - lo, esz, last - first)
+            else:
+                ptr, esz, shape, strides, image_strides = args
+                table.add_device(ptr, first - lo, esz, shape, strides, image_stride=image_strides)
+        return table.to_array()
+
+    def _upload(self, stream, lo: int, image: torch.Tensor, span: int, cur, stats) -> None:
+        fd = stream.fileno() if self._use_file_io else -1
+        if fd >= 0:
+            st = self._get_engine().h2d_fd(fd, METADATA_SIZE + lo, image.data_ptr(), span, cur.cuda_stream)
+        else:
+            st = self._get_engine().h2d(stream.data_address(lo), image.data_ptr(), span, cur.cuda_stream)
+        stats["h2d_s"] += st.seconds
+        stats["h2d_bytes"] += span
+
+    def _unpack(self, items, image: torch.Tensor, span: int, cur, payload_bytes: int) -> None:
+        """Launches the unpack of ``items`` out of ``image`` and waits for it: the targets are complete, and the
+        image may be reused or freed, when this returns."""
+        plan = hip_plan.Plan(items, b"", span, tile_bytes=self._tile_bytes, block_threads=self._block_threads,
+                             align_to_tensor=True)
+        try:
             if self.record_kernel_events:
                 begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 begin.record(cur)
                 plan.unpack(image, cur.cuda_stream)
                 end.record(cur)
-                self.kernel_events.append((begin, end, stats["device_payload_bytes"]))
+                self.kernel_events.append((begin, end, payload_bytes))
             else:
                 plan.unpack(image, cur.cuda_stream)
-            cur.synchronize()  # targets are complete (and the image may be freed) when read_data returns
+            cur.synchronize()
+        finally:
             plan.destroy()
-        for req, target, *_ in device_reqs:
-            planner.commit_tensor(req, target)
-        stats["device_items"] += len(device_reqs)
+
+    def _restore_range(self, object_id, stream, device, rows, lo, hi, sidecar, stats) -> None:
+        """One upload of [lo, hi), checksum on the GPU if the object has a sidecar, one unpack."""
+        span = hi - lo
+        image = torch.empty(span, dtype=torch.uint8, device=device)
+        cur = torch.cuda.current_stream(device)
+        self._upload(stream, lo, image, span, cur, stats)
+        if sidecar is not None:
+            chunk_bytes, data_bytes, want = sidecar
+            got = hip_plan.crc32c_device(image, data_bytes, chunk_bytes, cur.cuda_stream)
+            self._compare_checksums(object_id, got, want, chunk_bytes)
+        self._unpack(self._table_of(rows, lo), image, span, cur, stats["device_payload_bytes"])
+
+    @staticmethod
+    def _compare_checksums(object_id, got, want, chunk_bytes) -> None:
+        bad = [int(i) for i in (got != want).nonzero()[0]]
+        if bad:
+            raise integrity.ChecksumMismatchError(
+                f"'{object_id.data}': CRC-32C mismatch in chunk(s) {bad[:8]} of {len(want)} "
+                f"(chunk size {chunk_bytes})")
+
+    def _restore_windowed(self, object_id, stream, device, rows, limit, sidecar, stats) -> None:
+        """Fallback for an object whose requested range does not fit in HBM beside the live state: the rows are
+        sorted by position and restored window by window through one device buffer of at most ``limit`` bytes.  A
+        contiguous row larger than a window is cut into pieces; a strided one cannot be.  With a sidecar the whole
+        object is checked first, on the host (the windows do not coincide with the checksum chunks)."""
+        _LOGGER.warning("requested range of '%s' exceeds the HBM limit of %d bytes; restoring window by window",
+                        object_id, limit)
+        if sidecar is not None:
+            chunk_bytes, data_bytes, want = sidecar
+            fd = stream.fileno()
+            own_fd = fd < 0
+            if own_fd:
+                fd = os.open(object_id.data, os.O_RDONLY)
+            try:
+                got = hip_plan.crc32c_file(fd, METADATA_SIZE, data_bytes, chunk_bytes,
+                                           self._engine_config.resolved_copy_threads())
+            finally:
+                if own_fd:
+                    os.close(fd)
+            self._compare_checksums(object_id, got, want, chunk_bytes)
+        usable = limit - _UPLOAD_ALIGN  # a window starts on an upload boundary at or below its first row
+        piece = usable // 65536 * 65536  # a multiple of every element size
+        if piece <= 0:
+            raise ValueError(f"max_image_bytes={limit} is too small to restore anything")
+        pieces = []
+        for first, last, contiguous, args in sorted(rows, key=lambda r: r[0]):
+            if last - first <= usable:
+                pieces.append((first, last, contiguous, args))
+            elif contiguous:
+                ptr, esz = args
+                for begin in range(first, last, piece):
+                    pieces.append((begin, min(begin + piece, last), True, (ptr + (begin - first), esz)))
+            else:
+                raise NotImplementedError(
+                    f"'{object_id.data}': a strided or partial read spanning {last - first} bytes does not fit the "
+                    f"HBM limit of {limit} bytes")
+        windows, current, lo = [], [], 0
+        for row in pieces:
+            if current and row[1] - lo > limit:
+                windows.append((lo, current))
+                current = []
+            if not current:
+                lo = row[0] // _UPLOAD_ALIGN * _UPLOAD_ALIGN
+            current.append(row)
+        windows.append((lo, current))
+        cur = torch.cuda.current_stream(device)
+        image = torch.empty(max(max(r[1] for r in rs) - lo for lo, rs in windows), dtype=torch.uint8, device=device)
+        for lo, window_rows in windows:
+            span = max(r[1] for r in window_rows) - lo
+            self._upload(stream, lo, image, span, cur, stats)
+            self._unpack(self._table_of(window_rows, lo), image, span, cur,
+                         sum(r[1] - r[0] for r in window_rows if r[2]))
+        stats["windows"] = stats.get("windows", 0) + len(windows)
 
     # ---- discovery (core/checkpoint_discovery.py) ----------------------------------------------------------
     def _object_is_intact(self, path: str) -> bool:

@@ -405,6 +405,66 @@ def test_object_larger_than_the_hbm_limit_is_saved_window_by_window(shm_dir, man
     assert raw == image and got_spans == spans
 
 
+@pytest.mark.parametrize("load_file_io", [True, False])
+def test_restore_larger_than_the_hbm_limit_goes_window_by_window(shm_dir, manager_future, load_file_io):
+    """With ``max_image_bytes`` far below the object size the loader uploads and unpacks windows of rows through
+    one small device buffer (contiguous rows larger than a window are cut); the restored bits are the same, the
+    CRC sidecar is still honoured (on the host), and a strided read that cannot be cut says so."""
+    from ml_flashpoint.hip import integrity
+
+    sd_cpu = dict(_mixed_state_dict())
+    sd_cpu["big"] = torch.arange(200_000, dtype=torch.float32)          # 800 kB: several windows of its own
+    sd_cpu["wide"] = torch.arange(512 * 300, dtype=torch.int32).reshape(512, 300)
+    sd_dev = _to_dev(sd_cpu, keep_on_host=("w.i64",))
+    ckpt = os.path.join(shm_dir, "step-9_ckpt")
+    dcp.save(sd_dev, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(_saver(crc_chunk_bytes=1 << 16), manager_future),
+             no_dist=True)
+
+    def targets(transposed_wide=False):
+        out = {}
+        for k, v in sd_dev.items():
+            if not isinstance(v, torch.Tensor):
+                out[k] = None
+            elif v.dtype == torch.float8_e4m3fn:
+                out[k] = torch.zeros(v.shape, dtype=torch.uint8, device=v.device).view(torch.float8_e4m3fn)
+            else:
+                out[k] = torch.zeros(v.shape, dtype=v.dtype, device=v.device)
+        if transposed_wide:  # a strided target: its row cannot be cut into windows
+            out["wide"] = torch.zeros(300, 512, dtype=torch.int32, device=DEV).t()
+        return out
+
+    loader = _loader(max_image_bytes=256 << 10, use_file_io=load_file_io)
+    target = targets()
+    dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), no_dist=True)
+    assert loader.last_load_stats["windows"] >= 5
+    assert target["obj.step"] == 123
+    for k, v in sd_cpu.items():
+        if isinstance(v, torch.Tensor):
+            assert torch.equal(_bits(target[k]), _bits(v)), k
+
+    # a strided target small enough for one window is fine ...
+    target = targets(transposed_wide=True)
+    roomy = _loader(max_image_bytes=700 << 10, use_file_io=load_file_io)
+    dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, roomy), no_dist=True)
+    assert roomy.last_load_stats["windows"] >= 2 and torch.equal(target["wide"].cpu(), sd_cpu["wide"])
+    # ... one that is larger than a window is refused, not mangled
+    with pytest.raises(BaseException) as exc:
+        dcp.load(targets(transposed_wide=True), checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), no_dist=True)
+    cause = exc.value.failures[0][0] if hasattr(exc.value, "failures") else exc.value
+    assert isinstance(cause, NotImplementedError) and "does not fit the HBM limit" in str(cause)
+
+    obj = os.path.join(ckpt, "__0__0_src0.distcp")
+    with open(obj, "r+b") as f:  # one flipped bit: found by the host-side check before any window is uploaded
+        f.seek(METADATA_SIZE + 5 * (1 << 16) + 77)
+        byte = f.read(1)
+        f.seek(-1, os.SEEK_CUR)
+        f.write(bytes([byte[0] ^ 0x01]))
+    with pytest.raises(BaseException) as exc:
+        dcp.load(targets(), checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), no_dist=True)
+    cause = exc.value.failures[0][0] if hasattr(exc.value, "failures") else exc.value
+    assert isinstance(cause, integrity.ChecksumMismatchError) and "chunk(s) [5]" in str(cause)
+
+
 def test_legacy_torch_save_objects_are_still_readable(shm_dir):
     """An object whose signature is TORCH___ holds torch.save records; the loader reads it on the host."""
     from ml_flashpoint.core.defaults import CheckpointFormat
