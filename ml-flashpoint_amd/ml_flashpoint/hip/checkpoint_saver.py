@@ -454,8 +454,13 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                     plan.destroy()
                     xfer["d2h_s"] += st.seconds
                     xfer["d2h_bytes"] += end - begin
-        if self._crc_chunk_bytes:
-            _LOGGER.warning("no CRC sidecar is written for '%s': it was saved window by window", object_id)
+            fd = writer.fileno() if self._crc_chunk_bytes and nbytes else -1
+            if fd >= 0:
+                # windows end where records end, not where checksum chunks end, so the checksums of this (already
+                # blocking) mode are taken on the host, from the pages that were just written
+                crcs = hip_plan.crc32c_file(fd, METADATA_SIZE + start, nbytes, self._crc_chunk_bytes,
+                                            self._engine_config.resolved_copy_threads())
+                integrity.write_sidecar(str(object_id), self._crc_chunk_bytes, nbytes, crcs)
         stats["objects"] += 1
         stats["windows"] = stats.get("windows", 0) + len(windows)
         stats["device_payload_bytes"] += layout.device_payload_bytes

@@ -396,13 +396,27 @@ def test_object_larger_than_the_hbm_limit_is_saved_window_by_window(shm_dir, man
     sd_cpu["big"] = torch.arange(200_000, dtype=torch.float32)  # one record larger than the limit
     sd_dev = _to_dev(sd_cpu, keep_on_host=("w.i64",))
     ckpt = os.path.join(shm_dir, "step-8_ckpt")
-    saver = _saver(max_image_bytes=64 << 10)
+    saver = _saver(max_image_bytes=64 << 10, crc_chunk_bytes=1 << 16)
     dcp.save(sd_dev, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(saver, manager_future), no_dist=True)
     assert saver.last_save_stats["windows"] >= 4
     raw = open(os.path.join(ckpt, "__0__0_src0.distcp"), "rb").read()
     metadata = pickle.load(open(os.path.join(ckpt, ".metadata"), "rb"))
     image, spans, got_spans = _expected_file(sd_cpu, metadata, raw)
     assert raw == image and got_spans == spans
+    # the sidecar of a windowed save comes from the host routine; the GPU check of an ordinary restore accepts it
+    from ml_flashpoint.hip import integrity
+
+    chunk, nbytes, crcs = integrity.read_sidecar(os.path.join(ckpt, "__0__0_src0.distcp"))
+    assert chunk == 1 << 16 and nbytes == len(raw) - METADATA_SIZE and len(crcs) == -(-nbytes // chunk)
+    target = {k: (torch.zeros_like(v) if isinstance(v, torch.Tensor) and v.dtype != torch.float8_e4m3fn else
+                  (torch.zeros(v.shape, dtype=torch.uint8, device=v.device).view(v.dtype) if isinstance(v, torch.Tensor) else None))
+              for k, v in sd_dev.items()}
+    loader = _loader()
+    dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), no_dist=True)
+    assert "windows" not in loader.last_load_stats
+    for k, v in sd_cpu.items():
+        if isinstance(v, torch.Tensor):
+            assert torch.equal(_bits(target[k]), _bits(v)), k
 
 
 @pytest.mark.parametrize("load_file_io", [True, False])
