@@ -233,7 +233,23 @@ class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
 
         staged = [dataclasses.replace(bucket, tensor_data=on_host(bucket.tensor_data)) for bucket in write_buckets]
         if non_blocking and torch.cuda.is_available():
-            torch.cuda.synchronize()
+            # Placeholders know the event behind their pack; waiting for those is enough and, unlike a device-wide
+            # synchronize, does not also wait for an earlier checkpoint that is still crossing the host link.
+            waits = {}
+            for bucket in write_buckets:
+                for _, entry in bucket.tensor_data:
+                    wait = getattr(entry, "wait_until_packed", None)
+                    if wait is None:
+                        waits = None
+                        break
+                    waits[id(getattr(entry, "staged", entry))] = wait
+                if waits is None:
+                    break
+            if waits is None:
+                torch.cuda.synchronize()
+            else:
+                for wait in waits.values():
+                    wait()
         return staged
 
     @_timed(logger=_LOGGER, name="write_staged_write_buckets", level=logging.INFO)

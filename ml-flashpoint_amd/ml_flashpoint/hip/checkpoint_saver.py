@@ -95,6 +95,7 @@ class StagedObject:
         self.future: Optional[concurrent.futures.Future] = None
         self.done_marker: Optional[str] = None
         self.collected = False
+        self.packed_event: Optional[torch.cuda.Event] = None  # recorded behind the pack on the producer's stream
 
     def __reduce__(self):
         if self.future is None or self.done_marker is None:
@@ -155,6 +156,14 @@ class StagedTensorRef:
 
     def detach(self):
         return self
+
+    def wait_until_packed(self) -> None:
+        """Returns once the pack that read this tensor has finished, i.e. once the live tensor may be overwritten.
+        Staging code that finds this method on every entry can call it instead of synchronizing the whole device,
+        which would also wait for an earlier checkpoint that is still crossing the host link."""
+        event = getattr(self.staged, "packed_event", None)
+        if event is not None:
+            event.synchronize()
 
     def numel(self) -> int:
         return self.shape.numel()
@@ -387,7 +396,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         if device is None:
             device = torch.device("cuda", torch.cuda.current_device())
         items = [item for item, _ in tensor_data] + [item for item, _ in bytes_data]
-        plan = image = None
+        plan = image = packed = None
         stream = 0
         if layout.image_bytes and object_id is not None and layout.image_bytes > self._image_limit(device):
             return self._stage_windowed(layout, items, object_id, object_name, device, stats)
@@ -400,17 +409,21 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                 stream = torch.cuda.current_stream(device).cuda_stream
                 stats["plan_build_s"] += time.perf_counter() - t0
                 if self.record_kernel_events:
-                    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    begin, packed = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                     begin.record()
                     plan.pack(image, stream)
-                    end.record()
-                    self.kernel_events.append((begin, end, layout.device_payload_bytes))
+                    packed.record()
+                    self.kernel_events.append((begin, packed, layout.device_payload_bytes))
                 else:
                     plan.pack(image, stream)
+                    packed = torch.cuda.Event()
+                    packed.record()
         stats["objects"] += 1
         stats["device_payload_bytes"] += layout.device_payload_bytes
         stats["image_bytes"] += layout.image_bytes
-        return StagedObject(layout, plan, image, device.index or 0, stream, items)
+        staged = StagedObject(layout, plan, image, device.index or 0, stream, items)
+        staged.packed_event = packed if layout.image_bytes else None
+        return staged
 
     def _stage_windowed(self, layout, items, object_id, object_name, device, stats: dict) -> StagedObject:
         """Fallback for an object whose image does not fit in HBM beside the live state: consecutive records are

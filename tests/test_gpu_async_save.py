@@ -137,3 +137,43 @@ def test_failure_in_the_background_write_reaches_the_waiter(shm_dir, manager_fut
         saver.write_data(cid, remote, replicate_after_write=False)
     with pytest.raises(RuntimeError, match="injected"):
         saver.write_data(cid, buckets, replicate_after_write=False)
+
+
+def test_next_save_does_not_wait_for_the_previous_transfer(shm_dir, manager_future):
+    """The blocking part of a save ends when *its* pack has finished: staging waits for the event behind that pack,
+    not for the whole device, so a checkpoint that is still crossing the host link does not hold up the next one."""
+    saver = _make_saver(background_write=True)
+    dist = _DistWrapper(None, False, 0)
+    big = {f"big.{i}": torch.full((1 << 28,), float(i), device=DEV) for i in range(6)}  # 6 GiB: >= 0.1 s on the link
+    small = _state_dict()
+
+    def begin(step, sd):
+        cid = CheckpointContainerId(os.path.join(shm_dir, f"step-{step}_ckpt"))
+        saver.initialize_checkpoint(cid)
+        writer = MemoryStorageWriter(saver, manager_future)
+        writer.reset(cid.data)
+        buckets, metadata, *_ = statedictsaver.generate_plan(cid, sd, writer, DefaultSavePlanner(), dist)
+        staged = MemoryStorageWriter.stage_write_data_buckets(cid, buckets, non_blocking=True)
+        return cid, writer, metadata, staged
+
+    first = begin(10, big)
+    first_transfer = saver._staged_of(first[3][0]).future
+    t0 = time.perf_counter()
+    second = begin(11, small)
+    blocked_s = time.perf_counter() - t0
+    assert not first_transfer.done(), "the second save's blocking part outlasted the first save's transfer"
+    assert blocked_s < 0.1
+    snapshot = {k: v.cpu() for k, v in small.items()}
+    for v in small.values():
+        v.add_(1.0)
+    def complete(cid, writer, metadata, staged):
+        statedictsaver.write_data(cid, writer, staged, replicate_after_write=False)
+        statedictsaver.finish_write(cid, writer, metadata, dist)
+        saver.finalize_checkpoint(cid)
+
+    complete(*first)
+    with open(os.path.join(first[0].data, "__0__0_src0.distcp"), "rb") as raw:
+        raw.seek(-(1 << 20), os.SEEK_END)
+        assert raw.read() == torch.full((1 << 18,), 5.0).numpy().tobytes()  # the tail of the last big tensor
+    complete(*second)  # finalizing the newer checkpoint removes the older one in the background
+    _check_files(second[0], snapshot)
