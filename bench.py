@@ -167,8 +167,19 @@ def cpu_baseline(sd, sample_bytes, root, device):
         "blocking_stage_ms": round(stage * 1e3, 1),
         "write_GBps": round(gb / write, 3),
         "host_cpus": os.cpu_count(),
+        "usable_cpus": len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else None,
+        "numa_nodes_online": _read_text("/sys/devices/system/node/online"),
+        "tmpfs_root": root,
         "restored_ok": bool(ok),
     }
+
+
+def _read_text(path):
+    try:
+        with open(path) as f:
+            return f.read().strip()
+    except OSError:
+        return None
 
 
 def _rewrite_warm(path, tensors):
