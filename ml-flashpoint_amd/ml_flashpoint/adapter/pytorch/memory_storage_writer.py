@@ -60,6 +60,21 @@ class _StorageDataContext:
     prefix: str
 
 
+def _pack_waits(write_buckets: list[ObjectWriteBucket]):
+    """One ``wait_until_packed`` callable per packed image if every tensor entry of every bucket is a placeholder
+    that has one, else None.  Waiting for the events behind the packs is enough to know that the live tensors may be
+    overwritten, and unlike a device-wide synchronize it does not also wait for an earlier checkpoint that is
+    still crossing the host link."""
+    per_image = {}
+    for bucket in write_buckets:
+        for _, entry in bucket.tensor_data:
+            wait = getattr(entry, "wait_until_packed", None)
+            if wait is None:
+                return None
+            per_image.setdefault(id(getattr(entry, "staged", entry)), wait)
+    return list(per_image.values())
+
+
 class _WriteLedger:
     """Completion events and write results per checkpoint id, shared between the process that prepares a save and
     the one that writes it.  Empty until ``open`` is given a manager; a ledger that travelled to another process
@@ -233,22 +248,11 @@ class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
 
         staged = [dataclasses.replace(bucket, tensor_data=on_host(bucket.tensor_data)) for bucket in write_buckets]
         if non_blocking and torch.cuda.is_available():
-            # Placeholders know the event behind their pack; waiting for those is enough and, unlike a device-wide
-            # synchronize, does not also wait for an earlier checkpoint that is still crossing the host link.
-            waits = {}
-            for bucket in write_buckets:
-                for _, entry in bucket.tensor_data:
-                    wait = getattr(entry, "wait_until_packed", None)
-                    if wait is None:
-                        waits = None
-                        break
-                    waits[id(getattr(entry, "staged", entry))] = wait
-                if waits is None:
-                    break
+            waits = _pack_waits(write_buckets)
             if waits is None:
                 torch.cuda.synchronize()
             else:
-                for wait in waits.values():
+                for wait in waits:
                     wait()
         return staged
 

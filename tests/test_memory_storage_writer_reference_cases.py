@@ -215,6 +215,36 @@ def test_stage_write_data_buckets_is_static_and_keeps_host_tensors():
         sync.assert_called_once()
 
 
+def test_stage_waits_for_the_packs_of_placeholders_instead_of_the_device():
+    """Entries that stand for an image already being packed offer ``wait_until_packed``; when all of them do, those
+    waits (one per image) replace the device-wide synchronize.  (Not in the reference: its entries are tensors.)"""
+
+    class Placeholder:
+        def __init__(self, staged):
+            self.staged = staged
+
+        def to(self, **kwargs):
+            return self
+
+        def wait_until_packed(self):
+            self.staged.append("waited")
+
+    cid = CheckpointContainerId("/test_checkpoint")
+    image_a, image_b = [], []
+    buckets = _buckets(cid, count=2)
+    buckets[0].tensor_data = [(buckets[0].tensor_data[0][0], Placeholder(image_a)), (mock.MagicMock(), Placeholder(image_a))]
+    buckets[1].tensor_data = [(buckets[1].tensor_data[0][0], Placeholder(image_b))]
+    with mock.patch("torch.cuda.is_available", return_value=True), mock.patch("torch.cuda.synchronize") as sync:
+        staged = MemoryStorageWriter.stage_write_data_buckets(cid, buckets, non_blocking=True)
+        sync.assert_not_called()
+        assert image_a == ["waited"] and image_b == ["waited"]          # once per image, not once per entry
+        assert staged[0].tensor_data[0][1] is buckets[0].tensor_data[0][1]
+        buckets[1].tensor_data.append((mock.MagicMock(), torch.tensor([1])))  # one real tensor among them
+        MemoryStorageWriter.stage_write_data_buckets(cid, buckets, non_blocking=True)
+        sync.assert_called_once()
+        assert image_a == ["waited"] and image_b == ["waited"]
+
+
 # ---- write_staged_data_buckets / write_data (:615-888) --------------------------------------------------------------------
 @pytest.mark.parametrize("thread_count", [1, 4, 8])
 def test_write_staged_data_buckets(saver, mp_manager_future, thread_count):
