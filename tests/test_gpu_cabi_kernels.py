@@ -276,6 +276,54 @@ def test_strided_views_with_long_rows(dtype):
         assert torch.equal(got_b[mask], want_b[mask]) and int(got_b[~mask].count_nonzero()) == 0
 
 
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.bfloat16, torch.float32, torch.complex128])
+def test_views_of_the_maximum_rank_and_the_rank_limit(dtype):
+    """Eight dimensions is what a descriptor holds.  Views of that rank whose dimensions cannot be merged (reversed
+    order, every other element along several axes) pack and unpack like any other; one more dimension is fine as
+    long as the tensor is contiguous (it is a run of bytes) and refused otherwise."""
+    from ml_flashpoint.hip import plan as P
+
+    gen = torch.Generator().manual_seed(88)
+    shape = (3, 2, 4, 2, 3, 2, 2, 5)
+    base_cpu = _rand_tensor(gen, shape, dtype)
+    base_dev = base_cpu.to(DEV)
+
+    def views(t):
+        return [
+            t.permute(7, 6, 5, 4, 3, 2, 1, 0),                       # nothing merges
+            t[:, :, ::2, :, ::2, :, :, 1::3],                        # steps along three axes
+            t.permute(0, 2, 1, 4, 3, 6, 5, 7)[1:, 1:, :, :2],        # pairs swapped, then narrowed
+            t[2, 1],                                                 # a contiguous 6-d piece in the middle
+        ]
+
+    cpu, dev = views(base_cpu), views(base_dev)
+    assert all(v.dim() == 8 for v in cpu[:3]) and not any(v.is_contiguous() for v in cpu[:3])
+    layout, plan, image, got = _pack_image(dev)
+    assert got == oracle_fmt.data_section(cpu)[0]
+    assert got == b"".join(oracle_fmt.header_bytes(oracle_fmt.dtype_name(t.dtype), tuple(t.shape)) +
+                           oracle_fmt.payload_bytes_bruteforce(t) for t in cpu)
+    # unpack the same image into the same views of a zeroed parent: covered elements come back, the rest stays zero
+    zero_dev = torch.zeros_like(base_dev)
+    esz = base_cpu.element_size()
+    table = P.ItemTable()
+    for src, tgt, (off, length) in zip(cpu, views(zero_dev), layout.spans):
+        table.add_device(tgt.data_ptr(), off + length - src.numel() * esz, esz, tuple(src.shape), tuple(tgt.stride()))
+    P.Plan(table.to_array(), b"", layout.image_bytes, align_to_tensor=True).unpack(image)
+    torch.cuda.synchronize()
+    mask = torch.zeros(shape, dtype=torch.bool)
+    for m in views(mask):
+        m.fill_(True)
+    got_b = zero_dev.cpu().reshape(-1).view(torch.uint8).reshape(*shape, esz)
+    ref_b = base_cpu.reshape(-1).view(torch.uint8).reshape(*shape, esz)
+    assert torch.equal(got_b[mask], ref_b[mask]) and int(got_b[~mask].count_nonzero()) == 0
+
+    nine_cpu = _rand_tensor(gen, (2, 2, 2, 2, 2, 2, 2, 2, 3), dtype)
+    nine_dev = nine_cpu.to(DEV)
+    assert _pack_image([nine_dev])[3] == oracle_fmt.data_section([nine_cpu])[0]
+    with pytest.raises(NotImplementedError, match="rank > 8"):
+        P.build_save_layout([nine_dev.transpose(0, 8)])
+
+
 def test_pack_large_rows_go_through_flat_kernel():
     gen = torch.Generator().manual_seed(15)
     base_cpu = _rand_tensor(gen, (64, 8192), torch.bfloat16)
