@@ -189,6 +189,10 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         t_start = time.perf_counter()
         stats = {"h2d_s": 0.0, "h2d_bytes": 0, "device_payload_bytes": 0, "host_items": 0, "device_items": 0}
         with gc_paused(), self._checkpoint_object_manager.get_buffer(checkpoint_object_id) as stream:
+            recorded, held = stream.len_written_data, stream.buffer_obj.get_capacity() - METADATA_SIZE
+            if recorded > held:  # cut short after it was written: never read past the end of the file or its mapping
+                raise ValueError(f"'{checkpoint_object_id.data}' is truncated: its metadata block records {recorded} "
+                                 f"bytes of data, the file holds {held}")
             optimized = stream.format_signature == CheckpointFormat.MLF_FORMAT
             device_reqs = []  # (req, target, dtype, shape, payload_off, stored payload bytes)
             whole = stream.raw_view()

@@ -479,6 +479,23 @@ def test_restore_larger_than_the_hbm_limit_goes_window_by_window(shm_dir, manage
     assert isinstance(cause, integrity.ChecksumMismatchError) and "chunk(s) [5]" in str(cause)
 
 
+@pytest.mark.parametrize("load_file_io", [True, False])
+def test_truncated_object_is_refused_before_anything_is_read(shm_dir, manager_future, load_file_io):
+    """An object cut short after it was written (its metadata block still records the full length) must end in an
+    error, in both IO modes - not in a read past the end of the file or of its mapping."""
+    sd = {"a": torch.randn(300_000, device=DEV), "b": torch.ones(1000, device=DEV)}
+    ckpt = os.path.join(shm_dir, "step-3_ckpt")
+    dcp.save(sd, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(_saver(), manager_future), no_dist=True)
+    obj = os.path.join(ckpt, "__0__0_src0.distcp")
+    os.truncate(obj, os.path.getsize(obj) - 70_000)
+    target = {k: torch.zeros_like(v) for k, v in sd.items()}
+    with pytest.raises(BaseException) as exc:
+        dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, _loader(use_file_io=load_file_io)), no_dist=True)
+    cause = exc.value.failures[0][0] if hasattr(exc.value, "failures") else exc.value
+    assert isinstance(cause, ValueError) and "is truncated" in str(cause)
+    assert all(float(t.abs().sum()) == 0 for t in target.values())
+
+
 def test_legacy_torch_save_objects_are_still_readable(shm_dir):
     """An object whose signature is TORCH___ holds torch.save records; the loader reads it on the host."""
     from ml_flashpoint.core.defaults import CheckpointFormat
