@@ -34,7 +34,9 @@ typedef struct mlf_buffer mlf_buffer; /* opaque */
 
 /* Creates (or, with overwrite != 0, truncates and re-creates) the file `object_id`, sizes it to
  * `capacity` bytes and maps it read-write.  Parent directories are created.  Without overwrite an
- * existing path fails with MLF_ALREADY_EXISTS.
+ * existing path fails with MLF_ALREADY_EXISTS.  A capacity that the file system cannot hold at that
+ * moment (free space per fstatvfs) fails with MLF_INTERNAL and leaves no file: stores into pages a full
+ * tmpfs cannot back would otherwise end in SIGBUS (the reference has no such check).
  * Replaces BufferObject(object_id, capacity, overwrite): buffer_object.cpp:25-49,
  * buffer_helper.cpp:43-120. */
 int mlf_buffer_create(const char* object_id, size_t capacity, int overwrite, mlf_buffer** out);
@@ -53,8 +55,9 @@ int mlf_buffer_close(mlf_buffer* b, int has_truncate, size_t truncate_size);
 /* Closes (without truncation) if still open and frees the handle. Replaces ~BufferObject. */
 void mlf_buffer_destroy(mlf_buffer* b);
 
-/* munmap + ftruncate + mmap to a new capacity; the data pointer changes.  Fails on closed or read-only
- * handles and on new_capacity == 0.
+/* New capacity for file and mapping (mremap, so the surviving range keeps its page-table entries; the
+ * data pointer may change).  Fails on closed or read-only handles, on new_capacity == 0, and on growth
+ * beyond the free space of the file system, in which case the buffer stays as it was.
  * Replaces BufferObject::resize: buffer_object.cpp:178-197, buffer_helper.cpp:273-314. */
 int mlf_buffer_resize(mlf_buffer* b, size_t new_capacity);
 

@@ -16,6 +16,7 @@
 #endif
 #include <sys/mman.h>
 #include <sys/stat.h>
+#include <sys/statvfs.h>
 #include <unistd.h>
 
 #include <algorithm>
@@ -70,6 +71,22 @@ int make_parent_dirs(const std::string& path) {
   return S_ISDIR(st.st_mode) ? 0 : ENOTDIR;
 }
 
+// A store into a page of a MAP_SHARED file that the file system cannot back (a full tmpfs) does not fail with an
+// error code: the process gets SIGBUS.  So a file is never made larger than what its file system can hold at that
+// moment.  Returns 0 if `new_size` fits or nothing can be said (no limit reported), else the failure code.
+int check_space(int fd, size_t new_size, const std::string& id) {
+  struct stat st;
+  struct statvfs vfs;
+  if (fstat(fd, &st) != 0 || fstatvfs(fd, &vfs) != 0 || vfs.f_blocks == 0) return 0;
+  const unsigned long long allocated = (unsigned long long)st.st_blocks * 512ull;
+  if (new_size <= allocated) return 0;
+  const unsigned long long needed = new_size - allocated;
+  const unsigned long long available = (unsigned long long)vfs.f_bavail * (unsigned long long)vfs.f_frsize;
+  if (needed <= available) return 0;
+  return fail(MLF_INTERNAL, "not enough space on the file system that holds " + id + ": " + std::to_string(needed) +
+                                " more bytes needed, " + std::to_string(available) + " available");
+}
+
 bool is_open(const mlf_buffer* b) {
   return b && !b->closed && b->ptr != nullptr && b->ptr != MAP_FAILED && b->fd != -1;
 }
@@ -97,6 +114,11 @@ int mlf_buffer_create(const char* object_id, size_t capacity, int overwrite, mlf
       return fail(MLF_ALREADY_EXISTS,
                   "open() failed for file: " + id + ". File already exists and overwrite is set to false.");
     return fail_errno("open() failed for file: " + id, e);
+  }
+  if (int rc = check_space(fd, capacity, id)) {
+    close(fd);
+    unlink(object_id);  // it is empty: either just created or just truncated by O_TRUNC
+    return rc;
   }
   if (ftruncate(fd, (off_t)capacity) == -1) {
     int e = errno;
@@ -191,6 +213,8 @@ int mlf_buffer_resize(mlf_buffer* b, size_t new_capacity) {
   // change), but mremap carries the page-table entries of the surviving range over, so a pooled buffer that is
   // trimmed after one save and grown again for the next is written without taking a minor fault per page.
   const bool shrinking = new_capacity < b->cap;
+  if (!shrinking)
+    if (int rc = check_space(b->fd, new_capacity, b->id)) return rc;  // the buffer stays as it is
   if (!shrinking && ftruncate(b->fd, (off_t)new_capacity) == -1) return fail_errno("ftruncate() failed during resize", errno);
   void* p = mremap(b->ptr, b->cap, new_capacity, MREMAP_MAYMOVE);
   if (p == MAP_FAILED) {

@@ -320,3 +320,22 @@ def test_manager_prefers_pool_then_falls_back(tmp_path, no_pool):
     mgr.close_buffer(wb)  # closing a closed buffer is ignored
     # another manager in the same process shares the pool
     assert CheckpointObjectManager()._get_or_create_buffer_pool() is CheckpointObjectManager._worker_pool
+
+
+def test_a_buffer_is_never_made_larger_than_its_file_system_can_hold(shm_dir):
+    """Stores into pages a full tmpfs cannot back end in SIGBUS, so creation and growth beyond the free space are
+    refused with an error instead (the file is sparse: asking costs nothing)."""
+    free = os.statvfs(shm_dir)
+    too_much = free.f_bavail * free.f_frsize + (1 << 30)
+    path = os.path.join(shm_dir, "too_large.bin")
+    with pytest.raises(RuntimeError, match="not enough space on the file system"):
+        BufferObject(path, capacity=too_much, overwrite=True)
+    assert not os.path.exists(path)                                # nothing is left behind
+    bo = BufferObject(path, capacity=METADATA_SIZE + 100, overwrite=True)
+    memoryview(bo)[:3] = b"abc"
+    with pytest.raises(RuntimeError, match="not enough space on the file system"):
+        bo.resize(too_much)
+    assert not bo.closed and bo.get_capacity() == METADATA_SIZE + 100  # refused growth leaves the buffer as it was
+    assert bytes(memoryview(bo)[:3]) == b"abc"
+    bo.resize(METADATA_SIZE + 200)
+    bo.close()
