@@ -490,7 +490,6 @@ __global__ void __launch_bounds__(256) mlf_strided_kernel(const StridedDesc* __r
 // accesses are bound by the number of lane accesses, not by bytes); LDS is addressed per element on the transposed side.  T = 128 / 64 / 64 / 32 / 16 elements for esz = 1 / 2 / 4 / 8 / 16;
 // rows of the LDS tile are padded so that a column walk does not stay in one bank.
 constexpr uint32_t kTransThreads = 256;
-constexpr uint32_t kTransBand = 8;   // tile-rows per band of the visiting order (measured: 8 beats 1 by 10-40 %)
 constexpr uint32_t kTransPatch = 8;  // neighbouring tile-rows per XCD where 64 tile-rows are left (then 4, 2, 1)
 constexpr uint32_t kTransLdsBytes = 128 * (128 + 16);
 
