@@ -99,7 +99,7 @@ def cpu_baseline(sd, sample_bytes, root, device):
     """The reference's CPU path, restated by the oracle, on a prefix of the state dict of about ``sample_bytes``."""
     import torch
 
-    from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId, CheckpointObjectId
+    from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId
     from oracle import cpu_path
 
     sample, total = {}, 0

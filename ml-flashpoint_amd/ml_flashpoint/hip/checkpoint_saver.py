@@ -16,7 +16,6 @@ them (checkpoint_saver.py:340-343,533-619,709-762).
 
 import concurrent.futures
 import dataclasses
-import io
 import logging
 import os
 import pickle

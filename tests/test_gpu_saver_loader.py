@@ -177,7 +177,6 @@ def test_megatron_style_sequence_with_pool_and_finalize(shm_dir, manager_future)
     """initialize -> prepare buckets (pack) -> generic stage step -> write -> finish -> finalize, into pooled buffers,
     twice (the second save reuses a pool buffer and removes the first step)."""
     from torch.distributed.checkpoint import DefaultSavePlanner
-    from torch.distributed.checkpoint.default_planner import create_default_local_save_plan
 
     pool_cfg = BufferPoolConfig(os.path.join(shm_dir, "pool"), 0, 2, METADATA_SIZE + 4096)
     manager = CheckpointObjectManager(pool_cfg)

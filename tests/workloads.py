@@ -4,7 +4,6 @@ Values are generated with ``torch.Generator`` seeds fixed per config, on the req
 config for quick tests by dividing layer counts / widths, keeping the tensor structure.
 """
 
-import math
 from typing import Dict, List, Tuple
 
 import torch
