@@ -495,6 +495,38 @@ def test_truncated_object_is_refused_before_anything_is_read(shm_dir, manager_fu
     assert all(float(t.abs().sum()) == 0 for t in target.values())
 
 
+def test_several_objects_are_written_and_read_back_concurrently(shm_dir, manager_future):
+    """``thread_count=3`` splits a save into three objects; the reader then hands each object to the loader on a
+    thread of its own, so three ``read_data`` calls share one copy engine and one device."""
+    g = torch.Generator().manual_seed(17)
+    sd_cpu = {f"p{i}": torch.randn(40_000 + 1111 * i, generator=g) for i in range(9)}
+    sd_cpu["view"] = torch.randn(300, 200, generator=g).t()
+    sd_cpu["note"] = "three objects"
+    sd_dev = _to_dev(sd_cpu)
+    ckpt = os.path.join(shm_dir, "step-6_ckpt")
+    saver = _saver(crc_chunk_bytes=1 << 16)
+    dcp.save(sd_dev, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(saver, manager_future, thread_count=3), no_dist=True)
+    objects = sorted(n for n in os.listdir(ckpt) if n.endswith(".distcp"))
+    assert objects == ["__0__0_src0.distcp", "__0__1_src0.distcp", "__0__2_src0.distcp"]
+    metadata = pickle.load(open(os.path.join(ckpt, ".metadata"), "rb"))
+    for name in objects:  # each object is the oracle's image of the items the plan put there, in offset order
+        here = sorted(((i, s) for i, s in metadata.storage_data.items() if s.relative_path == name), key=lambda kv: kv[1].offset)
+        raw = open(os.path.join(ckpt, name), "rb").read()
+        tensors = [sd_cpu[i.fqn] for i, _ in here if isinstance(sd_cpu[i.fqn], torch.Tensor)]
+        blobs = [raw[METADATA_SIZE + s.offset : METADATA_SIZE + s.offset + s.length] for i, s in here
+                 if not isinstance(sd_cpu[i.fqn], torch.Tensor)]
+        assert raw == fmt.file_image(tensors, blobs)[0]
+    for _ in range(3):  # the interleaving of the three reader threads differs from run to run
+        target = {k: (torch.zeros(v.shape, dtype=v.dtype, device=DEV) if isinstance(v, torch.Tensor) else None)
+                  for k, v in sd_cpu.items()}
+        loader = _loader()
+        dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), no_dist=True)
+        assert target["note"] == "three objects"
+        for k, v in sd_cpu.items():
+            if isinstance(v, torch.Tensor):
+                assert torch.equal(_bits(target[k]), _bits(v)), k
+
+
 def test_legacy_torch_save_objects_are_still_readable(shm_dir):
     """An object whose signature is TORCH___ holds torch.save records; the loader reads it on the host."""
     from ml_flashpoint.core.defaults import CheckpointFormat
