@@ -19,6 +19,7 @@ import pickle
 import struct
 import threading
 import time
+import warnings
 from pathlib import Path
 from typing import IO, Callable, List, Optional, cast
 
@@ -144,7 +145,9 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                     try:
                         header = pickle.loads(buffer_slice.read(header_len))
                         data = buffer_slice.read()
-                        tensor = torch.frombuffer(data, dtype=header.dtype).reshape(header.shape)
+                        with warnings.catch_warnings():  # `data` is immutable and the tensor over it is only read
+                            warnings.filterwarnings("ignore", message="The given buffer is not writable")
+                            tensor = torch.frombuffer(data, dtype=header.dtype).reshape(header.shape)
                     except Exception:
                         _LOGGER.exception("Failed to parse tensor header")
                         raise
