@@ -108,7 +108,8 @@ def cpu_baseline(sd, sample_bytes, root, device):
             break
         sample[k] = v
         total += v.numel() * v.element_size()
-    saver = cpu_path.OracleCheckpointSaver(initial_buffer_size_bytes=total + (1 << 20))
+    capacity = total + 256 * len(sample) + (1 << 20)  # payloads + record headers (~140 B each) + slack
+    saver = cpu_path.OracleCheckpointSaver(initial_buffer_size_bytes=capacity)
     threads = saver.torch_thread_count(1)
     cid = CheckpointContainerId(os.path.join(root, "cpu_baseline", "step-0_ckpt"))
     path = os.path.join(cid.data, "sample.distcp")
@@ -123,7 +124,7 @@ def cpu_baseline(sd, sample_bytes, root, device):
         torch.set_num_threads(threads)
         try:
             if rep == 0:
-                spans = cpu_path.write_object(path, list(staged.values()), [], total + (1 << 20))
+                spans = cpu_path.write_object(path, list(staged.values()), [], capacity)
                 t2 = time.perf_counter()
             else:
                 # rewrite in place over warm pages: what a pooled buffer gives the reference from the second save on

@@ -104,6 +104,14 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
 int mlf_plan_destroy(mlf_plan* plan);
 int mlf_plan_get_info(const mlf_plan* plan, mlf_plan_info* out);
 
+/* Replaces the bytes of the plan's blob (same size as at creation) for a plan that is kept from one save to the
+ * next: the record headers in it repeat, step counters and other host-resident items do not.  The upload is
+ * enqueued on `stream`, so it is ordered behind launches already enqueued there (which still read the old bytes)
+ * and ahead of later ones; use the stream the plan is launched on.  No reference counterpart: the reference
+ * rebuilds everything per save (checkpoint_saver.py:622-707); its plan caching (save_strategies.py:182-212) is the
+ * model for keeping the tables. */
+int mlf_plan_update_blob(mlf_plan* plan, const void* host_blob, uint64_t blob_bytes, void* stream);
+
 /* Save direction: tensors (+ blob) -> image.  Asynchronous on `stream`; the image is complete when the
  * stream reaches the point after this call.  Replaces the per-tensor .to("cpu") staging
  * (checkpoint_saver.py:347-360; memory_storage_writer.py:213-233) and the per-tensor

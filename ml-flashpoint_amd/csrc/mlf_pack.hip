@@ -628,6 +628,9 @@ struct mlf_plan {
   TransDesc* d_tdescs = nullptr;
   TransWork* d_twork = nullptr;
   char* d_blob = nullptr;
+  uint64_t blob_size = 0;
+  char* h_blob = nullptr;            // pinned staging of mlf_plan_update_blob, allocated on first use
+  hipEvent_t blob_copied = nullptr;  // recorded behind the last upload out of h_blob
   uint32_t block_threads = 256;
   uint32_t unroll = 1;
   uint32_t cut_mask = 15;     // tile cuts sit on multiples of cut_mask + 1 bytes ...
@@ -646,6 +649,8 @@ struct mlf_plan {
     (void)hipFree(d_tdescs);
     (void)hipFree(d_twork);
     (void)hipFree(d_blob);
+    if (h_blob) (void)hipHostFree(h_blob);
+    if (blob_copied) (void)hipEventDestroy(blob_copied);
   }
 };
 
@@ -777,6 +782,7 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
   if (plan->grid_x_log2 > widest) return fail(MLF_HIP_BAD_ARG, "grid_x_log2: a grid row of that many workgroups exceeds 2^32 threads");
   if (plan->unroll != 1 && plan->unroll != 2 && plan->unroll != 4 && plan->unroll != 8)
     return fail(MLF_HIP_BAD_ARG, "unroll must be 1, 2, 4 or 8");
+  plan->blob_size = blob_bytes;
   if (blob_bytes) {
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&plan->d_blob), blob_bytes));
     HIP_TRY(hipMemcpy(plan->d_blob, host_blob, blob_bytes, hipMemcpyHostToDevice));
@@ -984,6 +990,27 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
 
 int mlf_plan_destroy(mlf_plan* plan) {
   delete plan;  // the destructor frees the device tables
+  return MLF_HIP_OK;
+}
+
+int mlf_plan_update_blob(mlf_plan* plan, const void* host_blob, uint64_t blob_bytes, void* stream) {
+  if (!plan) return fail(MLF_HIP_BAD_ARG, "null plan");
+  if (blob_bytes != plan->blob_size)
+    return fail(MLF_HIP_BAD_ARG, "blob of " + std::to_string(blob_bytes) + " bytes for a plan built with " +
+                                     std::to_string(plan->blob_size));
+  if (blob_bytes == 0) return MLF_HIP_OK;
+  if (!host_blob) return fail(MLF_HIP_BAD_ARG, "null host_blob");
+  HIP_TRY(hipSetDevice(plan->device));
+  if (!plan->h_blob) {
+    HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&plan->h_blob), blob_bytes, hipHostMallocDefault));
+    HIP_TRY(hipEventCreateWithFlags(&plan->blob_copied, hipEventDisableTiming));
+  } else {
+    HIP_TRY(hipEventSynchronize(plan->blob_copied));  // the previous upload has left the staging buffer
+  }
+  memcpy(plan->h_blob, host_blob, blob_bytes);
+  // ordered on the caller's stream: behind the launches that still read the old bytes, ahead of those to come
+  HIP_TRY(hipMemcpyAsync(plan->d_blob, plan->h_blob, blob_bytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream)));
+  HIP_TRY(hipEventRecord(plan->blob_copied, static_cast<hipStream_t>(stream)));
   return MLF_HIP_OK;
 }
 

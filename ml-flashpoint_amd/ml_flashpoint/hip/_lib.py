@@ -84,6 +84,7 @@ _SIGNATURES = {
     "mlf_plan_create": (_INT, [_VP, _U64, _VP, _U64, _U64, ctypes.POINTER(PlanOpts), ctypes.POINTER(_VP)]),
     "mlf_plan_destroy": (_INT, [_VP]),
     "mlf_plan_get_info": (_INT, [_VP, ctypes.POINTER(PlanInfo)]),
+    "mlf_plan_update_blob": (_INT, [_VP, _VP, _U64, _VP]),
     "mlf_pack_launch": (_INT, [_VP, _VP, _VP]),
     "mlf_unpack_launch": (_INT, [_VP, _VP, _VP]),
     "mlf_crc32c_device": (_INT, [_VP, _U64, _U64, _VP, _U64, _VP]),

@@ -120,6 +120,11 @@ class ItemTable:
         return arr
 
 
+def host_tensor_bytes(t: torch.Tensor) -> bytes:
+    """C-contiguous bytes of a host-resident tensor (what its record's payload is)."""
+    return t.detach().contiguous().reshape(-1).view(torch.uint8).numpy().tobytes()
+
+
 @dataclasses.dataclass
 class SaveLayout:
     """Where every item of one checkpoint object lies, and the table that packs it."""
@@ -130,6 +135,9 @@ class SaveLayout:
     blob: bytes
     device_payload_bytes: int
     device_tensors: List[torch.Tensor]  # kept alive while the plan may run
+    # pieces of the blob whose bytes are not determined by dtypes and shapes: (blob offset, nbytes, "tensor" | "blob",
+    # index into the tensors / blobs argument).  A layout that is reused for the next save refreshes exactly these.
+    variable_parts: List[Tuple[int, int, str, int]] = dataclasses.field(default_factory=list)
 
 
 def build_save_layout(tensors: Sequence[torch.Tensor], blobs: Sequence[bytes] = ()) -> SaveLayout:
@@ -142,9 +150,10 @@ def build_save_layout(tensors: Sequence[torch.Tensor], blobs: Sequence[bytes] = 
     blob = bytearray()
     spans: List[Tuple[int, int]] = []
     keep: List[torch.Tensor] = []
+    variable: List[Tuple[int, int, str, int]] = []
     pos = 0
     device_bytes = 0
-    for t in tensors:
+    for index, t in enumerate(tensors):
         start = pos
         hdr = header_bytes(t.dtype, t.shape)
         table.add_blob(len(blob), pos, len(hdr))
@@ -154,9 +163,9 @@ def build_save_layout(tensors: Sequence[torch.Tensor], blobs: Sequence[bytes] = 
         if nbytes:
             if t.device.type == "cpu":
                 # host-resident item (step counters, RNG state ...): its bytes travel with the headers
-                flat = t.detach().contiguous().reshape(-1).view(torch.uint8)
+                variable.append((len(blob), nbytes, "tensor", index))
                 table.add_blob(len(blob), pos, nbytes)
-                blob += flat.numpy().tobytes()
+                blob += host_tensor_bytes(t)
             else:
                 if t.is_contiguous():
                     table.add_contiguous(t.data_ptr(), pos, t.element_size(), nbytes)
@@ -166,8 +175,9 @@ def build_save_layout(tensors: Sequence[torch.Tensor], blobs: Sequence[bytes] = 
                 device_bytes += nbytes
             pos += nbytes
         spans.append((start, pos - start))
-    for data in blobs:
+    for index, data in enumerate(blobs):
         if len(data):
+            variable.append((len(blob), len(data), "blob", index))
             table.add_blob(len(blob), pos, len(data))
             blob += data
         spans.append((pos, len(data)))
@@ -179,6 +189,7 @@ def build_save_layout(tensors: Sequence[torch.Tensor], blobs: Sequence[bytes] = 
         blob=bytes(blob),
         device_payload_bytes=device_bytes,
         device_tensors=keep,
+        variable_parts=variable,
     )
 
 
@@ -222,6 +233,17 @@ class Plan:
         out = _lib.PlanInfo()
         _lib.check(_lib.load().mlf_plan_get_info(self._handle, ctypes.byref(out)), "mlf_plan_get_info")
         return out
+
+    def update_blob(self, blob: bytes, stream: int) -> None:
+        """New bytes (same length) for the blob of a plan that is kept across saves; ordered on ``stream``."""
+        if self._handle is None:
+            raise ValueError("plan already destroyed")
+        buf = (ctypes.c_char * len(blob)).from_buffer_copy(blob) if blob else None
+        _lib.check(
+            _lib.load().mlf_plan_update_blob(self._handle, ctypes.addressof(buf) if buf is not None else None,
+                                             len(blob), stream),
+            "mlf_plan_update_blob",
+        )
 
     def pack(self, image: torch.Tensor, stream: Optional[int] = None) -> None:
         """Enqueues tensors -> image on ``stream`` (default: torch's current stream)."""

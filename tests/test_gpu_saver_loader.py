@@ -527,6 +527,49 @@ def test_several_objects_are_written_and_read_back_concurrently(shm_dir, manager
                 assert torch.equal(_bits(target[k]), _bits(v)), k
 
 
+def test_plans_are_kept_from_save_to_save_and_rebuilt_when_the_tensors_change(shm_dir, manager_future):
+    """The second save of the same tensors reuses layout and device tables; new values, a new step counter (host
+    tensor) and new pickled objects of the same length only refresh bytes.  A changed shape, address or blob length
+    rebuilds.  Every file is the oracle's image of what was live at that save."""
+    g = torch.Generator().manual_seed(23)
+    sd_cpu = dict(_mixed_state_dict())
+    sd_cpu["opt.step"] = torch.tensor([1, 0, 0], dtype=torch.int64)      # stays on the host: its bytes change per save
+    sd_dev = _to_dev(sd_cpu, keep_on_host=("w.i64", "opt.step"))
+    saver = _saver()
+
+    def save(step, sd_d):
+        ckpt = os.path.join(shm_dir, f"step-{step}_ckpt")
+        dcp.save(sd_d, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(saver, manager_future), no_dist=True)
+        raw = open(os.path.join(ckpt, "__0__0_src0.distcp"), "rb").read()
+        metadata = pickle.load(open(os.path.join(ckpt, ".metadata"), "rb"))
+        host = {k: (v.cpu() if isinstance(v, torch.Tensor) else v) for k, v in sd_d.items()}
+        image, spans, got_spans = _expected_file(host, metadata, raw)
+        assert raw == image and got_spans == spans, f"save {step}"
+        return dict(saver.last_save_stats)
+
+    assert "plans_reused" not in save(1, sd_dev)
+    for step in (2, 3):  # training moves on: new values everywhere, same tensors
+        for k, v in sd_dev.items():
+            if isinstance(v, torch.Tensor) and v.is_floating_point() and v.dtype not in (torch.float8_e4m3fn,):
+                v.mul_(-1.5).add_(float(step))
+        sd_dev["opt.step"][0] = step
+        sd_dev["obj.step"] = 123 + step                     # pickles to the same number of bytes
+        assert save(step, sd_dev)["plans_reused"] == 1
+    sd_dev["obj.cfg"] = "lr=1e-4;name=a-longer-one"          # serialises into the same (padded) number of bytes
+    assert save(4, sd_dev)["plans_reused"] == 1
+    sd_dev["obj.cfg"] = "lr=1e-4;" + "x" * 300                # a blob of another length moves what lies behind it
+    assert "plans_reused" not in save(40, sd_dev)
+    assert save(5, sd_dev)["plans_reused"] == 1
+    sd_dev["w.fp32"] = torch.randn(129, 66, generator=g).to(DEV)  # same byte count, another shape and address
+    assert "plans_reused" not in save(6, sd_dev)
+    assert save(7, sd_dev)["plans_reused"] == 1
+    saver.release_device_memory()                               # drops the kept plans too
+    assert "plans_reused" not in save(8, sd_dev)
+    fresh = _saver(reuse_plans=False)
+    saver = fresh
+    assert "plans_reused" not in save(9, sd_dev) and "plans_reused" not in save(10, sd_dev)
+
+
 def test_legacy_torch_save_objects_are_still_readable(shm_dir):
     """An object whose signature is TORCH___ holds torch.save records; the loader reads it on the host."""
     from ml_flashpoint.core.defaults import CheckpointFormat
