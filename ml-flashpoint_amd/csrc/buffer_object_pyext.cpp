@@ -109,6 +109,23 @@ PyObject* bo_resize(PyObject* self_, PyObject* args, PyObject* kwargs) {
   Py_RETURN_NONE;
 }
 
+PyObject* bo_reserve(PyObject* self_, PyObject* args, PyObject* kwargs) {
+  auto* self = reinterpret_cast<PyBufferObject*>(self_);
+  static const char* kwlist[] = {"offset", "nbytes", nullptr};
+  PyObject *off_obj = nullptr, *len_obj = nullptr;
+  if (!PyArg_ParseTupleAndKeywords(args, kwargs, "OO", const_cast<char**>(kwlist), &off_obj, &len_obj)) return nullptr;
+  size_t off = PyLong_AsSize_t(off_obj);
+  if (off == (size_t)-1 && PyErr_Occurred()) return nullptr;
+  size_t len = PyLong_AsSize_t(len_obj);
+  if (len == (size_t)-1 && PyErr_Occurred()) return nullptr;
+  int rc;
+  Py_BEGIN_ALLOW_THREADS
+  rc = mlf_buffer_reserve(self->handle, off, len);
+  Py_END_ALLOW_THREADS
+  if (rc != MLF_OK) return raise_last();
+  Py_RETURN_NONE;
+}
+
 PyObject* bo_get_id(PyObject* self_, PyObject*) {
   auto* self = reinterpret_cast<PyBufferObject*>(self_);
   return PyUnicode_FromString(mlf_buffer_id(self->handle));
@@ -170,6 +187,8 @@ int bo_getbuffer(PyObject* self_, Py_buffer* view, int flags) {
 PyMethodDef bo_methods[] = {
     {"close", (PyCFunction)(void (*)(void))bo_close, METH_VARARGS | METH_KEYWORDS, "Closes the buffer object."},
     {"resize", (PyCFunction)(void (*)(void))bo_resize, METH_VARARGS | METH_KEYWORDS, "Resizes the buffer object."},
+    {"reserve", (PyCFunction)(void (*)(void))bo_reserve, METH_VARARGS | METH_KEYWORDS,
+     "Allocates the pages of a byte range of the file now instead of at first touch."},
     {"get_id", bo_get_id, METH_NOARGS, "Gets the buffer object id."},
     {"get_capacity", bo_get_capacity, METH_NOARGS, "Gets the buffer object capacity."},
     {"get_data_ptr", bo_get_data_ptr, METH_NOARGS, "Returns the raw memory address of the buffer as an integer."},

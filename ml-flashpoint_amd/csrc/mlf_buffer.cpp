@@ -242,6 +242,25 @@ int mlf_buffer_resize(mlf_buffer* b, size_t new_capacity) {
   return MLF_OK;
 }
 
+int mlf_buffer_reserve(mlf_buffer* b, size_t offset, size_t nbytes) {
+  if (!is_open(b)) return fail(MLF_FAILED_PRECONDITION, "Cannot reserve pages of a closed buffer.");
+  if (!b->writable) return fail(MLF_FAILED_PRECONDITION, "Cannot reserve pages of a read-only buffer.");
+  if (offset > b->cap || nbytes > b->cap - offset) return fail(MLF_INVALID_ARGUMENT, "range lies outside the buffer");
+  if (nbytes == 0) return MLF_OK;
+  struct stat st;
+  // a pooled buffer that is written for the second time has its pages already: nothing to do, and walking 100 GB of
+  // page cache to find that out would cost more than it saves
+  if (fstat(b->fd, &st) == 0 && (unsigned long long)st.st_blocks * 512ull >= (unsigned long long)(offset + nbytes))
+    return MLF_OK;
+  if (fallocate(b->fd, 0, (off_t)offset, (off_t)nbytes) == 0) return MLF_OK;
+  const int e = errno;
+  if (e == EOPNOTSUPP || e == ENOSYS) return MLF_OK;  // the file system allocates on first touch only: as before
+  if (e == ENOSPC)
+    return fail(MLF_INTERNAL, "not enough space on the file system that holds " + b->id + " for " +
+                                  std::to_string(nbytes) + " more bytes");
+  return fail_errno("fallocate() failed for file: " + b->id, e);
+}
+
 void* mlf_buffer_data_ptr(const mlf_buffer* b) { return is_open(b) ? b->ptr : nullptr; }
 size_t mlf_buffer_capacity(const mlf_buffer* b) { return is_open(b) ? b->cap : 0; }
 int mlf_buffer_is_closed(const mlf_buffer* b) { return is_open(b) ? 0 : 1; }

@@ -227,6 +227,15 @@ class BufferIO:
         self._check_validity()
         return self.buffer_obj.get_data_ptr() + METADATA_SIZE + pos
 
+    def reserve(self, nbytes: int) -> None:
+        """Has the file system allocate the pages of the next ``nbytes`` of the data section now (they are zero
+        until written).  For writers that know what they are about to fill: page allocation inside a page fault is
+        several times slower than ahead of time.  A no-op where the buffer object cannot do it."""
+        self._check_validity("write")
+        ahead = getattr(self.buffer_obj, "reserve", None)
+        if ahead is not None and nbytes > 0:
+            ahead(METADATA_SIZE + self._pos, nbytes)
+
     def fileno(self) -> int:
         """Descriptor of the mapped file, for engines that read/write the file directly; -1 if the underlying
         buffer object does not expose one."""

@@ -686,6 +686,9 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                 ensure = getattr(writer, "ensure_capacity", None)
                 if ensure is not None:
                     ensure(nbytes)  # pooled buffers grow once, to the exact total
+                reserve = getattr(writer, "reserve", None)
+                if reserve is not None:
+                    reserve(nbytes)  # pages allocated ahead of the copy threads (first use of a buffer file only)
                 with torch.cuda.device(staged.device_index):
                     _lib.check(_lib.load().mlf_hip_set_device(staged.device_index), "mlf_hip_set_device")
                     start = writer.tell()

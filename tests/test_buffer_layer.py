@@ -339,3 +339,28 @@ def test_a_buffer_is_never_made_larger_than_its_file_system_can_hold(shm_dir):
     assert bytes(memoryview(bo)[:3]) == b"abc"
     bo.resize(METADATA_SIZE + 200)
     bo.close()
+
+
+def test_reserve_allocates_the_pages_of_a_range_ahead_of_the_writer(shm_dir):
+    path = os.path.join(shm_dir, "reserve.bin")
+    bo = BufferObject(path, capacity=METADATA_SIZE + (8 << 20), overwrite=True)
+    assert os.stat(path).st_blocks * 512 < (1 << 20)             # sparse: nothing allocated yet
+    bo.reserve(offset=METADATA_SIZE, nbytes=4 << 20)
+    allocated = os.stat(path).st_blocks * 512
+    assert (4 << 20) <= allocated < (6 << 20)                     # that range and nothing like the whole file
+    assert bytes(memoryview(bo)[METADATA_SIZE : METADATA_SIZE + 16]) == bytes(16)   # reserved pages read as zeros
+    bo.reserve(METADATA_SIZE, 4 << 20)                            # already there: nothing to do
+    assert os.stat(path).st_blocks * 512 == allocated
+    with pytest.raises(RuntimeError, match="outside the buffer"):
+        bo.reserve(METADATA_SIZE, 9 << 20)
+    stream = BufferIO(bo)
+    stream.write(b"x" * 100)
+    stream.reserve(6 << 20)                                       # from the current position on
+    assert os.stat(path).st_blocks * 512 >= METADATA_SIZE + 100 + (6 << 20) - 4096
+    stream.close()
+    ro = BufferIO(BufferObject(path))
+    with pytest.raises(TypeError, match="read-only"):
+        ro.reserve(10)
+    with pytest.raises(RuntimeError, match="read-only"):
+        ro.buffer_obj.reserve(0, 10)
+    ro.close()
