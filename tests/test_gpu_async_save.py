@@ -162,7 +162,7 @@ def test_next_save_does_not_wait_for_the_previous_transfer(shm_dir, manager_futu
     second = begin(11, small)
     blocked_s = time.perf_counter() - t0
     assert not first_transfer.done(), "the second save's blocking part outlasted the first save's transfer"
-    assert blocked_s < 0.1
+    assert blocked_s < 0.25
     snapshot = {k: v.cpu() for k, v in small.items()}
     for v in small.values():
         v.add_(1.0)
