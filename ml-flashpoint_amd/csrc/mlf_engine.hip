@@ -205,6 +205,17 @@ int mlf_engine_create(uint64_t slot_bytes, uint32_t n_slots, uint32_t n_threads,
 
 namespace {
 
+// Copies still in flight when a transfer gives up target the pinned slots: they must have landed before the engine
+// (or the next transfer) touches the slots again.  Disarmed on the success path, where the streams are already idle.
+struct DrainOnExit {
+  mlf_engine* e;
+  bool armed = true;
+  ~DrainOnExit() {
+    if (!armed) return;
+    for (hipStream_t s : e->streams) (void)hipStreamSynchronize(s);
+  }
+};
+
 struct CrcRequest {
   uint64_t chunk_bytes = 0;  // 0: no checksum
   uint32_t* out_host = nullptr;
@@ -251,9 +262,7 @@ int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t
     HIP_TRY(hipEventRecord(e->slot_done[s], st));
     return MLF_HIP_OK;
   };
-  auto drain_streams = [&] {
-    for (hipStream_t s : e->streams) (void)hipStreamSynchronize(s);
-  };
+  DrainOnExit drain{e};
   for (uint64_t c = 0; c < std::min(n_chunks, n_slots); ++c)
     if (int rc = issue(c)) return rc;
   double wait = 0;
@@ -263,13 +272,12 @@ int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t
     const double w0 = now_s();
     HIP_TRY(hipEventSynchronize(e->slot_done[s]));
     if (c == 0) wait = now_s() - w0;
-    if (int err = pool_host_copy(*e->pool, host, off, e->slots[s], len, true)) {
-      drain_streams();  // copies still in flight target the slots: let them land before anyone reuses them
+    if (int err = pool_host_copy(*e->pool, host, off, e->slots[s], len, true))
       return fail(MLF_HIP_RUNTIME, std::string("pwrite() to the buffer file failed: ") + strerror(err));
-    }
     if (c + n_slots < n_chunks)
       if (int rc = issue(c + n_slots)) return rc;
   }
+  drain.armed = false;  // every chunk's event has been waited for
   if (want_crc) {
     crc_guard.armed = false;
     if (int rc = crc_finish(&crc_job, crc.out_host)) return rc;
@@ -294,14 +302,13 @@ int engine_h2d(mlf_engine* e, const HostEnd& host, void* dst_dev, uint64_t nbyte
   const uint64_t slot = e->slot_bytes;
   const uint64_t n_chunks = (nbytes + slot - 1) / slot;
   const uint64_t n_slots = e->slots.size();
+  DrainOnExit drain{e};
   for (uint64_t c = 0; c < n_chunks; ++c) {
     const uint64_t off = c * slot, len = std::min(slot, nbytes - off);
     const uint64_t s = c % n_slots;
     if (c >= n_slots) HIP_TRY(hipEventSynchronize(e->slot_done[s]));  // the slot's previous upload has left it
-    if (int err = pool_host_copy(*e->pool, host, off, e->slots[s], len, false)) {
-      for (hipStream_t st : e->streams) (void)hipStreamSynchronize(st);
+    if (int err = pool_host_copy(*e->pool, host, off, e->slots[s], len, false))
       return fail(MLF_HIP_RUNTIME, std::string("pread() from the buffer file failed: ") + strerror(err));
-    }
     hipStream_t st = e->streams[c & 1];
     HIP_TRY(hipMemcpyAsync(dst + off, e->slots[s], len, hipMemcpyHostToDevice, st));
     HIP_TRY(hipEventRecord(e->slot_done[s], st));
@@ -312,6 +319,7 @@ int engine_h2d(mlf_engine* e, const HostEnd& host, void* dst_dev, uint64_t nbyte
     HIP_TRY(hipStreamWaitEvent(static_cast<hipStream_t>(consumer_stream), e->gate, 0));
     HIP_TRY(hipStreamSynchronize(s));
   }
+  drain.armed = false;
   if (stats) {
     stats->seconds = now_s() - t0;
     stats->wait_seconds = 0;

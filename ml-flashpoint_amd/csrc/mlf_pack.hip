@@ -760,6 +760,7 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
   *out = nullptr;
   if (n_items && !items) return fail(MLF_HIP_BAD_ARG, "null items");
   if (blob_bytes && !host_blob) return fail(MLF_HIP_BAD_ARG, "null host_blob with blob_bytes > 0");
+  if (image_bytes >> 60) return fail(MLF_HIP_BAD_ARG, "image_bytes is not a plausible size");  // keeps the checks below from wrapping
   uint32_t tile = opts && opts->tile_bytes ? opts->tile_bytes : kDefaultTileBytes;
   uint32_t threads = opts && opts->block_threads ? opts->block_threads : 256;
   const bool align_to_tensor = opts && opts->align_to_tensor;
@@ -825,24 +826,25 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
     }
     uint64_t numel = 1;
     bool bad = false;
-    for (uint32_t d = 0; d < it.ndim; ++d) {
-      if (it.shape[d] <= 0) bad = true;
-      numel *= (uint64_t)it.shape[d];
-    }
-    if (bad || numel * esz != it.nbytes) {
+    for (uint32_t d = 0; d < it.ndim && !bad; ++d)
+      bad = it.shape[d] <= 0 || __builtin_mul_overflow(numel, (uint64_t)it.shape[d], &numel);
+    if (bad || numel > it.nbytes || numel * esz != it.nbytes) {
       rc = fail(MLF_HIP_BAD_ARG, "item " + std::to_string(k) + ": shape does not match nbytes");
       break;
     }
     // the image side must stay inside the item's declared span of the image
     {
       int64_t lo = 0, hi = 0;
+      bool wraps = false;
       for (uint32_t d = 0; d < it.ndim; ++d) {
-        const int64_t reach = (it.shape[d] - 1) * it.image_stride[d];
-        (reach < 0 ? lo : hi) += reach;
+        int64_t reach = 0;
+        wraps |= __builtin_mul_overflow(it.shape[d] - 1, it.image_stride[d], &reach);
+        wraps |= __builtin_add_overflow(reach < 0 ? lo : hi, reach, reach < 0 ? &lo : &hi);
       }
-      const int64_t first = (int64_t)it.image_off + lo * (int64_t)esz;
-      const uint64_t last = it.image_off + (uint64_t)hi * esz + esz;
-      if (first < 0 || last > image_bytes) {
+      wraps |= lo < -((int64_t)1 << 56) || hi > ((int64_t)1 << 56);  // times at most 16 bytes per element below
+      const int64_t first = wraps ? -1 : (int64_t)it.image_off + lo * (int64_t)esz;
+      const uint64_t last = wraps ? 0 : it.image_off + (uint64_t)hi * esz + esz;
+      if (wraps || first < 0 || last > image_bytes) {
         rc = fail(MLF_HIP_BAD_ARG, "item " + std::to_string(k) + ": image-side strides reach outside the image");
         break;
       }
@@ -1002,8 +1004,8 @@ int mlf_plan_update_blob(mlf_plan* plan, const void* host_blob, uint64_t blob_by
   if (!host_blob) return fail(MLF_HIP_BAD_ARG, "null host_blob");
   HIP_TRY(hipSetDevice(plan->device));
   if (!plan->h_blob) {
+    if (!plan->blob_copied) HIP_TRY(hipEventCreateWithFlags(&plan->blob_copied, hipEventDisableTiming));
     HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&plan->h_blob), blob_bytes, hipHostMallocDefault));
-    HIP_TRY(hipEventCreateWithFlags(&plan->blob_copied, hipEventDisableTiming));
   } else {
     HIP_TRY(hipEventSynchronize(plan->blob_copied));  // the previous upload has left the staging buffer
   }

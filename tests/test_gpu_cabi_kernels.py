@@ -492,6 +492,33 @@ def test_plan_rejects_items_outside_image():
         P.Plan(table.to_array(), b"12345678", 64)
 
 
+def test_plan_rejects_descriptors_whose_arithmetic_wraps():
+    """Shapes whose product wraps 2^64 back onto nbytes, and image-side strides whose reach wraps past the image's
+    bounds check, are refused on the host: no kernel is launched with them."""
+    from ml_flashpoint.hip import _lib, plan as P
+
+    t = torch.zeros(64, dtype=torch.float32, device=DEV)
+
+    def row(shape, image_stride):
+        table = P.ItemTable()
+        table.add_device(t.data_ptr(), 0, 4, (8, 8), (8, 1))
+        arr = table.to_array()
+        arr["ndim"][0] = len(shape)
+        arr["shape"][0, : len(shape)] = shape
+        arr["stride"][0, : len(shape)] = [1] * len(shape)
+        arr["image_stride"][0, : len(shape)] = image_stride
+        return arr
+
+    with pytest.raises(_lib.HipError, match="shape does not match nbytes"):
+        P.Plan(row((1 << 32, 1 << 32, 64), (0, 0, 1)), b"", 256)  # 2^64 * 64 elements == 64 (mod 2^64)
+    with pytest.raises(_lib.HipError, match="reach outside the image"):
+        P.Plan(row((2, 32), (1 << 62, 1)), b"", 256)
+    with pytest.raises(_lib.HipError, match="reach outside the image"):
+        P.Plan(row((2, 2, 16), (1 << 62, 1 << 62, 1)), b"", 256)  # 2^62 + 2^62 wraps a signed 64-bit sum
+    with pytest.raises(_lib.HipError, match="not a plausible size"):
+        P.Plan(row((8, 8), (8, 1)), b"", 1 << 61)
+
+
 @pytest.mark.parametrize("nbytes", [1, 15, 1023, 1024, 65535, 65536, 65537, 3 * 65536 + 1024 + 7, (5 << 20) + 13])
 def test_crc32c_device_matches_oracle(nbytes, oracle_c):
     from ml_flashpoint.hip import plan as P
