@@ -54,6 +54,12 @@ MIXED = [
     ((4, 0, 3), torch.int16),
     ((2, 3), torch.complex64),
     ((5,), torch.complex128),
+    ((33,), torch.uint16),
+    ((9, 11), torch.uint32),
+    ((1027,), torch.uint64),
+    ((129, 3), torch.float8_e5m2),
+    ((4099,), torch.float8_e4m3fnuz),
+    ((2, 515), torch.float8_e5m2fnuz),
     ((1 << 20,), torch.float32),
     ((777, 513), torch.float64),
 ]

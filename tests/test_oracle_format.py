@@ -44,7 +44,8 @@ def test_header_vectors_unpickle_to_the_package_class(case):
 
 @settings(max_examples=200, deadline=None)
 @given(
-    st.sampled_from(["float32", "bfloat16", "int64", "uint8", "float8_e4m3fn", "bool", "complex64"]),
+    st.sampled_from(["float32", "bfloat16", "int64", "uint8", "float8_e4m3fn", "bool", "complex64", "uint16", "uint64",
+                     "float8_e5m2", "float8_e4m3fnuz", "float8_e5m2fnuz", "complex128", "float64", "int8"]),
     st.lists(st.one_of(st.integers(0, 300), st.integers(0, 1 << 40)), min_size=0, max_size=9),
 )
 def test_header_pickle_closed_form_equals_cpython_pickler(dtype_name, shape):
