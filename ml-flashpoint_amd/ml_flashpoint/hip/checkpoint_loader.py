@@ -250,9 +250,14 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         # whole stored tensor into a contiguous target (the common case) is one run of bytes; anything else is a box
         # over the stored C-contiguous payload (offsets/strides) with the target's strides on the other side.
         rows = []  # (first, last, contiguous?, table arguments)
+        conversions = []  # (target, buffer of the stored dtype): the reference's `copy_` converts, so this does too
         for req, target, dtype, shape, payload_off, stored_bytes in device_reqs:
             if target.dtype != dtype:
-                raise TypeError(f"req {req.storage_index}: stored dtype {dtype} differs from target dtype {target.dtype}")
+                # restored bit-exact into a buffer of the stored dtype; torch converts on the device afterwards,
+                # on the stream the unpack runs on (checkpoint_loader.py:335 does the same conversion on the host)
+                stored_as = torch.empty(target.size(), dtype=dtype, device=device)
+                conversions.append((target, stored_as))
+                target = stored_as
             if payload_off + stored_bytes > written:
                 raise ValueError(f"req {req.storage_index}: record reaches past the written data of '{object_id.data}'")
             esz = _element_size(dtype)
@@ -303,6 +308,8 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                     self._restore_range(object_id, stream, device, rows, lo, hi, sidecar, stats)
                 else:
                     self._restore_windowed(object_id, stream, device, rows, limit, sidecar, stats)
+                for target, stored_as in conversions:
+                    target.copy_(stored_as)
         for req, target, *_ in device_reqs:
             planner.commit_tensor(req, target)
         stats["device_items"] += len(device_reqs)

@@ -371,6 +371,45 @@ def test_direct_saver_calls_offsets_names_and_sub_box_reads(shm_dir):
         _loader().read_data(CheckpointObjectId(oid.data + ".gone"), reqs, planner, storage)
 
 
+def test_targets_of_another_dtype_are_converted_as_copy_does(shm_dir):
+    """The reference ends a read with ``target.copy_(stored)`` (checkpoint_loader.py:335), which converts between
+    dtypes; a device target of another dtype gets the same values here, converted on the device."""
+    g = torch.Generator().manual_seed(9)
+    w = torch.randn(40, 30, generator=g)
+    steps = torch.arange(-50, 50, dtype=torch.int64)
+    data = {"w": w.to(DEV), "steps": steps.to(DEV), "same": w[:5].clone().to(DEV)}
+    cid, _, info = _write_direct(shm_dir, data)
+    oid = CheckpointObjectId.from_container(cid, "data_0_src0.distcp")
+    storage = {0: info["w"], 1: info["steps"], 2: info["same"]}
+    parent = torch.zeros(30, 40, dtype=torch.float64, device=DEV)
+    targets = {
+        "w_bf16": torch.zeros(40, 30, dtype=torch.bfloat16, device=DEV),
+        "w_f64_view": parent.t(),                                          # non-contiguous target of another dtype
+        "box_f16": torch.zeros(10, 7, dtype=torch.float16, device=DEV),    # sub-box of the stored tensor
+        "steps_f32": torch.zeros(100, dtype=torch.float32, device=DEV),
+        "same": torch.zeros(5, 30, device=DEV),
+    }
+    whole = lambda name, idx, shape: ReadItem(  # noqa: E731
+        type=LoadItemType.TENSOR, dest_index=MetadataIndex(name), dest_offsets=torch.Size([0] * len(shape)),
+        storage_index=idx, storage_offsets=torch.Size([0] * len(shape)), lengths=torch.Size(shape))
+    reqs = [
+        whole("w_bf16", 0, (40, 30)),
+        whole("w_f64_view", 0, (40, 30)),
+        ReadItem(type=LoadItemType.TENSOR, dest_index=MetadataIndex("box_f16"), dest_offsets=torch.Size([0, 0]),
+                 storage_index=0, storage_offsets=torch.Size([20, 3]), lengths=torch.Size([10, 7])),
+        whole("steps_f32", 1, (100,)),
+        whole("same", 2, (5, 30)),
+    ]
+    planner = _Planner(targets)
+    _loader().read_data(oid, reqs, planner, storage)
+    assert torch.equal(targets["w_bf16"].cpu(), w.to(torch.bfloat16))
+    assert torch.equal(parent.cpu(), w.to(torch.float64).t())
+    assert torch.equal(targets["box_f16"].cpu(), w[20:30, 3:10].to(torch.float16))
+    assert torch.equal(targets["steps_f32"].cpu(), steps.to(torch.float32))
+    assert torch.equal(targets["same"].cpu(), w[:5])
+    assert sorted(planner.committed) == sorted(targets)
+
+
 def test_multiple_buckets_and_overwrite_of_existing_object(shm_dir):
     data = {f"t{i}": torch.full((1000 + i,), float(i), device=DEV) for i in range(5)}
     data["b0"], data["b1"] = io.BytesIO(b"zero"), io.BytesIO(b"one")
