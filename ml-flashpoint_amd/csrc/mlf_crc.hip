@@ -1,9 +1,9 @@
 // CRC-32C (Castagnoli) of a checkpoint image: per-chunk values computed on the GPU, the same function on host
 // memory and on a byte range of a file, and the combine law.  Part of the library behind include/mlf_hip.h.
 //
-// Device side: per wavefront a 64 KiB segment is read as coalesced 1 KiB rows; every lane keeps four Horner
-// accumulators advanced by x^8192 through LDS tables, then lanes are folded with GF(2) multiplies; a second, tiny
-// kernel chains the segment values of every chunk.
+// Device side: per wavefront a segment (64 KiB to 512 KiB, by the size of the buffer) is read as coalesced 1 KiB
+// rows; every lane keeps four Horner accumulators advanced by x^8192 through LDS tables, then lanes are folded with
+// GF(2) multiplies; a second, tiny kernel chains the segment values of every chunk.
 #include "mlf_internal.h"
 
 #include <nmmintrin.h>
@@ -20,7 +20,6 @@ namespace mlf {
 struct CrcConsts {
   uint32_t row_tab[4][256];  // state advanced by one 1 KiB row, sliced by state byte
   uint32_t x4, x16, x32, x64, x128, x256, x512;  // x^(8*n) for the fold steps
-  uint32_t xseg;             // x^(8*kCrcSegBytes)
 };
 
 }  // namespace mlf
@@ -33,7 +32,10 @@ namespace {
 // CRC-32C
 // ---------------------------------------------------------------------------------------------------------
 constexpr uint32_t kPolyReflected = 0x82F63B78u;
-constexpr uint32_t kCrcSegBytes = 64 * 1024;  // bytes per wavefront
+constexpr uint32_t kCrcSegBytes = 64 * 1024;  // smallest segment (bytes per wavefront); chunks are multiples of it
+constexpr uint32_t kCrcMaxSegBytes = 512 * 1024;
+constexpr int kCrcTableCopies = 16;           // copies of the lookup tables in LDS, interleaved over the banks
+constexpr int kCrcThreads = 512;
 constexpr uint32_t kCrcRowBytes = 1024;       // one coalesced wavefront row: 64 lanes x 16 bytes
 
 // a(x) * b(x) mod P in the reflected representation (bit 31 is x^0).
@@ -67,23 +69,52 @@ __device__ __forceinline__ uint32_t crc_byte_step(uint32_t s, uint8_t b) {
 }
 
 // One wavefront per segment: raw remainder (zero initial state, no final xor) of the segment's bytes.
-__global__ void __launch_bounds__(256) mlf_crc_segments_kernel(const char* __restrict__ data, uint64_t nbytes,
-                                                               const CrcConsts* __restrict__ consts,
-                                                               uint32_t* __restrict__ seg_crc, uint32_t n_segs) {
-  __shared__ uint32_t tab[4][256];
-  for (uint32_t i = threadIdx.x; i < 1024; i += blockDim.x) tab[i >> 8][i & 255] = consts->row_tab[i >> 8][i & 255];
+//
+// The four 256-entry tables are kept R times in LDS, entry v of copy c at word v * R + c, and lane l reads copy
+// l % R: lookups with random v then spread over R times as many banks as a single copy would let them (measured on
+// random bytes: 4.2 conflict cycles per lookup with one copy, 2.0 with sixteen).  Folding the lanes costs about
+// 1 800 vector instructions per segment, as much as 50 rows of lookups: hence segments as long as the buffer allows.
+template <int R>
+__global__ void __launch_bounds__(kCrcThreads) mlf_crc_segments_kernel(const char* __restrict__ data, uint64_t nbytes,
+                                                                       const CrcConsts* __restrict__ consts,
+                                                                       uint32_t* __restrict__ seg_crc, uint32_t n_segs,
+                                                                       uint32_t seg_bytes) {
+  __shared__ uint32_t tab[4 * 256 * R];
+  for (uint32_t i = threadIdx.x; i < 1024; i += blockDim.x) {
+    const uint32_t v = consts->row_tab[i >> 8][i & 255];
+#pragma unroll
+    for (int c = 0; c < R; ++c) tab[i * R + c] = v;
+  }
   __syncthreads();
   const uint32_t seg = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (seg >= n_segs) return;
   const uint32_t lane = threadIdx.x & 63;
-  const uint64_t seg_off = (uint64_t)seg * kCrcSegBytes;
+  const uint32_t* my = tab + (lane & (R - 1));
+  const uint64_t seg_off = (uint64_t)seg * seg_bytes;
   const uint64_t remaining = nbytes - seg_off;
-  const uint32_t seg_len = remaining < kCrcSegBytes ? (uint32_t)remaining : kCrcSegBytes;
+  const uint32_t seg_len = remaining < seg_bytes ? (uint32_t)remaining : seg_bytes;
   const uint32_t rows = seg_len / kCrcRowBytes;
   const u32x4* p = reinterpret_cast<const u32x4*>(data + seg_off) + lane;
   uint32_t a0 = 0, a1 = 0, a2 = 0, a3 = 0;
-#define MLF_ROW_ADV(a) (tab[0][(a) & 255] ^ tab[1][((a) >> 8) & 255] ^ tab[2][((a) >> 16) & 255] ^ tab[3][(a) >> 24])
-  for (uint32_t r = 0; r < rows; ++r) {
+#define MLF_ROW_ADV(a)                                                                                   \
+  (my[((a) & 255u) * R] ^ my[(256u + (((a) >> 8) & 255u)) * R] ^ my[(512u + (((a) >> 16) & 255u)) * R] ^ \
+   my[(768u + ((a) >> 24)) * R])
+  uint32_t r = 0;
+  // four rows are requested before the first of them is used: bytes in flight per wavefront that cover the memory
+  // latency at the occupancy the tables leave
+  for (; r + 4 <= rows; r += 4) {
+    u32x4 v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] = __builtin_nontemporal_load(p + (size_t)(r + k) * 64);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      a0 = MLF_ROW_ADV(a0) ^ v[k].x;
+      a1 = MLF_ROW_ADV(a1) ^ v[k].y;
+      a2 = MLF_ROW_ADV(a2) ^ v[k].z;
+      a3 = MLF_ROW_ADV(a3) ^ v[k].w;
+    }
+  }
+  for (; r < rows; ++r) {
     const u32x4 v = __builtin_nontemporal_load(p + (size_t)r * 64);
     a0 = MLF_ROW_ADV(a0) ^ v.x;
     a1 = MLF_ROW_ADV(a1) ^ v.y;
@@ -140,7 +171,6 @@ void crc_init_host() {
   g_crc_host.x128 = x_pow_bytes(128);
   g_crc_host.x256 = x_pow_bytes(256);
   g_crc_host.x512 = x_pow_bytes(512);
-  g_crc_host.xseg = x_pow_bytes(kCrcSegBytes);
 }
 
 }  // namespace
@@ -164,8 +194,11 @@ int crc_enqueue(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint
   if (chunk_bytes == 0 || chunk_bytes % kCrcSegBytes)
     return fail(MLF_HIP_BAD_ARG, "chunk_bytes must be a positive multiple of 65536");
   const uint64_t n_chunks = (nbytes + chunk_bytes - 1) / chunk_bytes;
-  const uint64_t n_segs = (nbytes + kCrcSegBytes - 1) / kCrcSegBytes;
   if (n_out < n_chunks) return fail(MLF_HIP_BAD_ARG, "output array too small");
+  // the longest segment that divides the chunks and still leaves every CU several blocks of wavefronts
+  uint64_t seg_bytes = kCrcSegBytes;
+  while (seg_bytes < kCrcMaxSegBytes && chunk_bytes % (2 * seg_bytes) == 0 && nbytes / (2 * seg_bytes) >= 8192) seg_bytes *= 2;
+  const uint64_t n_segs = (nbytes + seg_bytes - 1) / seg_bytes;
   if (n_segs > 0xFFFFFFF0ull) return fail(MLF_HIP_BAD_ARG, "buffer too large for one CRC call");
   std::call_once(g_crc_once, crc_init_host);
   job->n_chunks = n_chunks;
@@ -183,13 +216,15 @@ int crc_enqueue(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint
   CRC_TRY(hipMalloc(reinterpret_cast<void**>(&job->d_out), n_chunks * sizeof(uint32_t)));
   CRC_TRY(hipHostMalloc(reinterpret_cast<void**>(&job->h_out), n_chunks * sizeof(uint32_t), hipHostMallocDefault));
   CRC_TRY(hipMemcpyAsync(job->d_consts, &g_crc_host, sizeof(CrcConsts), hipMemcpyHostToDevice, stream));
-  const uint32_t grid = (uint32_t)((n_segs + 3) / 4);
-  hipLaunchKernelGGL(mlf_crc_segments_kernel, dim3(grid), dim3(256), 0, stream, static_cast<const char*>(dev_ptr),
-                     nbytes, job->d_consts, job->d_seg, (uint32_t)n_segs);
+  const uint32_t waves_per_block = kCrcThreads / 64;
+  const uint32_t grid = (uint32_t)((n_segs + waves_per_block - 1) / waves_per_block);
+  hipLaunchKernelGGL(mlf_crc_segments_kernel<kCrcTableCopies>, dim3(grid), dim3(kCrcThreads), 0, stream,
+                     static_cast<const char*>(dev_ptr), nbytes, job->d_consts, job->d_seg, (uint32_t)n_segs,
+                     (uint32_t)seg_bytes);
   CRC_TRY(hipGetLastError());
-  const uint64_t last_seg_len = nbytes - (n_segs - 1) * kCrcSegBytes;
+  const uint64_t last_seg_len = nbytes - (n_segs - 1) * seg_bytes;
   hipLaunchKernelGGL(mlf_crc_chunks_kernel, dim3((uint32_t)((n_chunks + 63) / 64)), dim3(64), 0, stream, job->d_seg,
-                     (uint32_t)(chunk_bytes / kCrcSegBytes), (uint32_t)n_segs, g_crc_host.xseg,
+                     (uint32_t)(chunk_bytes / seg_bytes), (uint32_t)n_segs, x_pow_bytes(seg_bytes),
                      x_pow_bytes(last_seg_len), job->d_out, (uint32_t)n_chunks);
   CRC_TRY(hipGetLastError());
   CRC_TRY(hipMemcpyAsync(job->h_out, job->d_out, n_chunks * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));

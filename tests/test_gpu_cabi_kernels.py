@@ -546,6 +546,41 @@ def test_crc32c_device_matches_oracle(nbytes, oracle_c):
         assert whole == oracle_c.oracle_crc32c(raw, nbytes)
 
 
+@pytest.mark.parametrize("gib_x2,chunk", [(3, 32 << 20), (17, 32 << 20), (17, 3 << 16)])
+def test_crc32c_device_on_buffers_large_enough_for_long_segments(gib_x2, chunk, oracle_c):
+    """Buffers of 1.5 and 8.5 GiB are cut into segments of 128 and 512 KiB per wavefront (64 KiB where the chunk size
+    allows nothing longer).  Every chunk value, the ragged last one included, is compared with the host routine's
+    (SSE4.2, itself held to the oracle by the small cases) and a sample of them with the oracle's byte-table routine;
+    the chunk values chain to the checksum of the whole buffer."""
+    from ml_flashpoint.hip import plan as P
+
+    gen = torch.Generator().manual_seed(gib_x2)
+    block = torch.randint(0, 256, (1 << 29,), dtype=torch.uint8, generator=gen)
+    nbytes = gib_x2 * (1 << 29) - 54321
+    dev = block.to(DEV).repeat(gib_x2)
+    dev[(5 << 28) + 77 :: 1 << 29] ^= 0x5A  # the repeats differ, at places inside segments
+    got = P.crc32c_device(dev, nbytes, chunk)
+    n_chunks = -(-nbytes // chunk)
+    assert len(got) == n_chunks
+    sampled = {0, 1, n_chunks // 2, n_chunks - 2, n_chunks - 1}
+    step = (1 << 29) // chunk * chunk  # host copies are cut on chunk boundaries
+    whole = None
+    for start in range(0, nbytes, step):
+        raw = dev[start : min(start + step, nbytes)].cpu().numpy()
+        for off in range(0, raw.size, chunk):
+            k = (start + off) // chunk
+            n = min(chunk, raw.size - off)
+            assert P.crc32c_host(raw.ctypes.data + off, n) == int(got[k]), f"chunk {k}"
+            if k in sampled:
+                assert oracle_c.oracle_crc32c(ctypes.cast(ctypes.c_void_p(raw.ctypes.data + off), ctypes.c_char_p), n) == int(got[k]), f"chunk {k}"
+        part = P.crc32c_host(raw.ctypes.data, raw.size)
+        whole = part if whole is None else P.crc32c_combine(whole, part, raw.size)
+    chained = int(got[0])
+    for k in range(1, n_chunks):
+        chained = P.crc32c_combine(chained, int(got[k]), min(chunk, nbytes - k * chunk))
+    assert chained == whole
+
+
 def test_crc32c_known_vectors_on_device(oracle_c):
     from ml_flashpoint.hip import plan as P
 
