@@ -1,4 +1,4 @@
-"""BASELINE config 1 on the CPU: a GPT-2-small-shaped fp32 state dict goes through the PyTorch DCP adapters into
+"""The benchmark's CPU-runnable configuration: a GPT-2-small-shaped fp32 state dict goes through the PyTorch DCP adapters into
 buffer files and back, bit-exactly, with the CPU oracle's saver/loader as the plug-ins.
 
 This exercises the host logic of the adapters (plan -> buckets -> results -> metadata -> read plan) without a GPU and

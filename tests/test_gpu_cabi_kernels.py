@@ -122,7 +122,7 @@ def test_pack_misaligned_sources():
 
 
 def _views(base):
-    """Non-contiguous views of a 3-D base, the kinds BASELINE's strided config names plus a few more."""
+    """Non-contiguous views of a 3-D base, the kinds the benchmark's strided-views configuration names plus a few more."""
     m = base[0]
     return [
         m.t(),  # transposed

@@ -159,7 +159,7 @@ def test_dcp_save_bytes_equal_oracle_and_load_is_bit_exact(shm_dir, manager_futu
 
 
 def test_gpt2_small_config_on_device(shm_dir, manager_future):
-    """BASELINE config 1's state dict, resident on the GPU, saved by the gfx950 saver: same bytes as the oracle."""
+    """The GPT-2-small-shaped fp32 state dict (the benchmark's CPU-runnable configuration), resident on the GPU, saved by the gfx950 saver: same bytes as the oracle."""
     sd_dev = workloads.gpt2_small(device=DEV, layers=3, d=256, vocab=5003, ctx=128)
     sd_cpu = {k: v.cpu() for k, v in sd_dev.items()}
     ckpt = os.path.join(shm_dir, "step-1_ckpt")

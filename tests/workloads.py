@@ -1,4 +1,4 @@
-"""Seeded synthetic state dicts in the shapes BASELINE.json's configs name (shared by the tests and bench.py).
+"""Seeded synthetic state dicts in the shapes of the benchmark's configurations (shared by the tests and bench.py).
 
 Values are generated with ``torch.Generator`` seeds fixed per config, on the requested device; ``scale`` shrinks a
 config for quick tests by dividing layer counts / widths, keeping the tensor structure.
