@@ -168,6 +168,17 @@ int mlf_engine_d2h_crc(mlf_engine* engine, const void* src_dev, void* dst_host, 
                        void* producer_stream, uint64_t crc_chunk_bytes, uint32_t* crc_out_host,
                        uint64_t n_crc_out, mlf_xfer_stats* stats);
 
+/* mlf_engine_d2h_crc (`crc_chunk_bytes` may be 0: no checksums) that also publishes its progress: whenever a
+ * further slot has reached `dst_host`, the number of leading bytes of the range that are in place is stored into
+ * `*landed` (8-byte aligned host memory of the caller) with release ordering; a reader that loads it with acquire
+ * ordering may read that many bytes of the destination.  0 is stored before the first copy, `nbytes` with the
+ * last.  For a sender that forwards an object to its replica while the rest is still crossing the link: the
+ * reference hands the buffer to its replication manager only after the whole object is written
+ * (checkpoint_saver.py:700-707, replication_manager.py:248-300). */
+int mlf_engine_d2h_watched(mlf_engine* engine, const void* src_dev, void* dst_host, uint64_t nbytes,
+                           void* producer_stream, uint64_t crc_chunk_bytes, uint32_t* crc_out_host,
+                           uint64_t n_crc_out, uint64_t* landed, mlf_xfer_stats* stats);
+
 /* Host -> device.  Copies `nbytes` from `src_host` (pageable, e.g. the read-only mapping) to `dst_dev`
  * and makes `consumer_stream` wait for the last chunk, so an unpack launched on it afterwards sees the data.
  * Returns once all chunks are enqueued and the host source is no longer needed.  Replaces BufferIO.read()'s

@@ -220,6 +220,7 @@ struct CrcRequest {
   uint64_t chunk_bytes = 0;  // 0: no checksum
   uint32_t* out_host = nullptr;
   uint64_t n_out = 0;
+  uint64_t* landed = nullptr;  // progress counter of the caller, or null
 };
 
 int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t nbytes, void* producer_stream,
@@ -233,6 +234,7 @@ int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t
   HIP_TRY(hipEventRecord(e->gate, static_cast<hipStream_t>(producer_stream)));
   for (hipStream_t s : e->streams) HIP_TRY(hipStreamWaitEvent(s, e->gate, 0));
   const char* src = static_cast<const char*>(src_dev);
+  if (crc.landed) __atomic_store_n(crc.landed, (uint64_t)0, __ATOMIC_RELEASE);
   CrcJob crc_job;
   const bool want_crc = crc.chunk_bytes != 0 && nbytes != 0;
   if (want_crc) {
@@ -274,6 +276,7 @@ int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t
     if (c == 0) wait = now_s() - w0;
     if (int err = pool_host_copy(*e->pool, host, off, e->slots[s], len, true))
       return fail(MLF_HIP_RUNTIME, std::string("pwrite() to the buffer file failed: ") + strerror(err));
+    if (crc.landed) __atomic_store_n(crc.landed, off + len, __ATOMIC_RELEASE);  // the host threads' stores come first
     if (c + n_slots < n_chunks)
       if (int rc = issue(c + n_slots)) return rc;
   }
@@ -356,6 +359,21 @@ int mlf_engine_d2h_crc(mlf_engine* e, const void* src_dev, void* dst_host, uint6
   crc.chunk_bytes = crc_chunk_bytes;
   crc.out_host = crc_out_host;
   crc.n_out = n_crc_out;
+  return engine_d2h(e, src_dev, host, nbytes, producer_stream, stats, crc);
+}
+
+int mlf_engine_d2h_watched(mlf_engine* e, const void* src_dev, void* dst_host, uint64_t nbytes, void* producer_stream,
+                           uint64_t crc_chunk_bytes, uint32_t* crc_out_host, uint64_t n_crc_out, uint64_t* landed,
+                           mlf_xfer_stats* stats) {
+  if (crc_chunk_bytes && !crc_out_host) return fail(MLF_HIP_BAD_ARG, "null checksum output");
+  if (reinterpret_cast<uintptr_t>(landed) & 7) return fail(MLF_HIP_BAD_ARG, "progress counter must be 8-byte aligned");
+  HostEnd host;
+  host.ptr = static_cast<char*>(dst_host);
+  CrcRequest crc;
+  crc.chunk_bytes = crc_chunk_bytes;
+  crc.out_host = crc_out_host;
+  crc.n_out = n_crc_out;
+  crc.landed = landed;
   return engine_d2h(e, src_dev, host, nbytes, producer_stream, stats, crc);
 }
 

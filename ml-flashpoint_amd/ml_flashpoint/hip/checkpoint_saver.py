@@ -15,6 +15,7 @@ them (checkpoint_saver.py:340-343,533-619,709-762).
 """
 
 import concurrent.futures
+import ctypes
 import dataclasses
 import logging
 import os
@@ -123,6 +124,15 @@ class StagedObject:
         self.collected = False
         self.packed_event: Optional[torch.cuda.Event] = None  # recorded behind the pack on the producer's stream
         self.owns_plan = True  # False: the plan is kept by the saver for the next save
+        self._landed = ctypes.c_uint64(0)  # kept current by the copy engine while the image crosses the link
+        self.data_offset: Optional[int] = None  # position of the image's first byte in the object's data section
+
+    def landed_bytes(self) -> int:
+        """Leading bytes of the image that are in place in the buffer file (from byte 4096 + ``data_offset`` of the
+        file on; ``data_offset`` is None until the transfer has begun).  Grows while the transfer runs: a sender
+        that forwards the object to a replica can follow it instead of waiting for the whole object, which is
+        when the reference starts (checkpoint_saver.py:700-707)."""
+        return int(self._landed.value)
 
     def __reduce__(self):
         if self.future is None or self.done_marker is None:
@@ -699,12 +709,14 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                         if self._crc_chunk_bytes:
                             crcs = hip_plan.crc32c_device(staged.image, nbytes, self._crc_chunk_bytes, staged.stream)
                         st = engine.d2h_fd(staged.image.data_ptr(), fd, METADATA_SIZE + start, nbytes, staged.stream)
-                    elif self._crc_chunk_bytes:
-                        # checksum kernels run on the engine's third stream while the chunks cross the link
-                        st, crcs = engine.d2h_crc(staged.image.data_ptr(), writer.data_address(start), nbytes,
-                                                  staged.stream, self._crc_chunk_bytes)
                     else:
-                        st = engine.d2h(staged.image.data_ptr(), writer.data_address(start), nbytes, staged.stream)
+                        # checksum kernels (if asked for) run on the engine's third stream while the chunks cross
+                        # the link; the engine keeps the object's progress counter current
+                        staged.data_offset = start
+                        st, crcs = engine.d2h_watched(staged.image.data_ptr(), writer.data_address(start), nbytes,
+                                                      staged.stream, self._crc_chunk_bytes, staged._landed)
+                    staged.data_offset = start
+                    staged._landed.value = nbytes
                     xfer["d2h_s"] += st.seconds
                     xfer["d2h_wait_s"] += st.wait_seconds
                     xfer["d2h_bytes"] += nbytes

@@ -306,6 +306,21 @@ class CopyEngine:
         )
         return stats, crcs[:n_chunks]
 
+    def d2h_watched(self, src_dev_ptr: int, dst_host_ptr: int, nbytes: int, producer_stream: int, crc_chunk_bytes: int,
+                    landed: "ctypes.c_uint64"):
+        """``d2h_crc`` (``crc_chunk_bytes`` 0: no checksums) that keeps ``landed`` at the number of leading bytes
+        that have reached the destination, for a reader on another thread.  Returns (stats, checksums or None)."""
+        stats = _lib.XferStats()
+        n_chunks = (nbytes + crc_chunk_bytes - 1) // crc_chunk_bytes if crc_chunk_bytes else 0
+        crcs = np.zeros(max(n_chunks, 1), dtype=np.uint32)
+        _lib.check(
+            _lib.load().mlf_engine_d2h_watched(self._handle, src_dev_ptr, dst_host_ptr, nbytes, producer_stream,
+                                               crc_chunk_bytes, crcs.ctypes.data, len(crcs), ctypes.addressof(landed),
+                                               ctypes.byref(stats)),
+            "mlf_engine_d2h_watched",
+        )
+        return stats, (crcs[:n_chunks] if crc_chunk_bytes else None)
+
     def h2d(self, src_host_ptr: int, dst_dev_ptr: int, nbytes: int, consumer_stream: int = 0) -> _lib.XferStats:
         stats = _lib.XferStats()
         _lib.check(

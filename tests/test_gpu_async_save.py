@@ -177,3 +177,42 @@ def test_next_save_does_not_wait_for_the_previous_transfer(shm_dir, manager_futu
         assert raw.read() == torch.full((1 << 18,), 5.0).numpy().tobytes()  # the tail of the last big tensor
     complete(*second)  # finalizing the newer checkpoint removes the older one in the background
     _check_files(second[0], snapshot)
+
+
+def test_a_follower_can_forward_the_object_while_it_is_still_being_written(shm_dir, manager_future):
+    """The staged object publishes how much of its image has reached the buffer file; a follower that reads the file
+    behind that mark (what a replication sender would do instead of waiting for the whole object) ends up with the
+    object's data section, and has seen the transfer under way."""
+    from ml_flashpoint.checkpoint_object_manager.buffer_metadata import METADATA_SIZE
+
+    saver = _make_saver(background_write=True)
+    sd = {f"big.{i}": torch.randn(1 << 28, device=DEV) for i in range(2)}  # 2 GiB: some 65 slots of 32 MiB
+    cid = CheckpointContainerId(os.path.join(shm_dir, "step-20_ckpt"))
+    saver.initialize_checkpoint(cid)
+    writer = MemoryStorageWriter(saver, manager_future)
+    writer.reset(cid.data)
+    dist = _DistWrapper(None, False, 0)
+    buckets, metadata, *_ = statedictsaver.generate_plan(cid, sd, writer, DefaultSavePlanner(), dist)
+    staged = saver._staged_of(buckets[0])
+    total = staged.layout.image_bytes
+    path = str(buckets[0].object_id)
+    marks, replica = [], bytearray()
+    deadline = time.perf_counter() + 60
+    fd = None
+    while len(replica) < total and time.perf_counter() < deadline:
+        mark = staged.landed_bytes()
+        if mark > len(replica):
+            fd = fd if fd is not None else os.open(path, os.O_RDONLY)
+            marks.append(mark)
+            replica += os.pread(fd, mark - len(replica), METADATA_SIZE + staged.data_offset + len(replica))
+        else:
+            time.sleep(0.001)
+    assert len(replica) == total and marks == sorted(marks)
+    assert len(marks) >= 3, "the follower only ever saw the finished object"
+    statedictsaver.write_data(cid, writer, buckets, replicate_after_write=False)
+    statedictsaver.finish_write(cid, writer, metadata, dist)
+    saver.finalize_checkpoint(cid)
+    os.close(fd)
+    with open(path, "rb") as f:
+        f.seek(METADATA_SIZE)
+        assert f.read() == replica

@@ -639,3 +639,59 @@ def test_copy_engine_round_trip(nbytes, shm_dir, oracle_c):
     bo.close()
     bo2.close()
     engine.destroy()
+
+
+def test_watched_transfer_publishes_only_bytes_that_are_in_place(shm_dir, oracle_c):
+    """While a 200 MiB image crosses the link in 1 MiB slots, a second thread follows the progress counter and copies
+    whatever prefix it announces out of the mapping: the counter only grows, never runs ahead of the data, ends at the
+    full size, and the follower's copy is the image.  Checksums equal those of the unwatched call."""
+    import threading
+
+    from ml_flashpoint.checkpoint_object_manager.buffer_object.buffer_object_ext import BufferObject
+    from ml_flashpoint.hip import plan as P
+
+    nbytes = (200 << 20) + 4321
+    gen = torch.Generator().manual_seed(200)
+    host = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=gen)
+    want = host.numpy()
+    dev = host.to(DEV)
+    engine = P.CopyEngine(slot_bytes=1 << 20, n_slots=3, n_threads=4)
+    bo = BufferObject(f"{shm_dir}/watched.bin", 4096 + nbytes, True)
+    view = np.frombuffer(memoryview(bo), dtype=np.uint8)[4096:]
+    landed = ctypes.c_uint64(12345)  # whatever was there before is overwritten with 0 first
+    replica = np.zeros(nbytes, dtype=np.uint8)
+    seen, done = [], threading.Event()
+
+    def follow():
+        have = 0
+        while have < nbytes and not done.wait(0.0005):
+            now = int(landed.value)
+            if now == 12345:
+                continue  # the call has not begun
+            if now != have:
+                seen.append(now)
+                replica[have:now] = view[have:now]
+                have = now
+        now = int(landed.value)
+        replica[have:now] = view[have:now]
+        seen.append(now)
+
+    follower = threading.Thread(target=follow)
+    follower.start()
+    stream = torch.cuda.current_stream().cuda_stream
+    stats, crcs = engine.d2h_watched(dev.data_ptr(), bo.get_data_ptr() + 4096, nbytes, stream, 1 << 20, landed)
+    follower.join(30)
+    done.set()
+    follower.join()
+    assert int(landed.value) == nbytes and stats.bytes == nbytes
+    assert seen == sorted(seen) and seen[-1] == nbytes
+    assert len(set(seen)) >= 3, "the follower never saw the transfer under way"
+    assert all(v % (1 << 20) == 0 for v in seen if v != nbytes)  # whole slots
+    assert np.array_equal(replica, want) and np.array_equal(view, want)
+    _, plain = engine.d2h_crc(dev.data_ptr(), bo.get_data_ptr() + 4096, nbytes, stream, 1 << 20)
+    assert crcs.tolist() == plain.tolist()
+    _, none = engine.d2h_watched(dev.data_ptr(), bo.get_data_ptr() + 4096, 4097, stream, 0, landed)
+    assert none is None and int(landed.value) == 4097
+    del view
+    bo.close()
+    engine.destroy()
