@@ -188,7 +188,7 @@ void crc_release(CrcJob* job) {
 
 // Enqueues the two CRC kernels and the copy of the per-chunk values on `stream`; does not wait.
 int crc_enqueue(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint64_t n_out, hipStream_t stream,
-                CrcJob* job) {
+                CrcJob* job, bool background) {
   if (!dev_ptr) return fail(MLF_HIP_BAD_ARG, "null pointer");
   if (reinterpret_cast<uintptr_t>(dev_ptr) & 15) return fail(MLF_HIP_BAD_ARG, "device buffer must be 16-byte aligned");
   if (chunk_bytes == 0 || chunk_bytes % kCrcSegBytes)
@@ -216,11 +216,19 @@ int crc_enqueue(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint
   CRC_TRY(hipMalloc(reinterpret_cast<void**>(&job->d_out), n_chunks * sizeof(uint32_t)));
   CRC_TRY(hipHostMalloc(reinterpret_cast<void**>(&job->h_out), n_chunks * sizeof(uint32_t), hipHostMallocDefault));
   CRC_TRY(hipMemcpyAsync(job->d_consts, &g_crc_host, sizeof(CrcConsts), hipMemcpyHostToDevice, stream));
-  const uint32_t waves_per_block = kCrcThreads / 64;
-  const uint32_t grid = (uint32_t)((n_segs + waves_per_block - 1) / waves_per_block);
-  hipLaunchKernelGGL(mlf_crc_segments_kernel<kCrcTableCopies>, dim3(grid), dim3(kCrcThreads), 0, stream,
-                     static_cast<const char*>(dev_ptr), nbytes, job->d_consts, job->d_seg, (uint32_t)n_segs,
-                     (uint32_t)seg_bytes);
+  if (background) {
+    // one copy of the tables (4 KiB of LDS per workgroup instead of 64 KiB): the CUs' LDS stays available to the
+    // kernels this pass runs beside
+    const uint32_t grid = (uint32_t)((n_segs + 3) / 4);
+    hipLaunchKernelGGL(mlf_crc_segments_kernel<1>, dim3(grid), dim3(256), 0, stream, static_cast<const char*>(dev_ptr),
+                       nbytes, job->d_consts, job->d_seg, (uint32_t)n_segs, (uint32_t)seg_bytes);
+  } else {
+    const uint32_t waves_per_block = kCrcThreads / 64;
+    const uint32_t grid = (uint32_t)((n_segs + waves_per_block - 1) / waves_per_block);
+    hipLaunchKernelGGL(mlf_crc_segments_kernel<kCrcTableCopies>, dim3(grid), dim3(kCrcThreads), 0, stream,
+                       static_cast<const char*>(dev_ptr), nbytes, job->d_consts, job->d_seg, (uint32_t)n_segs,
+                       (uint32_t)seg_bytes);
+  }
   CRC_TRY(hipGetLastError());
   const uint64_t last_seg_len = nbytes - (n_segs - 1) * seg_bytes;
   hipLaunchKernelGGL(mlf_crc_chunks_kernel, dim3((uint32_t)((n_chunks + 63) / 64)), dim3(64), 0, stream, job->d_seg,
@@ -312,7 +320,7 @@ int mlf_crc32c_device(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes
                       uint64_t n_out, void* stream_) {
   if (nbytes == 0) return MLF_HIP_OK;
   CrcJob job;
-  if (int rc = crc_enqueue(dev_ptr, nbytes, chunk_bytes, n_out, static_cast<hipStream_t>(stream_), &job)) return rc;
+  if (int rc = crc_enqueue(dev_ptr, nbytes, chunk_bytes, n_out, static_cast<hipStream_t>(stream_), &job, false)) return rc;
   return crc_finish(&job, out_host);
 }
 

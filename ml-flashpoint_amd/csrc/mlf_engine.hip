@@ -241,7 +241,7 @@ int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t
     // the image is complete once the gate has passed and is not modified afterwards, so its checksum can be
     // computed while the link-bound copies run: it costs neither blocking time nor transfer time
     HIP_TRY(hipStreamWaitEvent(e->crc_stream, e->gate, 0));
-    if (int rc = crc_enqueue(src_dev, nbytes, crc.chunk_bytes, crc.n_out, e->crc_stream, &crc_job)) return rc;
+    if (int rc = crc_enqueue(src_dev, nbytes, crc.chunk_bytes, crc.n_out, e->crc_stream, &crc_job, true)) return rc;
   }
   struct CrcGuard {  // scratch is released on every exit path, after the kernels that use it have finished
     CrcJob* job;
