@@ -186,6 +186,11 @@ int mlf_engine_d2h_watched(mlf_engine* engine, const void* src_dev, void* dst_ho
 int mlf_engine_h2d(mlf_engine* engine, const void* src_host, void* dst_dev, uint64_t nbytes,
                    void* consumer_stream, mlf_xfer_stats* stats);
 
+/* Host -> host on the engine's threads: `nbytes` from `src_host` to `dst_host` (ranges must not overlap).  For
+ * checkpoint items that are resident in host memory - the reference copies those into the mapping with torch's
+ * intra-op threads (checkpoint_saver.py:443-450,797-800); they do not visit the device here either. */
+int mlf_engine_host_copy(mlf_engine* engine, void* dst_host, const void* src_host, uint64_t nbytes);
+
 /* The same two transfers with the pageable end given as a byte range of an open file instead of a pointer:
  * the host threads pwrite()/pread() the pinned slots straight to/from the buffer file (`fd` from
  * mlf_buffer_fd(), `file_offset` = 4096 + position in the data section).  The bytes land in the same page-cache

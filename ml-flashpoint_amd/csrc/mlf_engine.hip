@@ -377,6 +377,14 @@ int mlf_engine_d2h_watched(mlf_engine* e, const void* src_dev, void* dst_host, u
   return engine_d2h(e, src_dev, host, nbytes, producer_stream, stats, crc);
 }
 
+int mlf_engine_host_copy(mlf_engine* e, void* dst_host, const void* src_host, uint64_t nbytes) {
+  if (!e) return fail(MLF_HIP_BAD_ARG, "null engine");
+  if (nbytes && (!dst_host || !src_host)) return fail(MLF_HIP_BAD_ARG, "null pointer");
+  std::lock_guard<std::mutex> g(e->busy);  // the threads are the ones a transfer uses
+  pool_memcpy(*e->pool, static_cast<char*>(dst_host), static_cast<const char*>(src_host), nbytes);
+  return MLF_HIP_OK;
+}
+
 int mlf_engine_d2h_fd(mlf_engine* e, const void* src_dev, int fd, uint64_t file_offset, uint64_t nbytes,
                       void* producer_stream, mlf_xfer_stats* stats) {
   if (fd < 0) return fail(MLF_HIP_BAD_ARG, "bad file descriptor");

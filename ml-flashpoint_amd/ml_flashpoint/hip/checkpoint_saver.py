@@ -75,6 +75,10 @@ class EngineConfig:
         return max(1, min(16, cpus))
 
 
+# host-resident tensors of at least this many bytes go from host memory straight into the buffer; smaller ones ride
+# in the image with the headers (one copy more, no extra pieces in the transfer)
+_HOST_DIRECT_MIN_BYTES = 256 << 10
+
 _MAX_KEPT_PLANS = 64  # objects per save are few (one per writer thread); beyond this the oldest is rebuilt
 
 
@@ -83,7 +87,8 @@ class _KeptPlan:
 
     def __init__(self, key, layout: hip_plan.SaveLayout, plan: hip_plan.Plan, device: torch.device):
         self.key, self.plan, self.device = key, plan, device
-        self.layout = dataclasses.replace(layout, device_tensors=[])  # the table has the addresses; hold no tensors
+        # the table has the device addresses and host tensors are looked up again by index: hold no tensors
+        self.layout = dataclasses.replace(layout, device_tensors=[], host_tensors=[])
         self.blob = layout.blob
 
     def refreshed_blob(self, tensors, blobs) -> Optional[bytes]:
@@ -441,9 +446,13 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             device = kept.device
             fresh_blob = kept.refreshed_blob(tensors, blobs)
             layout = dataclasses.replace(kept.layout, blob=kept.blob,
-                                         device_tensors=[t for t in tensors if t.device.type != "cpu"])
+                                         device_tensors=[t for t in tensors if t.device.type != "cpu"],
+                                         host_tensors=[tensors[i] for _, _, i in kept.layout.host_spans])
         else:
-            layout = hip_plan.build_save_layout(tensors, blobs)
+            # through the file descriptor (pwrite) everything goes through the image; the direct host copy
+            # writes into the mapping
+            layout = hip_plan.build_save_layout(tensors, blobs,
+                                                None if self._use_file_io else _HOST_DIRECT_MIN_BYTES)
             device = next((t.device for t in tensors if t.device.type != "cpu"), None)
             if any(t.device != device for t in tensors if t.device.type != "cpu"):
                 raise ValueError("all device tensors of one checkpoint object must live on the same device")
@@ -454,6 +463,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         stream = 0
         if layout.image_bytes and object_id is not None and layout.image_bytes > self._image_limit(device):
             self._drop_kept_plan(object_name)
+            if layout.host_spans:  # the windowed mode sends one image, whole: lay the host items out inside it
+                layout = hip_plan.build_save_layout(tensors, blobs)
             return self._stage_windowed(layout, items, object_id, object_name, device, stats)
         if layout.image_bytes:
             with torch.cuda.device(device):
@@ -686,7 +697,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
 
     def _transfer_bucket(self, staged: StagedObject, bucket: ObjectWriteBucket, xfer: dict) -> list[WriteResult]:
         layout = staged.layout
-        nbytes = layout.image_bytes
+        nbytes = layout.data_bytes
         crcs = None
         with self._chkpt_obj_manager.acquire_buffer(
             bucket.object_id, max(self._initial_buffer_size_bytes, nbytes, 1)
@@ -703,23 +714,23 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                     _lib.check(_lib.load().mlf_hip_set_device(staged.device_index), "mlf_hip_set_device")
                     start = writer.tell()
                     writer.next_buffer_slice(nbytes).release()  # bounds check + position/high-water mark
+                    staged.data_offset = start
                     fd = writer.fileno() if self._use_file_io else -1
                     engine = self._get_engine()
-                    if fd >= 0:
+                    if layout.host_spans:
+                        crcs = self._transfer_in_pieces(staged, writer, start, xfer)
+                    elif fd >= 0:
                         if self._crc_chunk_bytes:
                             crcs = hip_plan.crc32c_device(staged.image, nbytes, self._crc_chunk_bytes, staged.stream)
                         st = engine.d2h_fd(staged.image.data_ptr(), fd, METADATA_SIZE + start, nbytes, staged.stream)
+                        self._count_transfer(xfer, st, nbytes)
                     else:
                         # checksum kernels (if asked for) run on the engine's third stream while the chunks cross
                         # the link; the engine keeps the object's progress counter current
-                        staged.data_offset = start
                         st, crcs = engine.d2h_watched(staged.image.data_ptr(), writer.data_address(start), nbytes,
                                                       staged.stream, self._crc_chunk_bytes, staged._landed)
-                    staged.data_offset = start
+                        self._count_transfer(xfer, st, nbytes)
                     staged._landed.value = nbytes
-                    xfer["d2h_s"] += st.seconds
-                    xfer["d2h_wait_s"] += st.wait_seconds
-                    xfer["d2h_bytes"] += nbytes
         staged.consumed = True
         staged.image = None
         if staged.plan is not None and staged.owns_plan:
@@ -728,6 +739,42 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         if crcs is not None:
             integrity.write_sidecar(str(bucket.object_id), self._crc_chunk_bytes, nbytes, crcs)
         return self._results_of(staged, bucket.object_name)
+
+    @staticmethod
+    def _count_transfer(xfer: dict, st, nbytes: int) -> None:
+        xfer["d2h_s"] += st.seconds
+        xfer["d2h_wait_s"] += st.wait_seconds
+        xfer["d2h_bytes"] += nbytes
+
+    def _transfer_in_pieces(self, staged: StagedObject, writer, start: int, xfer: dict):
+        """The transfer of an object some of whose tensors live in host memory: the runs of the image between them
+        cross the host link, the host-resident payloads are copied from where they are into their places in the
+        buffer, in the order of the data section.  Returns the chunk checksums (taken on the host, from the pages
+        just written: the image alone is not the object) or None."""
+        layout = staged.layout
+        engine = self._get_engine()
+        pieces = [(data_off, n, image_off, None) for image_off, data_off, n in layout.segments]
+        pieces += [(data_off, n, None, t) for (data_off, n, _), t in zip(layout.host_spans, layout.host_tensors)]
+        t_host = 0.0
+        for data_off, n, image_off, tensor in sorted(pieces, key=lambda piece: piece[0]):
+            dst = writer.data_address(start + data_off)
+            if tensor is None:
+                st = engine.d2h(staged.image.data_ptr() + image_off, dst, n, staged.stream)
+                self._count_transfer(xfer, st, n)
+            else:
+                t0 = time.perf_counter()
+                source = tensor.detach().contiguous()  # a copy only if the tensor is a strided view
+                assert source.numel() * source.element_size() == n
+                engine.host_copy(dst, source.data_ptr(), n)
+                t_host += time.perf_counter() - t0
+                xfer["host_copy_bytes"] = xfer.get("host_copy_bytes", 0) + n
+            staged._landed.value = data_off + n
+        xfer["host_copy_s"] = xfer.get("host_copy_s", 0.0) + t_host
+        fd = writer.fileno() if self._crc_chunk_bytes else -1
+        if fd < 0:
+            return None
+        return hip_plan.crc32c_file(fd, METADATA_SIZE + start, layout.data_bytes, self._crc_chunk_bytes,
+                                    self._engine_config.resolved_copy_threads())
 
     # ---- replication hand-off, metadata, finalize (host logic kept as in the reference) -------------------
     @log_execution_time(logger=_LOGGER, name="async_replicate_object")

@@ -127,10 +127,15 @@ def host_tensor_bytes(t: torch.Tensor) -> bytes:
 
 @dataclasses.dataclass
 class SaveLayout:
-    """Where every item of one checkpoint object lies, and the table that packs it."""
+    """Where every item of one checkpoint object lies, and the table that packs it.
+
+    ``image_bytes`` is what the image takes in HBM, ``data_bytes`` what the object's data section takes in the buffer
+    file.  They differ only when large host-resident tensors go from host memory straight into the buffer
+    (``host_spans``): their payloads are left out of the image, which then consists of ``segments`` - runs of image
+    bytes that belong at consecutive offsets of the data section."""
 
     image_bytes: int
-    spans: List[Tuple[int, int]]  # (offset, length) of each record: tensors in order, then byte blobs in order
+    spans: List[Tuple[int, int]]  # (data offset, length) of each record: tensors in order, then byte blobs in order
     items: np.ndarray
     blob: bytes
     device_payload_bytes: int
@@ -138,58 +143,95 @@ class SaveLayout:
     # pieces of the blob whose bytes are not determined by dtypes and shapes: (blob offset, nbytes, "tensor" | "blob",
     # index into the tensors / blobs argument).  A layout that is reused for the next save refreshes exactly these.
     variable_parts: List[Tuple[int, int, str, int]] = dataclasses.field(default_factory=list)
+    data_bytes: int = -1  # -1: same as image_bytes
+    host_spans: List[Tuple[int, int, int]] = dataclasses.field(default_factory=list)  # (data offset, nbytes, tensor index)
+    host_tensors: List[torch.Tensor] = dataclasses.field(default_factory=list)  # one per host span
+    segments: List[Tuple[int, int, int]] = dataclasses.field(default_factory=list)  # (image offset, data offset, nbytes)
+
+    def __post_init__(self):
+        if self.data_bytes < 0:
+            self.data_bytes = self.image_bytes
 
 
-def build_save_layout(tensors: Sequence[torch.Tensor], blobs: Sequence[bytes] = ()) -> SaveLayout:
+def build_save_layout(tensors: Sequence[torch.Tensor], blobs: Sequence[bytes] = (),
+                      host_direct_min: Optional[int] = None) -> SaveLayout:
     """Lays out records for ``tensors`` (device or host) followed by ``blobs`` and returns the descriptor table.
 
     Device tensors become DEVICE items (any strides; the image side is the C-contiguous payload).  Record headers,
-    payloads of host-resident tensors and byte blobs are collected into one host blob that the plan uploads once.
+    payloads of host-resident tensors and byte blobs are collected into one host blob that the plan uploads once -
+    except host-resident tensors of at least ``host_direct_min`` bytes (None: no such exception), which never
+    visit the device: the layout only notes where in the data section they belong (``host_spans``).
     """
     table = ItemTable()
     blob = bytearray()
     spans: List[Tuple[int, int]] = []
     keep: List[torch.Tensor] = []
     variable: List[Tuple[int, int, str, int]] = []
-    pos = 0
+    host_spans: List[Tuple[int, int, int]] = []
+    host_tensors: List[torch.Tensor] = []
+    pos = 0   # in the data section
+    ipos = 0  # in the image
     device_bytes = 0
     for index, t in enumerate(tensors):
         start = pos
         hdr = header_bytes(t.dtype, t.shape)
-        table.add_blob(len(blob), pos, len(hdr))
+        table.add_blob(len(blob), ipos, len(hdr))
         blob += hdr
         pos += len(hdr)
+        ipos += len(hdr)
         nbytes = t.numel() * t.element_size()
         if nbytes:
-            if t.device.type == "cpu":
+            if t.device.type == "cpu" and host_direct_min is not None and nbytes >= host_direct_min:
+                # large host-resident item (an optimizer state kept in host memory ...): host to buffer directly
+                host_spans.append((pos, nbytes, index))
+                host_tensors.append(t)
+            elif t.device.type == "cpu":
                 # host-resident item (step counters, RNG state ...): its bytes travel with the headers
                 variable.append((len(blob), nbytes, "tensor", index))
-                table.add_blob(len(blob), pos, nbytes)
+                table.add_blob(len(blob), ipos, nbytes)
                 blob += host_tensor_bytes(t)
+                ipos += nbytes
             else:
                 if t.is_contiguous():
-                    table.add_contiguous(t.data_ptr(), pos, t.element_size(), nbytes)
+                    table.add_contiguous(t.data_ptr(), ipos, t.element_size(), nbytes)
                 else:
-                    table.add_device(t.data_ptr(), pos, t.element_size(), tuple(t.shape), tuple(t.stride()))
+                    table.add_device(t.data_ptr(), ipos, t.element_size(), tuple(t.shape), tuple(t.stride()))
                 keep.append(t)
                 device_bytes += nbytes
+                ipos += nbytes
             pos += nbytes
         spans.append((start, pos - start))
     for index, data in enumerate(blobs):
         if len(data):
             variable.append((len(blob), len(data), "blob", index))
-            table.add_blob(len(blob), pos, len(data))
+            table.add_blob(len(blob), ipos, len(data))
             blob += data
         spans.append((pos, len(data)))
         pos += len(data)
+        ipos += len(data)
+    segments: List[Tuple[int, int, int]] = []
+    image_at = data_at = 0
+    for offset, nbytes, _ in host_spans:
+        if offset > data_at:
+            segments.append((image_at, data_at, offset - data_at))
+            image_at += offset - data_at
+        data_at = offset + nbytes
+    if pos > data_at:
+        segments.append((image_at, data_at, pos - data_at))
+        image_at += pos - data_at
+    assert image_at == ipos
     return SaveLayout(
-        image_bytes=pos,
+        image_bytes=ipos,
         spans=spans,
         items=table.to_array(),
         blob=bytes(blob),
         device_payload_bytes=device_bytes,
         device_tensors=keep,
         variable_parts=variable,
+        data_bytes=pos,
+        host_spans=host_spans,
+        host_tensors=host_tensors,
+        segments=segments,
     )
 
 
@@ -320,6 +362,10 @@ class CopyEngine:
             "mlf_engine_d2h_watched",
         )
         return stats, (crcs[:n_chunks] if crc_chunk_bytes else None)
+
+    def host_copy(self, dst_host_ptr: int, src_host_ptr: int, nbytes: int) -> None:
+        """Host memory to host memory on the engine's threads (checkpoint items that are resident on the host)."""
+        _lib.check(_lib.load().mlf_engine_host_copy(self._handle, dst_host_ptr, src_host_ptr, nbytes), "mlf_engine_host_copy")
 
     def h2d(self, src_host_ptr: int, dst_dev_ptr: int, nbytes: int, consumer_stream: int = 0) -> _lib.XferStats:
         stats = _lib.XferStats()

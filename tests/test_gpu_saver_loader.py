@@ -2,6 +2,7 @@
 with the CPU oracle on the same seeded state dicts (bit-exact)."""
 
 import concurrent.futures
+import ctypes
 import io
 import os
 import pickle
@@ -607,6 +608,63 @@ def test_plans_are_kept_from_save_to_save_and_rebuilt_when_the_tensors_change(sh
     fresh = _saver(reuse_plans=False)
     saver = fresh
     assert "plans_reused" not in save(9, sd_dev) and "plans_reused" not in save(10, sd_dev)
+
+
+@pytest.mark.parametrize("background_write", [False, True])
+def test_large_host_resident_tensors_go_from_host_memory_into_the_buffer(shm_dir, manager_future, background_write):
+    """A state dict with part of it kept in host memory (offloaded optimizer state): the large host tensors never visit
+    the device - the image holds the rest, in runs that are sent to their places around them - and the file is still
+    the oracle's, byte for byte, with a valid checksum sidecar; a second save through the kept plan picks up the
+    host tensors' new contents; the file restores into device and host targets alike."""
+    from ml_flashpoint.hip import integrity
+    from ml_flashpoint.hip import plan as P
+
+    g = torch.Generator().manual_seed(21)
+    sd_cpu = {
+        "dev.w": torch.randn(300, 1000, generator=g),
+        "host.m": torch.randn(700, 800, generator=g),                       # 2.2 MB, stays on the host
+        "dev.b": torch.randn(4097, generator=g).to(torch.bfloat16),
+        "host.v_view": torch.randn(900, 600, generator=g).t(),              # 2.2 MB, a strided view on the host
+        "host.small": torch.arange(50, dtype=torch.int64),                  # rides in the image with the headers
+        "dev.tail": torch.randint(0, 255, (70001,), dtype=torch.uint8, generator=g),
+        "host.last": torch.randn(1 << 18, generator=g),                     # 1 MiB, host, possibly the last record
+        "obj.step": 7,
+    }
+    on_host = {k for k in sd_cpu if k.startswith("host.")}
+    sd = {k: (v.to(DEV) if isinstance(v, torch.Tensor) and k not in on_host else v) for k, v in sd_cpu.items()}
+    saver = _saver(crc_chunk_bytes=1 << 18, background_write=background_write)
+    big_host_bytes = sum(sd_cpu[k].numel() * sd_cpu[k].element_size() for k in ("host.m", "host.v_view", "host.last"))
+    for step in (1, 2):
+        ckpt = os.path.join(shm_dir, f"step-{step}_ckpt")
+        dcp.save(sd, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(saver, manager_future), no_dist=True)
+        obj = os.path.join(ckpt, "__0__0_src0.distcp")
+        raw = open(obj, "rb").read()
+        metadata = pickle.load(open(os.path.join(ckpt, ".metadata"), "rb"))
+        image, spans, got_spans = _expected_file(sd_cpu, metadata, raw)
+        assert raw == image and got_spans == spans
+        if not background_write:  # (the background thread keeps its own transfer statistics)
+            stats = saver.last_save_stats
+            assert stats["host_copy_bytes"] == big_host_bytes
+            assert stats["d2h_bytes"] == len(raw) - METADATA_SIZE - big_host_bytes == stats["image_bytes"]
+            assert stats.get("plans_reused", 0) == (1 if step == 2 else 0)
+        chunk, nbytes, crcs = integrity.read_sidecar(obj)
+        assert nbytes == len(raw) - METADATA_SIZE
+        for k, c in enumerate(crcs):
+            piece = raw[METADATA_SIZE + k * chunk : METADATA_SIZE + (k + 1) * chunk]
+            buf = ctypes.create_string_buffer(piece, len(piece))
+            assert P.crc32c_host(ctypes.addressof(buf), len(piece)) == int(c)
+        target = {k: (torch.zeros(v.shape, dtype=v.dtype, device=sd[k].device) if isinstance(v, torch.Tensor) else None)
+                  for k, v in sd_cpu.items()}
+        dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, _loader()), no_dist=True)
+        assert target["obj.step"] == 7
+        for k, v in sd_cpu.items():
+            if isinstance(v, torch.Tensor):
+                assert torch.equal(_bits(target[k]), _bits(v)), k
+        # the next step's values, in place: on the host for the host tensors, on the device for the others
+        for k in ("host.m", "host.v_view", "host.small", "dev.w"):
+            sd_cpu[k].mul_(3).add_(1)
+        sd["dev.w"].mul_(3).add_(1)
+    saver.release_device_memory()
 
 
 def test_legacy_torch_save_objects_are_still_readable(shm_dir):

@@ -3,7 +3,8 @@
 The descriptor table is built on the host from addresses, shapes and strides only, so the whole rule set - record
 order, header bytes, offsets with no padding, blobs behind the tensors, what becomes a contiguous run and what a
 strided descriptor - can be compared with the oracle on CPU tensors.  (For host-resident tensors the payload
-travels in the plan's blob, which then *is* the data section; for device tensors only the table rows differ.)"""
+travels in the plan's blob, which then *is* the data section - unless they are large, when they stay out of the image
+altogether; for device tensors only the table rows differ.)"""
 
 import numpy as np
 import pytest
@@ -53,6 +54,47 @@ def test_layout_of_host_tensors_is_the_oracles_data_section(data):
         ends = items["image_off"] + items["nbytes"]
         assert items["image_off"][0] == 0 and (items["image_off"][1:] == ends[:-1]).all()
         assert (items["ptr"] == items["image_off"]).all()
+
+
+@settings(max_examples=60, deadline=None)
+@given(st.data())
+def test_host_tensors_above_the_threshold_are_left_out_of_the_image(data):
+    """With a threshold, large host tensors are only noted (``host_spans``); the image holds everything else in
+    ``segments``.  Putting the segments and the host payloads where the layout says reproduces the oracle's data
+    section, the records' spans are those of the layout without a threshold, and nothing overlaps or is left out."""
+    threshold = data.draw(st.sampled_from([1, 16, 64]))
+    tensors = []
+    for _ in range(data.draw(st.integers(0, 7))):
+        dtype = data.draw(st.sampled_from(DTYPES))
+        shape = tuple(data.draw(st.lists(st.integers(0, 6), min_size=0, max_size=3)))
+        t = _tensor(lambda k: data.draw(st.lists(st.integers(0, 255), min_size=k, max_size=k)), dtype, shape)
+        if t.dim() >= 2 and data.draw(st.booleans()):
+            t = t.transpose(0, -1)
+        tensors.append(t)
+    blobs = data.draw(st.lists(st.binary(min_size=0, max_size=40), min_size=0, max_size=2))
+    layout = P.build_save_layout(tensors, blobs, host_direct_min=threshold)
+    want, spans = fmt.data_section(tensors, blobs)
+    assert layout.spans == spans and layout.data_bytes == len(want)
+    big = [i for i, t in enumerate(tensors) if t.numel() * t.element_size() >= threshold]
+    assert [i for _, _, i in layout.host_spans] == big and [id(t) for t in layout.host_tensors] == [id(tensors[i]) for i in big]
+    assert layout.image_bytes == len(want) - sum(n for _, n, _ in layout.host_spans)
+    # the image, as the pack kernel would fill it from the table (every row is a piece of the blob here)
+    image = bytearray(layout.image_bytes)
+    for row in layout.items:
+        assert row["kind"] == _lib.ITEM_BLOB
+        image[int(row["image_off"]) : int(row["image_off"] + row["nbytes"])] = layout.blob[int(row["ptr"]) : int(row["ptr"] + row["nbytes"])]
+    built = bytearray(b"\xEE" * len(want))
+    covered = 0
+    for image_off, data_off, n in layout.segments:
+        built[data_off : data_off + n] = image[image_off : image_off + n]
+        covered += n
+    for (data_off, n, _), t in zip(layout.host_spans, layout.host_tensors):
+        built[data_off : data_off + n] = P.host_tensor_bytes(t)
+        covered += n
+    assert covered == len(want) and bytes(built) == want
+    pieces = sorted([(d, n) for _, d, n in layout.segments] + [(d, n) for d, n, _ in layout.host_spans])
+    assert all(a[0] + a[1] == b[0] for a, b in zip(pieces, pieces[1:])) and (not pieces or pieces[0][0] == 0)
+    assert [io for io, _, _ in layout.segments] == [sum(n for _, _, n in layout.segments[:k]) for k in range(len(layout.segments))]
 
 
 class _FakeDeviceTensor:
