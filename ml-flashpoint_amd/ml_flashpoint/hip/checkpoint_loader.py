@@ -175,6 +175,18 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                 _HEADER_CACHE[raw] = parsed
         return parsed[0], parsed[1], offset + 4 + header_len, parsed[2]
 
+    @staticmethod
+    def _payload_view(whole: memoryview, written: int, object_id, req, dtype, shape, payload_off: int, stored_bytes: int):
+        """A host tensor over a record's payload where it lies in the (read-only) mapping: nothing is copied."""
+        if payload_off + stored_bytes > written:
+            raise ValueError(f"req {req.storage_index}: record reaches past the written data of '{object_id.data}'")
+        if stored_bytes == 0:
+            return torch.empty(shape, dtype=dtype)
+        with warnings.catch_warnings():  # the mapping is read-only and the tensor over it is only read
+            warnings.filterwarnings("ignore", message="The given buffer is not writable")
+            flat = torch.frombuffer(whole, dtype=dtype, count=shape.numel(), offset=METADATA_SIZE + payload_off)
+        return flat.reshape(shape)
+
     # ---- read_data ------------------------------------------------------------------------------------
     @override
     @log_execution_time(logger=_LOGGER, name="read_data", level=logging.INFO)
@@ -209,7 +221,20 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                     continue
                 target = planner.resolve_tensor(req).detach()
                 parsed = self._parse_header(whole, item_md.offset, item_md.length) if optimized else None
-                if parsed is None or target.device.type == "cpu":
+                if parsed is not None and target.device.type == "cpu":
+                    # host-resident target: one copy, from a tensor laid over the record's payload in the mapping
+                    # into the target (the reference reads the record into a bytes object first,
+                    # checkpoint_loader.py:195-208)
+                    tensor = self._payload_view(whole, recorded, checkpoint_object_id, req, *parsed)
+                    tensor = narrow_tensor_by_index(tensor, req.storage_offsets, req.lengths)
+                    assert target.size() == tensor.size(), (
+                        f"req {req.storage_index} mismatch sizes {target.size()} vs {tensor.size()}"
+                    )
+                    target.copy_(tensor)
+                    planner.commit_tensor(req, target)
+                    stats["host_items"] += 1
+                    continue
+                if parsed is None:
                     view = cast(IO[bytes], _create_file_view(stream, item_md.offset, item_md.length))
                     tensor = self.read_tensor(view, req, use_optimized_loader=optimized)
                     assert target.size() == tensor.size(), (
