@@ -234,6 +234,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         remote_wait_timeout_s: float = 1800.0,
         max_image_bytes: Optional[int] = None,
         reuse_plans: bool = True,
+        snapshot_host_tensors: bool = False,
     ):
         """Same positional arguments as the reference's default saver (checkpoint_saver.py:290-321).
 
@@ -249,7 +250,10 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         by window inside ``prepare_write_data``, which then blocks for the whole transfer), ``reuse_plans`` (keep
         the layout and the device-resident tables of every object from one save to the next and use them again
         when the tensors' addresses, shapes, strides and dtypes are the same; only the bytes of host-resident items
-        are refreshed.  With 20 000 tensors this takes 60 ms out of the blocking part of each save after the first).
+        are refreshed.  With 20 000 tensors this takes 60 ms out of the blocking part of each save after the first),
+        ``snapshot_host_tensors`` (large host-resident tensors are copied from where they are into the buffer while
+        the transfer runs, as the reference copies them while it writes; True: they are cloned inside
+        ``prepare_write_data`` instead, for training loops that update them before the transfer has ended).
         """
         if not use_optimized_save:
             raise ValueError(
@@ -273,6 +277,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         self._remote_wait_timeout_s = remote_wait_timeout_s
         self._max_image_bytes = max_image_bytes
         self._reuse_plans = reuse_plans
+        self._snapshot_host_tensors = snapshot_host_tensors
         self._init_runtime_state()
 
     def _init_runtime_state(self):
@@ -458,6 +463,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                 raise ValueError("all device tensors of one checkpoint object must live on the same device")
             if device is None:
                 device = torch.device("cuda", torch.cuda.current_device())
+        if layout.host_tensors and self._snapshot_host_tensors:
+            layout.host_tensors = [t.detach().clone(memory_format=torch.contiguous_format) for t in layout.host_tensors]
         items = [item for item, _ in tensor_data] + [item for item, _ in bytes_data]
         plan = image = packed = None
         stream = 0

@@ -667,6 +667,28 @@ def test_large_host_resident_tensors_go_from_host_memory_into_the_buffer(shm_dir
     saver.release_device_memory()
 
 
+def test_host_tensors_can_be_snapshotted_inside_the_blocking_part(shm_dir):
+    """With ``snapshot_host_tensors=True`` the staged object holds clones of the large host tensors: what is written
+    is what they held when ``prepare_write_data`` returned, whatever happens to them before ``write_data``."""
+    from torch.distributed.checkpoint.planner_helpers import _create_write_items
+
+    host = torch.arange(1 << 17, dtype=torch.float32)  # 512 KiB on the host
+    data = {"host": host, "dev": torch.ones(1000, device=DEV)}
+    before = host.clone()
+    for snapshot in (True, False):
+        saver = _saver(snapshot_host_tensors=snapshot)
+        cid = CheckpointContainerId(os.path.join(shm_dir, f"step-{int(snapshot)}_ckpt"))
+        items = [wi for k, v in data.items() for wi in _create_write_items(k, v)]
+        buckets = saver.prepare_write_data(cid, items, _Resolver(data), "data", 1)
+        host.add_(1.0)  # the training loop moves on before the transfer
+        results = saver.write_data(cid, buckets, replicate_after_write=False)
+        where = {r.index.fqn: r.storage_data for r in results}["host"]
+        raw = open(os.path.join(cid.data, "data_0_src0.distcp"), "rb").read()
+        payload = raw[METADATA_SIZE + where.offset + where.length - host.numel() * 4 : METADATA_SIZE + where.offset + where.length]
+        assert payload == (before if snapshot else host).numpy().tobytes()
+        before = host.clone()
+
+
 def test_legacy_torch_save_objects_are_still_readable(shm_dir):
     """An object whose signature is TORCH___ holds torch.save records; the loader reads it on the host."""
     from ml_flashpoint.core.defaults import CheckpointFormat
