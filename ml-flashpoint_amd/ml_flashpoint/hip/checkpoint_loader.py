@@ -47,6 +47,11 @@ _LOGGER = get_logger(__name__)
 
 _MAX_HEADER_LEN = 1024 * 1024  # a larger "length" means the record is not in the MLF_TENS format
 _UPLOAD_ALIGN = 4096
+# A read that asks for part of an object (the weights out of weights + optimizer state, say) uploads only the
+# neighbourhoods of what it asks for, when that leaves out at least this much; requested ranges closer than the gap
+# are fetched together.
+_PARTIAL_READ_MIN_SAVING = 256 << 20
+_PARTIAL_READ_GAP = 16 << 20
 _U32 = struct.Struct("<I")
 _HEADER_CACHE: dict = {}  # header pickle bytes -> (dtype, shape, stored payload bytes)
 _ESZ_CACHE: dict = {}
@@ -326,13 +331,25 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
             if sidecar is not None:
                 lo, hi = 0, written  # checksums cover the whole data section
             lo = lo // _UPLOAD_ALIGN * _UPLOAD_ALIGN
+            clusters = None
+            if (hi - lo) - sum(r[1] - r[0] for r in rows) >= _PARTIAL_READ_MIN_SAVING:
+                clusters = self._clusters_of(rows, sidecar[0] if sidecar is not None else None, written)
+                if (hi - lo) - sum(c_hi - c_lo for c_lo, c_hi, _ in clusters) < _PARTIAL_READ_MIN_SAVING:
+                    clusters = None
             with torch.cuda.device(device):
                 _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
                 limit = self._image_limit(device)
-                if hi - lo <= limit:
-                    self._restore_range(object_id, stream, device, rows, lo, hi, sidecar, stats)
+                # one buffer for the range (or for the largest neighbourhood of a partial read) if the allocator
+                # has a block of that size; through a smaller buffer, window by window, if it has not
+                need = max(c_hi - c_lo for c_lo, c_hi, _ in clusters) if clusters is not None else hi - lo
+                image = hip_plan.try_allocate(need, device) if need <= limit else None
+                if image is None:
+                    self._restore_windowed(object_id, stream, device, rows, min(limit, need), sidecar, stats)
+                elif clusters is not None:
+                    self._restore_clusters(object_id, stream, device, clusters, sidecar, stats, image)
                 else:
-                    self._restore_windowed(object_id, stream, device, rows, limit, sidecar, stats)
+                    self._restore_range(object_id, stream, device, rows, lo, hi, sidecar, stats, image)
+                del image
                 for target, stored_as in conversions:
                     target.copy_(stored_as)
         for req, target, *_ in device_reqs:
@@ -379,10 +396,9 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         finally:
             plan.destroy()
 
-    def _restore_range(self, object_id, stream, device, rows, lo, hi, sidecar, stats) -> None:
-        """One upload of [lo, hi), checksum on the GPU if the object has a sidecar, one unpack."""
+    def _restore_range(self, object_id, stream, device, rows, lo, hi, sidecar, stats, image) -> None:
+        """One upload of [lo, hi) into ``image``, checksum on the GPU if the object has a sidecar, one unpack."""
         span = hi - lo
-        image = torch.empty(span, dtype=torch.uint8, device=device)
         cur = torch.cuda.current_stream(device)
         self._upload(stream, lo, image, span, cur, stats)
         if sidecar is not None:
@@ -392,12 +408,44 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         self._unpack(self._table_of(rows, lo), image, span, cur, stats["device_payload_bytes"])
 
     @staticmethod
-    def _compare_checksums(object_id, got, want, chunk_bytes) -> None:
-        bad = [int(i) for i in (got != want).nonzero()[0]]
+    def _compare_checksums(object_id, got, want, chunk_bytes, first_chunk: int = 0, n_chunks: Optional[int] = None) -> None:
+        bad = [first_chunk + int(i) for i in (got != want).nonzero()[0]]
         if bad:
             raise integrity.ChecksumMismatchError(
-                f"'{object_id.data}': CRC-32C mismatch in chunk(s) {bad[:8]} of {len(want)} "
+                f"'{object_id.data}': CRC-32C mismatch in chunk(s) {bad[:8]} of {n_chunks if n_chunks is not None else len(want)} "
                 f"(chunk size {chunk_bytes})")
+
+    @staticmethod
+    def _clusters_of(rows, chunk_bytes: Optional[int], written: int):
+        """Groups the requested rows into ranges of the data section that are worth one upload each: rows closer than
+        the gap go together; a range starts and ends on upload boundaries - on checksum chunks when the object has a
+        sidecar, so that every chunk that is read can be checked.  Returns [(lo, hi, rows)], ascending, disjoint."""
+        align = chunk_bytes or _UPLOAD_ALIGN
+        clusters = []
+        for row in sorted(rows, key=lambda r: r[0]):
+            lo = row[0] // align * align
+            hi = min(-(-row[1] // align) * align, written) if chunk_bytes else row[1]
+            if clusters and lo - clusters[-1][1] <= _PARTIAL_READ_GAP:
+                clusters[-1][1] = max(clusters[-1][1], hi)
+                clusters[-1][2].append(row)
+            else:
+                clusters.append([lo, hi, [row]])
+        return [(lo, hi, members) for lo, hi, members in clusters]
+
+    def _restore_clusters(self, object_id, stream, device, clusters, sidecar, stats, image) -> None:
+        """A partial read: every cluster is uploaded into ``image``, checked against the sidecar's values for exactly
+        the chunks it covers, and unpacked.  What the request does not touch is neither read nor checked."""
+        cur = torch.cuda.current_stream(device)
+        for lo, hi, members in clusters:
+            span = hi - lo
+            self._upload(stream, lo, image, span, cur, stats)
+            if sidecar is not None:
+                chunk_bytes, _, want = sidecar
+                got = hip_plan.crc32c_device(image, span, chunk_bytes, cur.cuda_stream)
+                first = lo // chunk_bytes
+                self._compare_checksums(object_id, got, want[first : first + len(got)], chunk_bytes, first, len(want))
+            self._unpack(self._table_of(members, lo), image, span, cur, sum(r[1] - r[0] for r in members if r[2]))
+        stats["partial_read_ranges"] = stats.get("partial_read_ranges", 0) + len(clusters)
 
     def _restore_windowed(self, object_id, stream, device, rows, limit, sidecar, stats) -> None:
         """Fallback for an object whose requested range does not fit in HBM beside the live state: the rows are
@@ -419,10 +467,17 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                 if own_fd:
                     os.close(fd)
             self._compare_checksums(object_id, got, want, chunk_bytes)
+        image = None
+        while image is None:  # the largest buffer the allocator really has, at most the limit
+            if limit - _UPLOAD_ALIGN < 65536:
+                if self._max_image_bytes is not None:
+                    raise ValueError(f"max_image_bytes={self._max_image_bytes} is too small to restore anything")
+                raise torch.OutOfMemoryError(f"no device buffer to restore '{object_id.data}' through")
+            image = hip_plan.try_allocate(limit, device)
+            if image is None:
+                limit //= 2
         usable = limit - _UPLOAD_ALIGN  # a window starts on an upload boundary at or below its first row
         piece = usable // 65536 * 65536  # a multiple of every element size
-        if piece <= 0:
-            raise ValueError(f"max_image_bytes={limit} is too small to restore anything")
         pieces = []
         for first, last, contiguous, args in sorted(rows, key=lambda r: r[0]):
             if last - first <= usable:
@@ -445,7 +500,6 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
             current.append(row)
         windows.append((lo, current))
         cur = torch.cuda.current_stream(device)
-        image = torch.empty(max(max(r[1] for r in rs) - lo for lo, rs in windows), dtype=torch.uint8, device=device)
         for lo, window_rows in windows:
             span = max(r[1] for r in window_rows) - lo
             self._upload(stream, lo, image, span, cur, stats)

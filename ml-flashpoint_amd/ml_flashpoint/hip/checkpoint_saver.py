@@ -79,6 +79,9 @@ class EngineConfig:
 # in the image with the headers (one copy more, no extra pieces in the transfer)
 _HOST_DIRECT_MIN_BYTES = 256 << 10
 
+# when the allocator has no single block for an object's image, the image is held in pieces of about this size
+_IMAGE_PIECE_BYTES = 8 << 30
+
 _MAX_KEPT_PLANS = 64  # objects per save are few (one per writer thread); beyond this the oldest is rebuilt
 
 
@@ -131,6 +134,8 @@ class StagedObject:
         self.owns_plan = True  # False: the plan is kept by the saver for the next save
         self._landed = ctypes.c_uint64(0)  # kept current by the copy engine while the image crosses the link
         self.data_offset: Optional[int] = None  # position of the image's first byte in the object's data section
+        # an image that is held in several device buffers: [(plan, buffer, first image byte, end)], in order
+        self.pieces: Optional[list] = None
 
     def landed_bytes(self) -> int:
         """Leading bytes of the image that are in place in the buffer file (from byte 4096 + ``data_offset`` of the
@@ -468,11 +473,20 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         items = [item for item, _ in tensor_data] + [item for item, _ in bytes_data]
         plan = image = packed = None
         stream = 0
-        if layout.image_bytes and object_id is not None and layout.image_bytes > self._image_limit(device):
-            self._drop_kept_plan(object_name)
-            if layout.host_spans:  # the windowed mode sends one image, whole: lay the host items out inside it
-                layout = hip_plan.build_save_layout(tensors, blobs)
-            return self._stage_windowed(layout, items, object_id, object_name, device, stats)
+        if layout.image_bytes and object_id is not None:
+            if layout.image_bytes <= self._image_limit(device):
+                with torch.cuda.device(device):
+                    image = hip_plan.try_allocate(layout.image_bytes, device)
+            if image is None:
+                # no room for the image in one block: in pieces, all resident, if the device has that much left
+                # in smaller blocks (the save stays asynchronous); else window by window through one buffer
+                self._drop_kept_plan(object_name)
+                if layout.host_spans:  # both modes send one image, whole: lay the host items out inside it
+                    layout = hip_plan.build_save_layout(tensors, blobs)
+                staged = self._stage_in_pieces(layout, items, device, stats)
+                if staged is not None:
+                    return staged
+                return self._stage_windowed(layout, items, object_id, object_name, device, stats)
         if layout.image_bytes:
             with torch.cuda.device(device):
                 _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
@@ -487,7 +501,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                                          block_threads=self._block_threads)
                     if key is not None:
                         self._keep_plan(object_name, _KeptPlan(key, layout, plan, device))
-                image = torch.empty(layout.image_bytes, dtype=torch.uint8, device=device)
+                if image is None:
+                    image = torch.empty(layout.image_bytes, dtype=torch.uint8, device=device)
                 stats["plan_build_s"] += time.perf_counter() - t0
                 if self.record_kernel_events:
                     begin, packed = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -533,6 +548,70 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         if kept is not None:
             kept.plan.destroy()  # releasing device memory waits for the kernels that still use it
 
+    @staticmethod
+    def _windows_of(layout: hip_plan.SaveLayout, limit: int) -> list:
+        """Consecutive rows of the layout's table grouped into windows of at most ``limit`` image bytes (a single
+        larger row gets a window of its own): [(first row, end row, first image byte, end)]."""
+        arr = layout.items
+        ends = (arr["image_off"] + arr["nbytes"]).tolist()
+        starts = arr["image_off"].tolist()
+        windows, r0, n = [], 0, len(arr)
+        while r0 < n:
+            r1 = r0 + 1
+            while r1 < n and ends[r1] - starts[r0] <= limit:
+                r1 += 1
+            windows.append((r0, r1, starts[r0], ends[r1 - 1]))
+            r0 = r1
+        return windows
+
+    def _stage_in_pieces(self, layout, items, device, stats: dict) -> Optional[StagedObject]:
+        """The image in several device buffers, all packed now: for a device whose free memory is there but not in
+        one block.  The transfer sends them one after the other, so the save is as asynchronous as with one
+        image.  None (and nothing allocated) if the buffers cannot be had either."""
+        if self._max_image_bytes is not None and layout.image_bytes > self._max_image_bytes:
+            return None
+        windows = self._windows_of(layout, _IMAGE_PIECE_BYTES)
+        with torch.cuda.device(device):
+            _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
+            buffers = []
+            for _, _, begin, end in windows:
+                buffers.append(hip_plan.try_allocate(end - begin, device))
+                if buffers[-1] is None:
+                    del buffers
+                    return None
+            if self._max_image_bytes is None and torch.cuda.mem_get_info(device)[0] < (1 << 30):
+                del buffers  # that would leave the training step nothing to allocate from
+                torch.cuda.empty_cache()
+                return None
+            _LOGGER.warning("no single block of %d bytes of device memory: the checkpoint image is held in %d pieces",
+                            layout.image_bytes, len(windows))
+            stream = torch.cuda.current_stream(device).cuda_stream
+            pieces = []
+            t0 = time.perf_counter()
+            begin_event = torch.cuda.Event(enable_timing=True) if self.record_kernel_events else None
+            if begin_event is not None:
+                begin_event.record()
+            for (r0, r1, begin, end), buf in zip(windows, buffers):
+                sub = layout.items[r0:r1].copy()
+                sub["image_off"] -= begin
+                plan = hip_plan.Plan(sub, layout.blob, end - begin, tile_bytes=self._tile_bytes,
+                                     block_threads=self._block_threads)
+                plan.pack(buf, stream)
+                pieces.append((plan, buf, begin, end))
+            packed = torch.cuda.Event(enable_timing=self.record_kernel_events)
+            packed.record()
+            if begin_event is not None:
+                self.kernel_events.append((begin_event, packed, layout.device_payload_bytes))
+            stats["plan_build_s"] += time.perf_counter() - t0
+        stats["objects"] += 1
+        stats["image_pieces"] = stats.get("image_pieces", 0) + len(pieces)
+        stats["device_payload_bytes"] += layout.device_payload_bytes
+        stats["image_bytes"] += layout.image_bytes
+        staged = StagedObject(layout, None, None, device.index or 0, stream, items)
+        staged.pieces = pieces
+        staged.packed_event = packed
+        return staged
+
     def _stage_windowed(self, layout, items, object_id, object_name, device, stats: dict) -> StagedObject:
         """Fallback for an object whose image does not fit in HBM beside the live state: consecutive records are
         grouped into windows of at most the image limit (a single larger record gets a window of its own), and each
@@ -541,16 +620,11 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         _LOGGER.warning("checkpoint image of %d bytes exceeds the HBM limit; saving '%s' window by window (blocking)",
                         layout.image_bytes, object_id)
         arr = layout.items
-        ends = (arr["image_off"] + arr["nbytes"]).tolist()
-        starts = arr["image_off"].tolist()
-        limit = max(self._image_limit(device), 1)
-        windows, r0, n = [], 0, len(arr)
-        while r0 < n:
-            r1 = r0 + 1
-            while r1 < n and ends[r1] - starts[r0] <= limit:
-                r1 += 1
-            windows.append((r0, r1, starts[r0], ends[r1 - 1]))
-            r0 = r1
+        limit = self._max_image_bytes
+        if limit is None:  # what the driver reports free now, the allocator's unused segments included
+            torch.cuda.empty_cache()
+            limit = max(torch.cuda.mem_get_info(device)[0] - (2 << 30), 64 << 20)
+        windows = self._windows_of(layout, max(limit, 1))
         nbytes = layout.image_bytes
         xfer = {"d2h_s": 0.0, "d2h_wait_s": 0.0, "d2h_bytes": 0}
         with self._chkpt_obj_manager.acquire_buffer(object_id, max(self._initial_buffer_size_bytes, nbytes)) as writer:
@@ -724,7 +798,9 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                     staged.data_offset = start
                     fd = writer.fileno() if self._use_file_io else -1
                     engine = self._get_engine()
-                    if layout.host_spans:
+                    if staged.pieces is not None:
+                        crcs = self._transfer_image_pieces(staged, writer, start, xfer)
+                    elif layout.host_spans:
                         crcs = self._transfer_in_pieces(staged, writer, start, xfer)
                     elif fd >= 0:
                         if self._crc_chunk_bytes:
@@ -753,6 +829,28 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         xfer["d2h_wait_s"] += st.wait_seconds
         xfer["d2h_bytes"] += nbytes
 
+    def _host_side_checksums(self, writer, start: int, nbytes: int):
+        """Chunk checksums of a data section that was not sent as one image: taken from the pages just written."""
+        fd = writer.fileno() if self._crc_chunk_bytes else -1
+        if fd < 0:
+            return None
+        return hip_plan.crc32c_file(fd, METADATA_SIZE + start, nbytes, self._crc_chunk_bytes,
+                                    self._engine_config.resolved_copy_threads())
+
+    def _transfer_image_pieces(self, staged: StagedObject, writer, start: int, xfer: dict):
+        """The transfer of an image that is held in several device buffers: one after the other, each released as
+        soon as it has been sent."""
+        engine = self._get_engine()
+        for k, (plan, buf, begin, end) in enumerate(staged.pieces):
+            st = engine.d2h(buf.data_ptr(), writer.data_address(start + begin), end - begin, staged.stream)
+            self._count_transfer(xfer, st, end - begin)
+            staged._landed.value = end
+            staged.pieces[k] = None
+            plan.destroy()
+            del buf
+        staged.pieces = None
+        return self._host_side_checksums(writer, start, staged.layout.data_bytes)
+
     def _transfer_in_pieces(self, staged: StagedObject, writer, start: int, xfer: dict):
         """The transfer of an object some of whose tensors live in host memory: the runs of the image between them
         cross the host link, the host-resident payloads are copied from where they are into their places in the
@@ -777,11 +875,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                 xfer["host_copy_bytes"] = xfer.get("host_copy_bytes", 0) + n
             staged._landed.value = data_off + n
         xfer["host_copy_s"] = xfer.get("host_copy_s", 0.0) + t_host
-        fd = writer.fileno() if self._crc_chunk_bytes else -1
-        if fd < 0:
-            return None
-        return hip_plan.crc32c_file(fd, METADATA_SIZE + start, layout.data_bytes, self._crc_chunk_bytes,
-                                    self._engine_config.resolved_copy_threads())
+        return self._host_side_checksums(writer, start, layout.data_bytes)
 
     # ---- replication hand-off, metadata, finalize (host logic kept as in the reference) -------------------
     @log_execution_time(logger=_LOGGER, name="async_replicate_object")

@@ -235,6 +235,19 @@ def build_save_layout(tensors: Sequence[torch.Tensor], blobs: Sequence[bytes] = 
     )
 
 
+def try_allocate(nbytes: int, device) -> Optional[torch.Tensor]:
+    """A ``uint8`` device buffer of ``nbytes`` from torch's allocator, or None if it cannot provide one piece of
+    that size - also not after handing its unused segments back to the driver.  (A long-running job's free memory
+    is rarely one piece: what the device reports as free says little about the largest block to be had.)"""
+    for attempt in (0, 1):
+        try:
+            return torch.empty(nbytes, dtype=torch.uint8, device=device)
+        except torch.OutOfMemoryError:
+            if attempt == 0:
+                torch.cuda.empty_cache()
+    return None
+
+
 class Plan:
     """Owns a native ``mlf_plan``: device-resident descriptor and work tables for one set of items."""
 

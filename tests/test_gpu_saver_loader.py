@@ -458,6 +458,49 @@ def test_object_larger_than_the_hbm_limit_is_saved_window_by_window(shm_dir, man
             assert torch.equal(_bits(target[k]), _bits(v)), k
 
 
+@pytest.mark.parametrize("background_write", [False, True])
+def test_image_is_held_in_pieces_when_no_single_block_is_to_be_had(shm_dir, manager_future, monkeypatch, background_write):
+    """Free device memory that is not in one block (the usual state of a long-running job): the image is packed into
+    several smaller buffers, all resident, and sent piece by piece - same file, valid sidecar, and still an
+    asynchronous save - instead of failing or falling back to the blocking window-by-window mode."""
+    from ml_flashpoint.hip import checkpoint_saver as saver_mod
+    from ml_flashpoint.hip import integrity
+    from ml_flashpoint.hip import plan as P
+
+    sd_cpu = _mixed_state_dict()
+    sd_cpu["big"] = torch.arange(100_000, dtype=torch.float32)  # a record larger than a piece: a piece of its own
+    for i in range(8):
+        sd_cpu[f"mid.{i}"] = torch.full((60_000,), float(i))
+    sd_dev = _to_dev(sd_cpu)
+    real = P.try_allocate
+    refused = []
+
+    def fragmented(nbytes, device):  # no block above 512 KiB
+        if nbytes > (1 << 19):
+            refused.append(nbytes)
+            return None
+        return real(nbytes, device)
+
+    monkeypatch.setattr(P, "try_allocate", fragmented)
+    monkeypatch.setattr(saver_mod, "_IMAGE_PIECE_BYTES", 1 << 18)
+    saver = _saver(crc_chunk_bytes=1 << 16, background_write=background_write)
+    ckpt = os.path.join(shm_dir, "step-6_ckpt")
+    dcp.save(sd_dev, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(saver, manager_future), no_dist=True)
+    obj = os.path.join(ckpt, "__0__0_src0.distcp")
+    raw = open(obj, "rb").read()
+    metadata = pickle.load(open(os.path.join(ckpt, ".metadata"), "rb"))
+    image, spans, got_spans = _expected_file(sd_cpu, metadata, raw)
+    assert raw == image and got_spans == spans
+    assert refused == [len(raw) - METADATA_SIZE]  # the one image was asked for, once
+    assert saver.last_save_stats["image_pieces"] >= 4 and "windows" not in saver.last_save_stats
+    chunk, nbytes, crcs = integrity.read_sidecar(obj)
+    assert nbytes == len(raw) - METADATA_SIZE
+    for k, c in enumerate(crcs):
+        piece = raw[METADATA_SIZE + k * chunk : METADATA_SIZE + (k + 1) * chunk]
+        buf = ctypes.create_string_buffer(piece, len(piece))
+        assert P.crc32c_host(ctypes.addressof(buf), len(piece)) == int(c)
+
+
 @pytest.mark.parametrize("load_file_io", [True, False])
 def test_restore_larger_than_the_hbm_limit_goes_window_by_window(shm_dir, manager_future, load_file_io):
     """With ``max_image_bytes`` far below the object size the loader uploads and unpacks windows of rows through
@@ -516,6 +559,30 @@ def test_restore_larger_than_the_hbm_limit_goes_window_by_window(shm_dir, manage
         dcp.load(targets(), checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), no_dist=True)
     cause = exc.value.failures[0][0] if hasattr(exc.value, "failures") else exc.value
     assert isinstance(cause, integrity.ChecksumMismatchError) and "chunk(s) [5]" in str(cause)
+
+
+def test_restore_goes_through_a_smaller_buffer_when_no_single_block_is_to_be_had(shm_dir, manager_future, monkeypatch):
+    """The loader asks for one buffer for the whole range; when the allocator has no block of that size it halves
+    its request until it gets one and restores window by window through it - same tensors."""
+    from ml_flashpoint.hip import plan as P
+
+    sd_cpu = {f"t{i}": torch.randn(50_000, generator=torch.Generator().manual_seed(i)) for i in range(12)}  # 2.4 MB
+    sd_dev = _to_dev(sd_cpu)
+    ckpt = os.path.join(shm_dir, "step-8_ckpt")
+    dcp.save(sd_dev, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(_saver(crc_chunk_bytes=1 << 16), manager_future), no_dist=True)
+    real, asked = P.try_allocate, []
+
+    def fragmented(nbytes, device):  # no block above 512 KiB
+        asked.append(nbytes)
+        return real(nbytes, device) if nbytes <= (1 << 19) else None
+
+    monkeypatch.setattr(P, "try_allocate", fragmented)
+    target = {k: torch.zeros_like(v) for k, v in sd_dev.items()}
+    loader = _loader()
+    dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), no_dist=True)
+    assert all(torch.equal(target[k].cpu(), sd_cpu[k]) for k in sd_cpu)
+    assert len(asked) >= 3 and asked == sorted(asked, reverse=True) and asked[-1] <= (1 << 19)
+    assert loader.last_load_stats["windows"] >= 5
 
 
 @pytest.mark.parametrize("load_file_io", [True, False])
@@ -687,6 +754,63 @@ def test_host_tensors_can_be_snapshotted_inside_the_blocking_part(shm_dir):
         payload = raw[METADATA_SIZE + where.offset + where.length - host.numel() * 4 : METADATA_SIZE + where.offset + where.length]
         assert payload == (before if snapshot else host).numpy().tobytes()
         before = host.clone()
+
+
+@pytest.mark.parametrize("with_sidecar", [False, True])
+def test_a_partial_read_uploads_only_what_it_needs(shm_dir, monkeypatch, with_sidecar):
+    """Asking for two of sixteen tensors (weights without the optimizer state, say) uploads two neighbourhoods, not
+    the object; with a sidecar exactly the chunks that are read are checked: damage inside them is found, damage
+    elsewhere is not looked at."""
+    from torch.distributed.checkpoint.planner_helpers import _create_write_items
+
+    from ml_flashpoint.hip import checkpoint_loader as loader_mod
+    from ml_flashpoint.hip import integrity
+
+    monkeypatch.setattr(loader_mod, "_PARTIAL_READ_MIN_SAVING", 1 << 20)
+    monkeypatch.setattr(loader_mod, "_PARTIAL_READ_GAP", 1 << 16)
+    g = torch.Generator().manual_seed(33)
+    data_cpu = {f"t{i:02d}": torch.randn(1 << 16, generator=g) for i in range(16)}  # 256 KiB each, 4 MiB together
+    data = {k: v.to(DEV) for k, v in data_cpu.items()}
+    saver = _saver(crc_chunk_bytes=(1 << 16) if with_sidecar else 0)
+    cid = CheckpointContainerId(os.path.join(shm_dir, "step-9_ckpt"))
+    items = [wi for k, v in data.items() for wi in _create_write_items(k, v)]
+    buckets = saver.prepare_write_data(cid, items, _Resolver(data), "data", 1)
+    info = {r.index.fqn: r.storage_data for r in saver.write_data(cid, buckets, replicate_after_write=False)}
+    oid = CheckpointObjectId.from_container(cid, "data_0_src0.distcp")
+    by_offset = sorted(info, key=lambda k: info[k].offset)
+    wanted = [by_offset[2], by_offset[11]]  # far apart in the object
+    storage = {n: info[k] for n, k in enumerate(wanted)}
+
+    def read():
+        targets = {k: torch.zeros(1 << 16, device=DEV) for k in wanted}
+        reqs = [ReadItem(type=LoadItemType.TENSOR, dest_index=MetadataIndex(k), dest_offsets=torch.Size([0]), storage_index=n,
+                         storage_offsets=torch.Size([0]), lengths=torch.Size([1 << 16])) for n, k in enumerate(wanted)]
+        loader = _loader()
+        loader.read_data(oid, reqs, _Planner(targets), storage)
+        return targets, loader.last_load_stats
+
+    targets, stats = read()
+    assert all(torch.equal(targets[k].cpu(), data_cpu[k]) for k in wanted)
+    assert stats["partial_read_ranges"] == 2
+    assert stats["h2d_bytes"] <= 2 * ((1 << 18) + (3 << 16))  # two tensors and at most a chunk or two around each
+    untouched = info[by_offset[7]]
+    with open(oid.data, "r+b") as f:  # damage in a tensor nobody asked for
+        f.seek(METADATA_SIZE + untouched.offset + 5000)
+        f.write(b"\xff\x00\xff")
+    targets, _ = read()
+    assert all(torch.equal(targets[k].cpu(), data_cpu[k]) for k in wanted)
+    hit = info[wanted[1]]
+    with open(oid.data, "r+b") as f:  # damage in a tensor that is asked for
+        f.seek(METADATA_SIZE + hit.offset + hit.length - 1000)
+        byte = f.read(1)
+        f.seek(-1, os.SEEK_CUR)
+        f.write(bytes([byte[0] ^ 0x01]))
+    if with_sidecar:
+        with pytest.raises(integrity.ChecksumMismatchError, match=rf"chunk\(s\) \[{(hit.offset + hit.length - 1000) // (1 << 16)}\]"):
+            read()
+    else:
+        targets, _ = read()
+        assert torch.equal(targets[wanted[0]].cpu(), data_cpu[wanted[0]]) and not torch.equal(targets[wanted[1]].cpu(), data_cpu[wanted[1]])
 
 
 def test_legacy_torch_save_objects_are_still_readable(shm_dir):

@@ -227,3 +227,22 @@ def test_copy_threads_default_follows_the_cpus_available(monkeypatch):
     assert EngineConfig().resolved_copy_threads() == 16
     monkeypatch.setattr(os, "sched_getaffinity", lambda pid: {0, 1, 2})
     assert EngineConfig().resolved_copy_threads() == 3
+
+
+def test_partial_read_clusters_are_cut_on_the_right_boundaries(monkeypatch):
+    """Pure host arithmetic of the loader: which ranges of an object a partial read uploads."""
+    from ml_flashpoint.hip import checkpoint_loader as loader_mod
+
+    monkeypatch.setattr(loader_mod, "_PARTIAL_READ_GAP", 1000)
+    cluster = loader_mod.HipMLFlashpointCheckpointLoader._clusters_of
+    rows = [(50_000, 51_000, True, "c"), (5_000, 6_000, True, "a"), (6_500, 9_000, False, "b"), (100_000, 100_010, True, "d")]
+    # without a sidecar: starts on 4096-byte upload boundaries, ends where the last row ends
+    got = cluster(rows, None, 200_000)
+    assert [(lo, hi, [r[3] for r in members]) for lo, hi, members in got] == [
+        (4096, 9_000, ["a", "b"]), (49_152, 51_000, ["c"]), (98_304, 100_010, ["d"])]
+    # with a sidecar: whole checksum chunks, the last one cut at the end of the written data; ranges that come to
+    # touch after rounding are one
+    got = cluster(rows, 65536, 100_020)
+    assert [(lo, hi, [r[3] for r in members]) for lo, hi, members in got] == [(0, 100_020, ["a", "b", "c", "d"])]
+    monkeypatch.setattr(loader_mod, "_PARTIAL_READ_GAP", 0)
+    assert [(lo, hi) for lo, hi, _ in cluster(rows, 8192, 200_000)] == [(0, 16_384), (49_152, 57_344), (98_304, 106_496)]
