@@ -656,6 +656,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                 crcs = hip_plan.crc32c_file(fd, METADATA_SIZE + start, nbytes, self._crc_chunk_bytes,
                                             self._engine_config.resolved_copy_threads())
                 integrity.write_sidecar(str(object_id), self._crc_chunk_bytes, nbytes, crcs)
+            else:
+                integrity.remove_sidecar(str(object_id))
         stats["objects"] += 1
         stats["windows"] = stats.get("windows", 0) + len(windows)
         stats["device_payload_bytes"] += layout.device_payload_bytes
@@ -821,6 +823,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         staged.plan = None
         if crcs is not None:
             integrity.write_sidecar(str(bucket.object_id), self._crc_chunk_bytes, nbytes, crcs)
+        else:
+            integrity.remove_sidecar(str(bucket.object_id))
         return self._results_of(staged, bucket.object_name)
 
     @staticmethod

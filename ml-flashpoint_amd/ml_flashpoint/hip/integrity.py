@@ -30,6 +30,14 @@ def write_sidecar(object_path: str, chunk_bytes: int, data_bytes: int, crcs: np.
     os.rename(tmp, path)
 
 
+def remove_sidecar(object_path: str) -> None:
+    """Drops the sidecar of an object that has just been rewritten without checksums: an old one would condemn it."""
+    try:
+        os.unlink(sidecar_path(object_path))
+    except FileNotFoundError:
+        pass
+
+
 def read_sidecar(object_path: str) -> Optional[Tuple[int, int, np.ndarray]]:
     """Returns (chunk_bytes, data_bytes, crcs) or None if the object has no (valid) sidecar."""
     path = sidecar_path(object_path)

@@ -252,6 +252,11 @@ def test_crc_sidecar_written_and_corruption_detected(shm_dir, manager_future):
     cause = exc.value.failures[0][0] if hasattr(exc.value, "failures") else exc.value
     assert isinstance(cause, integrity.ChecksumMismatchError) and "chunk(s) [2]" in str(cause)
     dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, _loader(verify_crc=False)), no_dist=True)
+    # the same object written again without checksums: the old sidecar must not outlive the bytes it described
+    dcp.save(sd, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(_saver(), manager_future), no_dist=True)
+    assert integrity.read_sidecar(obj) is None and not os.path.exists(integrity.sidecar_path(obj))
+    dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, _loader()), no_dist=True)
+    assert all(torch.equal(target[k], sd[k]) for k in sd)
 
 
 @pytest.mark.parametrize("save_file_io,load_file_io", [(False, False), (False, True), (True, False), (True, True)])
