@@ -23,6 +23,7 @@ import warnings
 from pathlib import Path
 from typing import IO, Callable, List, Optional, cast
 
+import numpy as np
 import torch
 from torch.distributed._shard._utils import narrow_tensor_by_index
 from torch.distributed.checkpoint import Metadata
@@ -49,8 +50,12 @@ _MAX_HEADER_LEN = 1024 * 1024  # a larger "length" means the record is not in th
 _UPLOAD_ALIGN = 4096
 # A read that asks for part of an object (the weights out of weights + optimizer state, say) uploads only the
 # neighbourhoods of what it asks for, when that leaves out at least this much; requested ranges closer than the gap
-# are fetched together.
+# are fetched together (a range costs about 0.3 ms to set up, the time 17 MB take on the link; measured on the
+# weights of the 112 GB shard: 16 MiB 0.41 s, 128 MiB 0.47 s).
 _PARTIAL_READ_MIN_SAVING = 256 << 20
+# neighbourhoods that share a device buffer start on this boundary in it (uploads to less aligned device addresses
+# were measured at half the link's rate)
+_SLICE_ALIGN = 2 << 20
 _PARTIAL_READ_GAP = 16 << 20
 _U32 = struct.Struct("<I")
 _HEADER_CACHE: dict = {}  # header pickle bytes -> (dtype, shape, stored payload bytes)
@@ -341,8 +346,19 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                 limit = self._image_limit(device)
                 # one buffer for the range (or for the largest neighbourhood of a partial read) if the allocator
                 # has a block of that size; through a smaller buffer, window by window, if it has not
-                need = max(c_hi - c_lo for c_lo, c_hi, _ in clusters) if clusters is not None else hi - lo
-                image = hip_plan.try_allocate(need, device) if need <= limit else None
+                image = None
+                if clusters is not None:
+                    # all neighbourhoods side by side in one buffer (one unpack for all of them), or one after
+                    # the other through a buffer for the largest
+                    for need in (sum(-(-(c_hi - c_lo) // _SLICE_ALIGN) * _SLICE_ALIGN for c_lo, c_hi, _ in clusters),
+                                 max(c_hi - c_lo for c_lo, c_hi, _ in clusters)):
+                        image = hip_plan.try_allocate(need, device) if need <= limit else None
+                        if image is not None:
+                            break
+                    need = min(need, limit)
+                else:
+                    need = hi - lo
+                    image = hip_plan.try_allocate(need, device) if need <= limit else None
                 if image is None:
                     self._restore_windowed(object_id, stream, device, rows, min(limit, need), sidecar, stats)
                 elif clusters is not None:
@@ -433,18 +449,32 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         return [(lo, hi, members) for lo, hi, members in clusters]
 
     def _restore_clusters(self, object_id, stream, device, clusters, sidecar, stats, image) -> None:
-        """A partial read: every cluster is uploaded into ``image``, checked against the sidecar's values for exactly
-        the chunks it covers, and unpacked.  What the request does not touch is neither read nor checked."""
+        """A partial read: every cluster is uploaded into ``image`` and checked against the sidecar's values for
+        exactly the chunks it covers.  If ``image`` has room for all clusters they lie side by side and one unpack
+        serves them all; otherwise they pass through it one at a time.  What the request does not touch is
+        neither read nor checked."""
         cur = torch.cuda.current_stream(device)
-        for lo, hi, members in clusters:
+        bases, at = [], 0
+        for lo, hi, _ in clusters:
+            bases.append(at)
+            at += -(-(hi - lo) // _SLICE_ALIGN) * _SLICE_ALIGN
+        together = at <= image.numel()
+        tables = []
+        for (lo, hi, members), base in zip(clusters, bases if together else [0] * len(clusters)):
             span = hi - lo
-            self._upload(stream, lo, image, span, cur, stats)
+            part = image[base : base + span]
+            self._upload(stream, lo, part, span, cur, stats)
             if sidecar is not None:
                 chunk_bytes, _, want = sidecar
-                got = hip_plan.crc32c_device(image, span, chunk_bytes, cur.cuda_stream)
+                got = hip_plan.crc32c_device(part, span, chunk_bytes, cur.cuda_stream)
                 first = lo // chunk_bytes
                 self._compare_checksums(object_id, got, want[first : first + len(got)], chunk_bytes, first, len(want))
-            self._unpack(self._table_of(members, lo), image, span, cur, sum(r[1] - r[0] for r in members if r[2]))
+            if together:
+                tables.append(self._table_of(members, lo - base))
+            else:
+                self._unpack(self._table_of(members, lo), image, span, cur, sum(r[1] - r[0] for r in members if r[2]))
+        if together:
+            self._unpack(np.concatenate(tables), image, at, cur, stats["device_payload_bytes"])
         stats["partial_read_ranges"] = stats.get("partial_read_ranges", 0) + len(clusters)
 
     def _restore_windowed(self, object_id, stream, device, rows, limit, sidecar, stats) -> None:
