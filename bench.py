@@ -46,7 +46,8 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=3)
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--workload", default="llama3-8b-shard",
-                    choices=["llama3-8b-shard", "many-small", "mixtral-expert-shard", "strided-views", "gpt2-small"])
+                    choices=["llama3-8b-shard", "many-small", "mixtral-expert-shard", "strided-views", "gpt2-small",
+                             "offloaded-optimizer"])
     ap.add_argument("--scale", type=float, default=1.0, help="fraction of the workload's layers/tensors (debugging)")
     ap.add_argument("--tile-bytes", type=int, default=0)
     ap.add_argument("--block-threads", type=int, default=0)
@@ -65,6 +66,9 @@ def parse_args():
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run one plain elementwise kernel (torch.add, 4 GiB in, 4 GiB out) so that hardware byte "
                          "counters of a profiler run can be scaled against a kernel of known traffic")
+    ap.add_argument("--partial-restore-prefix", default=None,
+                    help="after the timed steps, also time a restore of only the entries whose names start with this "
+                         "(e.g. 'model.': the weights out of weights + optimizer state); reported as partial_restore")
     ap.add_argument("--root", default=None, help="directory on tmpfs for the pool and checkpoints")
     return ap.parse_args()
 
@@ -88,6 +92,9 @@ def build_workload(name, device, scale):
         sd = dict(sd)
         sd["__parents__"] = parents  # keep alive; not a tensor entry
         label = "2,000 transposed / strided / row-block views of bf16/fp8/fp32 parents"
+    elif name == "offloaded-optimizer":
+        sd = workloads.offloaded_optimizer_shard(device, layers=max(1, round(8 * scale)))
+        label = "bf16 weights on the device, fp32 master + Adam m,v in host memory"
     else:
         sd = workloads.gpt2_small(device)
         label = "GPT-2-small fp32"
@@ -360,7 +367,11 @@ def main():
                 rec["plan"].append(t_plan - t0)
                 rec["pack_launch"].append(t_launch - t_plan)
                 rec["d2h"].append(d2h.get("d2h_s", 0.0))
+                rec.setdefault("d2h_bytes", []).append(d2h.get("d2h_bytes", 0))
+                rec.setdefault("host_copy_s", []).append(d2h.get("host_copy_s", 0.0))
+                rec.setdefault("host_copy_bytes", []).append(d2h.get("host_copy_bytes", 0))
                 rec["h2d"].append(loader.last_load_stats.get("h2d_s", 0.0))
+                rec.setdefault("h2d_bytes", []).append(loader.last_load_stats.get("h2d_bytes", 0))
                 rec.setdefault("pack_ms", []).append(pack_ms)
                 rec.setdefault("unpack_ms", []).append(unpack_ms)
                 rec.setdefault("pack_bytes", []).append(pack_bytes)
@@ -368,6 +379,25 @@ def main():
         # parity after the timed region: restored bits == original bits
         mismatched = [k for k, v in sd.items() if workloads.fingerprint(v) != prints[k]]
         assert not mismatched, f"restored tensors differ from the originals: {mismatched[:5]}"
+        partial = None
+        if args.partial_restore_prefix:
+            subset = {k: v for k, v in sd.items() if k.startswith(args.partial_restore_prefix)}
+            assert subset and len(subset) < len(sd), "--partial-restore-prefix must select some, not all, entries"
+            times = []
+            for _ in range(3):
+                for v in subset.values():
+                    v.zero_() if v.is_contiguous() else v.fill_(0)
+                torch.cuda.synchronize()
+                t1 = time.perf_counter()
+                dcp.load(subset, checkpoint_id=prev.data, storage_reader=MemoryStorageReader(prev.data, loader), no_dist=True)
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t1)
+            assert all(workloads.fingerprint(v) == prints[k] for k, v in subset.items()), "partial restore differs"
+            stats = loader.last_load_stats
+            partial = {"prefix": args.partial_restore_prefix, "entries": len(subset),
+                       "payload_bytes": workloads.payload_bytes(subset), "seconds": round(min(times), 4),
+                       "uploaded_bytes": stats.get("h2d_bytes", 0), "ranges": stats.get("partial_read_ranges", 1)}
+            print(f"[bench] partial restore of '{args.partial_restore_prefix}*': {partial}", file=sys.stderr, flush=True)
         manager.delete_container(prev)
 
         mean = lambda xs: sum(xs) / len(xs)  # noqa: E731
@@ -393,6 +423,7 @@ def main():
                        "file_bytes": file_bytes, "scale": args.scale, "tile_bytes": args.tile_bytes or 4096,
                        "engine": {"slot_mib": args.slot_mib, "slots": args.slots, "copy_threads": engine_cfg.resolved_copy_threads()},
                        "crc_chunk_mib": args.crc_chunk_mib, "plan_cache": args.plan_cache, "save_io": args.save_io, "restore_io": args.restore_io},
+            **({"partial_restore": partial} if partial else {}),
             "save_GBps": round(gb / mean(rec["save"]), 3),
             "restore_GBps": round(gb / mean(rec["restore"]), 3),
             "blocking_save_ms": round(mean(rec["blocking"]) * 1e3, 2),
@@ -403,8 +434,10 @@ def main():
             "blocking_host_us_per_tensor": round((mean(rec["blocking"]) - pack_s) * 1e6 / max(len(sd), 1), 2),
             "pack_GBps": round(pack_gbps, 1),
             "unpack_GBps": round(2 * mean(rec["unpack_bytes"]) / 1e9 / unpack_s, 1) if unpack_s > 0 else None,
-            "d2h_GBps": round(gb / mean(rec["d2h"]), 2) if mean(rec["d2h"]) > 0 else None,
-            "h2d_GBps": round(gb / mean(rec["h2d"]), 2) if mean(rec["h2d"]) > 0 else None,
+            "d2h_GBps": round(mean(rec["d2h_bytes"]) / 1e9 / mean(rec["d2h"]), 2) if mean(rec["d2h"]) > 0 else None,
+            **({"host_copy_GBps": round(mean(rec["host_copy_bytes"]) / 1e9 / mean(rec["host_copy_s"]), 2),
+                "host_copy_bytes": int(mean(rec["host_copy_bytes"]))} if mean(rec["host_copy_s"]) > 0 else {}),
+            "h2d_GBps": round(mean(rec["h2d_bytes"]) / 1e9 / mean(rec["h2d"]), 2) if mean(rec["h2d"]) > 0 else None,
             "parity": "restored tensors bit-identical to originals (fingerprints)",
             "roofline": {"bound": "hbm", "kernel": "mlf_flat_kernel<pack>", "achieved": round(pack_gbps, 1),
                          "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(pack_gbps / HBM_PEAK_GBPS, 4),

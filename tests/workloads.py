@@ -67,6 +67,23 @@ def llama3_8b_shard(device, seed=2024, **dims) -> Dict[str, torch.Tensor]:
     return sd
 
 
+def offloaded_optimizer_shard(device, seed=31, layers=8, d=8192, ffn=16384) -> Dict[str, torch.Tensor]:
+    """Weights on the device, optimizer state in host memory (an offloaded optimizer): per layer one bf16 weight of
+    ``d`` x ``ffn`` on the device and its fp32 master copy, exp_avg and exp_avg_sq on the host.  At the default
+    sizes: 2.1 GB on the device, 12.9 GB on the host."""
+    g = _gen(device, seed)
+    host = torch.Generator().manual_seed(seed)
+    sd = {}
+    for i in range(layers):
+        master = torch.randn(d, ffn, generator=host, dtype=torch.float32) * 0.02
+        sd[f"model.layers.{i}.weight"] = master.to(torch.bfloat16).to(device)
+        sd[f"optimizer.master.{i}"] = master
+        sd[f"optimizer.exp_avg.{i}"] = torch.randn(d, ffn, generator=host, dtype=torch.float32) * 1e-3
+        sd[f"optimizer.exp_avg_sq.{i}"] = torch.randn(d, ffn, generator=host, dtype=torch.float32).abs_() * 1e-4
+    _ = g
+    return sd
+
+
 def many_small(device, seed=7, count=20000, min_log2=6, max_log2=22) -> Dict[str, torch.Tensor]:
     """C3: ``count`` tensors, byte sizes log-uniform in [2^min_log2, 2^max_log2], dtypes cycling fp32/bf16/int64."""
     cpu = torch.Generator().manual_seed(seed)
