@@ -695,3 +695,13 @@ def test_watched_transfer_publishes_only_bytes_that_are_in_place(shm_dir, oracle
     del view
     bo.close()
     engine.destroy()
+
+
+def test_try_allocate_reports_what_the_allocator_cannot_provide():
+    """A request the device cannot satisfy comes back as None (after the allocator has returned its unused segments
+    and been asked again), not as an exception; an ordinary one as a byte buffer."""
+    from ml_flashpoint.hip import plan as P
+
+    assert P.try_allocate(1 << 50, torch.device(DEV)) is None  # a pebibyte
+    buf = P.try_allocate(4096, torch.device(DEV))
+    assert buf.dtype == torch.uint8 and buf.numel() == 4096 and buf.device == torch.device(DEV)
