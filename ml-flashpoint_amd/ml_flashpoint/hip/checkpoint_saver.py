@@ -27,6 +27,7 @@ import time
 import uuid
 from typing import Callable, Optional, Union
 
+import numpy as np
 import torch
 from torch.distributed.checkpoint import metadata as torchdistmeta
 from torch.distributed.checkpoint.filesystem import _split_by_size_and_type, _StorageInfo
@@ -457,7 +458,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             fresh_blob = kept.refreshed_blob(tensors, blobs)
             layout = dataclasses.replace(kept.layout, blob=kept.blob,
                                          device_tensors=[t for t in tensors if t.device.type != "cpu"],
-                                         host_tensors=[tensors[i] for _, _, i in kept.layout.host_spans])
+                                         host_tensors=[tensors[i] if i >= 0 else blobs[-1 - i]
+                                                       for _, _, i in kept.layout.host_spans])
         else:
             # through the file descriptor (pwrite) everything goes through the image; the direct host copy
             # writes into the mapping
@@ -469,7 +471,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             if device is None:
                 device = torch.device("cuda", torch.cuda.current_device())
         if layout.host_tensors and self._snapshot_host_tensors:
-            layout.host_tensors = [t.detach().clone(memory_format=torch.contiguous_format) for t in layout.host_tensors]
+            layout.host_tensors = [t.detach().clone(memory_format=torch.contiguous_format) if isinstance(t, torch.Tensor)
+                                   else t for t in layout.host_tensors]  # (byte blobs are immutable as they are)
         items = [item for item, _ in tensor_data] + [item for item, _ in bytes_data]
         plan = image = packed = None
         stream = 0
@@ -872,9 +875,14 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                 self._count_transfer(xfer, st, n)
             else:
                 t0 = time.perf_counter()
-                source = tensor.detach().contiguous()  # a copy only if the tensor is a strided view
-                assert source.numel() * source.element_size() == n
-                engine.host_copy(dst, source.data_ptr(), n)
+                if isinstance(tensor, torch.Tensor):
+                    source = tensor.detach().contiguous()  # a copy only if the tensor is a strided view
+                    assert source.numel() * source.element_size() == n
+                    engine.host_copy(dst, source.data_ptr(), n)
+                else:  # the bytes of a large pickled object
+                    source = np.frombuffer(tensor, dtype=np.uint8)
+                    assert source.size == n
+                    engine.host_copy(dst, source.ctypes.data, n)
                 t_host += time.perf_counter() - t0
                 xfer["host_copy_bytes"] = xfer.get("host_copy_bytes", 0) + n
             staged._landed.value = data_off + n

@@ -144,8 +144,9 @@ class SaveLayout:
     # index into the tensors / blobs argument).  A layout that is reused for the next save refreshes exactly these.
     variable_parts: List[Tuple[int, int, str, int]] = dataclasses.field(default_factory=list)
     data_bytes: int = -1  # -1: same as image_bytes
-    host_spans: List[Tuple[int, int, int]] = dataclasses.field(default_factory=list)  # (data offset, nbytes, tensor index)
-    host_tensors: List[torch.Tensor] = dataclasses.field(default_factory=list)  # one per host span
+    # (data offset, nbytes, index): index >= 0 into the tensors, -1 - k for byte blob k
+    host_spans: List[Tuple[int, int, int]] = dataclasses.field(default_factory=list)
+    host_tensors: list = dataclasses.field(default_factory=list)  # one source per host span: a tensor, or the blob's bytes
     segments: List[Tuple[int, int, int]] = dataclasses.field(default_factory=list)  # (image offset, data offset, nbytes)
 
     def __post_init__(self):
@@ -159,8 +160,8 @@ def build_save_layout(tensors: Sequence[torch.Tensor], blobs: Sequence[bytes] = 
 
     Device tensors become DEVICE items (any strides; the image side is the C-contiguous payload).  Record headers,
     payloads of host-resident tensors and byte blobs are collected into one host blob that the plan uploads once -
-    except host-resident tensors of at least ``host_direct_min`` bytes (None: no such exception), which never
-    visit the device: the layout only notes where in the data section they belong (``host_spans``).
+    except host-resident tensors and byte blobs of at least ``host_direct_min`` bytes (None: no such exception),
+    which never visit the device: the layout only notes where in the data section they belong (``host_spans``).
     """
     table = ItemTable()
     blob = bytearray()
@@ -202,13 +203,16 @@ def build_save_layout(tensors: Sequence[torch.Tensor], blobs: Sequence[bytes] = 
             pos += nbytes
         spans.append((start, pos - start))
     for index, data in enumerate(blobs):
-        if len(data):
+        if host_direct_min is not None and len(data) >= max(host_direct_min, 1):
+            host_spans.append((pos, len(data), -1 - index))  # a large pickled object: host to buffer, like a tensor
+            host_tensors.append(data)
+        elif len(data):
             variable.append((len(blob), len(data), "blob", index))
             table.add_blob(len(blob), ipos, len(data))
             blob += data
+            ipos += len(data)
         spans.append((pos, len(data)))
         pos += len(data)
-        ipos += len(data)
     segments: List[Tuple[int, int, int]] = []
     image_at = data_at = 0
     for offset, nbytes, _ in host_spans:

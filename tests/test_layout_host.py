@@ -76,7 +76,9 @@ def test_host_tensors_above_the_threshold_are_left_out_of_the_image(data):
     want, spans = fmt.data_section(tensors, blobs)
     assert layout.spans == spans and layout.data_bytes == len(want)
     big = [i for i, t in enumerate(tensors) if t.numel() * t.element_size() >= threshold]
-    assert [i for _, _, i in layout.host_spans] == big and [id(t) for t in layout.host_tensors] == [id(tensors[i]) for i in big]
+    big += [-1 - k for k, b in enumerate(blobs) if len(b) >= threshold]  # byte blobs follow the same rule
+    assert [i for _, _, i in layout.host_spans] == big
+    assert [id(t) for t in layout.host_tensors] == [id(tensors[i]) if i >= 0 else id(blobs[-1 - i]) for i in big]
     assert layout.image_bytes == len(want) - sum(n for _, n, _ in layout.host_spans)
     # the image, as the pack kernel would fill it from the table (every row is a piece of the blob here)
     image = bytearray(layout.image_bytes)
@@ -89,7 +91,7 @@ def test_host_tensors_above_the_threshold_are_left_out_of_the_image(data):
         built[data_off : data_off + n] = image[image_off : image_off + n]
         covered += n
     for (data_off, n, _), t in zip(layout.host_spans, layout.host_tensors):
-        built[data_off : data_off + n] = P.host_tensor_bytes(t)
+        built[data_off : data_off + n] = P.host_tensor_bytes(t) if isinstance(t, torch.Tensor) else t
         covered += n
     assert covered == len(want) and bytes(built) == want
     pieces = sorted([(d, n) for _, d, n in layout.segments] + [(d, n) for d, n, _ in layout.host_spans])
