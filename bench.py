@@ -20,6 +20,7 @@ Synthetic data, seeded; the restored tensors are checked against fingerprints of
 
 import argparse
 import concurrent.futures
+import gc
 import json
 import os
 import shutil
@@ -319,6 +320,7 @@ def main():
                 manager.delete_container(prev)
             saver.kernel_events.clear()
             loader.kernel_events.clear()
+            gc.collect()  # outside the timed regions: a full collection of this process's heap takes ~60 ms
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             # ---- save: plan -> pack (blocking part ends at the synchronize) -> D2H -> metadata -> finalize ----
