@@ -126,3 +126,12 @@ class CheckpointObjectManager:
                 raise exc_info[1]
 
         shutil.rmtree(path, onerror=unless_already_gone)
+
+
+def _fresh_pool_lock_after_fork() -> None:
+    """The class-level lock may have been held by a thread of the parent that the forked child does not have."""
+    CheckpointObjectManager._worker_pool_lock = threading.Lock()
+
+
+if hasattr(os, "register_at_fork"):
+    os.register_at_fork(after_in_child=_fresh_pool_lock_after_fork)

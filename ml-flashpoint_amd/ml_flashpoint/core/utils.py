@@ -78,6 +78,21 @@ _gc_pause_depth = 0
 _gc_was_enabled = False
 
 
+def _fresh_gc_pause_state_after_fork() -> None:
+    """A forked child (an async framework's worker) inherits the lock in whatever state some other thread of the parent
+    left it, and none of those threads: start over with a free lock, no pause in progress, and the collector as it
+    was before the pause the fork may have fallen into."""
+    global _gc_pause_lock, _gc_pause_depth
+    if _gc_pause_depth > 0 and _gc_was_enabled:
+        gc.enable()
+    _gc_pause_lock = threading.Lock()
+    _gc_pause_depth = 0
+
+
+if hasattr(os, "register_at_fork"):
+    os.register_at_fork(after_in_child=_fresh_gc_pause_state_after_fork)
+
+
 @contextlib.contextmanager
 def gc_paused():
     """Suspends the cyclic garbage collector for the duration of the block (re-entrant, thread-safe, restores the

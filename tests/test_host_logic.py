@@ -246,3 +246,36 @@ def test_partial_read_clusters_are_cut_on_the_right_boundaries(monkeypatch):
     assert [(lo, hi, [r[3] for r in members]) for lo, hi, members in got] == [(0, 100_020, ["a", "b", "c", "d"])]
     monkeypatch.setattr(loader_mod, "_PARTIAL_READ_GAP", 0)
     assert [(lo, hi) for lo, hi, _ in cluster(rows, 8192, 200_000)] == [(0, 16_384), (49_152, 57_344), (98_304, 106_496)]
+
+
+def test_a_forked_child_starts_with_free_locks_and_a_running_collector():
+    """An async framework forks its worker from the training process at any moment: the child must not inherit a
+    held lock (the thread that held it does not exist there) or a collector that was paused by such a thread."""
+    import gc
+    import os
+
+    from ml_flashpoint.checkpoint_object_manager.checkpoint_object_manager import CheckpointObjectManager
+    from ml_flashpoint.core import utils
+
+    assert gc.isenabled()
+    with utils.gc_paused():
+        utils._gc_pause_lock.acquire()  # as if another thread were inside the bookkeeping right now
+        CheckpointObjectManager._worker_pool_lock.acquire()
+        try:
+            pid = os.fork()
+            if pid == 0:
+                ok = False
+                try:
+                    free = utils._gc_pause_lock.acquire(timeout=2) and CheckpointObjectManager._worker_pool_lock.acquire(timeout=2)
+                    utils._gc_pause_lock.release()
+                    with utils.gc_paused():
+                        paused = not gc.isenabled()
+                    ok = bool(free) and paused and gc.isenabled() and utils._gc_pause_depth == 0
+                finally:
+                    os._exit(0 if ok else 1)
+            _, status = os.waitpid(pid, 0)
+        finally:
+            utils._gc_pause_lock.release()
+            CheckpointObjectManager._worker_pool_lock.release()
+    assert os.WIFEXITED(status) and os.WEXITSTATUS(status) == 0
+    assert gc.isenabled()
