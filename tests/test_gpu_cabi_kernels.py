@@ -705,3 +705,17 @@ def test_try_allocate_reports_what_the_allocator_cannot_provide():
     assert P.try_allocate(1 << 50, torch.device(DEV)) is None  # a pebibyte
     buf = P.try_allocate(4096, torch.device(DEV))
     assert buf.dtype == torch.uint8 and buf.numel() == 4096 and buf.device == torch.device(DEV)
+
+
+def test_a_cpp_program_uses_the_two_libraries_without_python_or_torch(shm_dir):
+    """tests/cabi/direct_caller.cpp links libmlf_hip.so and libmlf_buffer.so and walks the whole path - plan, pack,
+    checksum, watched transfer into a buffer file, reopen, upload through the descriptor, unpack - checking every
+    stage against bytes it builds on the host.  Built by ``__graft_entry__.build()``."""
+    import os
+    import subprocess
+
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cabi", "_build", "direct_caller")
+    assert os.path.exists(exe), "run __graft_entry__.build() first"
+    done = subprocess.run([exe, shm_dir], capture_output=True, text=True, timeout=100)
+    assert done.returncode == 0, done.stderr + done.stdout
+    assert "direct C-ABI caller ok" in done.stdout
