@@ -128,6 +128,18 @@ int mlf_unpack_launch(const mlf_plan* plan, const void* image_dev, void* stream)
  * of the copy pipeline (values are kept beside the object, never inside it). */
 int mlf_crc32c_device(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint32_t* out_host,
                       uint64_t n_out, void* stream);
+/* mlf_crc32c_device for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc); it has no counterpart in the reference.  Same values, but nothing is
+ * allocated or freed by the call: the lookup constants and the per-segment values live in a fixed array of
+ * 1 056 768 bytes that is part of the library's code object on every device it runs on, the per-chunk values are
+ * written to `out_dev` (DEVICE memory of the caller, ceil(nbytes/chunk_bytes) values, 4-byte aligned), and
+ * the call only enqueues kernels on `stream`: the values are valid when the stream reaches the point after it.
+ * Limit: at most 262 144 segment values per call (segments are 64 KiB to 512 KiB by the size of the buffer and are
+ * doubled, while they still divide `chunk_bytes`, until their count fits); more than that, e.g. 16 GiB in 64 KiB
+ * chunks, is refused with a message.  All calls on one device share that device's array and every call
+ * overwrites it: calls that overlap in time on one device race; calls ordered on one stream do not. */
+int mlf_crc32c_device_noalloc(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint32_t* out_dev,
+                              uint64_t n_out, void* stream);
 /* Same function on host memory (SSE4.2), and the combine law crc(A||B) from crc(A), crc(B), len(B). */
 uint32_t mlf_crc32c_host(const void* data, uint64_t nbytes);
 uint32_t mlf_crc32c_combine(uint32_t crc_a, uint32_t crc_b, uint64_t len_b);

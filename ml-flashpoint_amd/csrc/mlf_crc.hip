@@ -157,8 +157,50 @@ __global__ void mlf_crc_chunks_kernel(const uint32_t* __restrict__ seg_crc, uint
   out[c] = s ^ 0xFFFFFFFFu;
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// scratch of the allocation-free entry point (mlf_crc32c_device_noalloc)
+// ---------------------------------------------------------------------------------------------------------
+// A fixed array in every device's copy of this code object: the lookup constants, then one value per segment.
+// 256 Ki segment values cover 128 GiB at 512 KiB segments.  The array's name is a host-side stand-in, not a device
+// address: host code uses the per-device address that hipGetSymbolAddress returned, never the name.
+constexpr uint32_t kNoAllocMaxSegs = 256 * 1024;
+constexpr size_t kNoAllocConstsBytes = 8192;  // sizeof(CrcConsts) rounded up; the segment values follow
+constexpr size_t kNoAllocScratchBytes = kNoAllocConstsBytes + (size_t)kNoAllocMaxSegs * sizeof(uint32_t);
+static_assert(sizeof(CrcConsts) <= kNoAllocConstsBytes, "the constants must fit in front of the segment values");
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+constexpr int kNoAllocMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kNoAllocMaxDevices];  // device address of `scratch` on each device, looked up on first use there
+
+struct CrcFoldConsts {
+  uint32_t xrow, x4, x16, x32, x64, x128, x256, x512;
+};
+
+// Writes the lookup constants where a later kernel on the same stream reads them: 1024 threads, one table entry each.
+__global__ void __launch_bounds__(1024) mlf_crc_fill_consts_kernel(CrcConsts* __restrict__ consts, CrcFoldConsts k) {
+  const uint32_t i = threadIdx.x;
+  consts->row_tab[i >> 8][i & 255u] = gf_mul(k.xrow, (i & 255u) << (8u * (i >> 8)));
+  if (i == 0) {
+    consts->x4 = k.x4;
+    consts->x16 = k.x16;
+    consts->x32 = k.x32;
+    consts->x64 = k.x64;
+    consts->x128 = k.x128;
+    consts->x256 = k.x256;
+    consts->x512 = k.x512;
+  }
+}
+
 std::once_flag g_crc_once;
 CrcConsts g_crc_host;
+
+// The longest segment that divides the chunks and still leaves every CU several blocks of wavefronts.
+uint64_t pick_seg_bytes(uint64_t nbytes, uint64_t chunk_bytes) {
+  uint64_t seg_bytes = kCrcSegBytes;
+  while (seg_bytes < kCrcMaxSegBytes && chunk_bytes % (2 * seg_bytes) == 0 && nbytes / (2 * seg_bytes) >= 8192) seg_bytes *= 2;
+  return seg_bytes;
+}
 
 void crc_init_host() {
   const uint32_t xrow = x_pow_bytes(kCrcRowBytes);
@@ -195,9 +237,7 @@ int crc_enqueue(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint
     return fail(MLF_HIP_BAD_ARG, "chunk_bytes must be a positive multiple of 65536");
   const uint64_t n_chunks = (nbytes + chunk_bytes - 1) / chunk_bytes;
   if (n_out < n_chunks) return fail(MLF_HIP_BAD_ARG, "output array too small");
-  // the longest segment that divides the chunks and still leaves every CU several blocks of wavefronts
-  uint64_t seg_bytes = kCrcSegBytes;
-  while (seg_bytes < kCrcMaxSegBytes && chunk_bytes % (2 * seg_bytes) == 0 && nbytes / (2 * seg_bytes) >= 8192) seg_bytes *= 2;
+  const uint64_t seg_bytes = pick_seg_bytes(nbytes, chunk_bytes);
   const uint64_t n_segs = (nbytes + seg_bytes - 1) / seg_bytes;
   if (n_segs > 0xFFFFFFF0ull) return fail(MLF_HIP_BAD_ARG, "buffer too large for one CRC call");
   std::call_once(g_crc_once, crc_init_host);
@@ -322,6 +362,73 @@ int mlf_crc32c_device(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes
   CrcJob job;
   if (int rc = crc_enqueue(dev_ptr, nbytes, chunk_bytes, n_out, static_cast<hipStream_t>(stream_), &job, false)) return rc;
   return crc_finish(&job, out_host);
+}
+
+int mlf_crc32c_device_noalloc(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint32_t* out_dev,
+                              uint64_t n_out, void* stream_) {
+  if (nbytes == 0) return MLF_HIP_OK;
+  if (!dev_ptr || !out_dev) return fail(MLF_HIP_BAD_ARG, "null pointer");
+  if (reinterpret_cast<uintptr_t>(dev_ptr) & 15) return fail(MLF_HIP_BAD_ARG, "device buffer must be 16-byte aligned");
+  if (reinterpret_cast<uintptr_t>(out_dev) & 3) return fail(MLF_HIP_BAD_ARG, "output array must be 4-byte aligned");
+  if (chunk_bytes == 0 || chunk_bytes % kCrcSegBytes)
+    return fail(MLF_HIP_BAD_ARG, "chunk_bytes must be a positive multiple of 65536");
+  const uint64_t n_chunks = (nbytes + chunk_bytes - 1) / chunk_bytes;
+  if (n_out < n_chunks) return fail(MLF_HIP_BAD_ARG, "output array too small");
+  if (n_chunks > 0xFFFFFFF0ull) return fail(MLF_HIP_BAD_ARG, "buffer too large for one CRC call");
+  // segments as the allocating entry point cuts them, doubled while their values would not fit in the fixed array
+  // (a segment must still divide the chunk size)
+  uint64_t seg_bytes = pick_seg_bytes(nbytes, chunk_bytes);
+  while ((nbytes + seg_bytes - 1) / seg_bytes > kNoAllocMaxSegs && chunk_bytes % (2 * seg_bytes) == 0 &&
+         2 * seg_bytes <= (1ull << 30))
+    seg_bytes *= 2;
+  const uint64_t n_segs = (nbytes + seg_bytes - 1) / seg_bytes;
+  if (n_segs > kNoAllocMaxSegs)
+    return fail(MLF_HIP_BAD_ARG,
+                "mlf_crc32c_device_noalloc: " + std::to_string(nbytes) + " bytes in chunks of " + std::to_string(chunk_bytes) +
+                    " need " + std::to_string(n_segs) + " segment values, the fixed scratch array holds " +
+                    std::to_string(kNoAllocMaxSegs) + " (use larger chunks, several calls, or mlf_crc32c_device)");
+  int device = 0;
+  HIP_TRY(hipGetDevice(&device));
+  if (device < 0 || device >= kNoAllocMaxDevices) return fail(MLF_HIP_BAD_ARG, "device index beyond the per-device table");
+  void* base = nullptr;
+  {
+    // once per device, with that device current: every device holds its own copy of the array at its own address
+    std::lock_guard<std::mutex> g(g_scratch_mu);
+    if (!g_scratch_ptr[device]) {
+      void* p = nullptr;
+      HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+      if (!p) return fail(MLF_HIP_RUNTIME, "hipGetSymbolAddress returned a null address for the scratch array");
+      g_scratch_ptr[device] = p;
+    }
+    base = g_scratch_ptr[device];
+  }
+  CrcConsts* consts = static_cast<CrcConsts*>(base);
+  uint32_t* seg = reinterpret_cast<uint32_t*>(static_cast<char*>(base) + kNoAllocConstsBytes);
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  // Every call writes all it later reads (the constants, then one value per segment of this call), in stream order:
+  // nothing has to start at zero and what an earlier call left behind is never looked at.
+  CrcFoldConsts k;
+  k.xrow = x_pow_bytes(kCrcRowBytes);
+  k.x4 = x_pow_bytes(4);
+  k.x16 = x_pow_bytes(16);
+  k.x32 = x_pow_bytes(32);
+  k.x64 = x_pow_bytes(64);
+  k.x128 = x_pow_bytes(128);
+  k.x256 = x_pow_bytes(256);
+  k.x512 = x_pow_bytes(512);
+  hipLaunchKernelGGL(mlf_crc_fill_consts_kernel, dim3(1), dim3(1024), 0, stream, consts, k);
+  HIP_TRY(hipGetLastError());
+  const uint32_t waves_per_block = kCrcThreads / 64;
+  const uint32_t grid = (uint32_t)((n_segs + waves_per_block - 1) / waves_per_block);
+  hipLaunchKernelGGL(mlf_crc_segments_kernel<kCrcTableCopies>, dim3(grid), dim3(kCrcThreads), 0, stream,
+                     static_cast<const char*>(dev_ptr), nbytes, consts, seg, (uint32_t)n_segs, (uint32_t)seg_bytes);
+  HIP_TRY(hipGetLastError());
+  const uint64_t last_seg_len = nbytes - (n_segs - 1) * seg_bytes;
+  hipLaunchKernelGGL(mlf_crc_chunks_kernel, dim3((uint32_t)((n_chunks + 63) / 64)), dim3(64), 0, stream, seg,
+                     (uint32_t)(chunk_bytes / seg_bytes), (uint32_t)n_segs, x_pow_bytes(seg_bytes),
+                     x_pow_bytes(last_seg_len), out_dev, (uint32_t)n_chunks);
+  HIP_TRY(hipGetLastError());
+  return MLF_HIP_OK;
 }
 
 }  // extern "C"

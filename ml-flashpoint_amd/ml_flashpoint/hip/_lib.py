@@ -88,6 +88,7 @@ _SIGNATURES = {
     "mlf_pack_launch": (_INT, [_VP, _VP, _VP]),
     "mlf_unpack_launch": (_INT, [_VP, _VP, _VP]),
     "mlf_crc32c_device": (_INT, [_VP, _U64, _U64, _VP, _U64, _VP]),
+    "mlf_crc32c_device_noalloc": (_INT, [_VP, _U64, _U64, _VP, _U64, _VP]),
     "mlf_crc32c_host": (_U32, [_VP, _U64]),
     "mlf_crc32c_combine": (_U32, [_U32, _U32, _U64]),
     "mlf_crc32c_file": (_INT, [_INT, _U64, _U64, _U64, _VP, _U64, _U32]),
