@@ -1,11 +1,15 @@
-"""The Llama-3-8B shard at its full size (1 164 tensors, 112.4 GB) through the gfx950 saver and loader.
+"""The benchmark's four device-resident configurations at their full sizes through the gfx950 saver and loader:
+the Llama-3-8B shard (1 164 tensors, 112.4 GB), 20 000 small tensors, the Mixtral expert shard (92.9 GB) and 2 000
+non-contiguous views of shared parents.
 
-At this size a second copy of the data cannot be held for a byte-by-byte comparison with the CPU oracle, so the
+At these sizes a second copy of the data cannot be held for a byte-by-byte comparison with the CPU oracle, so the
 file is checked through properties that do not depend on size: every record header and every offset against the
-oracle's closed forms, the payload of a sample of records against the live tensors' bytes, the CRC-32C of every
-chunk of the file (host instruction, and the oracle's table-driven C routine on a sample) against the value the GPU
-computed from the packed image, the whole-file CRC as the combination of the chunk CRCs, and the restored tensors
-against order-sensitive fingerprints of the originals.
+oracle's closed forms (offset of the first record 0, every next one where the previous ends, length = header +
+payload, as the reference's own tests assert at tests/core/test_checkpoint_saver.py:1297-1307,1394-1431), the payload
+of a sample of records against the live tensors' bytes (for a view: the bytes of ``t.contiguous()``), the CRC-32C of
+every chunk of the file (host instruction, and the oracle's table-driven C routine on a sample) against the value the
+GPU computed from the packed image, the whole-file CRC as the combination of the chunk CRCs, and the restored
+tensors against order-sensitive fingerprints of the originals.
 """
 
 import concurrent.futures
@@ -43,7 +47,25 @@ class _LocalManager:
         return threading.Event()
 
 
-def test_llama3_8b_shard_full_size_properties(shm_dir, oracle_c):
+def _build(config):
+    """(state dict, objects to keep alive, expected tensor count, expected payload bytes or None)."""
+    if config == "llama3-8b-shard":
+        return workloads.llama3_8b_shard(DEV), None, 1164, 112_423_657_472
+    if config == "many-small":
+        return workloads.many_small(DEV), None, 20000, None
+    if config == "mixtral-expert-shard":
+        return workloads.mixtral_expert_shard(DEV), None, 32 * (7 + 8 * 3), None
+    sd, parents = workloads.strided_views(DEV)
+    return sd, parents, 2000, None
+
+
+# free HBM (state + image) and tmpfs the configuration needs; the test is skipped where the box has less
+NEEDS = {"llama3-8b-shard": (240e9, 125e9), "many-small": (20e9, 10e9), "mixtral-expert-shard": (200e9, 100e9),
+         "strided-views": (60e9, 25e9)}
+
+
+@pytest.mark.parametrize("config", ["llama3-8b-shard", "many-small", "mixtral-expert-shard", "strided-views"])
+def test_full_size_properties(config, shm_dir, oracle_c):
     from ml_flashpoint.core.checkpoint_loader import DefaultMLFlashpointCheckpointLoader
     from ml_flashpoint.core.checkpoint_saver import DefaultMLFlashpointCheckpointSaver
     from ml_flashpoint.hip import integrity
@@ -52,11 +74,15 @@ def test_llama3_8b_shard_full_size_properties(shm_dir, oracle_c):
     torch.cuda.empty_cache()
     free, _ = torch.cuda.mem_get_info()
     st = os.statvfs(shm_dir)
-    if free < 240e9 or st.f_bavail * st.f_frsize < 125e9:
-        pytest.skip("needs 240 GB of free HBM and 125 GB of tmpfs")
-    sd = workloads.llama3_8b_shard(DEV)
+    need_hbm, need_tmpfs = NEEDS[config]
+    if free < need_hbm or st.f_bavail * st.f_frsize < need_tmpfs:
+        pytest.skip(f"needs {need_hbm / 1e9:.0f} GB of free HBM and {need_tmpfs / 1e9:.0f} GB of tmpfs")
+    sd, keep_alive, n_tensors, want_payload = _build(config)
     payload = workloads.payload_bytes(sd)
-    assert len(sd) == 1164 and payload == 112_423_657_472
+    assert len(sd) == n_tensors and (want_payload is None or payload == want_payload)
+    if config == "strided-views":
+        kinds = {(t.dtype, t.stride(-1) == 1, t.is_contiguous()) for t in sd.values()}
+        assert len({d for d, _, _ in kinds}) == 3 and not all(c for _, _, c in kinds)  # three dtypes, real views
     prints = {k: workloads.fingerprint(v) for k, v in sd.items()}
 
     CheckpointObjectManager._worker_pool = None
@@ -77,24 +103,31 @@ def test_llama3_8b_shard_full_size_properties(shm_dir, oracle_c):
     fd = os.open(obj, os.O_RDONLY)
     try:
         pos = 0
+        header_total = 0
         for index, info in by_offset:
             t = sd[index.fqn]
             header = fmt.header_bytes(fmt.dtype_name(t.dtype), tuple(t.shape))
             assert (info.offset, info.length) == (pos, len(header) + t.numel() * t.element_size()), index.fqn
             assert os.pread(fd, len(header), METADATA_SIZE + pos) == header, index.fqn
             pos += info.length
+            header_total += len(header)
         data_bytes = pos
         assert os.fstat(fd).st_size == METADATA_SIZE + data_bytes
         assert os.pread(fd, METADATA_SIZE, 0) == fmt.metadata_block(data_bytes)
-        assert data_bytes - payload == sum(len(fmt.header_bytes(fmt.dtype_name(t.dtype), tuple(t.shape))) for t in sd.values())
+        assert data_bytes - payload == header_total
 
-        # -- payload of a sample of records (first, last, smallest, one of the largest, a few in between) -------
+        # -- payload of a sample of records (first, last, smallest, largest, a few in between) -------------------
         order = [i.fqn for i, _ in by_offset]
         sample = {order[0], order[-1], order[len(order) // 3], order[len(order) // 2], order[2 * len(order) // 3],
-                  min(sd, key=lambda k: sd[k].numel()), "model.model.layers.17.mlp.down_proj.weight",
-                  "optimizer.exp_avg_sq.model.layers.31.self_attn.k_proj.weight", "optimizer.master.lm_head.weight"}
+                  min(sd, key=lambda k: sd[k].numel()), max(sd, key=lambda k: sd[k].numel())}
+        if config == "llama3-8b-shard":
+            sample |= {"model.model.layers.17.mlp.down_proj.weight", "optimizer.master.lm_head.weight",
+                       "optimizer.exp_avg_sq.model.layers.31.self_attn.k_proj.weight"}
+        if config == "strided-views":  # one of every (dtype, view kind) pair
+            n_parents = len(keep_alive)  # view i: parent i % n_parents (dtype by parent % 3), kind (i // n_parents) % 3
+            sample |= {f"views.{p + n_parents * k}" for p in range(3) for k in range(3)}
         where = {i.fqn: s for i, s in by_offset}
-        for fqn in sample:
+        for fqn in sorted(sample):
             t = sd[fqn]
             nbytes = t.numel() * t.element_size()
             start = METADATA_SIZE + where[fqn].offset + where[fqn].length - nbytes
@@ -102,8 +135,9 @@ def test_llama3_8b_shard_full_size_properties(shm_dir, oracle_c):
             done = 0
             while done < nbytes:
                 done += os.preadv(fd, [memoryview(got)[done:]], start + done)
-            assert np.array_equal(got, t.cpu().reshape(-1).view(torch.uint8).numpy()), fqn
-            del got
+            want = t.contiguous().cpu().reshape(-1).view(torch.uint8).numpy()  # the logical tensor, row-major
+            assert np.array_equal(got, want), fqn
+            del got, want
 
         # -- every chunk's CRC-32C: GPU value (from the packed image) == CRC of the bytes that reached the file ---
         chunk, recorded_bytes, crcs = integrity.read_sidecar(obj)
@@ -124,7 +158,7 @@ def test_llama3_8b_shard_full_size_properties(shm_dir, oracle_c):
                 n = min(CHUNK, data_bytes - k * CHUNK)
                 assert oracle_c.oracle_crc32c(ctypes.cast(base + k * CHUNK, ctypes.c_char_p), n) == int(crcs[k])
             # checksum of checksums: combining the last chunks' CRCs gives the CRC of their concatenation
-            tail = 4
+            tail = min(4, len(crcs))
             whole = int(crcs[-tail])
             for k in range(len(crcs) - tail + 1, len(crcs)):
                 whole = P.crc32c_combine(whole, int(crcs[k]), min(CHUNK, data_bytes - k * CHUNK))
@@ -138,12 +172,15 @@ def test_llama3_8b_shard_full_size_properties(shm_dir, oracle_c):
 
     # -- restore into zeroed tensors: bit patterns equal the originals' ------------------------------------------
     for v in sd.values():
-        v.zero_()
+        v.zero_() if v.is_contiguous() else v.fill_(0)
     loader = DefaultMLFlashpointCheckpointLoader(manager, None)
     dcp.load(sd, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), no_dist=True)
     torch.cuda.synchronize()
     wrong = [k for k, v in sd.items() if workloads.fingerprint(v) != prints[k]]
     assert not wrong, wrong[:5]
     assert loader.last_load_stats["device_items"] == len(sd)
-    del sd
+    loader_engine = getattr(loader, "_engine", None)
+    if loader_engine is not None:
+        loader_engine.destroy()
+    del sd, keep_alive
     torch.cuda.empty_cache()
