@@ -66,7 +66,12 @@ typedef struct mlf_plan_opts {
   uint32_t grid_x_log2;      /* 0 = default; k > 0: rows of 2^(k-1) workgroups in the copy kernel's grid (a row may
                                 not exceed 2^32 - 1 threads),
                                 the rest goes to gridDim.y of the same launch.  Small values are for tests.     */
-  uint32_t reserved;         /* 0 */
+  uint32_t crc_chunk_kib;    /* 0 = no checksums.  k > 0 (a multiple of 64): every pack / unpack launch of the plan also
+                                yields the CRC-32C of every k KiB chunk of the image (the last may be short), read with
+                                mlf_plan_crc_values().  Where a contiguous item covers whole 64 KiB pieces of the image, the
+                                kernel that copies them also folds their remainders, so those bytes are not read a second
+                                time; the rest of the image (record headers, item edges, strided and transposed items, a
+                                last partial chunk) is checksummed from the image after it is complete.                   */
 } mlf_plan_opts;
 
 typedef struct mlf_plan_info {
@@ -81,6 +86,8 @@ typedef struct mlf_plan_info {
   uint64_t image_bytes;
   uint64_t table_bytes;       /* device memory held by the plan's tables + blob                                */
   uint64_t n_small_items;     /* pieces of at most 1 KiB that are copied one per wavefront                     */
+  uint64_t fused_crc_bytes;   /* image bytes whose checksum remainders come out of the copy itself (crc_chunk_kib > 0) */
+  uint64_t crc_chunks;        /* values mlf_plan_crc_values() returns                                                   */
 } mlf_plan_info;
 
 typedef struct mlf_plan mlf_plan;
@@ -121,6 +128,13 @@ int mlf_pack_launch(const mlf_plan* plan, void* image_dev, void* stream);
 /* Restore direction: image -> tensors.  Asynchronous on `stream`.  Replaces frombuffer + narrow + copy_
  * (checkpoint_loader.py:206-219,331-336). */
 int mlf_unpack_launch(const mlf_plan* plan, const void* image_dev, void* stream);
+
+/* Per-chunk CRC-32C values of the image that the plan's most recent mlf_pack_launch / mlf_unpack_launch moved (plans
+ * created with crc_chunk_kib > 0): waits for that launch's checksum work and copies ceil(image_bytes / chunk) values
+ * to `out_host`.  Same values as mlf_crc32c_device over the image.  On save they go into the object's sidecar; on
+ * restore the caller compares them with the sidecar's.  Call it before the plan is launched again.  No reference
+ * counterpart (the reference has no checksum). */
+int mlf_plan_crc_values(mlf_plan* plan, uint32_t* out_host, uint64_t n_out);
 
 /* CRC-32C (Castagnoli, reflected, init/xorout 0xFFFFFFFF as in RFC 3720) of consecutive `chunk_bytes`
  * pieces of a device buffer; the last chunk may be short.  Writes ceil(nbytes/chunk_bytes) values to

@@ -24,31 +24,8 @@ struct CrcConsts {
 
 }  // namespace mlf
 
-using namespace mlf;
+namespace mlf {
 
-namespace {
-
-// ---------------------------------------------------------------------------------------------------------
-// CRC-32C
-// ---------------------------------------------------------------------------------------------------------
-constexpr uint32_t kPolyReflected = 0x82F63B78u;
-constexpr uint32_t kCrcSegBytes = 64 * 1024;  // smallest segment (bytes per wavefront); chunks are multiples of it
-constexpr uint32_t kCrcMaxSegBytes = 512 * 1024;
-constexpr int kCrcTableCopies = 16;           // copies of the lookup tables in LDS, interleaved over the banks
-constexpr int kCrcThreads = 512;
-constexpr uint32_t kCrcRowBytes = 1024;       // one coalesced wavefront row: 64 lanes x 16 bytes
-
-// a(x) * b(x) mod P in the reflected representation (bit 31 is x^0).
-__host__ __device__ inline uint32_t gf_mul(uint32_t a, uint32_t b) {
-  uint32_t p = 0;
-  for (int i = 31; i >= 0; --i) {
-    p ^= ((a >> i) & 1u) ? b : 0u;
-    b = (b >> 1) ^ ((b & 1u) ? kPolyReflected : 0u);
-  }
-  return p;
-}
-
-// x^(8*nbytes) mod P.
 uint32_t x_pow_bytes(uint64_t nbytes) {
   uint32_t result = 0x80000000u;      // x^0
   uint32_t sq = gf_mul(0x40000000u, 0x40000000u);  // x^2
@@ -61,6 +38,22 @@ uint32_t x_pow_bytes(uint64_t nbytes) {
   }
   return result;
 }
+
+}  // namespace mlf
+
+using namespace mlf;
+
+namespace {
+
+// ---------------------------------------------------------------------------------------------------------
+// CRC-32C
+// ---------------------------------------------------------------------------------------------------------
+constexpr uint32_t kPolyReflected = kCrcPolyReflected;
+constexpr uint32_t kCrcSegBytes = 64 * 1024;  // smallest segment (bytes per wavefront); chunks are multiples of it
+constexpr uint32_t kCrcMaxSegBytes = 512 * 1024;
+constexpr int kCrcTableCopies = 16;           // copies of the lookup tables in LDS, interleaved over the banks
+constexpr int kCrcThreads = 512;
+constexpr uint32_t kCrcRowBytes = 1024;       // one coalesced wavefront row: 64 lanes x 16 bytes
 
 __device__ __forceinline__ uint32_t crc_byte_step(uint32_t s, uint8_t b) {
   s ^= b;
@@ -78,7 +71,8 @@ template <int R>
 __global__ void __launch_bounds__(kCrcThreads) mlf_crc_segments_kernel(const char* __restrict__ data, uint64_t nbytes,
                                                                        const CrcConsts* __restrict__ consts,
                                                                        uint32_t* __restrict__ seg_crc, uint32_t n_segs,
-                                                                       uint32_t seg_bytes) {
+                                                                       uint32_t seg_bytes,
+                                                                       const uint32_t* __restrict__ seg_list) {
   __shared__ uint32_t tab[4 * 256 * R];
   for (uint32_t i = threadIdx.x; i < 1024; i += blockDim.x) {
     const uint32_t v = consts->row_tab[i >> 8][i & 255];
@@ -86,8 +80,10 @@ __global__ void __launch_bounds__(kCrcThreads) mlf_crc_segments_kernel(const cha
     for (int c = 0; c < R; ++c) tab[i * R + c] = v;
   }
   __syncthreads();
-  const uint32_t seg = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  if (seg >= n_segs) return;
+  // wavefront k takes segment k, or, with a list, segment seg_list[k] (and reports under that number)
+  const uint32_t slot = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (slot >= n_segs) return;
+  const uint32_t seg = seg_list ? seg_list[slot] : slot;
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t* my = tab + (lane & (R - 1));
   const uint64_t seg_off = (uint64_t)seg * seg_bytes;
@@ -158,6 +154,46 @@ __global__ void mlf_crc_chunks_kernel(const uint32_t* __restrict__ seg_crc, uint
 }
 
 // ---------------------------------------------------------------------------------------------------------
+// chaining the remainders of a plan whose copy kernels fold them as they copy (struct FusedCrc)
+// ---------------------------------------------------------------------------------------------------------
+constexpr uint32_t kCellBytes = 4096;
+constexpr uint32_t kEntryBytes = 65536;
+
+// One thread per group: the remainder of the group's bytes from (a) the values of its fused-copy workgroups -
+// workgroup w holds cells w, w + G, ..., so consecutive values are one cell apart - and (b) the values of its entries
+// that were checksummed from the image.  Both are taken relative to the group's end (the image's end for the last,
+// possibly partial, group).
+__global__ void mlf_crc_groups_kernel(const uint64_t* __restrict__ ent, const uint32_t* __restrict__ ent_val,
+                                      const uint32_t* __restrict__ fast_val, uint32_t G, uint32_t ents_per_group,
+                                      uint64_t fused_groups, uint64_t n_ent, uint64_t n_groups, uint32_t x_cell,
+                                      uint32_t x_entry, uint32_t x_last_entry, uint32_t* __restrict__ group_val) {
+  const uint64_t g = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (g >= n_groups) return;
+  uint32_t fast = 0;
+  if (g < fused_groups)
+    for (uint32_t w = 0; w < G; ++w) fast = gf_mul(x_cell, fast) ^ fast_val[g * G + w];
+  uint32_t slow = 0;
+  const uint64_t e0 = g * ents_per_group;
+  const uint64_t e1 = e0 + ents_per_group < n_ent ? e0 + ents_per_group : n_ent;
+  for (uint64_t e = e0; e < e1; ++e)
+    slow = gf_mul(e == n_ent - 1 ? x_last_entry : x_entry, slow) ^ (ent[e] ? 0u : ent_val[e]);
+  group_val[g] = fast ^ slow;
+}
+
+// One thread per chunk: chain the group remainders, apply init and final xor.
+__global__ void mlf_crc_group_chunks_kernel(const uint32_t* __restrict__ group_val, uint32_t groups_per_chunk,
+                                            uint64_t n_groups, uint32_t x_group, uint32_t x_last_group,
+                                            uint32_t* __restrict__ out, uint32_t n_chunks) {
+  const uint32_t c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= n_chunks) return;
+  uint32_t s = 0xFFFFFFFFu;
+  const uint64_t first = (uint64_t)c * groups_per_chunk;
+  const uint64_t last = first + groups_per_chunk < n_groups ? first + groups_per_chunk : n_groups;
+  for (uint64_t g = first; g < last; ++g) s = gf_mul(g == n_groups - 1 ? x_last_group : x_group, s) ^ group_val[g];
+  out[c] = s ^ 0xFFFFFFFFu;
+}
+
+// ---------------------------------------------------------------------------------------------------------
 // scratch of the allocation-free entry point (mlf_crc32c_device_noalloc)
 // ---------------------------------------------------------------------------------------------------------
 // A fixed array in every device's copy of this code object: the lookup constants, then one value per segment.
@@ -220,6 +256,81 @@ void crc_init_host() {
 namespace mlf {
 
 
+void crc_fused_destroy(FusedCrc* f) {
+  (void)hipFree(f->d_ent);
+  (void)hipFree(f->d_slow_list);
+  (void)hipFree(f->d_ent_val);
+  (void)hipFree(f->d_fast_val);
+  (void)hipFree(f->d_group_val);
+  (void)hipFree(f->d_row_tab);
+  (void)hipFree(f->d_lane_w);
+  (void)hipFree(f->d_consts);
+  (void)hipFree(f->d_out);
+  if (f->h_out) (void)hipHostFree(f->h_out);
+  if (f->done) (void)hipEventDestroy(f->done);
+  *f = FusedCrc();
+}
+
+int crc_fused_setup(FusedCrc* f) {
+  std::call_once(g_crc_once, crc_init_host);
+  const uint64_t group_bytes = (uint64_t)f->rows * f->wgs_per_group * kCellBytes;
+  f->n_groups = (f->image_bytes + group_bytes - 1) / group_bytes;
+  f->n_chunks = (f->image_bytes + f->chunk_bytes - 1) / f->chunk_bytes;
+  // state advanced by one row of the fused kernel's walk (its cells are wgs_per_group cells apart), sliced by byte
+  std::vector<uint32_t> row_tab(1024);
+  const uint32_t x_row = x_pow_bytes((uint64_t)kCellBytes * f->wgs_per_group);
+  for (int b = 0; b < 4; ++b)
+    for (uint32_t v = 0; v < 256; ++v) row_tab[b * 256 + v] = gf_mul(x_row, v << (8 * b));
+  // dword j of lane t's vector lies 4096 - 16 t - 4 j bytes in front of its cell's end (its own four bytes included)
+  std::vector<uint32_t> lane_w(1024);
+  for (uint32_t t = 0; t < 256; ++t)
+    for (uint32_t j = 0; j < 4; ++j) lane_w[t * 4 + j] = x_pow_bytes(kCellBytes - 16 * t - 4 * j);
+  const uint64_t n_fast = f->fused_groups * f->wgs_per_group;
+  HIP_TRY(hipMalloc(reinterpret_cast<void**>(&f->d_ent_val), std::max<uint64_t>(f->n_ent, 1) * sizeof(uint32_t)));
+  HIP_TRY(hipMemset(f->d_ent_val, 0, std::max<uint64_t>(f->n_ent, 1) * sizeof(uint32_t)));
+  HIP_TRY(hipMalloc(reinterpret_cast<void**>(&f->d_fast_val), std::max<uint64_t>(n_fast, 1) * sizeof(uint32_t)));
+  HIP_TRY(hipMalloc(reinterpret_cast<void**>(&f->d_group_val), std::max<uint64_t>(f->n_groups, 1) * sizeof(uint32_t)));
+  HIP_TRY(hipMalloc(reinterpret_cast<void**>(&f->d_row_tab), 4096));
+  HIP_TRY(hipMemcpy(f->d_row_tab, row_tab.data(), 4096, hipMemcpyHostToDevice));
+  HIP_TRY(hipMalloc(reinterpret_cast<void**>(&f->d_lane_w), 4096));
+  HIP_TRY(hipMemcpy(f->d_lane_w, lane_w.data(), 4096, hipMemcpyHostToDevice));
+  HIP_TRY(hipMalloc(reinterpret_cast<void**>(&f->d_consts), sizeof(CrcConsts)));
+  HIP_TRY(hipMemcpy(f->d_consts, &g_crc_host, sizeof(CrcConsts), hipMemcpyHostToDevice));
+  HIP_TRY(hipMalloc(reinterpret_cast<void**>(&f->d_out), std::max<uint64_t>(f->n_chunks, 1) * sizeof(uint32_t)));
+  HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&f->h_out), std::max<uint64_t>(f->n_chunks, 1) * sizeof(uint32_t), hipHostMallocDefault));
+  HIP_TRY(hipEventCreateWithFlags(&f->done, hipEventDisableTiming));
+  return MLF_HIP_OK;
+}
+
+int crc_fused_finish(FusedCrc* f, const void* image, hipStream_t stream) {
+  if (f->n_slow) {
+    // entries the copy kernels did not fold: one wavefront each, from the image that is complete at this point of
+    // the stream; values land in ent_val under the entry's number
+    const uint32_t waves_per_block = kCrcThreads / 64;
+    const uint32_t grid = (uint32_t)((f->n_slow + waves_per_block - 1) / waves_per_block);
+    hipLaunchKernelGGL(mlf_crc_segments_kernel<kCrcTableCopies>, dim3(grid), dim3(kCrcThreads), 0, stream,
+                       static_cast<const char*>(image), f->image_bytes, f->d_consts, f->d_ent_val, (uint32_t)f->n_slow,
+                       kEntryBytes, f->d_slow_list);
+    HIP_TRY(hipGetLastError());
+  }
+  const uint64_t group_bytes = (uint64_t)f->rows * f->wgs_per_group * kCellBytes;
+  const uint32_t ents_per_group = (uint32_t)(group_bytes / kEntryBytes);
+  const uint64_t last_entry_len = f->image_bytes - (f->n_ent - 1) * kEntryBytes;
+  hipLaunchKernelGGL(mlf_crc_groups_kernel, dim3((uint32_t)((f->n_groups + 63) / 64)), dim3(64), 0, stream, f->d_ent,
+                     f->d_ent_val, f->d_fast_val, f->wgs_per_group, ents_per_group, f->fused_groups, f->n_ent, f->n_groups,
+                     x_pow_bytes(kCellBytes), x_pow_bytes(kEntryBytes), x_pow_bytes(last_entry_len), f->d_group_val);
+  HIP_TRY(hipGetLastError());
+  const uint64_t last_group_len = f->image_bytes - (f->n_groups - 1) * group_bytes;
+  hipLaunchKernelGGL(mlf_crc_group_chunks_kernel, dim3((uint32_t)((f->n_chunks + 63) / 64)), dim3(64), 0, stream,
+                     f->d_group_val, (uint32_t)(f->chunk_bytes / group_bytes), f->n_groups, x_pow_bytes(group_bytes),
+                     x_pow_bytes(last_group_len), f->d_out, (uint32_t)f->n_chunks);
+  HIP_TRY(hipGetLastError());
+  HIP_TRY(hipMemcpyAsync(f->h_out, f->d_out, f->n_chunks * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+  HIP_TRY(hipEventRecord(f->done, stream));
+  f->launched = true;
+  return MLF_HIP_OK;
+}
+
 void crc_release(CrcJob* job) {
   (void)hipFree(job->d_consts);
   (void)hipFree(job->d_seg);
@@ -261,13 +372,13 @@ int crc_enqueue(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint
     // kernels this pass runs beside
     const uint32_t grid = (uint32_t)((n_segs + 3) / 4);
     hipLaunchKernelGGL(mlf_crc_segments_kernel<1>, dim3(grid), dim3(256), 0, stream, static_cast<const char*>(dev_ptr),
-                       nbytes, job->d_consts, job->d_seg, (uint32_t)n_segs, (uint32_t)seg_bytes);
+                       nbytes, job->d_consts, job->d_seg, (uint32_t)n_segs, (uint32_t)seg_bytes, nullptr);
   } else {
     const uint32_t waves_per_block = kCrcThreads / 64;
     const uint32_t grid = (uint32_t)((n_segs + waves_per_block - 1) / waves_per_block);
     hipLaunchKernelGGL(mlf_crc_segments_kernel<kCrcTableCopies>, dim3(grid), dim3(kCrcThreads), 0, stream,
                        static_cast<const char*>(dev_ptr), nbytes, job->d_consts, job->d_seg, (uint32_t)n_segs,
-                       (uint32_t)seg_bytes);
+                       (uint32_t)seg_bytes, nullptr);
   }
   CRC_TRY(hipGetLastError());
   const uint64_t last_seg_len = nbytes - (n_segs - 1) * seg_bytes;
@@ -421,7 +532,8 @@ int mlf_crc32c_device_noalloc(const void* dev_ptr, uint64_t nbytes, uint64_t chu
   const uint32_t waves_per_block = kCrcThreads / 64;
   const uint32_t grid = (uint32_t)((n_segs + waves_per_block - 1) / waves_per_block);
   hipLaunchKernelGGL(mlf_crc_segments_kernel<kCrcTableCopies>, dim3(grid), dim3(kCrcThreads), 0, stream,
-                     static_cast<const char*>(dev_ptr), nbytes, consts, seg, (uint32_t)n_segs, (uint32_t)seg_bytes);
+                     static_cast<const char*>(dev_ptr), nbytes, consts, seg, (uint32_t)n_segs, (uint32_t)seg_bytes,
+                     nullptr);
   HIP_TRY(hipGetLastError());
   const uint64_t last_seg_len = nbytes - (n_segs - 1) * seg_bytes;
   hipLaunchKernelGGL(mlf_crc_chunks_kernel, dim3((uint32_t)((n_chunks + 63) / 64)), dim3(64), 0, stream, seg,

@@ -67,6 +67,55 @@ inline int full_pread(int fd, char* buf, size_t len, uint64_t off) {
   return 0;
 }
 
+// ---- CRC-32C arithmetic shared by the checksum code and the copy kernels that fold remainders as they copy ----
+constexpr uint32_t kCrcPolyReflected = 0x82F63B78u;
+
+// a(x) * b(x) mod P in the reflected representation (bit 31 is x^0).
+__host__ __device__ inline uint32_t gf_mul(uint32_t a, uint32_t b) {
+  uint32_t p = 0;
+  for (int i = 31; i >= 0; --i) {
+    p ^= ((a >> i) & 1u) ? b : 0u;
+    b = (b >> 1) ^ ((b & 1u) ? kCrcPolyReflected : 0u);
+  }
+  return p;
+}
+
+// x^(8*nbytes) mod P.
+uint32_t x_pow_bytes(uint64_t nbytes);
+
+// Checksum state of a plan whose copy kernels fold remainders (plan option crc_chunk_kib).  The image is cut into
+// cells of 4 KiB, entries of 16 cells (64 KiB) and groups of rows * wgs_per_group cells; a chunk is a whole number
+// of groups.  `fast_val` holds one remainder per workgroup of the fused copy kernel (groups [0, fused_groups)),
+// `ent_val` one per entry that the copy kernels do not cover (listed in `slow_list`, taken from the finished image).
+struct CrcConsts;
+struct FusedCrc {
+  uint64_t image_bytes = 0, chunk_bytes = 0;
+  uint32_t rows = 16;           // cells per workgroup of the fused copy kernel
+  uint32_t wgs_per_group = 0;   // G: a workgroup's cells are G cells apart
+  uint64_t fused_groups = 0;
+  uint64_t n_ent = 0, n_groups = 0, n_chunks = 0, n_slow = 0;
+  uint64_t* d_ent = nullptr;      // per entry: tensor-side address of its first byte, 0 = not served by the fused kernel
+  uint32_t* d_slow_list = nullptr;
+  uint32_t* d_ent_val = nullptr;  // zero except at listed entries
+  uint32_t* d_fast_val = nullptr;
+  uint32_t* d_group_val = nullptr;
+  uint32_t* d_row_tab = nullptr;  // [4][256]: state advanced by wgs_per_group cells, sliced by state byte
+  u32x4* d_lane_w = nullptr;      // [256]: weight of each lane's four dwords within a cell
+  CrcConsts* d_consts = nullptr;  // lookup constants of the segment kernel
+  uint32_t* d_out = nullptr;
+  uint32_t* h_out = nullptr;      // pinned
+  hipEvent_t done = nullptr;
+  bool launched = false;
+};
+
+// Allocates and fills everything in `f` but d_ent / d_slow_list (the plan builds those); image_bytes, chunk_bytes,
+// wgs_per_group, fused_groups, n_ent must be set.  crc_fused_destroy frees all of it (d_ent and d_slow_list too).
+int crc_fused_setup(FusedCrc* f);
+void crc_fused_destroy(FusedCrc* f);
+// After the copy kernels of a launch are enqueued on `stream`: remainders of the listed entries from the image, the
+// chain over groups and chunks, the copy of the chunk values to the pinned array, and the event behind it.
+int crc_fused_finish(FusedCrc* f, const void* image, hipStream_t stream);
+
 // A CRC pass in flight: scratch on the device, results in a pinned host array, all ordered on `stream`.
 struct CrcConsts;
 struct CrcJob {

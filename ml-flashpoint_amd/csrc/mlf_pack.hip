@@ -608,6 +608,145 @@ __global__ void __launch_bounds__(kTransThreads) mlf_transpose_kernel(const Tran
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// fused copy + CRC-32C kernel
+// ---------------------------------------------------------------------------------------------------------
+// For plans that also checksum the image (plan option crc_chunk_kib).  The image is seen as cells of 4 KiB; an
+// "entry" is 16 cells (64 KiB), and the plan's entry table gives, for every entry that lies inside one contiguous
+// item, the tensor-side address of its first byte.  A workgroup moves kFusedRows cells that are G cells apart (G
+// workgroups form a group of kFusedRows * G consecutive cells, a chunk is a whole number of groups): at any moment
+// the workgroups of a group are working on G consecutive cells, which keeps the traffic as sequential as with one
+// tile per workgroup, while every lane sees kFusedRows vectors at a fixed distance and can carry four Horner
+// accumulators from one to the next through a byte-sliced table in LDS (advance by G cells, then add the new
+// vector).  At the end the accumulators are weighted by the lane's position in the cell and summed over the
+// workgroup: the remainder, relative to the end of the workgroup's last cell, of its cells laid G apart - one
+// value per workgroup, chained by mlf_crc_groups_kernel.  Cells of entries without an address (record headers, item
+// edges, strided items ...) are skipped here; the other kernels move them and their remainders are taken from the
+// finished image.  The checksum arithmetic hides behind the memory traffic (measured on 16 GiB: copy alone in this
+// order 4.7-5.6 TB/s, with the checksum 5.7-5.8; one 4 KiB tile per workgroup without checksum 6.2).
+constexpr uint32_t kFusedRows = 16;   // cells per workgroup; FusedCrc::rows
+constexpr uint32_t kFusedAhead = 4;   // rows requested before the first is used
+constexpr uint32_t kFusedMaxGroupWgs = 512;
+constexpr uint32_t kCellBytes = 4096;
+constexpr uint32_t kEntryBytes = 65536;
+constexpr uint32_t kCellsPerEntryLog2 = 4;
+
+template <bool PACK>
+__global__ void __launch_bounds__(256) mlf_fused_crc_kernel(const uint64_t* __restrict__ ent, char* __restrict__ image,
+                                                            uint32_t G, const uint32_t* __restrict__ row_tab,
+                                                            const u32x4* __restrict__ lane_w,
+                                                            uint32_t* __restrict__ fast_val) {
+  __shared__ uint32_t tab[1024];
+  __shared__ uint32_t part[4];
+  const uint32_t tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t group = blockIdx.x / G;
+  uint32_t w = blockIdx.x - group * G;
+  if ((G & 511u) == 0) {
+    // workgroups reach the eight XCDs round-robin: within every 512 of them XCD x takes 64 consecutive cells of a
+    // row, so that a source line that straddles a cell cut is served by one L2
+    const uint32_t lo = w & 511u;
+    w = (w & ~511u) + (lo & 7u) * 64u + (lo >> 3);
+  }
+  const uint64_t cell0 = (uint64_t)group * kFusedRows * G + w;
+  uint32_t* out = fast_val + (uint64_t)group * G + w;
+  // tensor-side address of each of this workgroup's cells, 0 = not ours (uniform over the workgroup: scalar loads)
+  uint64_t base[kFusedRows];
+  bool any = false;
+#pragma unroll
+  for (uint32_t k = 0; k < kFusedRows; ++k) {
+    const uint64_t cell = cell0 + (uint64_t)k * G;
+    const uint64_t e = ent[cell >> kCellsPerEntryLog2];
+    base[k] = e ? e + ((cell & ((1u << kCellsPerEntryLog2) - 1u)) << 12) : 0;
+    any |= e != 0;
+  }
+  if (!any) {
+    if (tid == 0) *out = 0u;
+    return;
+  }
+  u32x4 raw[kFusedAhead], far[kFusedAhead];
+  // PACK: the tensor side is read - directly where it is dword-aligned, else as aligned 16-byte granules that are
+  // realigned across lanes (lane 63 of a wavefront also fetches the granule its neighbour in the next wavefront
+  // holds).  UNPACK: the image cell is read as it lies.
+#define MLF_FUSED_REQUEST(k)                                                                                        \
+  if (base[k]) {                                                                                                    \
+    if (PACK) {                                                                                                     \
+      const uint32_t delta = (uint32_t)base[k] & 15u;                                                               \
+      if ((delta & 3u) == 0u) {                                                                                     \
+        raw[(k) % kFusedAhead] = __builtin_nontemporal_load(gload<u32x4_u>(reinterpret_cast<const char*>(base[k]) + tid * 16u)); \
+      } else {                                                                                                      \
+        const char* a = reinterpret_cast<const char*>(base[k] - delta);                                             \
+        raw[(k) % kFusedAhead] = __builtin_nontemporal_load(gload<u32x4>(a + tid * 16u));                           \
+        if (lane == 63u) far[(k) % kFusedAhead] = __builtin_nontemporal_load(gload<u32x4>(a + (tid + 1u) * 16u));   \
+      }                                                                                                             \
+    } else {                                                                                                        \
+      raw[(k) % kFusedAhead] = __builtin_nontemporal_load(gload<u32x4>(image + ((cell0 + (uint64_t)(k) * G) << 12) + tid * 16u)); \
+    }                                                                                                               \
+  }
+#pragma unroll
+  for (uint32_t k = 0; k < kFusedAhead; ++k) {
+    MLF_FUSED_REQUEST(k)
+  }
+#pragma unroll
+  for (uint32_t k = 0; k < 4; ++k) tab[tid + 256u * k] = row_tab[tid + 256u * k];
+  __syncthreads();
+#define MLF_FUSED_ADV(a) \
+  (tab[(a) & 255u] ^ tab[256u + (((a) >> 8) & 255u)] ^ tab[512u + (((a) >> 16) & 255u)] ^ tab[768u + ((a) >> 24)])
+  uint32_t a0 = 0, a1 = 0, a2 = 0, a3 = 0;
+#pragma unroll
+  for (uint32_t k = 0; k < kFusedRows; ++k) {
+    u32x4 v = raw[k % kFusedAhead];  // becomes the cell's vector as it lies in the image
+    if (PACK && base[k]) {
+      const uint32_t delta = (uint32_t)base[k] & 15u;
+      if ((delta & 3u) != 0u) {
+        const u32x4 lo = v;
+        u32x4 hi;
+        hi.x = (uint32_t)__shfl_down((int)lo.x, 1);
+        hi.y = (uint32_t)__shfl_down((int)lo.y, 1);
+        hi.z = (uint32_t)__shfl_down((int)lo.z, 1);
+        hi.w = (uint32_t)__shfl_down((int)lo.w, 1);
+        if (lane == 63u) hi = far[k % kFusedAhead];
+        const uint32_t q = delta >> 2, r = delta & 3u;
+        uint32_t w0, w1, w2, w3, w4;
+        switch (q) {
+          case 0: w0 = lo.x; w1 = lo.y; w2 = lo.z; w3 = lo.w; w4 = hi.x; break;
+          case 1: w0 = lo.y; w1 = lo.z; w2 = lo.w; w3 = hi.x; w4 = hi.y; break;
+          case 2: w0 = lo.z; w1 = lo.w; w2 = hi.x; w3 = hi.y; w4 = hi.z; break;
+          default: w0 = lo.w; w1 = hi.x; w2 = hi.y; w3 = hi.z; w4 = hi.w; break;
+        }
+        v.x = __builtin_amdgcn_alignbyte(w1, w0, r);
+        v.y = __builtin_amdgcn_alignbyte(w2, w1, r);
+        v.z = __builtin_amdgcn_alignbyte(w3, w2, r);
+        v.w = __builtin_amdgcn_alignbyte(w4, w3, r);
+      }
+    }
+    if (k + kFusedAhead < kFusedRows) {  // the slot just read is free again
+      MLF_FUSED_REQUEST(k + kFusedAhead)
+    }
+    if (base[k]) {
+      if (PACK) __builtin_nontemporal_store(v, gstore<u32x4>(image + ((cell0 + (uint64_t)k * G) << 12) + tid * 16u));
+      else __builtin_nontemporal_store(v, gstore<u32x4_u>(reinterpret_cast<char*>(base[k]) + tid * 16u));
+      a0 = MLF_FUSED_ADV(a0) ^ v.x;
+      a1 = MLF_FUSED_ADV(a1) ^ v.y;
+      a2 = MLF_FUSED_ADV(a2) ^ v.z;
+      a3 = MLF_FUSED_ADV(a3) ^ v.w;
+    } else {  // somebody else's cell: it contributes zeros at this position
+      a0 = MLF_FUSED_ADV(a0);
+      a1 = MLF_FUSED_ADV(a1);
+      a2 = MLF_FUSED_ADV(a2);
+      a3 = MLF_FUSED_ADV(a3);
+    }
+  }
+#undef MLF_FUSED_ADV
+#undef MLF_FUSED_REQUEST
+  const u32x4 wts = lane_w[tid];
+  uint32_t acc = gf_mul(a0, wts.x) ^ gf_mul(a1, wts.y) ^ gf_mul(a2, wts.z) ^ gf_mul(a3, wts.w);
+#pragma unroll
+  for (int s = 1; s < 64; s <<= 1) acc ^= (uint32_t)__shfl_xor((int)acc, s, 64);
+  if (lane == 0u) part[tid >> 6] = acc;
+  __syncthreads();
+  if (tid == 0) *out = part[0] ^ part[1] ^ part[2] ^ part[3];
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------------------------------------
@@ -639,6 +778,8 @@ struct mlf_plan {
   uint32_t flat_first[kFlatClasses] = {0, 0, 0};  // first workgroup of each span class in that launch
   uint32_t flat_total = 0;
   mlf_plan_info info{};
+  bool has_crc = false;      // launches also fold the image's CRC-32C (plan option crc_chunk_kib)
+  mutable FusedCrc crc;      // its tables and values; the values are rewritten by every launch
   mlf_plan() = default;
   mlf_plan(const mlf_plan&) = delete;
   mlf_plan& operator=(const mlf_plan&) = delete;
@@ -651,6 +792,7 @@ struct mlf_plan {
     (void)hipFree(d_blob);
     if (h_blob) (void)hipHostFree(h_blob);
     if (blob_copied) (void)hipEventDestroy(blob_copied);
+    crc_fused_destroy(&crc);
   }
 };
 
@@ -693,6 +835,34 @@ void cut_spans(SpanTables& out, uint64_t tensor_addr, uint64_t image_off, uint64
     done += len;
   }
 }
+
+// One contiguous run of an item.  With checksums, the whole 64 KiB entries of the image that the run covers (below
+// `fused_entries`) go to the fused copy + CRC kernel - the entry table gets their tensor-side addresses - and only
+// the edges go to the span tables.
+struct FlatSink {
+  SpanTables* tables;
+  std::vector<uint64_t>* ent;  // null: no checksums
+  uint64_t fused_entries;
+  uint64_t fused_bytes;
+  uint32_t tile;
+  bool align_to_tensor;
+  uint32_t cut_mask;
+  void add(uint64_t tensor_addr, uint64_t image_off, uint64_t n) {
+    if (ent) {
+      const uint64_t e0 = (image_off + kEntryBytes - 1) / kEntryBytes;
+      const uint64_t e1 = std::min<uint64_t>((image_off + n) / kEntryBytes, fused_entries);
+      if (e1 > e0) {
+        for (uint64_t e = e0; e < e1; ++e) (*ent)[e] = tensor_addr + (e * kEntryBytes - image_off);
+        fused_bytes += (e1 - e0) * kEntryBytes;
+        const uint64_t head = e0 * kEntryBytes - image_off, tail_at = e1 * kEntryBytes - image_off;
+        if (head) cut_spans(*tables, tensor_addr, image_off, head, tile, align_to_tensor, cut_mask);
+        if (tail_at < n) cut_spans(*tables, tensor_addr + tail_at, image_off + tail_at, n - tail_at, tile, align_to_tensor, cut_mask);
+        return;
+      }
+    }
+    cut_spans(*tables, tensor_addr, image_off, n, tile, align_to_tensor, cut_mask);
+  }
+};
 
 struct Collapsed {
   int ndim;
@@ -783,6 +953,28 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
   if (plan->grid_x_log2 > widest) return fail(MLF_HIP_BAD_ARG, "grid_x_log2: a grid row of that many workgroups exceeds 2^32 threads");
   if (plan->unroll != 1 && plan->unroll != 2 && plan->unroll != 4 && plan->unroll != 8)
     return fail(MLF_HIP_BAD_ARG, "unroll must be 1, 2, 4 or 8");
+  std::vector<uint64_t> ent;
+  uint64_t fused_entries = 0;
+  if (opts && opts->crc_chunk_kib && image_bytes) {
+    if (opts->crc_chunk_kib % 64) return fail(MLF_HIP_BAD_ARG, "crc_chunk_kib must be a multiple of 64");
+    FusedCrc& f = plan->crc;
+    f.image_bytes = image_bytes;
+    f.chunk_bytes = (uint64_t)opts->crc_chunk_kib << 10;
+    f.rows = kFusedRows;
+    // a chunk is a whole number of groups of rows * G cells: G = the largest divisor of chunk cells / rows up to 512
+    const uint64_t m = f.chunk_bytes / kCellBytes / kFusedRows;
+    uint32_t G = 1;
+    for (uint32_t d = 1; d <= kFusedMaxGroupWgs && d <= m; ++d)
+      if (m % d == 0) G = d;
+    f.wgs_per_group = G;
+    // whole groups only, and no more workgroups than one grid row holds
+    f.fused_groups = std::min<uint64_t>(image_bytes / kCellBytes / ((uint64_t)kFusedRows * G), ((1u << 24) - 1) / G);
+    f.n_ent = (image_bytes + kEntryBytes - 1) / kEntryBytes;
+    if (f.n_ent >= 0xFFFFFFF0ull) return fail(MLF_HIP_BAD_ARG, "image too large for per-chunk checksums");
+    fused_entries = f.fused_groups * kFusedRows * G / (kEntryBytes / kCellBytes);
+    ent.assign(f.n_ent, 0);
+    plan->has_crc = true;
+  }
   plan->blob_size = blob_bytes;
   if (blob_bytes) {
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&plan->d_blob), blob_bytes));
@@ -791,6 +983,7 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
   const uint64_t blob_base = reinterpret_cast<uint64_t>(plan->d_blob);
 
   SpanTables tiles;
+  FlatSink flat{&tiles, plan->has_crc ? &ent : nullptr, fused_entries, 0, tile, align_to_tensor, plan->cut_mask};
   std::vector<StridedDesc> descs;
   std::vector<StridedWork> work;
   std::vector<TransDesc> tdescs;
@@ -811,7 +1004,7 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
         rc = fail(MLF_HIP_BAD_ARG, "blob item " + std::to_string(k) + " lies outside the host blob");
         break;
       }
-      cut_spans(tiles, blob_base + it.ptr, it.image_off, it.nbytes, tile, align_to_tensor, plan->cut_mask);
+      flat.add(blob_base + it.ptr, it.image_off, it.nbytes);
       info.blob_bytes += it.nbytes;
       continue;
     }
@@ -852,7 +1045,7 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
     info.device_bytes += it.nbytes;
     const Collapsed c = collapse_dims(it);
     if (c.ndim == 0 || (c.ndim == 1 && c.ts[0] == 1 && c.is[0] == 1)) {
-      cut_spans(tiles, it.ptr, it.image_off, it.nbytes, tile, align_to_tensor, plan->cut_mask);
+      flat.add(it.ptr, it.image_off, it.nbytes);
       continue;
     }
     // rows that are contiguous on both sides and long enough go through the flat kernel, one row at a time
@@ -867,8 +1060,7 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
           toff += idx[d] * c.ts[d];
           ioff += idx[d] * c.is[d];
         }
-        cut_spans(tiles, it.ptr + (uint64_t)(toff * (int64_t)esz), it.image_off + (uint64_t)(ioff * (int64_t)esz),
-                  row_bytes, tile, align_to_tensor, plan->cut_mask);
+        flat.add(it.ptr + (uint64_t)(toff * (int64_t)esz), it.image_off + (uint64_t)(ioff * (int64_t)esz), row_bytes);
         for (int d = last - 1; d >= 0; --d) {
           if (++idx[d] < c.shape[d]) break;
           idx[d] = 0;
@@ -958,6 +1150,18 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
   if (rc == MLF_HIP_OK) rc = upload(work, &plan->d_work);
   if (rc == MLF_HIP_OK) rc = upload(tdescs, &plan->d_tdescs);
   if (rc == MLF_HIP_OK) rc = upload(twork, &plan->d_twork);
+  if (rc == MLF_HIP_OK && plan->has_crc) {
+    // entries the fused kernel does not serve are checksummed from the finished image
+    std::vector<uint32_t> slow;
+    for (uint64_t e = 0; e < ent.size(); ++e)
+      if (!ent[e]) slow.push_back((uint32_t)e);
+    plan->crc.n_slow = slow.size();
+    rc = upload(ent, &plan->crc.d_ent);
+    if (rc == MLF_HIP_OK) rc = upload(slow, &plan->crc.d_slow_list);
+    if (rc == MLF_HIP_OK) rc = crc_fused_setup(&plan->crc);
+    info.fused_crc_bytes = flat.fused_bytes;
+    info.crc_chunks = plan->crc.n_chunks;
+  }
   if (rc != MLF_HIP_OK) {
     const std::string keep = last_error();
     mlf_plan_destroy(plan.release());
@@ -1031,6 +1235,15 @@ int launch_plan(const mlf_plan* plan, char* image, hipStream_t stream) {
   if (!plan) return fail(MLF_HIP_BAD_ARG, "null plan");
   if (!image && plan->info.image_bytes) return fail(MLF_HIP_BAD_ARG, "null image");
   if (reinterpret_cast<uintptr_t>(image) & 255) return fail(MLF_HIP_BAD_ARG, "image must be 256-byte aligned");
+  if (plan->has_crc) {
+    const FusedCrc& f = plan->crc;
+    const uint64_t n_wg = f.fused_groups * f.wgs_per_group;
+    if (n_wg) {
+      hipLaunchKernelGGL((mlf_fused_crc_kernel<PACK>), dim3((uint32_t)n_wg), dim3(256), 0, stream, f.d_ent, image,
+                         f.wgs_per_group, f.d_row_tab, f.d_lane_w, f.d_fast_val);
+      HIP_TRY(hipGetLastError());
+    }
+  }
   if (plan->flat_total) {
     // gridDim.x * blockDim.x must stay below 2^32; what does not fit in one row of workgroups goes to gridDim.y
     const uint32_t row_log2 = plan->grid_x_log2, total = plan->flat_total;
@@ -1067,12 +1280,24 @@ int launch_plan(const mlf_plan* plan, char* image, hipStream_t stream) {
                        plan->d_work + first, image);
     HIP_TRY(hipGetLastError());
   }
+  // the image (pack) or its source (unpack) is complete at this point of the stream: the rest of the checksum
+  if (plan->has_crc) return crc_fused_finish(&plan->crc, image, stream);
   return MLF_HIP_OK;
 }
 
 }  // namespace
 
 extern "C" {
+
+int mlf_plan_crc_values(mlf_plan* plan, uint32_t* out_host, uint64_t n_out) {
+  if (!plan || !out_host) return fail(MLF_HIP_BAD_ARG, "null argument");
+  if (!plan->has_crc) return fail(MLF_HIP_BAD_ARG, "the plan was created without crc_chunk_kib");
+  if (!plan->crc.launched) return fail(MLF_HIP_BAD_ARG, "the plan has not been launched yet");
+  if (n_out < plan->crc.n_chunks) return fail(MLF_HIP_BAD_ARG, "output array too small");
+  HIP_TRY(hipEventSynchronize(plan->crc.done));
+  memcpy(out_host, plan->crc.h_out, plan->crc.n_chunks * sizeof(uint32_t));
+  return MLF_HIP_OK;
+}
 
 int mlf_pack_launch(const mlf_plan* plan, void* image_dev, void* stream) {
   return launch_plan<true>(plan, static_cast<char*>(image_dev), static_cast<hipStream_t>(stream));

@@ -39,7 +39,7 @@ class PlanOpts(ctypes.Structure):
         ("align_to_tensor", ctypes.c_uint32),
         ("unroll", ctypes.c_uint32),
         ("grid_x_log2", ctypes.c_uint32),
-        ("reserved", ctypes.c_uint32),
+        ("crc_chunk_kib", ctypes.c_uint32),
     ]
 
 
@@ -58,6 +58,8 @@ class PlanInfo(ctypes.Structure):
             "image_bytes",
             "table_bytes",
             "n_small_items",
+            "fused_crc_bytes",
+            "crc_chunks",
         )
     ]
 
@@ -85,6 +87,7 @@ _SIGNATURES = {
     "mlf_plan_destroy": (_INT, [_VP]),
     "mlf_plan_get_info": (_INT, [_VP, ctypes.POINTER(PlanInfo)]),
     "mlf_plan_update_blob": (_INT, [_VP, _VP, _U64, _VP]),
+    "mlf_plan_crc_values": (_INT, [_VP, _VP, _U64]),
     "mlf_pack_launch": (_INT, [_VP, _VP, _VP]),
     "mlf_unpack_launch": (_INT, [_VP, _VP, _VP]),
     "mlf_crc32c_device": (_INT, [_VP, _U64, _U64, _VP, _U64, _VP]),

@@ -266,10 +266,17 @@ class Plan:
         align_to_tensor: bool = False,
         unroll: int = 0,
         grid_x_log2: int = 0,
+        crc_chunk_bytes: int = 0,
     ):
+        """``crc_chunk_bytes`` > 0 (a multiple of 64 KiB): every pack / unpack launch also yields the CRC-32C of each
+        chunk of that size of the image, folded inside the copy kernel where a contiguous item covers whole 64 KiB
+        pieces of the image (``crc_values``)."""
         lib = _lib.load()
         assert items.dtype == ITEM_DTYPE and items.flags["C_CONTIGUOUS"]
-        opts = _lib.PlanOpts(tile_bytes, block_threads, 1 if align_to_tensor else 0, unroll, grid_x_log2, 0)
+        if crc_chunk_bytes % 65536:
+            raise ValueError("crc_chunk_bytes must be a multiple of 65536")
+        opts = _lib.PlanOpts(tile_bytes, block_threads, 1 if align_to_tensor else 0, unroll, grid_x_log2,
+                             crc_chunk_bytes >> 10)
         handle = ctypes.c_void_p()
         blob_buf = (ctypes.c_char * len(blob)).from_buffer_copy(blob) if blob else None
         _lib.check(
@@ -286,6 +293,18 @@ class Plan:
         )
         self._handle = handle
         self.image_bytes = image_bytes
+        self.crc_chunk_bytes = crc_chunk_bytes if image_bytes else 0
+
+    def crc_values(self) -> np.ndarray:
+        """Per-chunk CRC-32C of the image moved by the most recent launch (waits for that launch's checksum work)."""
+        if self._handle is None:
+            raise ValueError("plan already destroyed")
+        if not self.crc_chunk_bytes:
+            return np.zeros(0, dtype=np.uint32)
+        n = -(-self.image_bytes // self.crc_chunk_bytes)
+        out = np.zeros(n, dtype=np.uint32)
+        _lib.check(_lib.load().mlf_plan_crc_values(self._handle, out.ctypes.data, n), "mlf_plan_crc_values")
+        return out
 
     @property
     def info(self) -> _lib.PlanInfo:

@@ -1,0 +1,174 @@
+"""Plans that checksum the image while they copy it (plan option ``crc_chunk_kib``): the bytes moved are the same as
+without the option, and the per-chunk CRC-32C values equal those of the stand-alone checksum pass and of the CPU
+oracle's C routine - for every source/target misalignment, for chunks of 64 KiB to 32 MiB (one to 512 workgroups per
+group), with record headers, item edges, strided views and a short last chunk in the image."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import mlf_format as oracle_fmt
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _oracle_chunks(oracle_c, raw: bytes, chunk: int) -> np.ndarray:
+    want = np.zeros(-(-len(raw) // chunk), dtype=np.uint32)
+    oracle_c.oracle_crc32c_chunks(raw, len(raw), chunk, want.ctypes.data)
+    return want
+
+
+def _misaligned_tensors(sizes, seed):
+    """Contiguous uint8 device tensors whose addresses are off the 16-byte grid by 0, 1, 2 ... bytes."""
+    gen = torch.Generator(device=DEV).manual_seed(seed)
+    out = []
+    for k, n in enumerate(sizes):
+        parent = torch.randint(0, 256, (n + 64,), dtype=torch.uint8, device=DEV, generator=gen)
+        t = parent[k % 16 : k % 16 + n]
+        assert t.data_ptr() % 16 == (parent.data_ptr() + k % 16) % 16
+        out.append(t)
+    return out
+
+
+@pytest.mark.parametrize("chunk", [65536, 1 << 20, 4 << 20, 32 << 20])
+def test_pack_with_checksums_matches_plain_pack_and_oracle(chunk, oracle_c):
+    from ml_flashpoint.hip import plan as P
+
+    # 17 tensors of 0.3 .. 9 MB at every byte misalignment; record headers in between put the payloads at odd offsets
+    sizes = [(300 << 10) + 4099 * k + (k % 5) * (1 << 21) for k in range(17)]
+    if chunk == 32 << 20:
+        sizes += [(40 << 20) + 7]  # room for a whole group of 512 workgroups
+    tensors = _misaligned_tensors(sizes, seed=3)
+    layout = P.build_save_layout(tensors)
+    plain = P.Plan(layout.items, layout.blob, layout.image_bytes)
+    fused = P.Plan(layout.items, layout.blob, layout.image_bytes, crc_chunk_bytes=chunk)
+    info = fused.info
+    assert info.crc_chunks == -(-layout.image_bytes // chunk)
+    assert info.fused_crc_bytes > 0.5 * layout.image_bytes if chunk <= (4 << 20) else info.fused_crc_bytes >= (32 << 20)
+    image_a = torch.full((layout.image_bytes + 512,), 0xAB, dtype=torch.uint8, device=DEV)
+    image_b = torch.full((layout.image_bytes + 512,), 0xCD, dtype=torch.uint8, device=DEV)
+    plain.pack(image_a)
+    fused.pack(image_b)
+    got = fused.crc_values()
+    torch.cuda.synchronize()
+    assert torch.equal(image_a[: layout.image_bytes], image_b[: layout.image_bytes])
+    assert bool((image_b[layout.image_bytes :] == 0xCD).all()), "pack wrote past the end of the image"
+    raw = image_b[: layout.image_bytes].cpu().numpy().tobytes()
+    want, spans = oracle_fmt.data_section([t.cpu() for t in tensors])
+    assert raw == want and layout.spans == spans
+    assert got.tolist() == P.crc32c_device(image_b, layout.image_bytes, chunk).tolist()
+    assert got.tolist() == _oracle_chunks(oracle_c, raw, chunk).tolist()
+    # a second launch of the same plan over changed tensors: new bytes, new values, nothing left over
+    for t in tensors:
+        t.add_(1)
+    fused.pack(image_b)
+    got2 = fused.crc_values()
+    raw2 = image_b[: layout.image_bytes].cpu().numpy().tobytes()
+    assert raw2 == oracle_fmt.data_section([t.cpu() for t in tensors])[0]
+    assert got2.tolist() == _oracle_chunks(oracle_c, raw2, chunk).tolist() and got2.tolist() != got.tolist()
+
+
+def test_pack_with_checksums_mixed_items(oracle_c):
+    """Small items, strided and transposed views, host-resident items and byte blobs beside large contiguous ones."""
+    from ml_flashpoint.hip import plan as P
+
+    gen = torch.Generator(device=DEV).manual_seed(5)
+    big = torch.randint(0, 256, (6 << 20,), dtype=torch.uint8, device=DEV, generator=gen)
+    base = torch.randint(0, 2**15, (1024, 768), dtype=torch.int16, device=DEV, generator=gen)
+    tensors = [
+        torch.randn(3, 5, device=DEV, generator=gen),
+        big[3:].view(torch.uint8),
+        base.t(),
+        base[:, ::2],
+        torch.randn(700_001, device=DEV, generator=gen).to(torch.bfloat16),
+        torch.arange(40_000, dtype=torch.int64),  # host-resident: rides in the blob
+        base[16:528],
+        torch.randn(1 << 20, device=DEV, generator=gen),
+    ]
+    blobs = [b"", bytes(range(256)) * 300, b"tail"]
+    layout = P.build_save_layout(tensors, blobs)
+    chunk = 1 << 20
+    fused = P.Plan(layout.items, layout.blob, layout.image_bytes, crc_chunk_bytes=chunk)
+    image = torch.zeros(layout.image_bytes, dtype=torch.uint8, device=DEV)
+    fused.pack(image)
+    got = fused.crc_values()
+    raw = image.cpu().numpy().tobytes()
+    assert raw == oracle_fmt.data_section([t.cpu() for t in tensors], blobs)[0]
+    assert got.tolist() == _oracle_chunks(oracle_c, raw, chunk).tolist()
+    info = fused.info
+    assert info.fused_crc_bytes > 0 and info.n_strided_items > 0 and info.n_transposed_items > 0
+
+
+@pytest.mark.parametrize("nbytes", [1, 4095, 65535, 65536, 65537, (1 << 20) - 1, (1 << 20) + 4096, (3 << 20) + 12345])
+def test_pack_with_checksums_small_images(nbytes, oracle_c):
+    from ml_flashpoint.hip import plan as P
+
+    gen = torch.Generator(device=DEV).manual_seed(nbytes)
+    t = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device=DEV, generator=gen)
+    layout = P.build_save_layout([t])
+    for chunk in (65536, 1 << 20):
+        fused = P.Plan(layout.items, layout.blob, layout.image_bytes, crc_chunk_bytes=chunk)
+        image = torch.zeros(layout.image_bytes, dtype=torch.uint8, device=DEV)
+        fused.pack(image)
+        raw = image.cpu().numpy().tobytes()
+        assert fused.crc_values().tolist() == _oracle_chunks(oracle_c, raw, chunk).tolist()
+
+
+@pytest.mark.parametrize("chunk", [65536, 1 << 20, 32 << 20])
+def test_unpack_with_checksums_restores_and_reports_the_images_values(chunk, oracle_c):
+    from ml_flashpoint.hip import plan as P
+
+    sizes = [(200 << 10) + 8191 * k + (k % 3) * (3 << 20) for k in range(16)]
+    if chunk == 32 << 20:
+        sizes += [(36 << 20) + 3]
+    source = _misaligned_tensors(sizes, seed=11)
+    layout = P.build_save_layout(source)
+    packer = P.Plan(layout.items, layout.blob, layout.image_bytes)
+    image = torch.zeros(layout.image_bytes, dtype=torch.uint8, device=DEV)
+    packer.pack(image)
+    torch.cuda.synchronize()
+    raw = image.cpu().numpy().tobytes()
+    want = _oracle_chunks(oracle_c, raw, chunk)
+    # targets at other misalignments than the sources, with guard bytes around them
+    parents = [torch.full((n + 96,), 0x5A, dtype=torch.uint8, device=DEV) for n in sizes]
+    targets = [p[32 + (5 * k + 1) % 16 : 32 + (5 * k + 1) % 16 + n] for k, (p, n) in enumerate(zip(parents, sizes))]
+    table = P.ItemTable()
+    for (offset, length), t in zip(layout.spans, targets):
+        n = t.numel()
+        table.add_contiguous(t.data_ptr(), offset + length - n, 1, n)
+    for align_to_tensor in (True, False):
+        for p in parents:
+            p.fill_(0x5A)
+        plan = P.Plan(table.to_array(), b"", layout.image_bytes, align_to_tensor=align_to_tensor, crc_chunk_bytes=chunk)
+        plan.unpack(image)
+        got = plan.crc_values()
+        torch.cuda.synchronize()
+        assert got.tolist() == want.tolist()
+        for k, (p, t, s) in enumerate(zip(parents, targets, source)):
+            assert torch.equal(t, s), k
+            lo = 32 + (5 * k + 1) % 16
+            assert bool((p[:lo] == 0x5A).all()) and bool((p[lo + t.numel() :] == 0x5A).all()), f"guard bytes of {k}"
+    # a flipped bit in the image shows up in exactly the chunk it lies in
+    at = layout.image_bytes // 2
+    image[at] ^= 0x10
+    plan.unpack(image)
+    bad = plan.crc_values()
+    assert (bad != want).nonzero()[0].tolist() == [at // chunk]
+
+
+def test_checksum_option_argument_checks():
+    from ml_flashpoint.hip import _lib
+    from ml_flashpoint.hip import plan as P
+
+    t = torch.zeros(1 << 16, dtype=torch.uint8, device=DEV)
+    layout = P.build_save_layout([t])
+    with pytest.raises(ValueError):
+        P.Plan(layout.items, layout.blob, layout.image_bytes, crc_chunk_bytes=1000)
+    plain = P.Plan(layout.items, layout.blob, layout.image_bytes)
+    out = np.zeros(4, dtype=np.uint32)
+    assert _lib.load().mlf_plan_crc_values(plain._handle, out.ctypes.data, 4) != 0
+    fused = P.Plan(layout.items, layout.blob, layout.image_bytes, crc_chunk_bytes=65536)
+    assert _lib.load().mlf_plan_crc_values(fused._handle, out.ctypes.data, 4) != 0  # not launched yet
+    assert b"not been launched" in _lib.load().mlf_hip_last_error()
