@@ -58,6 +58,10 @@ def parse_args():
     ap.add_argument("--crc-chunk-mib", type=int, default=32,
                     help="CRC-32C per chunk of this size, computed on the GPU during the save and verified on the GPU during "
                          "the restore (0 = off)")
+    ap.add_argument("--save-crc", choices=["beside", "fused"], default="beside",
+                    help="where the save's checksums are computed: a pass of its own beside the transfer, or inside the pack kernel")
+    ap.add_argument("--restore-crc", choices=["fused", "before"], default="fused",
+                    help="how the restore verifies them: inside the unpack kernel, or a pass of its own before it")
     ap.add_argument("--cpu-baseline-gb", type=float, default=12.0, help="size of the CPU baseline's sample (0 = skip)")
     ap.add_argument("--plan-cache", action="store_true",
                     help="reuse the save plan across steps once two consecutive plans compared equal, as the reference's "
@@ -292,9 +296,10 @@ def main():
     saver = DefaultMLFlashpointCheckpointSaver(
         lambda: 0, lambda: 0, lambda: None, manager, None, initial_buffer_size_bytes=1 << 20,
         engine_config=engine_cfg, tile_bytes=args.tile_bytes, block_threads=args.block_threads,
-        crc_chunk_bytes=args.crc_chunk_mib << 20, use_file_io=args.save_io == "file")
+        crc_chunk_bytes=args.crc_chunk_mib << 20, crc_mode=args.save_crc, use_file_io=args.save_io == "file")
     loader = DefaultMLFlashpointCheckpointLoader(manager, None, engine_config=engine_cfg, tile_bytes=args.tile_bytes,
-                                                 block_threads=args.block_threads, use_file_io=args.restore_io == "file")
+                                                 block_threads=args.block_threads, use_file_io=args.restore_io == "file",
+                                                 crc_mode=args.restore_crc)
     saver.record_kernel_events = loader.record_kernel_events = True
     result = None
     if args.pmc_calibration:
@@ -424,7 +429,7 @@ def main():
             "config": {"workload": f"{args.workload}: {label}", "tensors": len(sd), "payload_bytes": payload,
                        "file_bytes": file_bytes, "scale": args.scale, "tile_bytes": args.tile_bytes or 4096,
                        "engine": {"slot_mib": args.slot_mib, "slots": args.slots, "copy_threads": engine_cfg.resolved_copy_threads()},
-                       "crc_chunk_mib": args.crc_chunk_mib, "plan_cache": args.plan_cache, "save_io": args.save_io, "restore_io": args.restore_io},
+                       "crc_chunk_mib": args.crc_chunk_mib, "save_crc": args.save_crc, "restore_crc": args.restore_crc, "plan_cache": args.plan_cache, "save_io": args.save_io, "restore_io": args.restore_io},
             **({"partial_restore": partial} if partial else {}),
             "save_GBps": round(gb / mean(rec["save"]), 3),
             "restore_GBps": round(gb / mean(rec["restore"]), 3),

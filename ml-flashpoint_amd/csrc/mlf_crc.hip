@@ -264,6 +264,7 @@ void crc_fused_destroy(FusedCrc* f) {
   (void)hipFree(f->d_group_val);
   (void)hipFree(f->d_row_tab);
   (void)hipFree(f->d_lane_w);
+  (void)hipFree(f->d_sink);
   (void)hipFree(f->d_consts);
   (void)hipFree(f->d_out);
   if (f->h_out) (void)hipHostFree(f->h_out);
@@ -294,6 +295,7 @@ int crc_fused_setup(FusedCrc* f) {
   HIP_TRY(hipMemcpy(f->d_row_tab, row_tab.data(), 4096, hipMemcpyHostToDevice));
   HIP_TRY(hipMalloc(reinterpret_cast<void**>(&f->d_lane_w), 4096));
   HIP_TRY(hipMemcpy(f->d_lane_w, lane_w.data(), 4096, hipMemcpyHostToDevice));
+  HIP_TRY(hipMalloc(reinterpret_cast<void**>(&f->d_sink), 4096));
   HIP_TRY(hipMalloc(reinterpret_cast<void**>(&f->d_consts), sizeof(CrcConsts)));
   HIP_TRY(hipMemcpy(f->d_consts, &g_crc_host, sizeof(CrcConsts), hipMemcpyHostToDevice));
   HIP_TRY(hipMalloc(reinterpret_cast<void**>(&f->d_out), std::max<uint64_t>(f->n_chunks, 1) * sizeof(uint32_t)));

@@ -101,6 +101,7 @@ struct FusedCrc {
   uint32_t* d_group_val = nullptr;
   uint32_t* d_row_tab = nullptr;  // [4][256]: state advanced by wgs_per_group cells, sliced by state byte
   u32x4* d_lane_w = nullptr;      // [256]: weight of each lane's four dwords within a cell
+  char* d_sink = nullptr;         // 4 KiB that the fused kernel writes instead of cells that are not its own
   CrcConsts* d_consts = nullptr;  // lookup constants of the segment kernel
   uint32_t* d_out = nullptr;
   uint32_t* h_out = nullptr;      // pinned

@@ -623,10 +623,19 @@ __global__ void __launch_bounds__(kTransThreads) mlf_transpose_kernel(const Tran
 // value per workgroup, chained by mlf_crc_groups_kernel.  Cells of entries without an address (record headers, item
 // edges, strided items ...) are skipped here; the other kernels move them and their remainders are taken from the
 // finished image.  The checksum arithmetic hides behind the memory traffic (measured on 16 GiB: copy alone in this
-// order 4.7-5.6 TB/s, with the checksum 5.7-5.8; one 4 KiB tile per workgroup without checksum 6.2).
+// order 4.7-5.6 TB/s, with the checksum 5.7-5.8; one 4 KiB tile per workgroup without checksum 6.2): what the kernel
+// gives up against the flat kernel - 39.3 against 34.3 ms on the 112 GB shard - is the price of workgroups that live
+// for sixteen rows instead of one, not of the arithmetic.  Eight or four rows per workgroup do not amortise the
+// closing multiplications (5.0 and 3.7 TB/s), thirty-two gain nothing.
 constexpr uint32_t kFusedRows = 16;   // cells per workgroup; FusedCrc::rows
 constexpr uint32_t kFusedAhead = 4;   // rows requested before the first is used
-constexpr uint32_t kFusedMaxGroupWgs = 512;
+// workgroups per group: 64 (groups of 4 MiB) and 512 (32 MiB) move the 112 GB shard equally fast when packing; unpacking
+// into byte-misaligned tensors is faster with 64 (5.5 against 4.7 TB/s), and chaining 64 values per group takes 0.05 ms
+// where 512 take 0.6
+constexpr uint32_t kFusedMaxGroupWgs = 64;
+// copies of the Horner table in LDS (4 KiB each): four copies changed nothing (11.07 against 10.84 ms on a 28 GB
+// shard), the lookups are not what bounds this kernel
+constexpr uint32_t kFusedTabCopies = 1;
 constexpr uint32_t kCellBytes = 4096;
 constexpr uint32_t kEntryBytes = 65536;
 constexpr uint32_t kCellsPerEntryLog2 = 4;
@@ -635,8 +644,10 @@ template <bool PACK>
 __global__ void __launch_bounds__(256) mlf_fused_crc_kernel(const uint64_t* __restrict__ ent, char* __restrict__ image,
                                                             uint32_t G, const uint32_t* __restrict__ row_tab,
                                                             const u32x4* __restrict__ lane_w,
-                                                            uint32_t* __restrict__ fast_val) {
-  __shared__ uint32_t tab[1024];
+                                                            uint32_t* __restrict__ fast_val, char* __restrict__ sink) {
+  // kFusedTabCopies copies of the table, entry v of copy c at word v * copies + c, lane l reads copy l % copies:
+  // lookups with random v then spread over that many times more banks
+  __shared__ uint32_t tab[1024 * kFusedTabCopies];
   __shared__ uint32_t part[4];
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
   const uint32_t group = blockIdx.x / G;
@@ -663,81 +674,50 @@ __global__ void __launch_bounds__(256) mlf_fused_crc_kernel(const uint64_t* __re
     if (tid == 0) *out = 0u;
     return;
   }
-  u32x4 raw[kFusedAhead], far[kFusedAhead];
-  // PACK: the tensor side is read - directly where it is dword-aligned, else as aligned 16-byte granules that are
-  // realigned across lanes (lane 63 of a wavefront also fetches the granule its neighbour in the next wavefront
-  // holds).  UNPACK: the image cell is read as it lies.
-#define MLF_FUSED_REQUEST(k)                                                                                        \
-  if (base[k]) {                                                                                                    \
-    if (PACK) {                                                                                                     \
-      const uint32_t delta = (uint32_t)base[k] & 15u;                                                               \
-      if ((delta & 3u) == 0u) {                                                                                     \
-        raw[(k) % kFusedAhead] = __builtin_nontemporal_load(gload<u32x4_u>(reinterpret_cast<const char*>(base[k]) + tid * 16u)); \
-      } else {                                                                                                      \
-        const char* a = reinterpret_cast<const char*>(base[k] - delta);                                             \
-        raw[(k) % kFusedAhead] = __builtin_nontemporal_load(gload<u32x4>(a + tid * 16u));                           \
-        if (lane == 63u) far[(k) % kFusedAhead] = __builtin_nontemporal_load(gload<u32x4>(a + (tid + 1u) * 16u));   \
-      }                                                                                                             \
-    } else {                                                                                                        \
-      raw[(k) % kFusedAhead] = __builtin_nontemporal_load(gload<u32x4>(image + ((cell0 + (uint64_t)(k) * G) << 12) + tid * 16u)); \
-    }                                                                                                               \
-  }
+  u32x4 raw[kFusedAhead];
+  // PACK reads the tensor side where it lies (dwordx4 loads at any byte address: the realignment across lanes that
+  // the flat kernel uses for such sources costs registers here and gains nothing), UNPACK the image cell.  There is
+  // no branch around a row that is not ours: it reads a 4 KiB table instead, writes to a 4 KiB sink nobody reads,
+  // and is masked out of the sums.  (Uniform branches here cost a quarter of the throughput: the compiler ends the
+  // waits for outstanding loads at every block boundary, and the rows no longer overlap.)
+  const char* const spare_src = reinterpret_cast<const char*>(lane_w);
+#define MLF_FUSED_SRC(k)                                                                          \
+  ((base[k] ? (PACK ? reinterpret_cast<const char*>(base[k])                                      \
+                    : const_cast<const char*>(image) + ((cell0 + (uint64_t)(k) * G) << 12))       \
+            : spare_src) + tid * 16u)
+#define MLF_FUSED_DST(k)                                                                          \
+  ((base[k] ? (PACK ? image + ((cell0 + (uint64_t)(k) * G) << 12) : reinterpret_cast<char*>(base[k])) : sink) + tid * 16u)
 #pragma unroll
-  for (uint32_t k = 0; k < kFusedAhead; ++k) {
-    MLF_FUSED_REQUEST(k)
-  }
+  for (uint32_t k = 0; k < kFusedAhead; ++k) raw[k] = __builtin_nontemporal_load(gload<u32x4_u>(MLF_FUSED_SRC(k)));
 #pragma unroll
-  for (uint32_t k = 0; k < 4; ++k) tab[tid + 256u * k] = row_tab[tid + 256u * k];
+  for (uint32_t k = 0; k < 4; ++k) {
+    const uint32_t t = row_tab[tid + 256u * k];
+#pragma unroll
+    for (uint32_t c = 0; c < kFusedTabCopies; ++c) tab[(tid + 256u * k) * kFusedTabCopies + c] = t;
+  }
   __syncthreads();
-#define MLF_FUSED_ADV(a) \
-  (tab[(a) & 255u] ^ tab[256u + (((a) >> 8) & 255u)] ^ tab[512u + (((a) >> 16) & 255u)] ^ tab[768u + ((a) >> 24)])
+  const uint32_t* my = tab + (lane & (kFusedTabCopies - 1u));
+#define MLF_FUSED_ADV(a)                                                                          \
+  (my[((a) & 255u) * kFusedTabCopies] ^ my[(256u + (((a) >> 8) & 255u)) * kFusedTabCopies] ^      \
+   my[(512u + (((a) >> 16) & 255u)) * kFusedTabCopies] ^ my[(768u + ((a) >> 24)) * kFusedTabCopies])
   uint32_t a0 = 0, a1 = 0, a2 = 0, a3 = 0;
 #pragma unroll
   for (uint32_t k = 0; k < kFusedRows; ++k) {
-    u32x4 v = raw[k % kFusedAhead];  // becomes the cell's vector as it lies in the image
-    if (PACK && base[k]) {
-      const uint32_t delta = (uint32_t)base[k] & 15u;
-      if ((delta & 3u) != 0u) {
-        const u32x4 lo = v;
-        u32x4 hi;
-        hi.x = (uint32_t)__shfl_down((int)lo.x, 1);
-        hi.y = (uint32_t)__shfl_down((int)lo.y, 1);
-        hi.z = (uint32_t)__shfl_down((int)lo.z, 1);
-        hi.w = (uint32_t)__shfl_down((int)lo.w, 1);
-        if (lane == 63u) hi = far[k % kFusedAhead];
-        const uint32_t q = delta >> 2, r = delta & 3u;
-        uint32_t w0, w1, w2, w3, w4;
-        switch (q) {
-          case 0: w0 = lo.x; w1 = lo.y; w2 = lo.z; w3 = lo.w; w4 = hi.x; break;
-          case 1: w0 = lo.y; w1 = lo.z; w2 = lo.w; w3 = hi.x; w4 = hi.y; break;
-          case 2: w0 = lo.z; w1 = lo.w; w2 = hi.x; w3 = hi.y; w4 = hi.z; break;
-          default: w0 = lo.w; w1 = hi.x; w2 = hi.y; w3 = hi.z; w4 = hi.w; break;
-        }
-        v.x = __builtin_amdgcn_alignbyte(w1, w0, r);
-        v.y = __builtin_amdgcn_alignbyte(w2, w1, r);
-        v.z = __builtin_amdgcn_alignbyte(w3, w2, r);
-        v.w = __builtin_amdgcn_alignbyte(w4, w3, r);
-      }
-    }
-    if (k + kFusedAhead < kFusedRows) {  // the slot just read is free again
-      MLF_FUSED_REQUEST(k + kFusedAhead)
-    }
-    if (base[k]) {
-      if (PACK) __builtin_nontemporal_store(v, gstore<u32x4>(image + ((cell0 + (uint64_t)k * G) << 12) + tid * 16u));
-      else __builtin_nontemporal_store(v, gstore<u32x4_u>(reinterpret_cast<char*>(base[k]) + tid * 16u));
-      a0 = MLF_FUSED_ADV(a0) ^ v.x;
-      a1 = MLF_FUSED_ADV(a1) ^ v.y;
-      a2 = MLF_FUSED_ADV(a2) ^ v.z;
-      a3 = MLF_FUSED_ADV(a3) ^ v.w;
-    } else {  // somebody else's cell: it contributes zeros at this position
-      a0 = MLF_FUSED_ADV(a0);
-      a1 = MLF_FUSED_ADV(a1);
-      a2 = MLF_FUSED_ADV(a2);
-      a3 = MLF_FUSED_ADV(a3);
-    }
+    const u32x4 v = raw[k % kFusedAhead];  // the cell's vector as it lies in the image
+    if (k + kFusedAhead < kFusedRows)      // the slot just read is free again
+      raw[k % kFusedAhead] = __builtin_nontemporal_load(gload<u32x4_u>(MLF_FUSED_SRC(k + kFusedAhead)));
+    __builtin_nontemporal_store(v, gstore<u32x4_u>(MLF_FUSED_DST(k)));
+    const uint32_t ours = base[k] ? 0xFFFFFFFFu : 0u;
+    a0 = MLF_FUSED_ADV(a0) ^ (v.x & ours);
+    a1 = MLF_FUSED_ADV(a1) ^ (v.y & ours);
+    a2 = MLF_FUSED_ADV(a2) ^ (v.z & ours);
+    a3 = MLF_FUSED_ADV(a3) ^ (v.w & ours);
+    // rows stay in this order (without the fence the compiler may hoist all sixteen loads to the top)
+    __asm__ volatile("" ::: "memory");
   }
+#undef MLF_FUSED_SRC
+#undef MLF_FUSED_DST
 #undef MLF_FUSED_ADV
-#undef MLF_FUSED_REQUEST
   const u32x4 wts = lane_w[tid];
   uint32_t acc = gf_mul(a0, wts.x) ^ gf_mul(a1, wts.y) ^ gf_mul(a2, wts.z) ^ gf_mul(a3, wts.w);
 #pragma unroll
@@ -1240,7 +1220,7 @@ int launch_plan(const mlf_plan* plan, char* image, hipStream_t stream) {
     const uint64_t n_wg = f.fused_groups * f.wgs_per_group;
     if (n_wg) {
       hipLaunchKernelGGL((mlf_fused_crc_kernel<PACK>), dim3((uint32_t)n_wg), dim3(256), 0, stream, f.d_ent, image,
-                         f.wgs_per_group, f.d_row_tab, f.d_lane_w, f.d_fast_val);
+                         f.wgs_per_group, f.d_row_tab, f.d_lane_w, f.d_fast_val, f.d_sink);
       HIP_TRY(hipGetLastError());
     }
   }

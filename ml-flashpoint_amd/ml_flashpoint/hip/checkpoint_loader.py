@@ -84,13 +84,17 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         tile_bytes: int = 0,
         block_threads: int = 0,
         verify_crc: bool = True,
+        crc_mode: str = "fused",
         use_file_io: bool = True,
         verify_on_discovery: bool = False,
         max_image_bytes: Optional[int] = None,
     ):
         """Arguments as the reference's default loader (checkpoint_loader.py:126-158), plus the copy-engine and
         kernel work-split knobs, ``verify_crc`` (check the CRC-32C sidecar of an object, when it has one, while
-        restoring it) and ``verify_on_discovery`` (also check it, on the host, while choosing the checkpoint to
+        restoring it), ``crc_mode`` (how a whole-object restore checks it: ``"fused"`` - the unpack kernel folds the
+        checksums of the image it reads, so the image is read once and a mismatch is reported after the targets were
+        written; ``"before"`` - a checksum pass over the image first, and nothing is written on a mismatch) and
+        ``verify_on_discovery`` (also check it, on the host, while choosing the checkpoint to
         recover from, so that a corrupted copy counts as missing) and ``max_image_bytes`` (largest range of an
         object that is uploaded to HBM in one piece; default: what the device has free minus 2 GiB.  A larger
         range is restored window by window through one buffer of that size)."""
@@ -106,6 +110,9 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         self._tile_bytes = tile_bytes
         self._block_threads = block_threads
         self._verify_crc = verify_crc
+        if crc_mode not in ("fused", "before"):
+            raise ValueError("crc_mode must be 'fused' or 'before'")
+        self._crc_mode = crc_mode
         # pread() the buffer file into the pinned slots instead of reading through the (fresh, read-only) mapping:
         # reads of tmpfs run in parallel, and no page-table entry per 4 KiB has to be built and torn down
         self._use_file_io = use_file_io
@@ -394,11 +401,12 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         stats["h2d_s"] += st.seconds
         stats["h2d_bytes"] += span
 
-    def _unpack(self, items, image: torch.Tensor, span: int, cur, payload_bytes: int) -> None:
+    def _unpack(self, items, image: torch.Tensor, span: int, cur, payload_bytes: int, crc_chunk_bytes: int = 0):
         """Launches the unpack of ``items`` out of ``image`` and waits for it: the targets are complete, and the
-        image may be reused or freed, when this returns."""
+        image may be reused or freed, when this returns.  With ``crc_chunk_bytes`` the unpack kernel also folds the
+        CRC-32C of every chunk of the image; those values are returned."""
         plan = hip_plan.Plan(items, b"", span, tile_bytes=self._tile_bytes, block_threads=self._block_threads,
-                             align_to_tensor=True)
+                             align_to_tensor=True, crc_chunk_bytes=crc_chunk_bytes)
         try:
             if self.record_kernel_events:
                 begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -409,6 +417,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
             else:
                 plan.unpack(image, cur.cuda_stream)
             cur.synchronize()
+            return plan.crc_values() if crc_chunk_bytes else None
         finally:
             plan.destroy()
 
@@ -419,6 +428,10 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         self._upload(stream, lo, image, span, cur, stats)
         if sidecar is not None:
             chunk_bytes, data_bytes, want = sidecar
+            if self._crc_mode == "fused" and chunk_bytes % 65536 == 0 and data_bytes == span:
+                got = self._unpack(self._table_of(rows, lo), image, span, cur, stats["device_payload_bytes"], chunk_bytes)
+                self._compare_checksums(object_id, got, want, chunk_bytes)
+                return
             got = hip_plan.crc32c_device(image, data_bytes, chunk_bytes, cur.cuda_stream)
             self._compare_checksums(object_id, got, want, chunk_bytes)
         self._unpack(self._table_of(rows, lo), image, span, cur, stats["device_payload_bytes"])

@@ -172,3 +172,83 @@ def test_checksum_option_argument_checks():
     fused = P.Plan(layout.items, layout.blob, layout.image_bytes, crc_chunk_bytes=65536)
     assert _lib.load().mlf_plan_crc_values(fused._handle, out.ctypes.data, 4) != 0  # not launched yet
     assert b"not been launched" in _lib.load().mlf_hip_last_error()
+
+
+@pytest.mark.filterwarnings("ignore:torch.distributed is disabled")
+@pytest.mark.parametrize("background_write", [False, True])
+def test_saver_and_loader_checksum_modes_agree(shm_dir, background_write):
+    """The saver's two ways to the sidecar (a pass beside the transfer, or inside the pack kernel) write the same
+    object and the same sidecar; the loader's two ways to check it (inside the unpack kernel, or a pass before it)
+    restore the same bits and reject the same corrupted chunk."""
+    import concurrent.futures
+    import os
+    import threading
+
+    import torch.distributed.checkpoint as dcp
+
+    import workloads
+    from ml_flashpoint.adapter.pytorch.memory_storage_reader import MemoryStorageReader
+    from ml_flashpoint.adapter.pytorch.memory_storage_writer import MemoryStorageWriter
+    from ml_flashpoint.checkpoint_object_manager.buffer_metadata import METADATA_SIZE
+    from ml_flashpoint.checkpoint_object_manager.checkpoint_object_manager import CheckpointObjectManager
+    from ml_flashpoint.core.checkpoint_loader import DefaultMLFlashpointCheckpointLoader
+    from ml_flashpoint.core.checkpoint_saver import DefaultMLFlashpointCheckpointSaver
+    from ml_flashpoint.hip import integrity
+
+    class LocalManager:
+        def dict(self):
+            return {}
+
+        def Event(self):
+            return threading.Event()
+
+    fut = concurrent.futures.Future()
+    fut.set_result(LocalManager())
+    CheckpointObjectManager._worker_pool = None
+    sd = workloads.llama3_8b_shard(DEV, layers=2, d=512, ffn=1792, kv=128, vocab=8000)
+    sd["extra.step"] = 7  # a pickled object behind the tensors
+    chunk = 1 << 20
+    files, sidecars = {}, {}
+    for mode in ("beside", "fused"):
+        saver = DefaultMLFlashpointCheckpointSaver(lambda: 0, lambda: 0, lambda: None, CheckpointObjectManager(), None,
+                                                   initial_buffer_size_bytes=1 << 20, crc_chunk_bytes=chunk, crc_mode=mode,
+                                                   background_write=background_write)
+        for step in (1, 2):  # the second save of a mode runs on the kept plan
+            ckpt = os.path.join(shm_dir, mode, f"step-{step}_ckpt")
+            dcp.save(sd, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(saver, fut), no_dist=True)
+            obj = os.path.join(ckpt, "__0__0_src0.distcp")
+            files[mode, step] = open(obj, "rb").read()
+            sidecars[mode, step] = integrity.read_sidecar(obj)
+        assert saver.last_save_stats.get("plans_reused") == 1
+    assert files["beside", 1] == files["fused", 1] == files["fused", 2]
+    want = sidecars["beside", 1]
+    assert want is not None and want[0] == chunk and want[1] == len(files["beside", 1]) - METADATA_SIZE
+    for key, got in sidecars.items():
+        assert got[:2] == want[:2] and got[2].tolist() == want[2].tolist(), key
+    with pytest.raises(ValueError):
+        DefaultMLFlashpointCheckpointSaver(lambda: 0, lambda: 0, lambda: None, CheckpointObjectManager(), None, crc_mode="x")
+
+    ckpt = os.path.join(shm_dir, "fused", "step-2_ckpt")
+    obj = os.path.join(ckpt, "__0__0_src0.distcp")
+    originals = {k: v.clone() for k, v in sd.items() if isinstance(v, torch.Tensor)}
+    for mode in ("fused", "before"):
+        loader = DefaultMLFlashpointCheckpointLoader(CheckpointObjectManager(), None, crc_mode=mode)
+        target = {k: (torch.zeros_like(v) if isinstance(v, torch.Tensor) else None) for k, v in sd.items()}
+        dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), no_dist=True)
+        assert target["extra.step"] == 7
+        assert all(torch.equal(target[k].view(torch.uint8), v.view(torch.uint8)) for k, v in originals.items()), mode
+    at = METADATA_SIZE + 5 * chunk + 4321
+    with open(obj, "r+b") as f:
+        f.seek(at)
+        byte = f.read(1)
+        f.seek(at)
+        f.write(bytes([byte[0] ^ 0x01]))
+    for mode in ("fused", "before"):
+        loader = DefaultMLFlashpointCheckpointLoader(CheckpointObjectManager(), None, crc_mode=mode)
+        target = {k: (torch.zeros_like(v) if isinstance(v, torch.Tensor) else None) for k, v in sd.items()}
+        with pytest.raises(BaseException) as exc:
+            dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), no_dist=True)
+        cause = exc.value.failures[0][0] if hasattr(exc.value, "failures") else exc.value
+        assert isinstance(cause, integrity.ChecksumMismatchError) and "chunk(s) [5]" in str(cause), mode
+        if mode == "before":  # nothing was written before the mismatch was found
+            assert all(not bool(v.any()) for v in target.values() if isinstance(v, torch.Tensor))
