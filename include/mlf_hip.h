@@ -205,6 +205,15 @@ int mlf_engine_d2h_watched(mlf_engine* engine, const void* src_dev, void* dst_ho
                            void* producer_stream, uint64_t crc_chunk_bytes, uint32_t* crc_out_host,
                            uint64_t n_crc_out, uint64_t* landed, mlf_xfer_stats* stats);
 
+/* mlf_engine_d2h_watched whose copies (and checksum pass) wait for an event instead of for a stream: `ready_event`
+ * is a hipEvent_t (passed as void*) that the caller recorded right behind the kernel that produced the source - the
+ * pack - or NULL to start at once.  A transfer that is started from another thread than the one that launched the
+ * pack then waits for the pack only, not for whatever the training step has enqueued on that stream since.  No
+ * reference counterpart: the reference's device synchronize (memory_storage_writer.py:229-231) waits for everything. */
+int mlf_engine_d2h_gated(mlf_engine* engine, const void* src_dev, void* dst_host, uint64_t nbytes, void* ready_event,
+                         uint64_t crc_chunk_bytes, uint32_t* crc_out_host, uint64_t n_crc_out, uint64_t* landed,
+                         mlf_xfer_stats* stats);
+
 /* Host -> device.  Copies `nbytes` from `src_host` (pageable, e.g. the read-only mapping) to `dst_dev`
  * and makes `consumer_stream` wait for the last chunk, so an unpack launched on it afterwards sees the data.
  * Returns once all chunks are enqueued and the host source is no longer needed.  Replaces BufferIO.read()'s

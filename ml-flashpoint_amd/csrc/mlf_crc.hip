@@ -333,17 +333,48 @@ int crc_fused_finish(FusedCrc* f, const void* image, hipStream_t stream) {
   return MLF_HIP_OK;
 }
 
-void crc_release(CrcJob* job) {
-  (void)hipFree(job->d_consts);
-  (void)hipFree(job->d_seg);
-  (void)hipFree(job->d_out);
-  if (job->h_out) (void)hipHostFree(job->h_out);
-  *job = CrcJob();
+void crc_scratch_free(CrcScratch* sc) {
+  (void)hipFree(sc->d_consts);
+  (void)hipFree(sc->d_seg);
+  (void)hipFree(sc->d_out);
+  if (sc->h_out) (void)hipHostFree(sc->h_out);
+  *sc = CrcScratch();
 }
+
+namespace {
+
+int crc_scratch_ensure(CrcScratch* sc, uint64_t n_segs, uint64_t n_chunks) {
+  if (!sc->d_consts) {
+    std::call_once(g_crc_once, crc_init_host);
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&sc->d_consts), sizeof(CrcConsts)));
+    HIP_TRY(hipMemcpy(sc->d_consts, &g_crc_host, sizeof(CrcConsts), hipMemcpyHostToDevice));
+  }
+  if (n_segs > sc->seg_cap) {
+    (void)hipFree(sc->d_seg);
+    sc->d_seg = nullptr;
+    sc->seg_cap = 0;
+    const uint64_t cap = std::max<uint64_t>(n_segs + n_segs / 4, 4096);  // some headroom: objects of one job differ little
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&sc->d_seg), cap * sizeof(uint32_t)));
+    sc->seg_cap = cap;
+  }
+  if (n_chunks > sc->out_cap) {
+    (void)hipFree(sc->d_out);
+    if (sc->h_out) (void)hipHostFree(sc->h_out);
+    sc->d_out = sc->h_out = nullptr;
+    sc->out_cap = 0;
+    const uint64_t cap = std::max<uint64_t>(n_chunks + n_chunks / 4, 1024);
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&sc->d_out), cap * sizeof(uint32_t)));
+    HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&sc->h_out), cap * sizeof(uint32_t), hipHostMallocDefault));
+    sc->out_cap = cap;
+  }
+  return MLF_HIP_OK;
+}
+
+}  // namespace
 
 // Enqueues the two CRC kernels and the copy of the per-chunk values on `stream`; does not wait.
 int crc_enqueue(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint64_t n_out, hipStream_t stream,
-                CrcJob* job, bool background) {
+                CrcScratch* sc, bool background) {
   if (!dev_ptr) return fail(MLF_HIP_BAD_ARG, "null pointer");
   if (reinterpret_cast<uintptr_t>(dev_ptr) & 15) return fail(MLF_HIP_BAD_ARG, "device buffer must be 16-byte aligned");
   if (chunk_bytes == 0 || chunk_bytes % kCrcSegBytes)
@@ -353,53 +384,34 @@ int crc_enqueue(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint
   const uint64_t seg_bytes = pick_seg_bytes(nbytes, chunk_bytes);
   const uint64_t n_segs = (nbytes + seg_bytes - 1) / seg_bytes;
   if (n_segs > 0xFFFFFFF0ull) return fail(MLF_HIP_BAD_ARG, "buffer too large for one CRC call");
-  std::call_once(g_crc_once, crc_init_host);
-  job->n_chunks = n_chunks;
-  job->stream = stream;
-#define CRC_TRY(expr)                                                                             \
-  do {                                                                                            \
-    hipError_t e__ = (expr);                                                                      \
-    if (e__ != hipSuccess) {                                                                      \
-      crc_release(job);                                                                           \
-      return fail(MLF_HIP_RUNTIME, std::string(#expr) + " failed: " + hipGetErrorString(e__));    \
-    }                                                                                             \
-  } while (0)
-  CRC_TRY(hipMalloc(reinterpret_cast<void**>(&job->d_consts), sizeof(CrcConsts)));
-  CRC_TRY(hipMalloc(reinterpret_cast<void**>(&job->d_seg), n_segs * sizeof(uint32_t)));
-  CRC_TRY(hipMalloc(reinterpret_cast<void**>(&job->d_out), n_chunks * sizeof(uint32_t)));
-  CRC_TRY(hipHostMalloc(reinterpret_cast<void**>(&job->h_out), n_chunks * sizeof(uint32_t), hipHostMallocDefault));
-  CRC_TRY(hipMemcpyAsync(job->d_consts, &g_crc_host, sizeof(CrcConsts), hipMemcpyHostToDevice, stream));
+  if (int rc = crc_scratch_ensure(sc, n_segs, n_chunks)) return rc;
   if (background) {
     // one copy of the tables (4 KiB of LDS per workgroup instead of 64 KiB): the CUs' LDS stays available to the
     // kernels this pass runs beside
     const uint32_t grid = (uint32_t)((n_segs + 3) / 4);
     hipLaunchKernelGGL(mlf_crc_segments_kernel<1>, dim3(grid), dim3(256), 0, stream, static_cast<const char*>(dev_ptr),
-                       nbytes, job->d_consts, job->d_seg, (uint32_t)n_segs, (uint32_t)seg_bytes, nullptr);
+                       nbytes, sc->d_consts, sc->d_seg, (uint32_t)n_segs, (uint32_t)seg_bytes, nullptr);
   } else {
     const uint32_t waves_per_block = kCrcThreads / 64;
     const uint32_t grid = (uint32_t)((n_segs + waves_per_block - 1) / waves_per_block);
     hipLaunchKernelGGL(mlf_crc_segments_kernel<kCrcTableCopies>, dim3(grid), dim3(kCrcThreads), 0, stream,
-                       static_cast<const char*>(dev_ptr), nbytes, job->d_consts, job->d_seg, (uint32_t)n_segs,
+                       static_cast<const char*>(dev_ptr), nbytes, sc->d_consts, sc->d_seg, (uint32_t)n_segs,
                        (uint32_t)seg_bytes, nullptr);
   }
-  CRC_TRY(hipGetLastError());
+  HIP_TRY(hipGetLastError());
   const uint64_t last_seg_len = nbytes - (n_segs - 1) * seg_bytes;
-  hipLaunchKernelGGL(mlf_crc_chunks_kernel, dim3((uint32_t)((n_chunks + 63) / 64)), dim3(64), 0, stream, job->d_seg,
+  hipLaunchKernelGGL(mlf_crc_chunks_kernel, dim3((uint32_t)((n_chunks + 63) / 64)), dim3(64), 0, stream, sc->d_seg,
                      (uint32_t)(chunk_bytes / seg_bytes), (uint32_t)n_segs, x_pow_bytes(seg_bytes),
-                     x_pow_bytes(last_seg_len), job->d_out, (uint32_t)n_chunks);
-  CRC_TRY(hipGetLastError());
-  CRC_TRY(hipMemcpyAsync(job->h_out, job->d_out, n_chunks * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
-#undef CRC_TRY
+                     x_pow_bytes(last_seg_len), sc->d_out, (uint32_t)n_chunks);
+  HIP_TRY(hipGetLastError());
+  HIP_TRY(hipMemcpyAsync(sc->h_out, sc->d_out, n_chunks * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
   return MLF_HIP_OK;
 }
 
-// Waits for the job, hands the values out and frees the scratch.
-int crc_finish(CrcJob* job, uint32_t* out_host) {
-  hipError_t e = hipStreamSynchronize(job->stream);
-  if (e == hipSuccess && out_host) memcpy(out_host, job->h_out, job->n_chunks * sizeof(uint32_t));
-  crc_release(job);
-  if (e != hipSuccess) return fail(MLF_HIP_RUNTIME, std::string("hipStreamSynchronize failed: ") + hipGetErrorString(e));
+int crc_finish(CrcScratch* sc, hipStream_t stream, uint64_t n_chunks, uint32_t* out_host) {
+  HIP_TRY(hipStreamSynchronize(stream));
   if (!out_host) return fail(MLF_HIP_BAD_ARG, "null pointer");
+  memcpy(out_host, sc->h_out, n_chunks * sizeof(uint32_t));
   return MLF_HIP_OK;
 }
 
@@ -472,9 +484,16 @@ int mlf_crc32c_file(int fd, uint64_t file_offset, uint64_t nbytes, uint64_t chun
 int mlf_crc32c_device(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint32_t* out_host,
                       uint64_t n_out, void* stream_) {
   if (nbytes == 0) return MLF_HIP_OK;
-  CrcJob job;
-  if (int rc = crc_enqueue(dev_ptr, nbytes, chunk_bytes, n_out, static_cast<hipStream_t>(stream_), &job, false)) return rc;
-  return crc_finish(&job, out_host);
+  // one scratch per device, kept for the life of the library; calls on one device take turns
+  static std::mutex mu[kNoAllocMaxDevices];
+  static CrcScratch scratch[kNoAllocMaxDevices];
+  int device = 0;
+  HIP_TRY(hipGetDevice(&device));
+  if (device < 0 || device >= kNoAllocMaxDevices) return fail(MLF_HIP_BAD_ARG, "device index beyond the per-device table");
+  std::lock_guard<std::mutex> g(mu[device]);
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (int rc = crc_enqueue(dev_ptr, nbytes, chunk_bytes, n_out, stream, &scratch[device], false)) return rc;
+  return crc_finish(&scratch[device], stream, (nbytes + chunk_bytes - 1) / chunk_bytes, out_host);
 }
 
 int mlf_crc32c_device_noalloc(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint32_t* out_dev,

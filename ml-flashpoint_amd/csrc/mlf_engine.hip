@@ -145,6 +145,7 @@ struct mlf_engine {
   hipStream_t streams[2] = {nullptr, nullptr};
   hipStream_t crc_stream = nullptr;  // checksum kernels run beside the copies, not before them
   hipEvent_t gate = nullptr;
+  CrcScratch crc;  // of the checksum passes that run beside transfers; allocated on first use, grown when too small
   std::unique_ptr<WorkerPool> pool;
   std::mutex busy;  // one transfer at a time per engine
 };
@@ -158,7 +159,11 @@ int mlf_engine_destroy(mlf_engine* e) {
   if (e->gate) (void)hipEventDestroy(e->gate);
   for (hipStream_t s : e->streams)
     if (s) (void)hipStreamDestroy(s);
-  if (e->crc_stream) (void)hipStreamDestroy(e->crc_stream);
+  if (e->crc_stream) {
+    (void)hipStreamSynchronize(e->crc_stream);
+    (void)hipStreamDestroy(e->crc_stream);
+  }
+  crc_scratch_free(&e->crc);
   delete e;
   return MLF_HIP_OK;
 }
@@ -223,36 +228,47 @@ struct CrcRequest {
   uint64_t* landed = nullptr;  // progress counter of the caller, or null
 };
 
-int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t nbytes, void* producer_stream,
+// What a device-to-host transfer waits for before its first copy: everything enqueued so far on a stream, or an
+// event the caller recorded behind the producing kernel (then later work on the producer's stream does not delay it).
+struct Gate {
+  void* producer_stream = nullptr;
+  hipEvent_t ready = nullptr;
+  bool by_event = false;
+};
+
+int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t nbytes, const Gate& gate,
                mlf_xfer_stats* stats, const CrcRequest& crc = CrcRequest()) {
   if (!e) return fail(MLF_HIP_BAD_ARG, "null engine");
   if (nbytes && (!src_dev || (host.fd < 0 && !host.ptr))) return fail(MLF_HIP_BAD_ARG, "null pointer");
   std::lock_guard<std::mutex> g(e->busy);
   HIP_TRY(hipSetDevice(e->device));
   const double t0 = now_s();
-  // the copy streams start after whatever the producer has enqueued so far (the pack)
-  HIP_TRY(hipEventRecord(e->gate, static_cast<hipStream_t>(producer_stream)));
-  for (hipStream_t s : e->streams) HIP_TRY(hipStreamWaitEvent(s, e->gate, 0));
+  hipEvent_t ready = gate.ready;
+  if (!gate.by_event) {
+    // the copy streams start after whatever the producer has enqueued so far (the pack)
+    HIP_TRY(hipEventRecord(e->gate, static_cast<hipStream_t>(gate.producer_stream)));
+    ready = e->gate;
+  }
+  if (ready)
+    for (hipStream_t s : e->streams) HIP_TRY(hipStreamWaitEvent(s, ready, 0));
   const char* src = static_cast<const char*>(src_dev);
   if (crc.landed) __atomic_store_n(crc.landed, (uint64_t)0, __ATOMIC_RELEASE);
-  CrcJob crc_job;
   const bool want_crc = crc.chunk_bytes != 0 && nbytes != 0;
+  const uint64_t n_crc = want_crc ? (nbytes + crc.chunk_bytes - 1) / crc.chunk_bytes : 0;
+  struct CrcGuard {  // on every exit path the checksum kernels have finished before the scratch can be used again
+    hipStream_t stream;
+    bool armed;
+    ~CrcGuard() {
+      if (armed) (void)hipStreamSynchronize(stream);
+    }
+  } crc_guard{e->crc_stream, false};
   if (want_crc) {
     // the image is complete once the gate has passed and is not modified afterwards, so its checksum can be
     // computed while the link-bound copies run: it costs neither blocking time nor transfer time
-    HIP_TRY(hipStreamWaitEvent(e->crc_stream, e->gate, 0));
-    if (int rc = crc_enqueue(src_dev, nbytes, crc.chunk_bytes, crc.n_out, e->crc_stream, &crc_job, true)) return rc;
+    if (ready) HIP_TRY(hipStreamWaitEvent(e->crc_stream, ready, 0));
+    crc_guard.armed = true;
+    if (int rc = crc_enqueue(src_dev, nbytes, crc.chunk_bytes, crc.n_out, e->crc_stream, &e->crc, true)) return rc;
   }
-  struct CrcGuard {  // scratch is released on every exit path, after the kernels that use it have finished
-    CrcJob* job;
-    bool armed;
-    ~CrcGuard() {
-      if (armed) {
-        (void)hipStreamSynchronize(job->stream);
-        crc_release(job);
-      }
-    }
-  } crc_guard{&crc_job, want_crc};
   const uint64_t slot = e->slot_bytes;
   const uint64_t n_chunks = (nbytes + slot - 1) / slot;
   const uint64_t n_slots = e->slots.size();
@@ -283,7 +299,7 @@ int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t
   drain.armed = false;  // every chunk's event has been waited for
   if (want_crc) {
     crc_guard.armed = false;
-    if (int rc = crc_finish(&crc_job, crc.out_host)) return rc;
+    if (int rc = crc_finish(&e->crc, e->crc_stream, n_crc, crc.out_host)) return rc;
   }
   if (stats) {
     stats->seconds = now_s() - t0;
@@ -340,7 +356,9 @@ int mlf_engine_d2h(mlf_engine* e, const void* src_dev, void* dst_host, uint64_t 
                    mlf_xfer_stats* stats) {
   HostEnd host;
   host.ptr = static_cast<char*>(dst_host);
-  return engine_d2h(e, src_dev, host, nbytes, producer_stream, stats);
+  Gate gate;
+  gate.producer_stream = producer_stream;
+  return engine_d2h(e, src_dev, host, nbytes, gate, stats);
 }
 
 int mlf_engine_h2d(mlf_engine* e, const void* src_host, void* dst_dev, uint64_t nbytes, void* consumer_stream,
@@ -359,7 +377,9 @@ int mlf_engine_d2h_crc(mlf_engine* e, const void* src_dev, void* dst_host, uint6
   crc.chunk_bytes = crc_chunk_bytes;
   crc.out_host = crc_out_host;
   crc.n_out = n_crc_out;
-  return engine_d2h(e, src_dev, host, nbytes, producer_stream, stats, crc);
+  Gate gate;
+  gate.producer_stream = producer_stream;
+  return engine_d2h(e, src_dev, host, nbytes, gate, stats, crc);
 }
 
 int mlf_engine_d2h_watched(mlf_engine* e, const void* src_dev, void* dst_host, uint64_t nbytes, void* producer_stream,
@@ -374,7 +394,27 @@ int mlf_engine_d2h_watched(mlf_engine* e, const void* src_dev, void* dst_host, u
   crc.out_host = crc_out_host;
   crc.n_out = n_crc_out;
   crc.landed = landed;
-  return engine_d2h(e, src_dev, host, nbytes, producer_stream, stats, crc);
+  Gate gate;
+  gate.producer_stream = producer_stream;
+  return engine_d2h(e, src_dev, host, nbytes, gate, stats, crc);
+}
+
+int mlf_engine_d2h_gated(mlf_engine* e, const void* src_dev, void* dst_host, uint64_t nbytes, void* ready_event,
+                         uint64_t crc_chunk_bytes, uint32_t* crc_out_host, uint64_t n_crc_out, uint64_t* landed,
+                         mlf_xfer_stats* stats) {
+  if (crc_chunk_bytes && !crc_out_host) return fail(MLF_HIP_BAD_ARG, "null checksum output");
+  if (reinterpret_cast<uintptr_t>(landed) & 7) return fail(MLF_HIP_BAD_ARG, "progress counter must be 8-byte aligned");
+  HostEnd host;
+  host.ptr = static_cast<char*>(dst_host);
+  CrcRequest crc;
+  crc.chunk_bytes = crc_chunk_bytes;
+  crc.out_host = crc_out_host;
+  crc.n_out = n_crc_out;
+  crc.landed = landed;
+  Gate gate;
+  gate.ready = static_cast<hipEvent_t>(ready_event);
+  gate.by_event = true;
+  return engine_d2h(e, src_dev, host, nbytes, gate, stats, crc);
 }
 
 int mlf_engine_host_copy(mlf_engine* e, void* dst_host, const void* src_host, uint64_t nbytes) {
@@ -391,7 +431,9 @@ int mlf_engine_d2h_fd(mlf_engine* e, const void* src_dev, int fd, uint64_t file_
   HostEnd host;
   host.fd = fd;
   host.file_off = file_offset;
-  return engine_d2h(e, src_dev, host, nbytes, producer_stream, stats);
+  Gate gate;
+  gate.producer_stream = producer_stream;
+  return engine_d2h(e, src_dev, host, nbytes, gate, stats);
 }
 
 int mlf_engine_h2d_fd(mlf_engine* e, int fd, uint64_t file_offset, void* dst_dev, uint64_t nbytes,

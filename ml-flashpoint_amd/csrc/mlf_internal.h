@@ -117,26 +117,28 @@ void crc_fused_destroy(FusedCrc* f);
 // chain over groups and chunks, the copy of the chunk values to the pinned array, and the event behind it.
 int crc_fused_finish(FusedCrc* f, const void* image, hipStream_t stream);
 
-// A CRC pass in flight: scratch on the device, results in a pinned host array, all ordered on `stream`.
-struct CrcConsts;
-struct CrcJob {
+// Scratch of the stand-alone checksum pass: lookup constants, one value per segment, one per chunk on the device and
+// a pinned copy of the latter.  Owned by whoever runs the passes (the copy engine, or the library per device) and
+// kept from pass to pass: allocating and releasing device memory per pass would synchronise the whole device.
+struct CrcScratch {
   CrcConsts* d_consts = nullptr;
   uint32_t* d_seg = nullptr;
+  uint64_t seg_cap = 0;
   uint32_t* d_out = nullptr;
   uint32_t* h_out = nullptr;  // pinned
-  uint64_t n_chunks = 0;
-  hipStream_t stream = nullptr;
+  uint64_t out_cap = 0;
 };
 
-// Enqueues the two CRC kernels and the copy of the per-chunk values on `stream`; does not wait.  `background`: the
-// pass runs beside other work on the device (a save's checksum beside the training step) and takes the variant
-// that leaves the CUs' LDS to that work, at 85 % of the speed of the one that fills it with table copies.
+// Enqueues the two CRC kernels and the copy of the per-chunk values on `stream`; does not wait.  Grows `scratch`
+// first if this pass needs more than it holds (its previous user must have finished).  `background`: the pass runs
+// beside other work on the device (a save's checksum beside the training step) and takes the variant that leaves the
+// CUs' LDS to that work, at 85 % of the speed of the one that fills it with table copies.
 int crc_enqueue(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint64_t n_out, hipStream_t stream,
-                CrcJob* job, bool background);
-// Waits for the job, hands the values out and frees the scratch.
-int crc_finish(CrcJob* job, uint32_t* out_host);
-// Frees the scratch of a job that is not going to be finished (its stream must be idle).
-void crc_release(CrcJob* job);
+                CrcScratch* scratch, bool background);
+// Waits for `stream` and hands out the values of the pass enqueued last (`n_chunks` of them).
+int crc_finish(CrcScratch* scratch, hipStream_t stream, uint64_t n_chunks, uint32_t* out_host);
+// Frees the scratch (its stream must be idle).
+void crc_scratch_free(CrcScratch* scratch);
 
 }  // namespace mlf
 

@@ -750,6 +750,8 @@ struct mlf_plan {
   uint64_t blob_size = 0;
   char* h_blob = nullptr;            // pinned staging of mlf_plan_update_blob, allocated on first use
   hipEvent_t blob_copied = nullptr;  // recorded behind the last upload out of h_blob
+  mutable hipEvent_t launched = nullptr;  // recorded behind the last launch (plans with a blob): an upload of new
+                                          // blob bytes on another stream waits for the kernels that read the old ones
   uint32_t block_threads = 256;
   uint32_t unroll = 1;
   uint32_t cut_mask = 15;     // tile cuts sit on multiples of cut_mask + 1 bytes ...
@@ -772,6 +774,7 @@ struct mlf_plan {
     (void)hipFree(d_blob);
     if (h_blob) (void)hipHostFree(h_blob);
     if (blob_copied) (void)hipEventDestroy(blob_copied);
+    if (launched) (void)hipEventDestroy(launched);
     crc_fused_destroy(&crc);
   }
 };
@@ -1194,7 +1197,9 @@ int mlf_plan_update_blob(mlf_plan* plan, const void* host_blob, uint64_t blob_by
     HIP_TRY(hipEventSynchronize(plan->blob_copied));  // the previous upload has left the staging buffer
   }
   memcpy(plan->h_blob, host_blob, blob_bytes);
-  // ordered on the caller's stream: behind the launches that still read the old bytes, ahead of those to come
+  // behind the launches that still read the old bytes - also when they ran on another stream than this one -
+  // and, ordered on the caller's stream, ahead of those to come
+  if (plan->launched) HIP_TRY(hipStreamWaitEvent(static_cast<hipStream_t>(stream), plan->launched, 0));
   HIP_TRY(hipMemcpyAsync(plan->d_blob, plan->h_blob, blob_bytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream)));
   HIP_TRY(hipEventRecord(plan->blob_copied, static_cast<hipStream_t>(stream)));
   return MLF_HIP_OK;
@@ -1259,6 +1264,10 @@ int launch_plan(const mlf_plan* plan, char* image, hipStream_t stream) {
     hipLaunchKernelGGL((mlf_strided_kernel<PACK>), dim3((uint32_t)count), dim3(256), 0, stream, plan->d_descs,
                        plan->d_work + first, image);
     HIP_TRY(hipGetLastError());
+  }
+  if (plan->blob_size) {
+    if (!plan->launched) HIP_TRY(hipEventCreateWithFlags(&plan->launched, hipEventDisableTiming));
+    HIP_TRY(hipEventRecord(plan->launched, stream));
   }
   // the image (pack) or its source (unpack) is complete at this point of the stream: the rest of the checksum
   if (plan->has_crc) return crc_fused_finish(&plan->crc, image, stream);

@@ -832,14 +832,13 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                         t0 = time.perf_counter()
                         crcs = staged.plan.crc_values()
                         xfer["crc_s"] = xfer.get("crc_s", 0.0) + time.perf_counter() - t0
-                        st, _ = engine.d2h_watched(staged.image.data_ptr(), writer.data_address(start), nbytes,
-                                                   staged.stream, 0, staged._landed)
+                        st, _ = self._send_image(engine, staged, writer.data_address(start), nbytes, 0)
                         self._count_transfer(xfer, st, nbytes)
                     else:
                         # checksum kernels (if asked for) run on the engine's third stream while the chunks cross
                         # the link; the engine keeps the object's progress counter current
-                        st, crcs = engine.d2h_watched(staged.image.data_ptr(), writer.data_address(start), nbytes,
-                                                      staged.stream, self._crc_chunk_bytes, staged._landed)
+                        st, crcs = self._send_image(engine, staged, writer.data_address(start), nbytes,
+                                                    self._crc_chunk_bytes)
                         self._count_transfer(xfer, st, nbytes)
                     staged._landed.value = nbytes
         staged.consumed = True
@@ -852,6 +851,17 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         else:
             integrity.remove_sidecar(str(bucket.object_id))
         return self._results_of(staged, bucket.object_name)
+
+    @staticmethod
+    def _send_image(engine, staged: StagedObject, dst_host_ptr: int, nbytes: int, crc_chunk_bytes: int):
+        """The image into the buffer.  The copies wait for the event recorded behind the pack, so a transfer that
+        runs on a background thread is not held up by what the training step has put on that stream since."""
+        event = staged.packed_event
+        if event is not None:
+            return engine.d2h_gated(staged.image.data_ptr(), dst_host_ptr, nbytes, event.cuda_event, crc_chunk_bytes,
+                                    staged._landed)
+        return engine.d2h_watched(staged.image.data_ptr(), dst_host_ptr, nbytes, staged.stream, crc_chunk_bytes,
+                                  staged._landed)
 
     @staticmethod
     def _count_transfer(xfer: dict, st, nbytes: int) -> None:

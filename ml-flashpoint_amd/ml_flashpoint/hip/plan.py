@@ -399,6 +399,21 @@ class CopyEngine:
         )
         return stats, (crcs[:n_chunks] if crc_chunk_bytes else None)
 
+    def d2h_gated(self, src_dev_ptr: int, dst_host_ptr: int, nbytes: int, ready_event: Optional[int],
+                  crc_chunk_bytes: int, landed: "ctypes.c_uint64"):
+        """``d2h_watched`` that waits for an event (a raw ``hipEvent_t``, e.g. ``torch.cuda.Event.cuda_event``, recorded
+        behind the pack; None: does not wait) instead of for everything on the producer's stream."""
+        stats = _lib.XferStats()
+        n_chunks = (nbytes + crc_chunk_bytes - 1) // crc_chunk_bytes if crc_chunk_bytes else 0
+        crcs = np.zeros(max(n_chunks, 1), dtype=np.uint32)
+        _lib.check(
+            _lib.load().mlf_engine_d2h_gated(self._handle, src_dev_ptr, dst_host_ptr, nbytes, ready_event,
+                                             crc_chunk_bytes, crcs.ctypes.data, len(crcs), ctypes.addressof(landed),
+                                             ctypes.byref(stats)),
+            "mlf_engine_d2h_gated",
+        )
+        return stats, (crcs[:n_chunks] if crc_chunk_bytes else None)
+
     def host_copy(self, dst_host_ptr: int, src_host_ptr: int, nbytes: int) -> None:
         """Host memory to host memory on the engine's threads (checkpoint items that are resident on the host)."""
         _lib.check(_lib.load().mlf_engine_host_copy(self._handle, dst_host_ptr, src_host_ptr, nbytes), "mlf_engine_host_copy")
