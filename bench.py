@@ -34,11 +34,15 @@ for _p in (REPO, os.path.join(REPO, "ml-flashpoint_amd"), os.path.join(REPO, "te
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, vendor figure
-# HBM bytes moved by one pack of the default workload, relative to its algorithmic bytes (2 x payload): measured
-# with `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`, each scaled against a torch.add kernel of known size
-# (summary: profiles/pmc_traffic_mlf_flat_kernel_llama3-8b-shard.md).  Hardware counters cannot be read from
-# inside this script, so the ratio is applied to the live algorithmic byte count of the same workload only.
-PACK_TRAFFIC_RATIO_LLAMA3_8B = 1.0008
+# HBM bytes moved by one pack, relative to its algorithmic bytes (2 x payload), by (workload, where the checksums are
+# computed): measured with `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`, each scaled against a torch.add kernel of
+# known size (summaries: profiles/pmc_traffic_*.md).  Hardware counters cannot be read from inside this script, so the
+# ratio of the same workload at full scale is applied to the live algorithmic byte count; other runs report null.
+PACK_TRAFFIC_RATIO = {
+    ("llama3-8b-shard", "beside"): 1.0008,
+    ("llama3-8b-shard", "fused"): 1.0010,
+    ("strided-views", "beside"): 1.253,
+}
 
 
 def parse_args():
@@ -74,6 +78,12 @@ def parse_args():
     ap.add_argument("--partial-restore-prefix", default=None,
                     help="after the timed steps, also time a restore of only the entries whose names start with this "
                          "(e.g. 'model.': the weights out of weights + optimizer state); reported as partial_restore")
+    ap.add_argument("--max-image-gb", type=float, default=0.0,
+                    help="cap on the image held in HBM at once (saver and loader): smaller than the object, the save "
+                         "goes window by window and blocks for the transfer; 0 = what the device has free")
+    ap.add_argument("--no-prefault", action="store_true", help="leave the pool file's pages to the first save, as the reference does")
+    ap.add_argument("--no-link-probe", action="store_true", help="skip the bare host-link measurement")
+    ap.add_argument("--no-crc-compare", action="store_true", help="skip the extra saves in the other checksum mode")
     ap.add_argument("--root", default=None, help="directory on tmpfs for the pool and checkpoints")
     return ap.parse_args()
 
@@ -127,7 +137,8 @@ def cpu_baseline(sd, sample_bytes, root, device):
     path = os.path.join(cid.data, "sample.distcp")
     tensors = list(sample.values())
     times = {"stage": [], "write": [], "restore": []}
-    for rep in range(2):  # the first pass faults the tmpfs pages in, like the GPU path's warm-up
+    passes = 5
+    for rep in range(1 + passes):  # the first pass faults the tmpfs pages in, like the GPU path's prime iteration
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         staged = saver.stage_data(cid, sample, non_blocking=True)
@@ -163,18 +174,24 @@ def cpu_baseline(sd, sample_bytes, root, device):
         t4 = time.perf_counter()
         ok = all(torch.equal(a.view(torch.uint8), b.contiguous().view(torch.uint8)) for a, b in zip(targets[:8], tensors[:8]))
         del targets
-        times["stage"].append(t1 - t0)
-        times["write"].append(t2 - t1)
-        times["restore"].append(t4 - t3)
+        if rep:  # the warm-up pass is not counted
+            times["stage"].append(t1 - t0)
+            times["write"].append(t2 - t1)
+            times["restore"].append(t4 - t3)
     shutil.rmtree(os.path.join(root, "cpu_baseline"), ignore_errors=True)
-    stage, write, restore = times["stage"][-1], times["write"][-1], times["restore"][-1]
+    import statistics
+
+    stage, write, restore = (statistics.median(times[k]) for k in ("stage", "write", "restore"))
     gb = total / 1e9
     return {
         "value": round(2 * gb / (stage + write + restore), 3),
         "unit": "GB/s",
         "cores": threads,
         "kind": "port",
-        "sample": f"first {len(sample)} tensors ({gb:.2f} GB) of the same state dict, second pass (warm tmpfs pages)",
+        "sample": f"first {len(sample)} tensors ({gb:.2f} GB) of the same state dict; one warm-up pass, then the median of {passes} "
+                  "(warm tmpfs pages)",
+        "passes": passes,
+        "spread": {k: [round(min(v), 3), round(max(v), 3)] for k, v in times.items()},
         "save_GBps": round(gb / (stage + write), 3),
         "restore_GBps": round(gb / restore, 3),
         "blocking_stage_ms": round(stage * 1e3, 1),
@@ -289,18 +306,32 @@ def main():
     fut = concurrent.futures.Future()
     fut.set_result(mgr)
     engine_cfg = EngineConfig(slot_bytes=args.slot_mib << 20, n_slots=args.slots, copy_threads=args.copy_threads)
-    # one pooled buffer: the previous step's object is deleted before the next save, as finalize_checkpoint's
-    # background cleanup would have done, so the same warm tmpfs pages are reused every step
+    # one pooled buffer of the object's size (payload + record headers + slack), created before the first save the
+    # way a job creates its pool at start-up: its pages are allocated and mapped on a background thread
+    # (BufferPoolConfig.prefault), and the previous step's object is deleted before the next save, as
+    # finalize_checkpoint's background cleanup would have done, so the same pages are reused every step
     CheckpointObjectManager._worker_pool = None
-    manager = CheckpointObjectManager(BufferPoolConfig(os.path.join(root, "pool"), 0, 1, METADATA_SIZE + (1 << 20)))
-    saver = DefaultMLFlashpointCheckpointSaver(
-        lambda: 0, lambda: 0, lambda: None, manager, None, initial_buffer_size_bytes=1 << 20,
-        engine_config=engine_cfg, tile_bytes=args.tile_bytes, block_threads=args.block_threads,
-        crc_chunk_bytes=args.crc_chunk_mib << 20, crc_mode=args.save_crc, use_file_io=args.save_io == "file")
+    pool_bytes = METADATA_SIZE + payload + 256 * len(sd) + (1 << 20)
+    manager = CheckpointObjectManager(BufferPoolConfig(os.path.join(root, "pool"), 0, 1, pool_bytes,
+                                                       prefault=not args.no_prefault))
+    t_pool = time.perf_counter()
+    manager.warm_up_pool()
+    max_image = int(args.max_image_gb * 1e9) if args.max_image_gb > 0 else None
+
+    def make_saver(crc_mode):
+        made = DefaultMLFlashpointCheckpointSaver(
+            lambda: 0, lambda: 0, lambda: None, manager, None, initial_buffer_size_bytes=1 << 20,
+            engine_config=engine_cfg, tile_bytes=args.tile_bytes, block_threads=args.block_threads,
+            crc_chunk_bytes=args.crc_chunk_mib << 20, crc_mode=crc_mode, use_file_io=args.save_io == "file",
+            max_image_bytes=max_image)
+        made.record_kernel_events = True
+        return made
+
+    saver = make_saver(args.save_crc)
     loader = DefaultMLFlashpointCheckpointLoader(manager, None, engine_config=engine_cfg, tile_bytes=args.tile_bytes,
                                                  block_threads=args.block_threads, use_file_io=args.restore_io == "file",
-                                                 crc_mode=args.restore_crc)
-    saver.record_kernel_events = loader.record_kernel_events = True
+                                                 crc_mode=args.restore_crc, max_image_bytes=max_image)
+    loader.record_kernel_events = True
     result = None
     if args.pmc_calibration:
         cal_src = torch.ones(1 << 30, dtype=torch.float32, device=device)
@@ -309,80 +340,92 @@ def main():
         torch.cuda.synchronize()
         del cal_src, cal_dst
         torch.cuda.empty_cache()
+    dist = _DistWrapper(None, False, 0)
+    state = {"cached": None, "metadata": None}
+
+    def one_save(the_saver, cid):
+        """The reference's three-call form of a save (plan / write / finish), as its async strategy drives it.
+        Returns the wall times of its parts; the blocking part ends where the training stream may go on."""
+        the_saver.kernel_events.clear()
+        gc.collect()  # outside the timed regions: a full collection of this process's heap takes ~60 ms
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        the_saver.initialize_checkpoint(cid)
+        writer = MemoryStorageWriter(the_saver, fut)
+        writer.reset(cid.data)
+        buckets, md, central, local, validated = state_dict_saver.generate_plan(
+            cid, sd, writer, DefaultSavePlanner(), dist, state["cached"] if args.plan_cache else None)
+        state["metadata"] = md if md is not None else state["metadata"]
+        state["cached"] = (central, local, validated)
+        if md is None:  # a cached plan: the caller holds the metadata object that goes with it
+            writer.expect_metadata(state["metadata"])
+        t_launch = time.perf_counter()
+        staged = MemoryStorageWriter.stage_write_data_buckets(cid, buckets, non_blocking=True)
+        t_block = time.perf_counter()
+        prepare_s = the_saver.last_save_stats.get("prepare_s", 0.0)
+        results = state_dict_saver.write_data(cid, writer, staged, replicate_after_write=False)
+        t_written = time.perf_counter()
+        state_dict_saver.finish_write(cid, writer, state["metadata"], dist)
+        the_saver.finalize_checkpoint(cid)
+        t_saved = time.perf_counter()
+        stats = dict(the_saver.last_save_stats)
+        del buckets, staged, results
+        return {"save": t_saved - t0, "blocking": t_block - t0, "plan": t_launch - prepare_s - t0, "pack_launch": prepare_s,
+                "tail": t_saved - t_written, "stats": stats,
+                "pack_ms": sum(b.elapsed_time(e) for b, e, _ in the_saver.kernel_events),
+                "pack_bytes": sum(n for _, _, n in the_saver.kernel_events)}
+
     try:
-        rec = {k: [] for k in ("step", "save", "restore", "blocking", "plan", "pack_launch", "d2h", "h2d")}
+        rec = {}
         file_bytes = 0
         prev = None
-        cached = metadata = None
-        dist = _DistWrapper(None, False, 0)
-        # iteration 0 ("prime") is set-up, not a warm-up step: it is the save that first touches the pool buffer's
-        # tmpfs pages (page allocation at ~5 GB/s, paid once per pool buffer in a real job) and the first read of
-        # them; the W warm-up steps and K timed steps that follow all run on the populated buffer
+        first = {}
+        pool_prefault_s = manager.warm_up_pool(wait=True)
+        pool_age_s = time.perf_counter() - t_pool
+        # iteration 0 ("prime") is the first save and the first restore of the job; with the pool file's pages in
+        # place it runs like any other, without them it pays for their allocation (~5 GB/s).  It is reported as
+        # first_save_s / first_restore_s and not counted among the W warm-up and K timed steps.
         for it in range(1 + args.warmup + args.steps):
             timed = it >= 1 + args.warmup
             cid = CheckpointContainerId(os.path.join(root, "run", f"step-{it}_ckpt"))
             if prev is not None:
                 manager.delete_container(prev)
-            saver.kernel_events.clear()
             loader.kernel_events.clear()
-            gc.collect()  # outside the timed regions: a full collection of this process's heap takes ~60 ms
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            # ---- save: plan -> pack (blocking part ends at the synchronize) -> D2H -> metadata -> finalize ----
-            saver.initialize_checkpoint(cid)
-            writer = MemoryStorageWriter(saver, fut)
-            writer.reset(cid.data)
-            # the reference's three-call form of a save (plan / write / finish), as its async strategy drives it
-            buckets, md, central, local, validated = state_dict_saver.generate_plan(
-                cid, sd, writer, DefaultSavePlanner(), dist, cached if args.plan_cache else None)
-            metadata = md if md is not None else metadata
-            cached = (central, local, validated)
-            t_launch = time.perf_counter()
-            staged = MemoryStorageWriter.stage_write_data_buckets(cid, buckets, non_blocking=True)
-            t_block = time.perf_counter()
-            prepare_s = saver.last_save_stats.get("prepare_s", 0.0)
-            t_plan = t_launch - prepare_s
-            results = state_dict_saver.write_data(cid, writer, staged, replicate_after_write=False)
-            state_dict_saver.finish_write(cid, writer, metadata, dist)
-            saver.finalize_checkpoint(cid)
-            t_saved = time.perf_counter()
-            d2h = dict(saver.last_save_stats)
-            pack_ms = sum(b.elapsed_time(e) for b, e, _ in saver.kernel_events)
-            pack_bytes = sum(n for _, _, n in saver.kernel_events)
-            del buckets, staged, results
+            sv = one_save(saver, cid)
+            d2h = sv["stats"]
             # ---- restore into zeroed live tensors ----
             for v in sd.values():
                 v.zero_() if v.is_contiguous() else v.fill_(0)
+            gc.collect()
             torch.cuda.synchronize()
             t1 = time.perf_counter()
             dcp.load(sd, checkpoint_id=cid.data, storage_reader=MemoryStorageReader(cid.data, loader), no_dist=True)
             torch.cuda.synchronize()
             t2 = time.perf_counter()
+            ld = dict(loader.last_load_stats)
             unpack_ms = sum(b.elapsed_time(e) for b, e, _ in loader.kernel_events)
             unpack_bytes = sum(n for _, _, n in loader.kernel_events)
             file_bytes = os.path.getsize(os.path.join(cid.data, "__0__0_src0.distcp"))
             prev = cid
-            line = (f"[bench] it {it} {'timed ' if timed else ('prime ' if it == 0 else 'warmup')} save {t_saved - t0:.3f}s (blocking "
-                    f"{(t_block - t0) * 1e3:.1f} ms, pack kernel {pack_ms:.2f} ms, d2h {d2h.get('d2h_s', 0):.3f}s) "
-                    f"restore {t2 - t1:.3f}s (h2d {loader.last_load_stats.get('h2d_s', 0):.3f}s, unpack {unpack_ms:.2f} ms)")
+            line = (f"[bench] it {it} {'timed ' if timed else ('prime ' if it == 0 else 'warmup')} save {sv['save']:.3f}s (blocking "
+                    f"{sv['blocking'] * 1e3:.1f} ms, pack kernel {sv['pack_ms']:.2f} ms, d2h {d2h.get('d2h_s', 0):.3f}s) "
+                    f"restore {t2 - t1:.3f}s (h2d {ld.get('h2d_s', 0):.3f}s, unpack {unpack_ms:.2f} ms)")
             print(line, file=sys.stderr, flush=True)
+            if it == 0:
+                first = {"save": sv["save"], "restore": t2 - t1, "blocking": sv["blocking"]}
             if timed:
-                rec["step"].append((t_saved - t0) + (t2 - t1))
-                rec["save"].append(t_saved - t0)
-                rec["restore"].append(t2 - t1)
-                rec["blocking"].append(t_block - t0)
-                rec["plan"].append(t_plan - t0)
-                rec["pack_launch"].append(t_launch - t_plan)
-                rec["d2h"].append(d2h.get("d2h_s", 0.0))
-                rec.setdefault("d2h_bytes", []).append(d2h.get("d2h_bytes", 0))
-                rec.setdefault("host_copy_s", []).append(d2h.get("host_copy_s", 0.0))
-                rec.setdefault("host_copy_bytes", []).append(d2h.get("host_copy_bytes", 0))
-                rec["h2d"].append(loader.last_load_stats.get("h2d_s", 0.0))
-                rec.setdefault("h2d_bytes", []).append(loader.last_load_stats.get("h2d_bytes", 0))
-                rec.setdefault("pack_ms", []).append(pack_ms)
-                rec.setdefault("unpack_ms", []).append(unpack_ms)
-                rec.setdefault("pack_bytes", []).append(pack_bytes)
-                rec.setdefault("unpack_bytes", []).append(unpack_bytes)
+                row = {"step": sv["save"] + (t2 - t1), "save": sv["save"], "restore": t2 - t1, "blocking": sv["blocking"],
+                       "plan": sv["plan"], "pack_launch": sv["pack_launch"], "save_tail": sv["tail"],
+                       "d2h": d2h.get("d2h_s", 0.0), "d2h_bytes": d2h.get("d2h_bytes", 0),
+                       "host_copy_s": d2h.get("host_copy_s", 0.0), "host_copy_bytes": d2h.get("host_copy_bytes", 0),
+                       "h2d": ld.get("h2d_s", 0.0), "h2d_bytes": ld.get("h2d_bytes", 0),
+                       "pack_ms": sv["pack_ms"], "unpack_ms": unpack_ms, "pack_bytes": sv["pack_bytes"], "unpack_bytes": unpack_bytes,
+                       "r_read": ld.get("read_s", 0.0), "r_parse": ld.get("parse_s", 0.0), "r_table": ld.get("table_s", 0.0),
+                       "r_crc": ld.get("crc_s", 0.0), "r_unpack_plan": ld.get("unpack_plan_s", 0.0),
+                       "r_unpack": ld.get("unpack_s", 0.0), "r_commit": ld.get("commit_s", 0.0),
+                       "windows": d2h.get("windows", 0), "image_pieces": d2h.get("image_pieces", 0)}
+                for k, v in row.items():
+                    rec.setdefault(k, []).append(v)
         # parity after the timed region: restored bits == original bits
         mismatched = [k for k, v in sd.items() if workloads.fingerprint(v) != prints[k]]
         assert not mismatched, f"restored tensors differ from the originals: {mismatched[:5]}"
@@ -405,14 +448,60 @@ def main():
                        "payload_bytes": workloads.payload_bytes(subset), "seconds": round(min(times), 4),
                        "uploaded_bytes": stats.get("h2d_bytes", 0), "ranges": stats.get("partial_read_ranges", 1)}
             print(f"[bench] partial restore of '{args.partial_restore_prefix}*': {partial}", file=sys.stderr, flush=True)
-        manager.delete_container(prev)
 
         mean = lambda xs: sum(xs) / len(xs)  # noqa: E731
+        pack_s = mean(rec["pack_ms"]) * 1e-3
+        algorithmic = 2 * mean(rec["pack_bytes"])
+        # ---- the other way to the checksums, for comparison: two more saves (the first builds its plan) ----
+        crc_modes = None
+        if args.crc_chunk_mib and not args.no_crc_compare and max_image is None:
+            image_bytes = file_bytes - METADATA_SIZE
+            crc_modes = {args.save_crc: {"pack_ms": round(pack_s * 1e3, 3), "blocking_save_ms": round(mean(rec["blocking"]) * 1e3, 2),
+                                         "save_s": round(mean(rec["save"]), 4)}}
+            other_mode = "fused" if args.save_crc == "beside" else "beside"
+            other = make_saver(other_mode)
+            runs = []
+            for k in range(2):
+                manager.delete_container(prev)
+                prev = CheckpointContainerId(os.path.join(root, "run", f"step-{1000 + k}_ckpt"))
+                runs.append(one_save(other, prev))
+            crc_modes[other_mode] = {"pack_ms": round(runs[-1]["pack_ms"], 3), "blocking_save_ms": round(runs[-1]["blocking"] * 1e3, 2),
+                                     "save_s": round(runs[-1]["save"], 4)}
+            for mode, entry in crc_modes.items():
+                # what one save moves through HBM: the pack reads and writes the payload, a checksum pass of its own
+                # reads the image once more, the copies to the host read it once
+                entry["save_hbm_bytes"] = {"pack": int(algorithmic), "checksum_pass": image_bytes if mode == "beside" else 0,
+                                           "transfer_read": image_bytes}
+                entry["save_hbm_bytes"]["total"] = sum(entry["save_hbm_bytes"].values())
+            other.release_device_memory()
+        manager.delete_container(prev)
+
+        # ---- the host link by itself: device <-> the engine's pinned slots, nothing behind them ----
+        link = None
+        if not args.no_link_probe:
+            probe_bytes = min(24 << 30, max(file_bytes, 64 << 20))  # long enough to be past the link's start-up
+            torch.cuda.empty_cache()
+            scratch = torch.zeros(probe_bytes, dtype=torch.uint8, device=device)
+            torch.cuda.synchronize()
+            engine = saver._get_engine()
+            down = min(engine.link_probe(scratch.data_ptr(), probe_bytes, True) for _ in range(3))
+            up = min(engine.link_probe(scratch.data_ptr(), probe_bytes, False) for _ in range(3))
+            del scratch
+            link = {"d2h_peak_GBps": round(probe_bytes / 1e9 / down, 2), "h2d_peak_GBps": round(probe_bytes / 1e9 / up, 2),
+                    "bytes": probe_bytes, "slot_mib": args.slot_mib, "streams": 2,
+                    "what": "pinned hipMemcpyAsync between HBM and the copy engine's own slots, no host-side copy"}
+
         step_s = mean(rec["step"])
         gb = file_bytes / 1e9
-        pack_s = mean(rec["pack_ms"]) * 1e-3
         unpack_s = mean(rec["unpack_ms"]) * 1e-3
-        pack_gbps = 2 * mean(rec["pack_bytes"]) / 1e9 / pack_s if pack_s > 0 else 0.0
+        pack_gbps = algorithmic / 1e9 / pack_s if pack_s > 0 else 0.0
+        save_gbps, restore_gbps = gb / mean(rec["save"]), gb / mean(rec["restore"])
+        if link:
+            link["save_frac"] = round(save_gbps / link["d2h_peak_GBps"], 4)
+            link["restore_frac"] = round(restore_gbps / link["h2d_peak_GBps"], 4)
+        ratio = PACK_TRAFFIC_RATIO.get((args.workload, args.save_crc)) if args.scale >= 1.0 and max_image is None else None
+        ms = lambda key: round(mean(rec[key]) * 1e3, 2)  # noqa: E731
+        restore_known = sum(mean(rec[k]) for k in ("r_parse", "r_table", "h2d", "r_crc", "r_unpack_plan", "r_unpack", "r_commit"))
         result = {
             "metric": "save/restore GB/s + blocking save ms, 8B bf16+fp32-Adam shard, 1 MI355X",
             "value": round(2 * gb / step_s, 3),
@@ -429,28 +518,50 @@ def main():
             "config": {"workload": f"{args.workload}: {label}", "tensors": len(sd), "payload_bytes": payload,
                        "file_bytes": file_bytes, "scale": args.scale, "tile_bytes": args.tile_bytes or 4096,
                        "engine": {"slot_mib": args.slot_mib, "slots": args.slots, "copy_threads": engine_cfg.resolved_copy_threads()},
-                       "crc_chunk_mib": args.crc_chunk_mib, "save_crc": args.save_crc, "restore_crc": args.restore_crc, "plan_cache": args.plan_cache, "save_io": args.save_io, "restore_io": args.restore_io},
+                       "crc_chunk_mib": args.crc_chunk_mib, "save_crc": args.save_crc, "restore_crc": args.restore_crc,
+                       "plan_cache": args.plan_cache, "save_io": args.save_io, "restore_io": args.restore_io,
+                       "max_image_gb": args.max_image_gb, "pool_prefault": not args.no_prefault},
             **({"partial_restore": partial} if partial else {}),
-            "save_GBps": round(gb / mean(rec["save"]), 3),
-            "restore_GBps": round(gb / mean(rec["restore"]), 3),
+            "save_GBps": round(save_gbps, 3),
+            "restore_GBps": round(restore_gbps, 3),
             "blocking_save_ms": round(mean(rec["blocking"]) * 1e3, 2),
-            "blocking_breakdown_ms": {"dcp_plan": round(mean(rec["plan"]) * 1e3, 2),
-                                      "layout_and_pack_launch": round(mean(rec["pack_launch"]) * 1e3, 2),
+            "blocking_breakdown_ms": {"dcp_plan": ms("plan"), "layout_and_pack_launch": ms("pack_launch"),
                                       "pack_kernel": round(pack_s * 1e3, 3)},
             # host work in the blocking window per tensor: planning + layout + launch, without the kernel itself
             "blocking_host_us_per_tensor": round((mean(rec["blocking"]) - pack_s) * 1e6 / max(len(sd), 1), 2),
+            # after the last byte is in the buffer: results, the .metadata file (pickled on a thread of its own while
+            # the image crosses the link; see MemoryStorageWriter), finalize
+            "save_tail_ms": ms("save_tail"),
+            # the first save and restore of the job (iteration 0), not among the timed steps; the pool's file was
+            # created `pool_age_s` before it and its pages took `pool_prefault_s` to allocate and map in the background
+            "first_save_s": round(first["save"], 3), "first_restore_s": round(first["restore"], 3),
+            "first_blocking_save_ms": round(first["blocking"] * 1e3, 2),
+            "pool_prefault_s": round(pool_prefault_s, 3), "pool_age_at_first_save_s": round(pool_age_s, 2),
+            "restore_breakdown_ms": {
+                "dcp_plan_and_metadata": round((mean(rec["restore"]) - mean(rec["r_read"])) * 1e3, 2),
+                "parse_headers_resolve_targets": ms("r_parse"), "descriptor_table": ms("r_table"), "h2d": ms("h2d"),
+                "checksum_pass": ms("r_crc"), "unpack_plan": ms("r_unpack_plan"),
+                "unpack_and_sync": ms("r_unpack"), "commit": ms("r_commit"),
+                "other_in_read_data": round((mean(rec["r_read"]) - restore_known) * 1e3, 2)},
             "pack_GBps": round(pack_gbps, 1),
             "unpack_GBps": round(2 * mean(rec["unpack_bytes"]) / 1e9 / unpack_s, 1) if unpack_s > 0 else None,
             "d2h_GBps": round(mean(rec["d2h_bytes"]) / 1e9 / mean(rec["d2h"]), 2) if mean(rec["d2h"]) > 0 else None,
             **({"host_copy_GBps": round(mean(rec["host_copy_bytes"]) / 1e9 / mean(rec["host_copy_s"]), 2),
                 "host_copy_bytes": int(mean(rec["host_copy_bytes"]))} if mean(rec["host_copy_s"]) > 0 else {}),
             "h2d_GBps": round(mean(rec["h2d_bytes"]) / 1e9 / mean(rec["h2d"]), 2) if mean(rec["h2d"]) > 0 else None,
+            **({"save_windows": int(mean(rec["windows"])), "save_image_pieces": int(mean(rec["image_pieces"]))}
+               if mean(rec["windows"]) or mean(rec["image_pieces"]) else {}),
+            **({"link_roofline": link} if link else {}),
+            **({"crc_modes": crc_modes} if crc_modes else {}),
             "parity": "restored tensors bit-identical to originals (fingerprints)",
-            "roofline": {"bound": "hbm", "kernel": "mlf_flat_kernel<pack>", "achieved": round(pack_gbps, 1),
+            "roofline": {"bound": "hbm",
+                         "kernel": "mlf_fused_crc_kernel<pack> (copy + CRC-32C)" if args.save_crc == "fused" else "mlf_flat_kernel<pack>",
+                         "achieved": round(pack_gbps, 1),
                          "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(pack_gbps / HBM_PEAK_GBPS, 4),
-                         "traffic": (int(PACK_TRAFFIC_RATIO_LLAMA3_8B * 2 * mean(rec["pack_bytes"]))
-                                     if args.workload == "llama3-8b-shard" and args.scale >= 1.0 else None),
-                         "algorithmic_bytes_per_launch": int(2 * mean(rec["pack_bytes"])),
+                         "traffic": int(ratio * algorithmic) if ratio else None,
+                         "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this workload at this scale (profiles/), "
+                                           "applied to this run's byte count" if ratio else None,
+                         "algorithmic_bytes_per_launch": int(algorithmic),
                          "avg_launch_ms": round(pack_s * 1e3, 3)},
         }
         if args.cpu_baseline_gb > 0:

@@ -221,6 +221,13 @@ int mlf_engine_d2h_gated(mlf_engine* engine, const void* src_dev, void* dst_host
 int mlf_engine_h2d(mlf_engine* engine, const void* src_host, void* dst_dev, uint64_t nbytes,
                    void* consumer_stream, mlf_xfer_stats* stats);
 
+/* Measurement aid: moves `nbytes` between `dev_buf` and the engine's own pinned slots over its two copy streams -
+ * device to slots (`to_host` != 0) or slots to device - with no host-side copy behind it, and reports the wall time.
+ * That is the rate the host link gives this engine's transfers at best; what mlf_engine_d2h / mlf_engine_h2d reach is
+ * to be read against it.  The slots' contents are left as they are (to the device go whatever bytes they hold).  No
+ * reference counterpart. */
+int mlf_engine_link_probe(mlf_engine* engine, void* dev_buf, uint64_t nbytes, int to_host, double* seconds);
+
 /* Host -> host on the engine's threads: `nbytes` from `src_host` to `dst_host` (ranges must not overlap).  For
  * checkpoint items that are resident in host memory - the reference copies those into the mapping with torch's
  * intra-op threads (checkpoint_saver.py:443-450,797-800); they do not visit the device here either. */

@@ -126,6 +126,24 @@ PyObject* bo_reserve(PyObject* self_, PyObject* args, PyObject* kwargs) {
   Py_RETURN_NONE;
 }
 
+PyObject* bo_prefault(PyObject* self_, PyObject* args, PyObject* kwargs) {
+  auto* self = reinterpret_cast<PyBufferObject*>(self_);
+  static const char* kwlist[] = {"offset", "nbytes", "threads", nullptr};
+  PyObject *off_obj = nullptr, *len_obj = nullptr;
+  int threads = 4;
+  if (!PyArg_ParseTupleAndKeywords(args, kwargs, "OO|i", const_cast<char**>(kwlist), &off_obj, &len_obj, &threads)) return nullptr;
+  size_t off = PyLong_AsSize_t(off_obj);
+  if (off == (size_t)-1 && PyErr_Occurred()) return nullptr;
+  size_t len = PyLong_AsSize_t(len_obj);
+  if (len == (size_t)-1 && PyErr_Occurred()) return nullptr;
+  int rc;
+  Py_BEGIN_ALLOW_THREADS
+  rc = mlf_buffer_prefault(self->handle, off, len, threads);
+  Py_END_ALLOW_THREADS
+  if (rc != MLF_OK) return raise_last();
+  Py_RETURN_NONE;
+}
+
 PyObject* bo_get_id(PyObject* self_, PyObject*) {
   auto* self = reinterpret_cast<PyBufferObject*>(self_);
   return PyUnicode_FromString(mlf_buffer_id(self->handle));
@@ -189,6 +207,8 @@ PyMethodDef bo_methods[] = {
     {"resize", (PyCFunction)(void (*)(void))bo_resize, METH_VARARGS | METH_KEYWORDS, "Resizes the buffer object."},
     {"reserve", (PyCFunction)(void (*)(void))bo_reserve, METH_VARARGS | METH_KEYWORDS,
      "Allocates the pages of a byte range of the file now instead of at first touch."},
+    {"prefault", (PyCFunction)(void (*)(void))bo_prefault, METH_VARARGS | METH_KEYWORDS,
+     "Allocates the pages of a byte range and maps them writable, so that the first stores take no page fault."},
     {"get_id", bo_get_id, METH_NOARGS, "Gets the buffer object id."},
     {"get_capacity", bo_get_capacity, METH_NOARGS, "Gets the buffer object capacity."},
     {"get_data_ptr", bo_get_data_ptr, METH_NOARGS, "Returns the raw memory address of the buffer as an integer."},

@@ -20,9 +20,14 @@
 #include <unistd.h>
 
 #include <algorithm>
+#include <atomic>
 #include <string>
 #include <thread>
 #include <vector>
+
+#ifndef MADV_POPULATE_WRITE
+#define MADV_POPULATE_WRITE 23  // Linux 5.14; older kernels answer EINVAL and the per-page store below takes over
+#endif
 
 struct mlf_buffer {
   std::string id;
@@ -259,6 +264,40 @@ int mlf_buffer_reserve(mlf_buffer* b, size_t offset, size_t nbytes) {
     return fail(MLF_INTERNAL, "not enough space on the file system that holds " + b->id + " for " +
                                   std::to_string(nbytes) + " more bytes");
   return fail_errno("fallocate() failed for file: " + b->id, e);
+}
+
+int mlf_buffer_prefault(mlf_buffer* b, size_t offset, size_t nbytes, int threads) {
+  if (int rc = mlf_buffer_reserve(b, offset, nbytes)) return rc;
+  if (nbytes == 0) return MLF_OK;
+  // page-table entries for the whole range, writable, so that the first stores into it take no fault at all
+  const size_t page = 4096;
+  char* base = static_cast<char*>(b->ptr);
+  const size_t begin = offset / page * page, end = std::min(b->cap, (offset + nbytes + page - 1) / page * page);
+  const size_t want = std::max<size_t>(1, std::min<size_t>((size_t)std::max(threads, 1), (end - begin) / ((size_t)64 << 20) + 1));
+  size_t per = ((end - begin + want - 1) / want + page - 1) / page * page;
+  std::atomic<int> err{0};
+  auto run = [&](size_t lo, size_t hi) {
+    const size_t step = (size_t)256 << 20;  // bounded calls: a signal or an error shows up between them
+    for (size_t at = lo; at < hi && !err.load(); at += step) {
+      const size_t len = std::min(step, hi - at);
+#ifdef MADV_POPULATE_WRITE
+      if (madvise(base + at, len, MADV_POPULATE_WRITE) == 0) continue;
+      if (errno != EINVAL && errno != ENOSYS) {
+        err.store(errno);
+        return;
+      }
+#endif
+      // a kernel without MADV_POPULATE_WRITE: a store that changes nothing, one per page
+      for (size_t p = at; p < at + len; p += page)
+        __atomic_fetch_or(reinterpret_cast<unsigned char*>(base + p), (unsigned char)0, __ATOMIC_RELAXED);
+    }
+  };
+  std::vector<std::thread> pool;
+  for (size_t lo = begin + per; lo < end; lo += per) pool.emplace_back(run, lo, std::min(end, lo + per));
+  run(begin, std::min(end, begin + per));
+  for (auto& t : pool) t.join();
+  if (int e = err.load()) return fail_errno("madvise(MADV_POPULATE_WRITE) failed for file: " + b->id, e);
+  return MLF_OK;
 }
 
 void* mlf_buffer_data_ptr(const mlf_buffer* b) { return is_open(b) ? b->ptr : nullptr; }

@@ -417,6 +417,30 @@ int mlf_engine_d2h_gated(mlf_engine* e, const void* src_dev, void* dst_host, uin
   return engine_d2h(e, src_dev, host, nbytes, gate, stats, crc);
 }
 
+int mlf_engine_link_probe(mlf_engine* e, void* dev_buf, uint64_t nbytes, int to_host, double* seconds) {
+  if (!e || !dev_buf || !seconds) return fail(MLF_HIP_BAD_ARG, "null argument");
+  if (nbytes == 0) return fail(MLF_HIP_BAD_ARG, "nothing to copy");
+  std::lock_guard<std::mutex> g(e->busy);
+  HIP_TRY(hipSetDevice(e->device));
+  char* dev = static_cast<char*>(dev_buf);
+  const uint64_t slot = e->slot_bytes, n_chunks = (nbytes + slot - 1) / slot, n_slots = e->slots.size();
+  DrainOnExit drain{e};
+  HIP_TRY(hipDeviceSynchronize());
+  const double t0 = now_s();
+  for (uint64_t c = 0; c < n_chunks; ++c) {
+    const uint64_t off = c * slot, len = std::min(slot, nbytes - off), s = c % n_slots;
+    if (c >= n_slots) HIP_TRY(hipEventSynchronize(e->slot_done[s]));  // the slot's previous copy has finished
+    hipStream_t st = e->streams[c & 1];
+    if (to_host) HIP_TRY(hipMemcpyAsync(e->slots[s], dev + off, len, hipMemcpyDeviceToHost, st));
+    else HIP_TRY(hipMemcpyAsync(dev + off, e->slots[s], len, hipMemcpyHostToDevice, st));
+    HIP_TRY(hipEventRecord(e->slot_done[s], st));
+  }
+  for (hipStream_t s : e->streams) HIP_TRY(hipStreamSynchronize(s));
+  drain.armed = false;
+  *seconds = now_s() - t0;
+  return MLF_HIP_OK;
+}
+
 int mlf_engine_host_copy(mlf_engine* e, void* dst_host, const void* src_host, uint64_t nbytes) {
   if (!e) return fail(MLF_HIP_BAD_ARG, "null engine");
   if (nbytes && (!dst_host || !src_host)) return fail(MLF_HIP_BAD_ARG, "null pointer");

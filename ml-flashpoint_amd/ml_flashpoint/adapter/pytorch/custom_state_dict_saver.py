@@ -65,6 +65,11 @@ def generate_plan(
             local_plan = storage_writer.prepare_local_plan(planner.create_local_plan())
             central_plan, global_metadata = _agree_on_plan(local_plan, storage_writer, planner, world_dist_wrapper)
         buckets = storage_writer.prepare_write_data_buckets(checkpoint_id, planner.finish_plan(central_plan), planner)
+        expect = getattr(storage_writer, "expect_metadata", None)
+        if expect is not None:
+            # one process on its own: the metadata object that finish_write will be given is known now, and the
+            # writer may pickle it while the data is on its way (with several ranks it depends on everyone's results)
+            expect(global_metadata if not world_dist_wrapper.use_dist else None)
         return buckets, global_metadata, central_plan, local_plan, cache.central_plan == central_plan
 
 

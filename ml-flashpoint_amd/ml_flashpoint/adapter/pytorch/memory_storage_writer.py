@@ -19,6 +19,8 @@ import concurrent.futures
 import dataclasses
 import logging
 import os
+import pickle
+import threading
 import time
 
 import torch
@@ -99,6 +101,35 @@ class _WriteLedger:
         return self.events[checkpoint_id].wait(timeout=timeout_s)
 
 
+class _EarlyMetadata:
+    """The checkpoint's metadata object pickled while its data is still on the way to the buffer.
+
+    Where every item ends up is decided when the object is laid out, long before the last byte is written, so when
+    one process plans, writes and finishes a save (no other rank's results to wait for) the metadata object - whose
+    pickling takes 150 ms for 20 000 tensors - need not wait for the write.  ``finish_checkpoint`` uses the bytes
+    only if they describe exactly what the write then reported; otherwise it pickles again, as without this."""
+
+    def __init__(self, checkpoint_id, metadata: Metadata, where: dict, storage_meta):
+        self.checkpoint_id, self.metadata, self.where, self.storage_meta = checkpoint_id, metadata, where, storage_meta
+        self.payload: bytes | None = None
+        self._thread = threading.Thread(target=self._run, name="mlf-early-metadata", daemon=True)
+        self._thread.start()
+
+    def _run(self):
+        try:
+            with utils.gc_paused():
+                filled = dataclasses.replace(self.metadata, storage_data=self.where, storage_meta=self.storage_meta)
+                self.payload = pickle.dumps(filled)
+        except Exception:  # the ordinary path takes over
+            _LOGGER.warning("could not pickle the metadata object ahead of time", exc_info=True)
+
+    def result_for(self, checkpoint_id, metadata: Metadata, where: dict, storage_meta) -> bytes | None:
+        self._thread.join()
+        same = (self.payload is not None and checkpoint_id == self.checkpoint_id and metadata is self.metadata
+                and storage_meta == self.storage_meta and where == self.where)
+        return self.payload if same else None
+
+
 class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
     def __init__(
         self,
@@ -118,6 +149,8 @@ class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
         self._ledger = _WriteLedger()
         self._current_checkpoint_id: CheckpointContainerId | None = None
         self._current_save_id: str | None = None
+        self._expected_metadata: Metadata | None = None  # see expect_metadata
+        self._early_metadata: _EarlyMetadata | None = None
 
     # the ledger's two dicts under the names other code (and the reference's tests) know them by
     @property
@@ -137,10 +170,19 @@ class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
         self._ledger.results = value
 
     def __getstate__(self):
-        return {k: v for k, v in self.__dict__.items() if k != "_main_process_torchmp_manager_future"}
+        left_behind = ("_main_process_torchmp_manager_future", "_expected_metadata", "_early_metadata")
+        return {k: v for k, v in self.__dict__.items() if k not in left_behind}
 
     def __setstate__(self, state):
-        self.__dict__.update(state, _main_process_torchmp_manager_future=None)
+        self.__dict__.update(state, _main_process_torchmp_manager_future=None, _expected_metadata=None,
+                             _early_metadata=None)
+
+    def expect_metadata(self, metadata: Metadata | None) -> None:
+        """Tells the writer which metadata object ``finish_checkpoint`` is going to be called with, for a save that
+        this one process plans, writes and finishes alone: the writer may then pickle it while the data is still
+        being written (see ``_EarlyMetadata``).  Optional; without it, or in a process that received the writer by
+        pickling, nothing changes."""
+        self._expected_metadata = metadata
 
     # ---- identity of the save in progress ------------------------------------------------------------------------
     def _require_reset(self) -> CheckpointContainerId:
@@ -267,6 +309,7 @@ class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
         """Synchronous write of prepared buckets; publishes the results for ``get_write_results`` (in whichever
         process that is called) and also returns them in a completed future.  A failing write publishes nothing."""
         began = time.perf_counter()
+        self._start_early_metadata(checkpoint_id, staged_write_buckets)
         outcome = self._checkpoint_saver.write_data(
             checkpoint_id,
             write_buckets=staged_write_buckets,
@@ -279,6 +322,20 @@ class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
         done: TorchFuture = TorchFuture()
         done.set_result(outcome)
         return done
+
+    def _start_early_metadata(self, checkpoint_id, buckets) -> None:
+        self._early_metadata = None
+        metadata, predict = self._expected_metadata, getattr(self._checkpoint_saver, "predict_write_results", None)
+        if metadata is None or predict is None or self._current_checkpoint_id != checkpoint_id:
+            return
+        try:
+            predicted = predict(buckets)
+        except Exception:
+            _LOGGER.warning("could not predict the write results", exc_info=True)
+            return
+        if predicted is not None:
+            where = {result.index: result.storage_data for result in predicted}
+            self._early_metadata = _EarlyMetadata(checkpoint_id, metadata, where, self.storage_meta())
 
     @_timed(logger=_LOGGER, name="get_write_results")
     def get_write_results(
@@ -317,6 +374,12 @@ class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
                 raise RuntimeError(complaint)
             where.update((result.index, result.storage_data) for result in rank_results)  # a repeated index: last wins
         metadata.storage_data, metadata.storage_meta = where, self.storage_meta()
-        self._checkpoint_saver.write_metadata(checkpoint_id, metadata)
+        early, self._early_metadata = self._early_metadata, None
+        ready = early.result_for(checkpoint_id, metadata, where, metadata.storage_meta) if early is not None else None
+        write_bytes = getattr(self._checkpoint_saver, "write_metadata_bytes", None)
+        if ready is not None and write_bytes is not None:
+            write_bytes(checkpoint_id, ready)  # pickled while the data was being written: same bytes, no wait
+        else:
+            self._checkpoint_saver.write_metadata(checkpoint_id, metadata)
         if self._ledger.results is not None:
             self._ledger.results.pop(checkpoint_id, None)

@@ -46,9 +46,21 @@ class CheckpointObjectManager:
                     wanted = self._pool_config
                     owner._worker_pool = BufferPool(pool_dir_path=wanted.pool_dir_path, rank=wanted.rank,
                                                     num_buffers=wanted.num_buffers, buffer_size=wanted.buffer_size)
+                    if getattr(wanted, "prefault", True):
+                        owner._worker_pool.start_prefault()
                 except Exception:
                     _LOGGER.exception("Failed to initialize BufferPool")
             return owner._worker_pool
+
+    def warm_up_pool(self, wait: bool = False) -> float:
+        """Creates this process's pool now instead of at the first ``acquire_buffer``, so that the background
+        allocation of its files' pages (``BufferPoolConfig.prefault``) runs while the job is still starting up.
+        ``wait``: return only when that has finished.  Returns the seconds the allocation has taken so far (0.0
+        without a pool, or while it is still running and ``wait`` is false)."""
+        pool = self._get_or_create_buffer_pool()
+        if pool is None:
+            return 0.0
+        return pool.wait_prefault() if wait else pool.prefault_seconds
 
     def teardown_pool(self):
         owner = CheckpointObjectManager

@@ -102,6 +102,7 @@ _SIGNATURES = {
     "mlf_engine_d2h_crc": (_INT, [_VP, _VP, _VP, _U64, _VP, _U64, _VP, _U64, ctypes.POINTER(XferStats)]),
     "mlf_engine_d2h_watched": (_INT, [_VP, _VP, _VP, _U64, _VP, _U64, _VP, _U64, _VP, ctypes.POINTER(XferStats)]),
     "mlf_engine_d2h_gated": (_INT, [_VP, _VP, _VP, _U64, _VP, _U64, _VP, _U64, _VP, ctypes.POINTER(XferStats)]),
+    "mlf_engine_link_probe": (_INT, [_VP, _VP, _U64, _INT, ctypes.POINTER(ctypes.c_double)]),
     "mlf_engine_host_copy": (_INT, [_VP, _VP, _VP, _U64]),
     "mlf_engine_d2h_fd": (_INT, [_VP, _VP, _INT, _U64, _U64, _VP, ctypes.POINTER(XferStats)]),
     "mlf_engine_h2d_fd": (_INT, [_VP, _INT, _U64, _VP, _U64, _VP, ctypes.POINTER(XferStats)]),

@@ -120,11 +120,19 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         self._max_image_bytes = max_image_bytes
         self._engine: Optional[hip_plan.CopyEngine] = None
         self._engine_lock = threading.Lock()
+        self._stats_local = threading.local()  # read_data runs on one executor thread per object
         self._init_discovery()
         self.last_load_stats: dict = {}
         # set to True to bracket every unpack launch with timing events; see the saver's attribute of the same name
         self.record_kernel_events = False
         self.kernel_events: list = []
+
+    @property
+    def _stats_in_progress(self) -> dict:
+        stats = getattr(self._stats_local, "current", None)
+        if stats is None:
+            stats = self._stats_local.current = {}
+        return stats
 
     def _get_engine(self) -> hip_plan.CopyEngine:
         with self._engine_lock:  # read_data runs on one executor thread per object
@@ -220,6 +228,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
             raise FileNotFoundError(msg)
         t_start = time.perf_counter()
         stats = {"h2d_s": 0.0, "h2d_bytes": 0, "device_payload_bytes": 0, "host_items": 0, "device_items": 0}
+        self._stats_local.current = stats
         with gc_paused(), self._checkpoint_object_manager.get_buffer(checkpoint_object_id) as stream:
             recorded, held = stream.len_written_data, stream.buffer_obj.get_capacity() - METADATA_SIZE
             if recorded > held:  # cut short after it was written: never read past the end of the file or its mapping
@@ -228,6 +237,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
             optimized = stream.format_signature == CheckpointFormat.MLF_FORMAT
             device_reqs = []  # (req, target, dtype, shape, payload_off, stored payload bytes)
             whole = stream.raw_view()
+            t_parse = time.perf_counter()
             for req in read_items:
                 item_md = storage_data[req.storage_index]
                 if req.type == LoadItemType.BYTE_IO:
@@ -262,6 +272,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                     stats["host_items"] += 1
                     continue
                 device_reqs.append((req, target) + parsed)
+            stats["parse_s"] = time.perf_counter() - t_parse  # headers parsed, targets resolved, host items served
             if device_reqs:
                 self._read_device_items(checkpoint_object_id, stream, device_reqs, planner, stats)
         stats["read_s"] = time.perf_counter() - t_start
@@ -291,6 +302,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         # and how to add it to a descriptor table once the offset of the uploaded range is known.  A request for a
         # whole stored tensor into a contiguous target (the common case) is one run of bytes; anything else is a box
         # over the stored C-contiguous payload (offsets/strides) with the target's strides on the other side.
+        t_rows = time.perf_counter()
         rows = []  # (first, last, contiguous?, table arguments)
         conversions = []  # (target, buffer of the stored dtype): the reference's `copy_` converts, so this does too
         for req, target, dtype, shape, payload_off, stored_bytes in device_reqs:
@@ -337,6 +349,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                              (target.data_ptr(), esz, tuple(lengths), tuple(target.stride()), tuple(stored_strides))))
                 stored_bytes = numel * esz
             stats["device_payload_bytes"] += stored_bytes
+        stats["table_s"] = time.perf_counter() - t_rows
         if rows:
             lo = min(r[0] for r in rows)
             hi = max(r[1] for r in rows)
@@ -375,8 +388,10 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                 del image
                 for target, stored_as in conversions:
                     target.copy_(stored_as)
+        t_commit = time.perf_counter()
         for req, target, *_ in device_reqs:
             planner.commit_tensor(req, target)
+        stats["commit_s"] = time.perf_counter() - t_commit
         stats["device_items"] += len(device_reqs)
 
     @staticmethod
@@ -405,8 +420,12 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         """Launches the unpack of ``items`` out of ``image`` and waits for it: the targets are complete, and the
         image may be reused or freed, when this returns.  With ``crc_chunk_bytes`` the unpack kernel also folds the
         CRC-32C of every chunk of the image; those values are returned."""
+        t0 = time.perf_counter()
         plan = hip_plan.Plan(items, b"", span, tile_bytes=self._tile_bytes, block_threads=self._block_threads,
                              align_to_tensor=True, crc_chunk_bytes=crc_chunk_bytes)
+        stats = self._stats_in_progress
+        stats["unpack_plan_s"] = stats.get("unpack_plan_s", 0.0) + time.perf_counter() - t0
+        t0 = time.perf_counter()
         try:
             if self.record_kernel_events:
                 begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -417,6 +436,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
             else:
                 plan.unpack(image, cur.cuda_stream)
             cur.synchronize()
+            stats["unpack_s"] = stats.get("unpack_s", 0.0) + time.perf_counter() - t0
             return plan.crc_values() if crc_chunk_bytes else None
         finally:
             plan.destroy()
@@ -432,7 +452,9 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                 got = self._unpack(self._table_of(rows, lo), image, span, cur, stats["device_payload_bytes"], chunk_bytes)
                 self._compare_checksums(object_id, got, want, chunk_bytes)
                 return
+            t0 = time.perf_counter()
             got = hip_plan.crc32c_device(image, data_bytes, chunk_bytes, cur.cuda_stream)
+            stats["crc_s"] = stats.get("crc_s", 0.0) + time.perf_counter() - t0
             self._compare_checksums(object_id, got, want, chunk_bytes)
         self._unpack(self._table_of(rows, lo), image, span, cur, stats["device_payload_bytes"])
 

@@ -944,6 +944,31 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             pickle.dump(metadata, f)
         os.rename(tmp_path, final_path)
 
+    def write_metadata_bytes(self, checkpoint_id: CheckpointContainerId, pickled: bytes,
+                             md_object_name: str = default_metadata_object_name()) -> None:
+        """``write_metadata`` for a metadata object that has been pickled already (same temporary name, same
+        rename)."""
+        final_path = os.path.join(checkpoint_id.data, md_object_name)
+        tmp_path = final_path + ".tmp"
+        os.makedirs(os.path.dirname(final_path), exist_ok=True)
+        with open(tmp_path, "wb") as f:
+            f.write(pickled)
+        os.rename(tmp_path, final_path)
+
+    def predict_write_results(self, write_buckets: list[ObjectWriteBucket]) -> Optional[list[WriteResult]]:
+        """What ``write_data`` is going to return for buckets this saver prepared in this process - offsets and
+        lengths are fixed when an object is laid out - or None if any bucket is not of that kind."""
+        results: list[WriteResult] = []
+        for bucket in write_buckets:
+            refs = [t for _, t in bucket.tensor_data]
+            if not refs or not all(isinstance(r, StagedTensorRef) for r in refs):
+                return None
+            staged = refs[0].staged
+            if not isinstance(staged, StagedObject) or any(r.staged is not staged for r in refs):
+                return None
+            results.extend(self._results_of(staged, bucket.object_name))
+        return results
+
     @override
     @log_execution_time(logger=_LOGGER, name="finalize_checkpoint")
     def finalize_checkpoint(self, checkpoint_id: CheckpointContainerId) -> Union[subprocess.Popen, None]:

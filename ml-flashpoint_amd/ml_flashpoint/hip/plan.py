@@ -414,6 +414,14 @@ class CopyEngine:
         )
         return stats, (crcs[:n_chunks] if crc_chunk_bytes else None)
 
+    def link_probe(self, dev_ptr: int, nbytes: int, to_host: bool) -> float:
+        """Seconds to move ``nbytes`` between device memory and the engine's pinned slots with nothing behind them:
+        the host link's own rate for this engine's slot size and streams."""
+        seconds = ctypes.c_double(0.0)
+        _lib.check(_lib.load().mlf_engine_link_probe(self._handle, dev_ptr, nbytes, 1 if to_host else 0,
+                                                     ctypes.byref(seconds)), "mlf_engine_link_probe")
+        return seconds.value
+
     def host_copy(self, dst_host_ptr: int, src_host_ptr: int, nbytes: int) -> None:
         """Host memory to host memory on the engine's threads (checkpoint items that are resident on the host)."""
         _lib.check(_lib.load().mlf_engine_host_copy(self._handle, dst_host_ptr, src_host_ptr, nbytes), "mlf_engine_host_copy")

@@ -364,3 +364,44 @@ def test_reserve_allocates_the_pages_of_a_range_ahead_of_the_writer(shm_dir):
     with pytest.raises(RuntimeError, match="read-only"):
         ro.buffer_obj.reserve(0, 10)
     ro.close()
+
+
+def test_pool_prefaults_its_files_in_the_background(shm_dir):
+    """A pool of files large enough to be worth it allocates and maps their pages on a background thread; a buffer
+    is lent out only once its own file is done, holds what is written into it, and shrinks to the exact size."""
+    import os
+
+    from ml_flashpoint.checkpoint_object_manager.buffer_metadata import METADATA_SIZE
+    from ml_flashpoint.checkpoint_object_manager.checkpoint_object_manager import CheckpointObjectManager
+    from ml_flashpoint.core.buffer_pool import BufferPool, BufferPoolConfig
+    from ml_flashpoint.core.checkpoint_id_types import CheckpointObjectId
+
+    size = 96 << 20
+    pool = BufferPool(os.path.join(shm_dir, "pool"), rank=3, num_buffers=2, buffer_size=size, prefault=True)
+    assert pool._prefault_worker is not None
+    stream = pool.acquire(os.path.join(shm_dir, "object.distcp"))  # waits for the file it gets
+    path = stream.buffer_obj.get_id()
+    assert os.stat(path).st_blocks * 512 >= size, "the file's pages were not allocated ahead of the writer"
+    payload = bytes(range(256)) * 4096
+    stream.write(payload)
+    stream.close()
+    assert os.path.getsize(path) == METADATA_SIZE + len(payload)
+    assert open(os.path.join(shm_dir, "object.distcp"), "rb").read()[METADATA_SIZE:] == payload
+    assert pool.wait_prefault() > 0.0
+    other = [p for p in os.listdir(os.path.join(shm_dir, "pool")) if not path.endswith(p)]
+    assert len(other) == 1 and os.stat(os.path.join(shm_dir, "pool", other[0])).st_blocks * 512 >= size
+    pool.teardown()
+    # small files, or prefault=False: no thread, pages left to the first write as in the reference
+    assert BufferPool(os.path.join(shm_dir, "small"), num_buffers=1, buffer_size=1 << 20, prefault=True)._prefault_worker is None
+    lazy = BufferPool(os.path.join(shm_dir, "lazy"), num_buffers=1, buffer_size=size)
+    assert lazy._prefault_worker is None and os.stat(lazy.free_buffers[0].buffer_obj.get_id()).st_blocks * 512 < size
+    lazy.teardown()
+    # through the manager: the pool can be created, and waited for, before the first save
+    CheckpointObjectManager._worker_pool = None
+    manager = CheckpointObjectManager(BufferPoolConfig(os.path.join(shm_dir, "managed"), 0, 1, size))
+    assert manager.warm_up_pool(wait=True) > 0.0
+    with manager.acquire_buffer(CheckpointObjectId(os.path.join(shm_dir, "ckpt", "a.distcp")), 1 << 20) as writer:
+        writer.write(b"abc")
+    assert open(os.path.join(shm_dir, "ckpt", "a.distcp"), "rb").read()[METADATA_SIZE:] == b"abc"
+    manager.teardown_pool()
+    assert CheckpointObjectManager(None).warm_up_pool() == 0.0

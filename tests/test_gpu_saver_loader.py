@@ -221,6 +221,54 @@ def test_megatron_style_sequence_with_pool_and_finalize(shm_dir, manager_future)
     assert _loader().get_latest_complete_checkpoint(CheckpointContainerId(os.path.join(shm_dir, "run"))).data.endswith("step-20_ckpt")
 
 
+def test_metadata_object_is_pickled_while_the_data_is_written(shm_dir, manager_future, monkeypatch):
+    """A save that one process plans, writes and finishes: the metadata object is pickled on a thread while the image
+    crosses the link, and ``finish_write`` only writes those bytes - the same file as the ordinary way produces.  If
+    what the write reported differs from what was predicted, or another metadata object arrives, the ordinary way
+    is taken."""
+    from torch.distributed.checkpoint import DefaultSavePlanner
+    from torch.distributed.checkpoint.utils import _DistWrapper
+
+    from ml_flashpoint.adapter.pytorch import custom_state_dict_saver as three_calls
+
+    sd_dev = {k: v for k, v in _to_dev(_mixed_state_dict()).items()}
+    saver = _saver()
+    dist = _DistWrapper(None, False, 0)
+    calls = []
+    real_bytes, real_object = saver.write_metadata_bytes, saver.write_metadata
+    monkeypatch.setattr(saver, "write_metadata_bytes", lambda *a, **k: (calls.append("bytes"), real_bytes(*a, **k))[1])
+    monkeypatch.setattr(saver, "write_metadata", lambda *a, **k: (calls.append("object"), real_object(*a, **k))[1])
+
+    def save(step, tamper=None):
+        cid = CheckpointContainerId(os.path.join(shm_dir, f"step-{step}_ckpt"))
+        writer = MemoryStorageWriter(saver, manager_future)
+        writer.reset(cid.data)
+        buckets, metadata, *_ = three_calls.generate_plan(cid, sd_dev, writer, DefaultSavePlanner(), dist)
+        staged = MemoryStorageWriter.stage_write_data_buckets(cid, buckets)
+        three_calls.write_data(cid, writer, staged, replicate_after_write=False)
+        if tamper == "other-object":
+            metadata = pickle.loads(pickle.dumps(metadata))
+        three_calls.finish_write(cid, writer, metadata, dist)
+        return cid, writer
+
+    cid, writer = save(1)
+    assert calls == ["bytes"]
+    early = pickle.load(open(os.path.join(cid.data, ".metadata"), "rb"))
+    assert early.storage_meta.checkpoint_id == cid.data and early.storage_meta.save_id == writer._current_save_id
+    cid2, _ = save(2, tamper="other-object")
+    assert calls == ["bytes", "object"]
+    late = pickle.load(open(os.path.join(cid2.data, ".metadata"), "rb"))
+    assert early.state_dict_metadata == late.state_dict_metadata and early.storage_data == late.storage_data
+    assert early.planner_data == late.planner_data
+    # the object the early bytes describe is the one that was written: it loads
+    target = {k: (torch.zeros_like(v) if isinstance(v, torch.Tensor) and v.dtype != torch.float8_e4m3fn else
+                  (torch.zeros(v.shape, dtype=torch.uint8, device=v.device).view(v.dtype) if isinstance(v, torch.Tensor) else None))
+              for k, v in sd_dev.items()}
+    dcp.load(target, checkpoint_id=cid.data, storage_reader=MemoryStorageReader(cid.data, _loader()), no_dist=True)
+    assert all(torch.equal(_bits(target[k]), _bits(v)) for k, v in sd_dev.items() if isinstance(v, torch.Tensor))
+    assert target["obj.step"] == 123
+
+
 def test_crc_sidecar_written_and_corruption_detected(shm_dir, manager_future):
     from ml_flashpoint.hip import integrity
 
