@@ -642,7 +642,8 @@ constexpr uint32_t kCellsPerEntryLog2 = 4;
 
 template <bool PACK>
 __global__ void __launch_bounds__(256) mlf_fused_crc_kernel(const uint64_t* __restrict__ ent, char* __restrict__ image,
-                                                            uint32_t G, const uint32_t* __restrict__ row_tab,
+                                                            uint32_t G, uint32_t xcd_sets,
+                                                            const uint32_t* __restrict__ row_tab,
                                                             const u32x4* __restrict__ lane_w,
                                                             uint32_t* __restrict__ fast_val, char* __restrict__ sink) {
   // kFusedTabCopies copies of the table, entry v of copy c at word v * copies + c, lane l reads copy l % copies:
@@ -650,13 +651,21 @@ __global__ void __launch_bounds__(256) mlf_fused_crc_kernel(const uint64_t* __re
   __shared__ uint32_t tab[1024 * kFusedTabCopies];
   __shared__ uint32_t part[4];
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
-  const uint32_t group = blockIdx.x / G;
+  uint32_t group = blockIdx.x / G;
   uint32_t w = blockIdx.x - group * G;
+  // Workgroups reach the eight XCDs round-robin, and a source line that straddles a cell cut should be served by one
+  // L2, not fetched from HBM by two: neighbouring cells go to the same XCD.
   if ((G & 511u) == 0) {
-    // workgroups reach the eight XCDs round-robin: within every 512 of them XCD x takes 64 consecutive cells of a
-    // row, so that a source line that straddles a cell cut is served by one L2
+    // within every 512 workgroups XCD x takes 64 consecutive cells of a row
     const uint32_t lo = w & 511u;
     w = (w & ~511u) + (lo & 7u) * 64u + (lo >> 3);
+  } else if (blockIdx.x < xcd_sets * 8u * G) {
+    // smaller groups: of every eight consecutive groups XCD x takes group x whole (measured on the 112 GB shard with
+    // groups of 64: fetched bytes 1.047 -> 1.030 x the payload, same time; what is left is one extra 128-byte line
+    // per misaligned cell, fetched again because the neighbour's row passed through that L2 some microseconds earlier)
+    const uint32_t set = blockIdx.x / (8u * G), lo = blockIdx.x - set * 8u * G;
+    group = set * 8u + (lo & 7u);
+    w = lo >> 3;
   }
   const uint64_t cell0 = (uint64_t)group * kFusedRows * G + w;
   uint32_t* out = fast_val + (uint64_t)group * G + w;
@@ -1225,7 +1234,7 @@ int launch_plan(const mlf_plan* plan, char* image, hipStream_t stream) {
     const uint64_t n_wg = f.fused_groups * f.wgs_per_group;
     if (n_wg) {
       hipLaunchKernelGGL((mlf_fused_crc_kernel<PACK>), dim3((uint32_t)n_wg), dim3(256), 0, stream, f.d_ent, image,
-                         f.wgs_per_group, f.d_row_tab, f.d_lane_w, f.d_fast_val, f.d_sink);
+                         f.wgs_per_group, (uint32_t)(f.fused_groups / 8), f.d_row_tab, f.d_lane_w, f.d_fast_val, f.d_sink);
       HIP_TRY(hipGetLastError());
     }
   }
