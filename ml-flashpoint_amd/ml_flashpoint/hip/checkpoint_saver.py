@@ -786,14 +786,46 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             except OSError:
                 pass
         else:
-            results = self._transfer_bucket(staged, bucket, xfer)
+            streaming = getattr(self._replication_manager, "async_replicate_streaming", None) if replicate_after_write else None
+            results = self._transfer_bucket(staged, bucket, xfer, streaming)
+            if streaming is not None:
+                return results  # the replication manager has been following the transfer since it began
         if replicate_after_write and self._replication_manager is not None:
             # without a replication manager (single node, or this package used on its own) there is no peer to
             # send to; an explicit async_replicate_object() call still raises
             self.async_replicate_object(bucket.object_id)
         return results
 
-    def _transfer_bucket(self, staged: StagedObject, bucket: ObjectWriteBucket, xfer: dict) -> list[WriteResult]:
+    def _transfer_bucket(self, staged: StagedObject, bucket: ObjectWriteBucket, xfer: dict,
+                         streaming=None) -> list[WriteResult]:
+        """``streaming``: a replication manager's ``async_replicate_streaming``, called when the transfer begins
+        (see ``_announce_transfer``)."""
+        outcome: Optional[concurrent.futures.Future] = concurrent.futures.Future() if streaming is not None else None
+        try:
+            results = self._transfer_bucket_inner(staged, bucket, xfer, streaming, outcome)
+        except BaseException as e:
+            if outcome is not None and not outcome.done():
+                outcome.set_exception(e)  # whoever follows the transfer learns that it will not complete
+            raise
+        if outcome is not None and not outcome.done():
+            outcome.set_result(True)
+        return results
+
+    def _announce_transfer(self, streaming, bucket: ObjectWriteBucket, staged: StagedObject, start: int, nbytes: int,
+                           outcome: concurrent.futures.Future) -> None:
+        """Hands the object to a replication manager that can forward it while it is still being written, where
+        the reference hands it over after the write (checkpoint_saver.py:700-707 -> replication_manager.py:248-300).
+        The manager is told: the object, the file offset of its data section's first byte (the 4096-byte metadata
+        block in front of it is final at this point), a callable that returns how many leading bytes of the data
+        section are in place - it only grows - their total, and a future that resolves when the transfer has ended
+        (its exception if it failed: the counter then stops short of the total)."""
+        try:
+            streaming(bucket.object_id, METADATA_SIZE + start, staged.landed_bytes, nbytes, outcome=outcome)
+        except Exception:
+            _LOGGER.exception("async_replicate_streaming failed for '%s'; the object is written all the same", bucket.object_id)
+
+    def _transfer_bucket_inner(self, staged: StagedObject, bucket: ObjectWriteBucket, xfer: dict, streaming,
+                               outcome) -> list[WriteResult]:
         layout = staged.layout
         nbytes = layout.data_bytes
         crcs = None
@@ -813,6 +845,9 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                     start = writer.tell()
                     writer.next_buffer_slice(nbytes).release()  # bounds check + position/high-water mark
                     staged.data_offset = start
+                    staged._landed.value = 0
+                    if streaming is not None:
+                        self._announce_transfer(streaming, bucket, staged, start, nbytes, outcome)
                     fd = writer.fileno() if self._use_file_io else -1
                     engine = self._get_engine()
                     if staged.pieces is not None:
@@ -841,6 +876,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                                                     self._crc_chunk_bytes)
                         self._count_transfer(xfer, st, nbytes)
                     staged._landed.value = nbytes
+            elif streaming is not None:  # an object without data: nothing to follow, but it is to be replicated
+                self._announce_transfer(streaming, bucket, staged, 0, 0, outcome)
         staged.consumed = True
         staged.image = None
         if staged.plan is not None and staged.owns_plan:
@@ -991,6 +1028,9 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             path = os.path.join(parent, name)
             if step is not None and step < limit and os.path.isdir(path):
                 doomed.append(path)
+                sidecars = integrity.sidecar_dir(path)  # the checksums of a removed step go with it
+                if os.path.isdir(sidecars):
+                    doomed.append(sidecars)
         if not doomed:
             return None
         try:

@@ -216,3 +216,172 @@ def test_a_follower_can_forward_the_object_while_it_is_still_being_written(shm_d
     with open(path, "rb") as f:
         f.seek(METADATA_SIZE)
         assert f.read() == replica
+
+
+def test_replication_manager_that_follows_the_transfer(shm_dir, manager_future):
+    """A replication manager with ``async_replicate_streaming`` is handed the object when its transfer begins: a
+    follower thread copies the metadata block and then whatever prefix of the data section the counter announces
+    into a second file, and ends with a byte-identical replica - identical, too, to the oracle's image.  A manager
+    without the method gets the reference's call after the write; a transfer that fails tells the follower so."""
+    import concurrent.futures
+    import threading
+
+    from ml_flashpoint.checkpoint_object_manager.buffer_metadata import METADATA_SIZE
+
+    class FollowingManager:
+        def __init__(self, replica_dir):
+            self.replica_dir, self.calls, self.after_write, self.threads, self.errors = replica_dir, [], [], [], []
+
+        def async_replicate(self, buffer_io):
+            self.after_write.append(buffer_io.buffer_obj.get_id())
+            buffer_io.close()
+            return []
+
+        def async_replicate_streaming(self, object_id, data_offset, landed_counter, total, *, outcome):
+            self.calls.append((str(object_id), data_offset, total))
+            done = concurrent.futures.Future()
+            target = os.path.join(self.replica_dir, os.path.basename(str(object_id)))
+
+            def follow():
+                try:
+                    seen, have = [], 0
+                    with open(str(object_id), "rb") as src, open(target, "wb") as dst:
+                        dst.write(os.pread(src.fileno(), data_offset, 0))  # the metadata block is final already
+                        while have < total:
+                            now = landed_counter()
+                            if now > have:
+                                seen.append(now)
+                                dst.write(os.pread(src.fileno(), now - have, data_offset + have))
+                                have = now
+                            elif outcome.done():
+                                outcome.result()  # raises if the transfer failed
+                                if landed_counter() == have:
+                                    break
+                            else:
+                                time.sleep(0.0002)
+                    done.set_result(seen)
+                except BaseException as e:
+                    self.errors.append(e)
+                    done.set_exception(e)
+
+            thread = threading.Thread(target=follow, daemon=True)
+            thread.start()
+            self.threads.append(thread)
+            return [done]
+
+    import torch.distributed.checkpoint as dcp
+
+    from ml_flashpoint.hip.checkpoint_saver import EngineConfig, HipMLFlashpointCheckpointSaver
+
+    def _saver(replication_manager, **kw):
+        CheckpointObjectManager._worker_pool = None
+        return HipMLFlashpointCheckpointSaver(_zero, _zero, _none, CheckpointObjectManager(), replication_manager,
+                                              initial_buffer_size_bytes=1 << 20, **kw)
+
+    replica_dir = os.path.join(shm_dir, "replica")
+    os.makedirs(replica_dir)
+    manager = FollowingManager(replica_dir)
+    g = torch.Generator(device=DEV).manual_seed(17)
+    sd = {f"layer.{i}.w": torch.randn(3 << 20, generator=g, device=DEV) for i in range(8)}  # 96 MiB
+    sd_cpu = {k: v.cpu() for k, v in sd.items()}
+    saver = _saver(manager, crc_chunk_bytes=1 << 20, engine_config=EngineConfig(slot_bytes=1 << 20, n_slots=3, copy_threads=4))
+    ckpt = os.path.join(shm_dir, "step-1_ckpt")
+    dcp.save(sd, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(saver, manager_future), no_dist=True)
+    for thread in manager.threads:
+        thread.join(30)
+    obj = os.path.join(ckpt, "__0__0_src0.distcp")
+    assert not manager.errors and not manager.after_write
+    assert [c[0] for c in manager.calls] == [obj] and manager.calls[0][1] == METADATA_SIZE
+    raw = open(obj, "rb").read()
+    assert manager.calls[0][2] == len(raw) - METADATA_SIZE
+    replica = open(os.path.join(replica_dir, "__0__0_src0.distcp"), "rb").read()
+    metadata = pickle.load(open(os.path.join(ckpt, ".metadata"), "rb"))
+    order = [i.fqn for i, _ in sorted(metadata.storage_data.items(), key=lambda kv: kv[1].offset)]
+    want, _ = fmt.file_image([sd_cpu[k] for k in order])
+    assert raw == want and replica == want
+    # a manager without the method: the reference's hand-over after the write
+    class PlainManager:
+        def __init__(self):
+            self.after_write = []
+
+        def async_replicate(self, buffer_io):
+            self.after_write.append(buffer_io.buffer_obj.get_id())
+            buffer_io.close()
+            return []
+
+    plain = PlainManager()
+    ckpt2 = os.path.join(shm_dir, "step-2_ckpt")
+    dcp.save(sd, checkpoint_id=ckpt2, storage_writer=MemoryStorageWriter(_saver(plain), manager_future), no_dist=True)
+    assert plain.after_write == [os.path.join(ckpt2, "__0__0_src0.distcp")]
+
+
+def test_discovery_with_checksums_of_objects_written_on_the_gpu(shm_dir, manager_future):
+    """Two steps saved by the gfx950 saver with checksums; a byte of the newer step's object is flipped afterwards.
+    Recovery discovery that verifies while choosing (host-side check against the sidecars the GPU produced, collectives
+    injected) picks the older step; discovery that only looks at what is present, as the reference's, the newer one.
+    The sidecars lie outside the containers, so no lister takes them for objects."""
+    import torch.distributed.checkpoint as dcp
+
+    from ml_flashpoint.checkpoint_object_manager.buffer_metadata import METADATA_SIZE
+    from ml_flashpoint.hip import integrity
+    from ml_flashpoint.hip.checkpoint_loader import HipMLFlashpointCheckpointLoader
+    from ml_flashpoint.hip.checkpoint_saver import HipMLFlashpointCheckpointSaver
+
+    CheckpointObjectManager._worker_pool = None
+    base = os.path.join(shm_dir, "job")
+    for crc_mode, step in (("beside", 1), ("fused", 2)):
+        saver = HipMLFlashpointCheckpointSaver(_zero, _zero, _none, CheckpointObjectManager(), None,
+                                               initial_buffer_size_bytes=1 << 20, crc_chunk_bytes=1 << 16, crc_mode=crc_mode)
+        cid = CheckpointContainerId(os.path.join(base, f"step-{step}_ckpt"))
+        sd = _state_dict()
+        dcp.save(sd, checkpoint_id=cid.data, storage_writer=MemoryStorageWriter(saver, manager_future), no_dist=True)
+        saver._remove_dirty_checkpoint_marker(cid)  # plain dcp.save leaves the marker to the strategy's finalize step
+        assert sorted(os.listdir(cid.data)) == [".metadata", "__0__0_src0.distcp"]  # no sidecar in the container
+        assert os.path.exists(integrity.sidecar_path(os.path.join(cid.data, "__0__0_src0.distcp")))
+    assert sorted(os.listdir(base)) == [".mlf_crc32c", "step-1_ckpt", "step-2_ckpt"]
+
+    calls = {"gather": 0, "broadcast": 0}
+
+    def all_gather(out_list, obj):
+        calls["gather"] += 1
+        out_list[0] = obj
+
+    def broadcast(obj_list, src=0):
+        calls["broadcast"] += 1
+
+    def loader(**kw):
+        made = HipMLFlashpointCheckpointLoader(CheckpointObjectManager(), None, all_gather_object_func=all_gather,
+                                               broadcast_object_list_func=broadcast, **kw)
+        made.common_state_object_name = None  # written by plain dcp.save: no common.pt
+        return made
+
+    base_id = CheckpointContainerId(base)
+    assert loader(verify_on_discovery=True).get_latest_complete_checkpoint(base_id).data.endswith("step-2_ckpt")
+    newer = os.path.join(base, "step-2_ckpt", "__0__0_src0.distcp")
+    with open(newer, "r+b") as f:
+        f.seek(METADATA_SIZE + 3 * (1 << 16) + 99)
+        byte = f.read(1)
+        f.seek(-1, os.SEEK_CUR)
+        f.write(bytes([byte[0] ^ 0x40]))
+    assert loader().get_latest_complete_checkpoint(base_id).data.endswith("step-2_ckpt")
+    checking = loader(verify_on_discovery=True)
+    assert checking.get_latest_complete_checkpoint(base_id).data.endswith("step-1_ckpt")
+    assert calls["gather"] >= 4 and calls["broadcast"] >= 2
+    # the older step restores; the corrupted one is refused by the restore as well
+    target = {k: torch.zeros_like(v) for k, v in _state_dict().items()}
+    older = os.path.join(base, "step-1_ckpt")
+    from ml_flashpoint.adapter.pytorch.memory_storage_reader import MemoryStorageReader
+
+    dcp.load(target, checkpoint_id=older, storage_reader=MemoryStorageReader(older, checking), no_dist=True)
+    assert all(torch.equal(target[k], v) for k, v in _state_dict().items())
+    with pytest.raises(BaseException) as exc:
+        bad = os.path.join(base, "step-2_ckpt")
+        dcp.load(target, checkpoint_id=bad, storage_reader=MemoryStorageReader(bad, checking), no_dist=True)
+    cause = exc.value.failures[0][0] if hasattr(exc.value, "failures") else exc.value
+    assert isinstance(cause, integrity.ChecksumMismatchError) and "chunk(s) [3]" in str(cause)
+    # finalize of a later step removes an older step's sidecars along with the step
+    saver = HipMLFlashpointCheckpointSaver(_zero, _zero, _none, CheckpointObjectManager(), None)
+    proc = saver._remove_older_checkpoints(CheckpointContainerId(os.path.join(base, "step-2_ckpt")))
+    proc.wait()
+    assert sorted(os.listdir(base)) == [".mlf_crc32c", "step-2_ckpt"]
+    assert os.listdir(os.path.join(base, ".mlf_crc32c")) == ["step-2_ckpt"]
