@@ -289,13 +289,15 @@ class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
             return [(item, tensor.to(device="cpu", non_blocking=non_blocking)) for item, tensor in pairs]
 
         staged = [dataclasses.replace(bucket, tensor_data=on_host(bucket.tensor_data)) for bucket in write_buckets]
-        if non_blocking and torch.cuda.is_available():
+        if torch.cuda.is_available():
             waits = _pack_waits(write_buckets)
-            if waits is None:
-                torch.cuda.synchronize()
-            else:
+            if waits is not None:
+                # placeholders: whether the caller asked for blocking copies or not, the live tensors may be
+                # overwritten once this returns, so the packs that read them must have finished
                 for wait in waits:
                     wait()
+            elif non_blocking:
+                torch.cuda.synchronize()
         return staged
 
     @_timed(logger=_LOGGER, name="write_staged_write_buckets", level=logging.INFO)

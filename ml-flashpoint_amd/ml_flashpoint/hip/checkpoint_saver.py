@@ -243,7 +243,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         reuse_plans: bool = True,
         snapshot_host_tensors: bool = False,
     ):
-        """Same positional arguments as the reference's default saver (checkpoint_saver.py:290-321).
+        """Same positional arguments as the reference's default saver (checkpoint_saver.py:290-321);
+        ``use_optimized_save=False`` writes the legacy format (``torch.save`` records) on the host, as the reference does.
 
         Keyword-only extras: ``engine_config`` (pinned ring), ``tile_bytes`` / ``block_threads`` (pack kernel work
         split, 0 = library default), ``crc_chunk_bytes`` (> 0: compute a CRC-32C per chunk of every object on the
@@ -265,11 +266,6 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         the transfer runs, as the reference copies them while it writes; True: they are cloned inside
         ``prepare_write_data`` instead, for training loops that update them before the transfer has ended).
         """
-        if not use_optimized_save:
-            raise ValueError(
-                "use_optimized_save=False asks for torch.save records, which are produced on the CPU only; "
-                "the gfx950 saver writes the MLF_TENS format."
-            )
         _lib.load()  # fail now, loudly, if the native library is not there
         self._global_rank_getter = global_rank_getter
         self._local_rank_getter = local_rank_getter
@@ -277,7 +273,10 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         self._chkpt_obj_manager = ckpt_obj_manager
         self._replication_manager = replication_manager
         self._initial_buffer_size_bytes = initial_buffer_size_bytes
-        self._use_optimized_save = True
+        # False: the legacy object format, one ``torch.save`` record per tensor.  Those records are produced by
+        # torch's serializer, on the host, as in the reference (checkpoint_saver.py:662-673); the kernels are not
+        # involved and the blocking part of such a save is the generic ``.to("cpu")`` staging.
+        self._use_optimized_save = use_optimized_save
         self._engine_config = engine_config or EngineConfig()
         self._tile_bytes = tile_bytes
         self._block_threads = block_threads
@@ -428,6 +427,13 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                 continue
             object_name = f"{object_name_prefix}_{len(write_buckets)}_src{rank}{_DEFAULT_OBJ_NAME_SUFFIX}"
             object_id = CheckpointObjectId.from_container(checkpoint_id, object_name)
+            if not self._use_optimized_save or not tensor_data:
+                # torch.save records, or an object of byte blobs only: written on the host by write_data, nothing
+                # to pack.  Host views are copied now, as the reference does (checkpoint_saver.py:390-398).
+                tensor_data = [(item, self._clone_if_needed(t)) for item, t in tensor_data]
+                write_buckets.append(ObjectWriteBucket(object_id=object_id, object_name=object_name,
+                                                       bytesio_data=bytes_data, tensor_data=tensor_data))
+                continue
             staged = self._stage_object(tensor_data, bytes_data, stats, object_id, object_name)
             refs = [
                 (item, StagedTensorRef(staged, i, t.dtype, t.shape)) for i, (item, t) in enumerate(tensor_data)
@@ -440,6 +446,13 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         stats["prepare_s"] = time.perf_counter() - t_start
         self.last_save_stats = stats
         return write_buckets
+
+    @staticmethod
+    def _clone_if_needed(tensor: torch.Tensor) -> torch.Tensor:
+        if tensor.device.type != "cpu":
+            return tensor
+        is_view = tensor.untyped_storage().size() != tensor.numel() * tensor.element_size()
+        return (tensor.clone() if is_view else tensor).contiguous()
 
     def _image_limit(self, device: torch.device) -> int:
         """Bytes of HBM an image may take: the explicit limit, or what the device and torch's allocator have free
@@ -768,7 +781,40 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
 
         threading.Thread(target=run, name=f"mlf-write-{bucket.object_name}", daemon=True).start()
 
+    def _write_bucket_on_host(self, bucket: ObjectWriteBucket, replicate_after_write: bool) -> list[WriteResult]:
+        """An object that the kernels have no part in: ``torch.save`` records (``use_optimized_save=False``) and/or
+        byte blobs, written through the buffer's file interface, tensors first (checkpoint_saver.py:655-698)."""
+        results: list[WriteResult] = []
+        with self._chkpt_obj_manager.acquire_buffer(bucket.object_id, self._initial_buffer_size_bytes) as writer:
+            legacy = not self._use_optimized_save
+            writer.set_format_signature(CheckpointFormat.TORCH_SAVE if legacy else CheckpointFormat.MLF_FORMAT)
+
+            def record(item, write):
+                offset = writer.tell()
+                write()
+                length = writer.tell() - offset
+                results.append(WriteResult(index=item.index, size_in_bytes=length,
+                                           storage_data=_StorageInfo(relative_path=bucket.object_name, offset=offset, length=length)))
+
+            for item, tensor in bucket.tensor_data:
+                record(item, lambda: torch.save(tensor, writer))
+            for item, data in bucket.bytesio_data:
+                data.seek(0)
+                record(item, lambda: writer.write(data.read()))
+            nbytes = writer.tell()
+            crcs = self._host_side_checksums(writer, 0, nbytes) if nbytes else None
+        if crcs is not None:
+            integrity.write_sidecar(str(bucket.object_id), self._crc_chunk_bytes, nbytes, crcs)
+        else:
+            integrity.remove_sidecar(str(bucket.object_id))
+        if replicate_after_write and self._replication_manager is not None:
+            self.async_replicate_object(bucket.object_id)
+        return results
+
     def _write_bucket(self, bucket: ObjectWriteBucket, replicate_after_write: bool, xfer: dict) -> list[WriteResult]:
+        if not bucket.tensor_data or (not self._use_optimized_save and not any(
+                isinstance(t, StagedTensorRef) for _, t in bucket.tensor_data)):
+            return self._write_bucket_on_host(bucket, replicate_after_write)
         staged = self._staged_of(bucket)
         if isinstance(staged, RemoteStagedObject):
             # this process only received the bucket: the process that owns the GPU is writing it

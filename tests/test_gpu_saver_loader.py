@@ -891,9 +891,65 @@ def test_legacy_torch_save_objects_are_still_readable(shm_dir):
     assert torch.equal(target.cpu(), t)
 
 
-def test_saver_rejects_cpu_only_format_and_is_picklable():
-    with pytest.raises(ValueError, match="MLF_TENS"):
-        _saver(use_optimized_save=False)
+def test_legacy_format_and_blob_only_objects_are_written_on_the_host(shm_dir, manager_future):
+    """``use_optimized_save=False`` (torch.save records, as the reference writes them) with the tensors on the device:
+    the generic staging step brings them to the host, the object carries the legacy signature and loads back through
+    the loader; a state dict of non-tensors only becomes an object of byte blobs without any image."""
+    sd_cpu = {k: v for k, v in _mixed_state_dict().items() if not (isinstance(v, torch.Tensor) and v.dtype == torch.float8_e4m3fn)}
+    sd_dev = _to_dev(sd_cpu)
+    saver = _saver(use_optimized_save=False, crc_chunk_bytes=1 << 16)
+    ckpt = os.path.join(shm_dir, "step-1_ckpt")
+    dcp.save(sd_dev, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(saver, manager_future), no_dist=True)
+    raw = open(os.path.join(ckpt, "__0__0_src0.distcp"), "rb").read()
+    assert raw[8:16] == b"TORCH___" and saver.last_save_stats.get("objects", 0) == 0  # nothing was packed
+    metadata = pickle.load(open(os.path.join(ckpt, ".metadata"), "rb"))
+    for index, info in metadata.storage_data.items():
+        if isinstance(sd_cpu[index.fqn], torch.Tensor):
+            record = raw[METADATA_SIZE + info.offset : METADATA_SIZE + info.offset + info.length]
+            got = torch.load(io.BytesIO(record), weights_only=True, map_location="cpu")
+            assert torch.equal(_bits(got), _bits(sd_cpu[index.fqn])), index.fqn
+    target = {k: (torch.zeros_like(v) if isinstance(v, torch.Tensor) else None) for k, v in sd_dev.items()}
+    dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, _loader()), no_dist=True)
+    assert all(torch.equal(_bits(target[k]), _bits(v)) for k, v in sd_cpu.items() if isinstance(v, torch.Tensor))
+    assert target["obj.step"] == 123
+    # byte blobs only, default format
+    saver = _saver()
+    ckpt2 = os.path.join(shm_dir, "step-2_ckpt")
+    only_objects = {"a": 1, "b": "two", "c": 3.5}
+    dcp.save(only_objects, checkpoint_id=ckpt2, storage_writer=MemoryStorageWriter(saver, manager_future), no_dist=True)
+    assert saver.last_save_stats.get("objects", 0) == 0 and saver._engine is None  # no image, no copy engine
+    target = {"a": None, "b": None, "c": None}
+    dcp.load(target, checkpoint_id=ckpt2, storage_reader=MemoryStorageReader(ckpt2, _loader()), no_dist=True)
+    assert target == only_objects
+
+
+def test_blocking_stage_call_waits_for_the_pack(shm_dir, manager_future):
+    """``stage_write_data_buckets(non_blocking=False)``: the reference's blocking copies return with the data staged;
+    with placeholders the call returns once the pack that read the live tensors has finished."""
+    from torch.distributed.checkpoint import DefaultSavePlanner
+    from torch.distributed.checkpoint.utils import _DistWrapper
+
+    from ml_flashpoint.adapter.pytorch import custom_state_dict_saver as three_calls
+
+    sd = {"w": torch.randn(64 << 20, device=DEV)}
+    want = sd["w"].cpu()
+    saver = _saver()
+    cid = CheckpointContainerId(os.path.join(shm_dir, "step-1_ckpt"))
+    writer = MemoryStorageWriter(saver, manager_future)
+    writer.reset(cid.data)
+    dist = _DistWrapper(None, False, 0)
+    buckets, metadata, *_ = three_calls.generate_plan(cid, sd, writer, DefaultSavePlanner(), dist)
+    staged = MemoryStorageWriter.stage_write_data_buckets(cid, buckets, non_blocking=False)
+    event = buckets[0].tensor_data[0][1].staged.packed_event
+    assert event.query(), "the call returned before the pack had finished"
+    sd["w"].zero_()  # the live tensor may be overwritten now
+    three_calls.write_data(cid, writer, staged, replicate_after_write=False)
+    three_calls.finish_write(cid, writer, metadata, dist)
+    raw = open(os.path.join(cid.data, "__0__0_src0.distcp"), "rb").read()
+    assert raw == fmt.file_image([want])[0]
+
+
+def test_saver_is_picklable():
     from ml_flashpoint.hip.checkpoint_saver import HipMLFlashpointCheckpointSaver
 
     s = HipMLFlashpointCheckpointSaver(_zero, _zero, _none, CheckpointObjectManager(), replication_manager=object())

@@ -11,6 +11,7 @@ import subprocess
 from unittest import mock
 
 import pytest
+import torch
 
 from ml_flashpoint.checkpoint_object_manager.buffer_io import BufferIO
 from ml_flashpoint.checkpoint_object_manager.checkpoint_object_manager import CheckpointObjectManager
@@ -207,5 +208,54 @@ def test_pickling_keeps_configuration_and_callables_but_not_the_replication_mana
     clone = pickle.loads(pickle.dumps(saver))
     assert clone._replication_manager is None and clone._initial_buffer_size_bytes == 1024
     assert clone._use_optimized_save is True and clone._global_rank_getter() == 0 and clone._plan_cache == {}
-    with pytest.raises(ValueError, match="MLF_TENS"):          # torch.save records are a CPU-only format
-        HipMLFlashpointCheckpointSaver(_zero, _zero, _none, CheckpointObjectManager(), None, use_optimized_save=False)
+    legacy = HipMLFlashpointCheckpointSaver(_zero, _zero, _none, CheckpointObjectManager(), None, use_optimized_save=False)
+    assert pickle.loads(pickle.dumps(legacy))._use_optimized_save is False  # (tests/core/test_checkpoint_saver.py:2207-2218)
+
+
+def test_write_data_with_optimized_save_false(tmp_path):
+    """The reference's case (tests/core/test_checkpoint_saver.py:188-230), same input: an object written with
+    ``use_optimized_save=False`` does not carry the MLF signature and its data section loads with ``torch.load``.
+    Plus what that case leaves out: offsets and lengths of several records, byte blobs behind the tensors, and the
+    loader reading such an object back."""
+    import io
+
+    from torch.distributed.checkpoint.metadata import MetadataIndex
+    from torch.distributed.checkpoint.planner import WriteItem, WriteItemType
+
+    from ml_flashpoint.checkpoint_object_manager.buffer_metadata import METADATA_SIZE
+    from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId
+    from ml_flashpoint.core.defaults import CheckpointFormat
+
+    class Resolver:
+        def __init__(self, data):
+            self.data = data
+
+        def resolve_data(self, item):
+            return self.data[item.index]
+
+    CheckpointObjectManager._worker_pool = None
+    manager = CheckpointObjectManager()
+    saver = HipMLFlashpointCheckpointSaver(_zero, _zero, _none, manager, None, initial_buffer_size_bytes=1 << 20,
+                                           use_optimized_save=False)
+    checkpoint_id = CheckpointContainerId(str(tmp_path / "ckpt_opt_false"))
+    tensor = torch.tensor([1, 2, 3], dtype=torch.int32)
+    view = torch.arange(24, dtype=torch.float32).reshape(4, 6)[:, ::2]
+    blob = io.BytesIO(b"pickled step counter")
+    data = {MetadataIndex("item_0"): tensor, MetadataIndex("item_1"): view, MetadataIndex("item_2"): blob}
+    items = [WriteItem(index=i, type=WriteItemType.BYTE_IO if isinstance(v, io.BytesIO) else WriteItemType.TENSOR)
+             for i, v in data.items()]
+    buckets = saver.prepare_write_data(checkpoint_id, items, Resolver(data), object_name_prefix="data", bucket_count=1)
+    assert len(buckets) == 1 and buckets[0].object_name == "data_0_src0.distcp"
+    assert all(isinstance(t, torch.Tensor) for _, t in buckets[0].tensor_data)  # real tensors, no placeholders
+    results = saver.write_data(checkpoint_id, buckets, replicate_after_write=False)
+    raw = open(buckets[0].object_id.data, "rb").read()
+    assert raw[8:16] == CheckpointFormat.TORCH_SAVE != CheckpointFormat.MLF_FORMAT
+    section = raw[METADATA_SIZE:]
+    assert torch.equal(torch.load(io.BytesIO(section), weights_only=False), tensor)  # the reference's assertion
+    by_name = {r.index.fqn: r.storage_data for r in results}
+    assert by_name["item_0"].offset == 0 and by_name["item_1"].offset == by_name["item_0"].length
+    assert by_name["item_2"].offset == by_name["item_1"].offset + by_name["item_1"].length
+    assert by_name["item_2"].offset + by_name["item_2"].length == len(section)
+    second = section[by_name["item_1"].offset : by_name["item_1"].offset + by_name["item_1"].length]
+    assert torch.equal(torch.load(io.BytesIO(second), weights_only=True), view)
+    assert section[by_name["item_2"].offset :] == b"pickled step counter"
