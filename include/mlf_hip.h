@@ -113,8 +113,9 @@ int mlf_plan_get_info(const mlf_plan* plan, mlf_plan_info* out);
 
 /* Replaces the bytes of the plan's blob (same size as at creation) for a plan that is kept from one save to the
  * next: the record headers in it repeat, step counters and other host-resident items do not.  The upload is
- * enqueued on `stream`, so it is ordered behind launches already enqueued there (which still read the old bytes)
- * and ahead of later ones; use the stream the plan is launched on.  No reference counterpart: the reference
+ * enqueued on `stream` and made to wait for the plan's last launch wherever that ran, so it is ordered behind
+ * the kernels that still read the old bytes and ahead of launches enqueued on `stream` afterwards; a launch on
+ * another stream must be ordered behind the upload by the caller.  No reference counterpart: the reference
  * rebuilds everything per save (checkpoint_saver.py:622-707); its plan caching (save_strategies.py:182-212) is the
  * model for keeping the tables. */
 int mlf_plan_update_blob(mlf_plan* plan, const void* host_blob, uint64_t blob_bytes, void* stream);
