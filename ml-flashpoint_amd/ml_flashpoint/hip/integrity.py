@@ -76,3 +76,56 @@ def read_sidecar(object_path: str) -> Optional[Tuple[int, int, np.ndarray]]:
 
 class ChecksumMismatchError(RuntimeError):
     """A restored object's bytes do not match the CRC-32C recorded when it was saved."""
+
+
+class ChunkChecksums:
+    """Per-chunk CRC-32C of a data section that is checksummed piece by piece.
+
+    An object that leaves the device in several transfers (windows, pieces) is cut where records end, not where
+    checksum chunks end.  Each piece is checksummed where it lies, cut on the chunk grid of the data section - the
+    first value covers the bytes up to the next chunk boundary, the following ones whole chunks, the last one what
+    is left - and the values of the parts of one chunk are joined here: crc(A || B) = crc(A) * x^(8 |B|) + crc(B)
+    over GF(2), the law ``mlf_crc32c_combine`` implements.  Pieces must arrive in ascending order and without gaps;
+    ``result`` refuses an incomplete section."""
+
+    def __init__(self, chunk_bytes: int, data_bytes: int, combine=None):
+        if chunk_bytes <= 0:
+            raise ValueError("chunk_bytes must be positive")
+        if combine is None:
+            from ml_flashpoint.hip import plan as hip_plan
+
+            combine = hip_plan.crc32c_combine
+        self._combine = combine
+        self.chunk_bytes, self.data_bytes = chunk_bytes, data_bytes
+        self._values = np.zeros(-(-data_bytes // chunk_bytes), dtype=np.uint32)
+        self._at = 0  # the section is covered up to here
+
+    @staticmethod
+    def cuts(offset: int, nbytes: int, chunk_bytes: int) -> list:
+        """[(first byte, length)] of the parts of [offset, offset + nbytes) between chunk boundaries."""
+        parts, at, end = [], offset, offset + nbytes
+        while at < end:
+            stop = min((at // chunk_bytes + 1) * chunk_bytes, end)
+            parts.append((at, stop - at))
+            at = stop
+        return parts
+
+    def add(self, offset: int, nbytes: int, values) -> None:
+        """``values``: one CRC-32C per part of ``cuts(offset, nbytes, chunk_bytes)``."""
+        if offset != self._at:
+            raise ValueError(f"piece at {offset} does not continue the section, which is covered up to {self._at}")
+        parts = self.cuts(offset, nbytes, self.chunk_bytes)
+        if len(values) != len(parts):
+            raise ValueError(f"{len(values)} checksums for {len(parts)} parts")
+        for (first, length), value in zip(parts, values):
+            k = first // self.chunk_bytes
+            if first % self.chunk_bytes == 0:
+                self._values[k] = int(value)
+            else:
+                self._values[k] = self._combine(int(self._values[k]), int(value), length)
+        self._at = offset + nbytes
+
+    def result(self) -> np.ndarray:
+        if self._at != self.data_bytes:
+            raise ValueError(f"checksums cover {self._at} of {self.data_bytes} bytes")
+        return self._values

@@ -479,6 +479,33 @@ def crc32c_device(buf: torch.Tensor, nbytes: int, chunk_bytes: int, stream: Opti
     return out
 
 
+def crc32c_device_cut(buf: torch.Tensor, buf_off: int, data_off: int, nbytes: int, chunk_bytes: int, host_ptr: int,
+                      stream: Optional[int] = None) -> list:
+    """CRC-32C of ``nbytes`` bytes of a data section, from byte ``data_off`` on, cut where the section's checksum
+    chunks end: one value per part of ``integrity.ChunkChecksums.cuts(data_off, nbytes, chunk_bytes)``.  The bytes
+    lie at ``buf[buf_off:]`` on the device and, already, at ``host_ptr`` on the host; buffer positions and section
+    positions must agree modulo 16, so that chunk boundaries are 16-byte aligned on the device (the checksum
+    kernels read vectors).  Only a first part that starts off that grid needs the host copy: its leading bytes, at
+    most 15, are checksummed there and joined with the device's value for the rest."""
+    if nbytes == 0:
+        return []
+    base = buf.data_ptr() + buf_off
+    if (base - data_off) % 16:
+        raise ValueError("buffer and data section positions differ modulo 16")
+    values = []
+    head = min(nbytes, -data_off % chunk_bytes)
+    if head:
+        skip = min(head, -base % 16)
+        value = crc32c_host(host_ptr, skip) if skip else None
+        if head > skip:
+            on_device = int(crc32c_device(buf[buf_off + skip : buf_off + head], head - skip, chunk_bytes, stream)[0])
+            value = on_device if value is None else crc32c_combine(value, on_device, head - skip)
+        values.append(value)
+    if nbytes > head:
+        values.extend(int(v) for v in crc32c_device(buf[buf_off + head : buf_off + nbytes], nbytes - head, chunk_bytes, stream))
+    return values
+
+
 def crc32c_host(ptr: int, nbytes: int) -> int:
     return int(_lib.load().mlf_crc32c_host(ptr, nbytes))
 
