@@ -526,23 +526,17 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
     def _restore_windowed(self, object_id, stream, device, rows, limit, sidecar, stats) -> None:
         """Fallback for an object whose requested range does not fit in HBM beside the live state: the rows are
         sorted by position and restored window by window through one device buffer of at most ``limit`` bytes.  A
-        contiguous row larger than a window is cut into pieces; a strided one cannot be.  With a sidecar the whole
-        object is checked first, on the host (the windows do not coincide with the checksum chunks)."""
+        contiguous row larger than a window is cut into pieces; a strided one cannot be.
+
+        With a sidecar and ``crc_mode="fused"`` every window starts on a checksum chunk, so the unpack of a window
+        yields the checksums of the chunks it holds completely; a chunk that a window ends in is held completely by
+        the next window when the rows continue there (it starts on that chunk: a few MiB are uploaded twice); chunks
+        that no window holds completely (where the rows do not continue; those of byte blobs behind the tensors)
+        are checked on the host at the end.  A mismatch raises before any tensor is committed.  With
+        ``crc_mode="before"``, or a buffer too small for that, the whole object is checked on the host first."""
         _LOGGER.warning("requested range of '%s' exceeds the HBM limit of %d bytes; restoring window by window",
                         object_id, limit)
-        if sidecar is not None:
-            chunk_bytes, data_bytes, want = sidecar
-            fd = stream.fileno()
-            own_fd = fd < 0
-            if own_fd:
-                fd = os.open(object_id.data, os.O_RDONLY)
-            try:
-                got = hip_plan.crc32c_file(fd, METADATA_SIZE, data_bytes, chunk_bytes,
-                                           self._engine_config.resolved_copy_threads())
-            finally:
-                if own_fd:
-                    os.close(fd)
-            self._compare_checksums(object_id, got, want, chunk_bytes)
+        chunk_bytes, data_bytes, want = sidecar if sidecar is not None else (0, 0, None)
         image = None
         while image is None:  # the largest buffer the allocator really has, at most the limit
             if limit - _UPLOAD_ALIGN < 65536:
@@ -552,7 +546,12 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
             image = hip_plan.try_allocate(limit, device)
             if image is None:
                 limit //= 2
-        usable = limit - _UPLOAD_ALIGN  # a window starts on an upload boundary at or below its first row
+        on_device = (sidecar is not None and self._crc_mode == "fused" and chunk_bytes % 65536 == 0
+                     and limit >= 4 * chunk_bytes)
+        if sidecar is not None and not on_device:
+            self._check_on_host(object_id, stream, sidecar, range(len(want)))
+        align = chunk_bytes if on_device else _UPLOAD_ALIGN
+        usable = limit - align  # a window starts on an upload boundary at or below its first row
         piece = usable // 65536 * 65536  # a multiple of every element size
         pieces = []
         for first, last, contiguous, args in sorted(rows, key=lambda r: r[0]):
@@ -572,16 +571,53 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                 windows.append((lo, current))
                 current = []
             if not current:
-                lo = row[0] // _UPLOAD_ALIGN * _UPLOAD_ALIGN
+                lo = row[0] // align * align
             current.append(row)
         windows.append((lo, current))
         cur = torch.cuda.current_stream(device)
+        checked = set()
         for lo, window_rows in windows:
             span = max(r[1] for r in window_rows) - lo
             self._upload(stream, lo, image, span, cur, stats)
-            self._unpack(self._table_of(window_rows, lo), image, span, cur,
-                         sum(r[1] - r[0] for r in window_rows if r[2]))
+            got = self._unpack(self._table_of(window_rows, lo), image, span, cur,
+                               sum(r[1] - r[0] for r in window_rows if r[2]), chunk_bytes if on_device else 0)
+            if on_device:
+                first = lo // chunk_bytes
+                whole = span // chunk_bytes + (1 if lo + span == data_bytes and span % chunk_bytes else 0)
+                self._compare_checksums(object_id, got[:whole], want[first : first + whole], chunk_bytes, first, len(want))
+                checked.update(range(first, first + whole))
+        if on_device:  # what no window held completely: chunks where the rows do not continue, and those of byte blobs
+            self._check_on_host(object_id, stream, sidecar, sorted(set(range(len(want))) - checked))
         stats["windows"] = stats.get("windows", 0) + len(windows)
+
+    def _check_on_host(self, object_id, stream, sidecar, chunks) -> None:
+        """Compares the given chunks of an object's data section with its sidecar, reading them on the host."""
+        chunk_bytes, data_bytes, want = sidecar
+        chunks = list(chunks)
+        if not chunks:
+            return
+        t0 = time.perf_counter()
+        fd = stream.fileno()
+        own_fd = fd < 0
+        if own_fd:
+            fd = os.open(object_id.data, os.O_RDONLY)
+        try:
+            threads = self._engine_config.resolved_copy_threads()
+            if chunks == list(range(chunks[0], chunks[-1] + 1)):  # one run: one threaded pass
+                first = chunks[0] * chunk_bytes
+                length = min((chunks[-1] + 1) * chunk_bytes, data_bytes) - first
+                got = hip_plan.crc32c_file(fd, METADATA_SIZE + first, length, chunk_bytes, threads)
+                self._compare_checksums(object_id, got, want[chunks[0] : chunks[-1] + 1], chunk_bytes, chunks[0], len(want))
+            else:
+                for k in chunks:
+                    length = min((k + 1) * chunk_bytes, data_bytes) - k * chunk_bytes
+                    got = hip_plan.crc32c_file(fd, METADATA_SIZE + k * chunk_bytes, length, chunk_bytes, threads)
+                    self._compare_checksums(object_id, got, want[k : k + 1], chunk_bytes, k, len(want))
+        finally:
+            if own_fd:
+                os.close(fd)
+        stats = self._stats_in_progress
+        stats["crc_s"] = stats.get("crc_s", 0.0) + time.perf_counter() - t0
 
     # ---- discovery (core/checkpoint_discovery.py) ----------------------------------------------------------
     def _object_is_intact(self, path: str) -> bool:

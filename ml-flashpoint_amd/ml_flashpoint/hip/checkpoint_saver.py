@@ -83,6 +83,9 @@ _HOST_DIRECT_MIN_BYTES = 256 << 10
 # when the allocator has no single block for an object's image, the image is held in pieces of about this size
 _IMAGE_PIECE_BYTES = 8 << 30
 
+# a window or piece of an image starts this many bytes (modulo) into its device buffer as into the image
+_WINDOW_PAD = 4096
+
 _MAX_KEPT_PLANS = 64  # objects per save are few (one per writer thread); beyond this the oldest is rebuilt
 
 
@@ -603,7 +606,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
             buffers = []
             for _, _, begin, end in windows:
-                buffers.append(hip_plan.try_allocate(end - begin, device))
+                buffers.append(hip_plan.try_allocate(begin % _WINDOW_PAD + end - begin, device))
                 if buffers[-1] is None:
                     del buffers
                     return None
@@ -620,9 +623,10 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             if begin_event is not None:
                 begin_event.record()
             for (r0, r1, begin, end), buf in zip(windows, buffers):
+                pad = begin % _WINDOW_PAD  # as in _stage_windowed
                 sub = layout.items[r0:r1].copy()
-                sub["image_off"] -= begin
-                plan = hip_plan.Plan(sub, layout.blob, end - begin, tile_bytes=self._tile_bytes,
+                sub["image_off"] -= begin - pad
+                plan = hip_plan.Plan(sub, layout.blob, pad + end - begin, tile_bytes=self._tile_bytes,
                                      block_threads=self._block_threads)
                 plan.pack(buf, stream)
                 pieces.append((plan, buf, begin, end))
@@ -665,25 +669,40 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                 start = writer.tell()
                 writer.next_buffer_slice(nbytes).release()
                 stream = torch.cuda.current_stream(device).cuda_stream
-                buf = torch.empty(max(e - b for _, _, b, e in windows), dtype=torch.uint8, device=device)
+                # a window lies in the buffer where it lies in the image modulo the pad, so that tiles and checksum
+                # chunks are cut on the same grid as in an image held whole
+                buf = torch.empty(max(e - b for _, _, b, e in windows) + _WINDOW_PAD, dtype=torch.uint8, device=device)
                 engine = self._get_engine()
+                sums = integrity.ChunkChecksums(self._crc_chunk_bytes, nbytes) if self._crc_chunk_bytes and nbytes else None
                 for r0, r1, begin, end in windows:
+                    pad = begin % _WINDOW_PAD
                     sub = arr[r0:r1].copy()
-                    sub["image_off"] -= begin
-                    plan = hip_plan.Plan(sub, layout.blob, end - begin, tile_bytes=self._tile_bytes,
+                    sub["image_off"] -= begin - pad
+                    plan = hip_plan.Plan(sub, layout.blob, pad + end - begin, tile_bytes=self._tile_bytes,
                                          block_threads=self._block_threads)
-                    plan.pack(buf, stream)
-                    st = engine.d2h(buf.data_ptr(), writer.data_address(start + begin), end - begin, stream)
+                    if self.record_kernel_events:
+                        t_begin, t_end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                        t_begin.record()
+                        plan.pack(buf, stream)
+                        t_end.record()
+                        self.kernel_events.append(
+                            (t_begin, t_end, int(sub["nbytes"][sub["kind"] == hip_plan.ITEM_DEVICE].sum())))
+                    else:
+                        plan.pack(buf, stream)
+                    dst = writer.data_address(start + begin)
+                    st = engine.d2h(buf.data_ptr() + pad, dst, end - begin, stream)
+                    if sums is not None:
+                        # windows end where records end, not where checksum chunks end: the parts are checksummed
+                        # where they lie in the buffer and joined per chunk
+                        t0 = time.perf_counter()
+                        sums.add(begin, end - begin, hip_plan.crc32c_device_cut(buf, pad, begin, end - begin,
+                                                                                 self._crc_chunk_bytes, dst, stream))
+                        xfer["crc_s"] = xfer.get("crc_s", 0.0) + time.perf_counter() - t0
                     plan.destroy()
                     xfer["d2h_s"] += st.seconds
                     xfer["d2h_bytes"] += end - begin
-            fd = writer.fileno() if self._crc_chunk_bytes and nbytes else -1
-            if fd >= 0:
-                # windows end where records end, not where checksum chunks end, so the checksums of this (already
-                # blocking) mode are taken on the host, from the pages that were just written
-                crcs = hip_plan.crc32c_file(fd, METADATA_SIZE + start, nbytes, self._crc_chunk_bytes,
-                                            self._engine_config.resolved_copy_threads())
-                integrity.write_sidecar(str(object_id), self._crc_chunk_bytes, nbytes, crcs)
+            if sums is not None:
+                integrity.write_sidecar(str(object_id), self._crc_chunk_bytes, nbytes, sums.result())
             else:
                 integrity.remove_sidecar(str(object_id))
         stats["objects"] += 1
@@ -964,15 +983,32 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         """The transfer of an image that is held in several device buffers: one after the other, each released as
         soon as it has been sent."""
         engine = self._get_engine()
+        nbytes = staged.layout.data_bytes
+        sums = integrity.ChunkChecksums(self._crc_chunk_bytes, nbytes) if self._crc_chunk_bytes and nbytes else None
+        # the checksum kernels get a stream of their own: this may be a background thread, and the training step's
+        # kernels are queued on the stream the pack ran on
+        side = torch.cuda.Stream(device=staged.device_index) if sums is not None else None
         for k, (plan, buf, begin, end) in enumerate(staged.pieces):
-            st = engine.d2h(buf.data_ptr(), writer.data_address(start + begin), end - begin, staged.stream)
+            pad = begin % _WINDOW_PAD
+            dst = writer.data_address(start + begin)
+            if staged.packed_event is not None:
+                st, _ = engine.d2h_gated(buf.data_ptr() + pad, dst, end - begin, staged.packed_event.cuda_event, 0,
+                                         ctypes.c_uint64(0))
+            else:
+                st = engine.d2h(buf.data_ptr() + pad, dst, end - begin, staged.stream)
             self._count_transfer(xfer, st, end - begin)
+            if sums is not None:
+                # the piece has left the device, so its pack is over: the side stream may read it at once
+                t0 = time.perf_counter()
+                sums.add(begin, end - begin, hip_plan.crc32c_device_cut(buf, pad, begin, end - begin,
+                                                                         self._crc_chunk_bytes, dst, side.cuda_stream))
+                xfer["crc_s"] = xfer.get("crc_s", 0.0) + time.perf_counter() - t0
             staged._landed.value = end
             staged.pieces[k] = None
             plan.destroy()
             del buf
         staged.pieces = None
-        return self._host_side_checksums(writer, start, staged.layout.data_bytes)
+        return sums.result() if sums is not None else None
 
     def _transfer_in_pieces(self, staged: StagedObject, writer, start: int, xfer: dict):
         """The transfer of an object some of whose tensors live in host memory: the runs of the image between them

@@ -495,11 +495,18 @@ def test_object_larger_than_the_hbm_limit_is_saved_window_by_window(shm_dir, man
     metadata = pickle.load(open(os.path.join(ckpt, ".metadata"), "rb"))
     image, spans, got_spans = _expected_file(sd_cpu, metadata, raw)
     assert raw == image and got_spans == spans
-    # the sidecar of a windowed save comes from the host routine; the GPU check of an ordinary restore accepts it
+    # windows end where records end, not where checksum chunks end: the sidecar is joined from the checksums the GPU
+    # took of the parts of each window; every value is the host's for that chunk of the file, and the GPU check of an
+    # ordinary restore accepts it
     from ml_flashpoint.hip import integrity
+    from ml_flashpoint.hip import plan as P
 
     chunk, nbytes, crcs = integrity.read_sidecar(os.path.join(ckpt, "__0__0_src0.distcp"))
     assert chunk == 1 << 16 and nbytes == len(raw) - METADATA_SIZE and len(crcs) == -(-nbytes // chunk)
+    for k, c in enumerate(crcs):
+        piece = raw[METADATA_SIZE + k * chunk : METADATA_SIZE + (k + 1) * chunk]
+        buf = ctypes.create_string_buffer(piece, len(piece))
+        assert P.crc32c_host(ctypes.addressof(buf), len(piece)) == int(c), k
     target = {k: (torch.zeros_like(v) if isinstance(v, torch.Tensor) and v.dtype != torch.float8_e4m3fn else
                   (torch.zeros(v.shape, dtype=torch.uint8, device=v.device).view(v.dtype) if isinstance(v, torch.Tensor) else None))
               for k, v in sd_dev.items()}
@@ -558,7 +565,8 @@ def test_image_is_held_in_pieces_when_no_single_block_is_to_be_had(shm_dir, mana
 def test_restore_larger_than_the_hbm_limit_goes_window_by_window(shm_dir, manager_future, load_file_io):
     """With ``max_image_bytes`` far below the object size the loader uploads and unpacks windows of rows through
     one small device buffer (contiguous rows larger than a window are cut); the restored bits are the same, the
-    CRC sidecar is still honoured (on the host), and a strided read that cannot be cut says so."""
+    CRC sidecar is still honoured (windows start on checksum chunks and the unpack kernel checks what it scatters),
+    and a strided read that cannot be cut says so."""
     from ml_flashpoint.hip import integrity
 
     sd_cpu = dict(_mixed_state_dict())
@@ -603,7 +611,28 @@ def test_restore_larger_than_the_hbm_limit_goes_window_by_window(shm_dir, manage
     assert isinstance(cause, NotImplementedError) and "does not fit the HBM limit" in str(cause)
 
     obj = os.path.join(ckpt, "__0__0_src0.distcp")
-    with open(obj, "r+b") as f:  # one flipped bit: found by the host-side check before any window is uploaded
+    assert loader.last_load_stats.get("crc_s", 0.0) >= 0.0
+    with open(obj, "r+b") as f:  # one flipped bit: found by the window that holds its chunk
+        f.seek(METADATA_SIZE + 5 * (1 << 16) + 77)
+        byte = f.read(1)
+        f.seek(-1, os.SEEK_CUR)
+        f.write(bytes([byte[0] ^ 0x01]))
+    for mode in ("fused", "before"):  # "before": the whole object is checked on the host ahead of the first window
+        picky = _loader(max_image_bytes=256 << 10, use_file_io=load_file_io, crc_mode=mode)
+        victim = targets()
+        with pytest.raises(BaseException) as exc:
+            dcp.load(victim, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, picky), no_dist=True)
+        cause = exc.value.failures[0][0] if hasattr(exc.value, "failures") else exc.value
+        assert isinstance(cause, integrity.ChecksumMismatchError) and "chunk(s) [5]" in str(cause), mode
+        if mode == "before":
+            assert all(not v.any() for v in victim.values()
+                       if isinstance(v, torch.Tensor) and v.is_cuda and v.dtype != torch.float8_e4m3fn)
+    with open(obj, "r+b") as f:  # the last chunk of the object, which no window holds completely: found on the host
+        f.seek(-3, os.SEEK_END)
+        byte = f.read(1)
+        f.seek(-1, os.SEEK_CUR)
+        f.write(bytes([byte[0] ^ 0x80]))
+    with open(obj, "r+b") as f:  # (the first flip undone)
         f.seek(METADATA_SIZE + 5 * (1 << 16) + 77)
         byte = f.read(1)
         f.seek(-1, os.SEEK_CUR)
@@ -611,7 +640,8 @@ def test_restore_larger_than_the_hbm_limit_goes_window_by_window(shm_dir, manage
     with pytest.raises(BaseException) as exc:
         dcp.load(targets(), checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), no_dist=True)
     cause = exc.value.failures[0][0] if hasattr(exc.value, "failures") else exc.value
-    assert isinstance(cause, integrity.ChecksumMismatchError) and "chunk(s) [5]" in str(cause)
+    n_chunks = -(-(os.path.getsize(obj) - METADATA_SIZE) // (1 << 16))
+    assert isinstance(cause, integrity.ChecksumMismatchError) and f"chunk(s) [{n_chunks - 1}]" in str(cause)
 
 
 def test_restore_goes_through_a_smaller_buffer_when_no_single_block_is_to_be_had(shm_dir, manager_future, monkeypatch):
