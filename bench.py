@@ -418,7 +418,7 @@ def main():
                        "plan": sv["plan"], "pack_launch": sv["pack_launch"], "save_tail": sv["tail"],
                        "d2h": d2h.get("d2h_s", 0.0), "d2h_bytes": d2h.get("d2h_bytes", 0),
                        "host_copy_s": d2h.get("host_copy_s", 0.0), "host_copy_bytes": d2h.get("host_copy_bytes", 0),
-                       "h2d": ld.get("h2d_s", 0.0), "h2d_bytes": ld.get("h2d_bytes", 0),
+                       "h2d": ld.get("h2d_s", 0.0), "h2d_bytes": ld.get("h2d_bytes", 0), "h2d_host": ld.get("h2d_host_s", 0.0),
                        "pack_ms": sv["pack_ms"], "unpack_ms": unpack_ms, "pack_bytes": sv["pack_bytes"], "unpack_bytes": unpack_bytes,
                        "r_read": ld.get("read_s", 0.0), "r_parse": ld.get("parse_s", 0.0), "r_table": ld.get("table_s", 0.0),
                        "r_crc": ld.get("crc_s", 0.0), "r_unpack_plan": ld.get("unpack_plan_s", 0.0),
@@ -540,6 +540,7 @@ def main():
             "restore_breakdown_ms": {
                 "dcp_plan_and_metadata": round((mean(rec["restore"]) - mean(rec["r_read"])) * 1e3, 2),
                 "parse_headers_resolve_targets": ms("r_parse"), "descriptor_table": ms("r_table"), "h2d": ms("h2d"),
+                "of_h2d_filling_pinned_slots": ms("h2d_host"),  # pread() into the slots, overlapped with the copies
                 "checksum_pass": ms("r_crc"), "unpack_plan": ms("r_unpack_plan"),
                 "unpack_and_sync": ms("r_unpack"), "commit": ms("r_commit"),
                 "other_in_read_data": round((mean(rec["r_read"]) - restore_known) * 1e3, 2)},

@@ -171,7 +171,8 @@ typedef struct mlf_engine mlf_engine;
 
 typedef struct mlf_xfer_stats {
   double seconds;        /* wall time of the call                                                             */
-  double wait_seconds;   /* of which the calling thread spent waiting for the producer stream (d2h only)      */
+  double wait_seconds;   /* d2h: of which the calling thread spent waiting for the producer stream;           */
+                         /* h2d: of which the host threads spent filling the pinned slots (pread / memcpy)    */
   uint64_t bytes;
   uint64_t chunks;
 } mlf_xfer_stats;

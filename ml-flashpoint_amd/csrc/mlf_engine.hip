@@ -322,12 +322,15 @@ int engine_h2d(mlf_engine* e, const HostEnd& host, void* dst_dev, uint64_t nbyte
   const uint64_t n_chunks = (nbytes + slot - 1) / slot;
   const uint64_t n_slots = e->slots.size();
   DrainOnExit drain{e};
+  double host_s = 0;  // spent filling slots from the file or the mapping
   for (uint64_t c = 0; c < n_chunks; ++c) {
     const uint64_t off = c * slot, len = std::min(slot, nbytes - off);
     const uint64_t s = c % n_slots;
     if (c >= n_slots) HIP_TRY(hipEventSynchronize(e->slot_done[s]));  // the slot's previous upload has left it
+    const double t_read = now_s();
     if (int err = pool_host_copy(*e->pool, host, off, e->slots[s], len, false))
       return fail(MLF_HIP_RUNTIME, std::string("pread() from the buffer file failed: ") + strerror(err));
+    host_s += now_s() - t_read;
     hipStream_t st = e->streams[c & 1];
     HIP_TRY(hipMemcpyAsync(dst + off, e->slots[s], len, hipMemcpyHostToDevice, st));
     HIP_TRY(hipEventRecord(e->slot_done[s], st));
@@ -341,7 +344,7 @@ int engine_h2d(mlf_engine* e, const HostEnd& host, void* dst_dev, uint64_t nbyte
   drain.armed = false;
   if (stats) {
     stats->seconds = now_s() - t0;
-    stats->wait_seconds = 0;
+    stats->wait_seconds = host_s;
     stats->bytes = nbytes;
     stats->chunks = n_chunks;
   }

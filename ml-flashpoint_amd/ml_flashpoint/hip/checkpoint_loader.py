@@ -414,6 +414,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         else:
             st = self._get_engine().h2d(stream.data_address(lo), image.data_ptr(), span, cur.cuda_stream)
         stats["h2d_s"] += st.seconds
+        stats["h2d_host_s"] = stats.get("h2d_host_s", 0.0) + st.wait_seconds  # filling the pinned slots
         stats["h2d_bytes"] += span
 
     def _unpack(self, items, image: torch.Tensor, span: int, cur, payload_bytes: int, crc_chunk_bytes: int = 0):
