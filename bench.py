@@ -480,12 +480,17 @@ def main():
         link = None
         if not args.no_link_probe:
             probe_bytes = min(24 << 30, max(file_bytes, 64 << 20))  # long enough to be past the link's start-up
-            torch.cuda.empty_cache()
+            # out of the allocator's cache, i.e. the memory the images of the timed steps lay in: a block that the
+            # driver has just handed out afresh, while it is still clearing what was released, has measured as low as
+            # 46 GB/s in one direction or the other
             scratch = torch.zeros(probe_bytes, dtype=torch.uint8, device=device)
             torch.cuda.synchronize()
             engine = saver._get_engine()
-            down = min(engine.link_probe(scratch.data_ptr(), probe_bytes, True) for _ in range(3))
-            up = min(engine.link_probe(scratch.data_ptr(), probe_bytes, False) for _ in range(3))
+            down, up = [], []
+            for _ in range(3):  # directions alternate, the best of each counts
+                down.append(engine.link_probe(scratch.data_ptr(), probe_bytes, True))
+                up.append(engine.link_probe(scratch.data_ptr(), probe_bytes, False))
+            down, up = min(down), min(up)
             del scratch
             link = {"d2h_peak_GBps": round(probe_bytes / 1e9 / down, 2), "h2d_peak_GBps": round(probe_bytes / 1e9 / up, 2),
                     "bytes": probe_bytes, "slot_mib": args.slot_mib, "streams": 2,

@@ -15,12 +15,14 @@ them (checkpoint_saver.py:340-343,533-619,709-762).
 """
 
 import concurrent.futures
+import contextlib
 import ctypes
 import dataclasses
 import logging
 import os
 import pickle
 import subprocess
+import sys
 import tempfile
 import threading
 import time
@@ -85,6 +87,8 @@ _IMAGE_PIECE_BYTES = 8 << 30
 
 # a window or piece of an image starts this many bytes (modulo) into its device buffer as into the image
 _WINDOW_PAD = 4096
+# the buffer that the windows of an image too large for HBM pass through: a quarter of the limit, at most this
+_WINDOW_BUFFER_BYTES = 8 << 30
 
 _MAX_KEPT_PLANS = 64  # objects per save are few (one per writer thread); beyond this the oldest is rebuilt
 
@@ -580,13 +584,14 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             kept.plan.destroy()  # releasing device memory waits for the kernels that still use it
 
     @staticmethod
-    def _windows_of(layout: hip_plan.SaveLayout, limit: int) -> list:
-        """Consecutive rows of the layout's table grouped into windows of at most ``limit`` image bytes (a single
-        larger row gets a window of its own): [(first row, end row, first image byte, end)]."""
+    def _windows_of(layout: hip_plan.SaveLayout, limit: int, stop: Optional[int] = None) -> list:
+        """Consecutive rows of the layout's table (the first ``stop`` of them) grouped into windows of at most
+        ``limit`` image bytes (a single larger row gets a window of its own): [(first row, end row, first image
+        byte, end)]."""
         arr = layout.items
         ends = (arr["image_off"] + arr["nbytes"]).tolist()
         starts = arr["image_off"].tolist()
-        windows, r0, n = [], 0, len(arr)
+        windows, r0, n = [], 0, len(arr) if stop is None else stop
         while r0 < n:
             r1 = r0 + 1
             while r1 < n and ends[r1] - starts[r0] <= limit:
@@ -645,10 +650,13 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         return staged
 
     def _stage_windowed(self, layout, items, object_id, object_name, device, stats: dict) -> StagedObject:
-        """Fallback for an object whose image does not fit in HBM beside the live state: consecutive records are
-        grouped into windows of at most the image limit (a single larger record gets a window of its own), and each
-        window is packed into one reusable device buffer and sent before the next is packed.  The live tensors are
-        read until the last window, so this runs to completion here, inside the blocking part of the save."""
+        """Fallback for an object whose image does not fit in HBM beside the live state.  The records at the end of
+        the object, as many as three quarters of the limit hold, are packed into an image that stays resident, like
+        the image of an ordinary save; the records before them are grouped into windows (a single larger record gets
+        a window of its own), each packed into one reusable buffer and sent before the next is packed.  The live
+        tensors of the windows are read until the last window has left, so that part runs here, inside the blocking
+        part of the save - at the link's rate; the resident image follows on a thread of this process while the
+        training step goes on.  Blocking time: (image - resident part) / link rate."""
         _LOGGER.warning("checkpoint image of %d bytes exceeds the HBM limit; saving '%s' window by window (blocking)",
                         layout.image_bytes, object_id)
         arr = layout.items
@@ -656,10 +664,19 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         if limit is None:  # what the driver reports free now, the allocator's unused segments included
             torch.cuda.empty_cache()
             limit = max(torch.cuda.mem_get_info(device)[0] - (2 << 30), 64 << 20)
-        windows = self._windows_of(layout, max(limit, 1))
+        limit = max(limit, 1)
         nbytes = layout.image_bytes
+        starts = arr["image_off"].tolist()
+        ends = (arr["image_off"] + arr["nbytes"]).tolist()
         xfer = {"d2h_s": 0.0, "d2h_wait_s": 0.0, "d2h_bytes": 0}
-        with self._chkpt_obj_manager.acquire_buffer(object_id, max(self._initial_buffer_size_bytes, nbytes)) as writer:
+        staged = StagedObject(layout, None, None, device.index or 0, 0, items)
+        staged.consumed = True
+        staged.future = concurrent.futures.Future()
+        staged.done_marker = os.path.join(tempfile.gettempdir(), f"mlf_write_{os.getpid()}_{uuid.uuid4().hex}.done")
+        held = contextlib.ExitStack()  # the buffer stays open until the resident part has been written
+        try:
+            writer = held.enter_context(
+                self._chkpt_obj_manager.acquire_buffer(object_id, max(self._initial_buffer_size_bytes, nbytes)))
             writer.set_format_signature(CheckpointFormat.MLF_FORMAT)
             ensure = getattr(writer, "ensure_capacity", None)
             if ensure is not None:
@@ -669,12 +686,13 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                 start = writer.tell()
                 writer.next_buffer_slice(nbytes).release()
                 stream = torch.cuda.current_stream(device).cuda_stream
-                # a window lies in the buffer where it lies in the image modulo the pad, so that tiles and checksum
-                # chunks are cut on the same grid as in an image held whole
-                buf = torch.empty(max(e - b for _, _, b, e in windows) + _WINDOW_PAD, dtype=torch.uint8, device=device)
                 engine = self._get_engine()
                 sums = integrity.ChunkChecksums(self._crc_chunk_bytes, nbytes) if self._crc_chunk_bytes and nbytes else None
-                for r0, r1, begin, end in windows:
+
+                def pack_rows(r0, r1, begin, end, buf):
+                    """Rows [r0, r1) = image bytes [begin, end) into ``buf``.  They lie in the buffer where they lie
+                    in the image modulo the pad, so that tiles and checksum chunks are cut on the same grid as in
+                    an image held whole.  Returns the plan and the pad."""
                     pad = begin % _WINDOW_PAD
                     sub = arr[r0:r1].copy()
                     sub["image_off"] -= begin - pad
@@ -689,34 +707,98 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                             (t_begin, t_end, int(sub["nbytes"][sub["kind"] == hip_plan.ITEM_DEVICE].sum())))
                     else:
                         plan.pack(buf, stream)
+                    return plan, pad
+
+                def checksum(buf, pad, begin, end, dst, on_stream):
+                    # windows end where records end, not where checksum chunks end: the parts are checksummed where
+                    # they lie in the buffer and joined per chunk
+                    t0 = time.perf_counter()
+                    sums.add(begin, end - begin,
+                             hip_plan.crc32c_device_cut(buf, pad, begin, end - begin, self._crc_chunk_bytes, dst, on_stream))
+                    xfer["crc_s"] = xfer.get("crc_s", 0.0) + time.perf_counter() - t0
+
+                # the resident part: the longest run of records at the end that fits beside the window buffer
+                cycle = max(min(limit // 4, _WINDOW_BUFFER_BYTES), 1)
+                room = limit - cycle - 2 * _WINDOW_PAD
+                tail_row = len(arr)
+                while tail_row > 0 and ends[-1] - starts[tail_row - 1] <= room:
+                    tail_row -= 1
+                tail = None  # (plan, image, pad, first byte, event)
+                if 0 < tail_row < len(arr):
+                    tail_begin = starts[tail_row]
+                    image = hip_plan.try_allocate(tail_begin % _WINDOW_PAD + nbytes - tail_begin, device)
+                    if image is not None:
+                        plan, pad = pack_rows(tail_row, len(arr), tail_begin, nbytes, image)
+                        packed = torch.cuda.Event()
+                        packed.record()
+                        tail = (plan, image, pad, tail_begin, packed)
+                if tail is None:
+                    tail_row, cycle = len(arr), limit
+                windows = self._windows_of(layout, cycle, tail_row)
+                buf = torch.empty(max(e - b for _, _, b, e in windows) + _WINDOW_PAD, dtype=torch.uint8, device=device)
+                for r0, r1, begin, end in windows:
+                    plan, pad = pack_rows(r0, r1, begin, end, buf)
                     dst = writer.data_address(start + begin)
                     st = engine.d2h(buf.data_ptr() + pad, dst, end - begin, stream)
                     if sums is not None:
-                        # windows end where records end, not where checksum chunks end: the parts are checksummed
-                        # where they lie in the buffer and joined per chunk
-                        t0 = time.perf_counter()
-                        sums.add(begin, end - begin, hip_plan.crc32c_device_cut(buf, pad, begin, end - begin,
-                                                                                 self._crc_chunk_bytes, dst, stream))
-                        xfer["crc_s"] = xfer.get("crc_s", 0.0) + time.perf_counter() - t0
+                        checksum(buf, pad, begin, end, dst, stream)
                     plan.destroy()
                     xfer["d2h_s"] += st.seconds
                     xfer["d2h_bytes"] += end - begin
-            if sums is not None:
-                integrity.write_sidecar(str(object_id), self._crc_chunk_bytes, nbytes, sums.result())
-            else:
-                integrity.remove_sidecar(str(object_id))
+                del buf
+        except BaseException:
+            held.__exit__(*sys.exc_info())
+            raise
+
+        def finish():
+            """The resident part, the sidecar, the buffer's close: on the caller's thread when there is no resident
+            part, else on a thread of its own."""
+            try:
+                with held:
+                    if tail is not None:
+                        plan, image, pad, tail_begin, packed = tail
+                        with torch.cuda.device(device):
+                            _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
+                            dst = writer.data_address(start + tail_begin)
+                            st, _ = engine.d2h_gated(image.data_ptr() + pad, dst, nbytes - tail_begin, packed.cuda_event, 0,
+                                                     ctypes.c_uint64(0))
+                            xfer["d2h_s"] += st.seconds
+                            xfer["d2h_bytes"] += nbytes - tail_begin
+                            if sums is not None:
+                                # on a stream of its own: the training step's kernels are queued on the pack's
+                                checksum(image, pad, tail_begin, nbytes, dst, torch.cuda.Stream(device=device).cuda_stream)
+                            plan.destroy()
+                if sums is not None:
+                    integrity.write_sidecar(str(object_id), self._crc_chunk_bytes, nbytes, sums.result())
+                else:
+                    integrity.remove_sidecar(str(object_id))
+                outcome = (True, self._results_of(staged, object_name))
+            except BaseException as e:  # reported to whoever waits; a thread must not die silently
+                _LOGGER.exception("Windowed write of '%s' failed", object_id)
+                outcome = (False, f"{type(e).__name__}: {e}", e)
+            stats.update({k: stats.get(k, 0) + v for k, v in xfer.items()})  # (the dict last_save_stats refers to)
+            if tail is None and not outcome[0]:
+                raise outcome[2]
+            try:
+                tmp = staged.done_marker + ".tmp"
+                with open(tmp, "wb") as f:
+                    pickle.dump(outcome[:2], f)
+                os.rename(tmp, staged.done_marker)
+            finally:
+                if outcome[0]:
+                    staged.future.set_result(outcome[1])
+                else:
+                    staged.future.set_exception(RuntimeError(outcome[1]))
+
         stats["objects"] += 1
         stats["windows"] = stats.get("windows", 0) + len(windows)
         stats["device_payload_bytes"] += layout.device_payload_bytes
         stats["image_bytes"] += nbytes
-        stats.update({k: stats.get(k, 0) + v for k, v in xfer.items()})
-        staged = StagedObject(layout, None, None, device.index or 0, 0, items)
-        staged.consumed = True
-        staged.future = concurrent.futures.Future()
-        staged.future.set_result(self._results_of(staged, object_name))
-        staged.done_marker = os.path.join(tempfile.gettempdir(), f"mlf_write_{os.getpid()}_{uuid.uuid4().hex}.done")
-        with open(staged.done_marker, "wb") as f:
-            pickle.dump((True, staged.future.result()), f)
+        if tail is None:
+            finish()
+        else:
+            stats["resident_bytes"] = stats.get("resident_bytes", 0) + nbytes - tail[3]
+            threading.Thread(target=finish, name=f"mlf-write-{object_name}", daemon=True).start()
         return staged
 
     @staticmethod
@@ -756,7 +838,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             except Exception as e:  # collected, first one re-raised: same contract as the reference's workers
                 _LOGGER.exception("Error writing object '%s'", bucket.object_id)
                 errors.append(e)
-        self.last_save_stats = {**self.last_save_stats, **xfer}
+        # (a save that went window by window has counted its transfers already)
+        self.last_save_stats = {**self.last_save_stats, **{k: self.last_save_stats.get(k, 0) + v for k, v in xfer.items()}}
         if errors:
             raise errors[0]
         return all_results

@@ -518,6 +518,75 @@ def test_object_larger_than_the_hbm_limit_is_saved_window_by_window(shm_dir, man
             assert torch.equal(_bits(target[k]), _bits(v)), k
 
 
+def test_windowed_save_keeps_the_end_of_the_object_resident_and_sends_it_behind_the_blocking_part(shm_dir):
+    """With room for part of the image only, the records at the end of the object stay in HBM as a snapshot and are
+    sent by a thread after ``prepare_write_data`` has returned; the records before them go window by window inside
+    it.  Overwriting every live tensor right after that call must not change what lands in the file."""
+    from torch.distributed.checkpoint.planner_helpers import _create_write_items
+
+    from ml_flashpoint.hip import integrity
+    from ml_flashpoint.hip import plan as P
+
+    g = torch.Generator().manual_seed(31)
+    data_cpu = {f"t{i:02d}": torch.randn(40_000 + 1_000 * i, generator=g) for i in range(14)}  # 2.6 MB
+    data_cpu["blob"] = io.BytesIO(b"x" * 1000)
+    data = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in data_cpu.items()}
+    saver = _saver(max_image_bytes=1 << 20, crc_chunk_bytes=1 << 16)
+    cid = CheckpointContainerId(os.path.join(shm_dir, "step-12_ckpt"))
+    items = [wi for k, v in data.items() for wi in _create_write_items(k, v)]
+    buckets = saver.prepare_write_data(cid, items, _Resolver(data), "data", 1)
+    stats = saver.last_save_stats
+    assert stats["windows"] >= 3 and 0 < stats["resident_bytes"] <= (1 << 20) * 3 // 4
+    for v in data.values():  # the training step goes on
+        if isinstance(v, torch.Tensor):
+            v.fill_(-1.0)
+    torch.cuda.synchronize()
+    results = saver.write_data(cid, buckets, replicate_after_write=False, thread_count=1)
+    assert saver.last_save_stats["d2h_bytes"] == sum(r.size_in_bytes for r in results)
+    path = os.path.join(cid.data, "data_0_src0.distcp")
+    raw = open(path, "rb").read()
+    order = sorted(results, key=lambda r: r.storage_data.offset)
+    tensors = [data_cpu[r.index.fqn] for r in order if r.index.fqn != "blob"]
+    assert raw == fmt.file_image(tensors, [b"x" * 1000])[0]
+    chunk, nbytes, crcs = integrity.read_sidecar(path)
+    assert nbytes == len(raw) - METADATA_SIZE and len(crcs) == -(-nbytes // chunk)
+    for k, c in enumerate(crcs):
+        piece = raw[METADATA_SIZE + k * chunk : METADATA_SIZE + (k + 1) * chunk]
+        buf = ctypes.create_string_buffer(piece, len(piece))
+        assert P.crc32c_host(ctypes.addressof(buf), len(piece)) == int(c), k
+    with pytest.raises(ValueError, match="already written"):
+        saver.write_data(cid, buckets, replicate_after_write=False, thread_count=1)
+
+
+def test_windowed_save_reports_a_failure_of_the_part_that_follows(shm_dir, monkeypatch):
+    """The resident part is written by a thread; what goes wrong there reaches ``write_data``, and the saver stays
+    usable."""
+    from torch.distributed.checkpoint.planner_helpers import _create_write_items
+
+    from ml_flashpoint.hip import integrity
+
+    data = {f"t{i}": torch.full((50_000,), float(i), device=DEV) for i in range(10)}
+    saver = _saver(max_image_bytes=1 << 20, crc_chunk_bytes=1 << 16)
+    items = [wi for k, v in data.items() for wi in _create_write_items(k, v)]
+
+    def refuse(*a, **kw):
+        raise OSError("no room for the sidecar")
+
+    monkeypatch.setattr(integrity, "write_sidecar", refuse)
+    cid = CheckpointContainerId(os.path.join(shm_dir, "step-13_ckpt"))
+    buckets = saver.prepare_write_data(cid, items, _Resolver(data), "data", 1)
+    assert saver.last_save_stats["resident_bytes"] > 0
+    with pytest.raises(RuntimeError, match="no room for the sidecar"):
+        saver.write_data(cid, buckets, replicate_after_write=False, thread_count=1)
+    monkeypatch.undo()
+    cid = CheckpointContainerId(os.path.join(shm_dir, "step-14_ckpt"))
+    buckets = saver.prepare_write_data(cid, items, _Resolver(data), "data", 1)
+    results = saver.write_data(cid, buckets, replicate_after_write=False, thread_count=1)
+    raw = open(os.path.join(cid.data, "data_0_src0.distcp"), "rb").read()
+    order = sorted(results, key=lambda r: r.storage_data.offset)
+    assert raw == fmt.file_image([data[r.index.fqn].cpu() for r in order])[0]
+
+
 @pytest.mark.parametrize("background_write", [False, True])
 def test_image_is_held_in_pieces_when_no_single_block_is_to_be_had(shm_dir, manager_future, monkeypatch, background_write):
     """Free device memory that is not in one block (the usual state of a long-running job): the image is packed into
