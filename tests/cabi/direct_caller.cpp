@@ -1,7 +1,9 @@
 // A caller of the two C-ABI libraries with no Python and no torch in the process: the way a C++ component of the
 // reference (its transfer service already links the buffer object) would use them.  One object with a contiguous
 // tensor, a transposed view and a record header is packed, checksummed, sent into a buffer file, read back through
-// the file descriptor and unpacked into fresh device memory; every stage is compared with bytes built on the host.
+// the file descriptor and unpacked into fresh device memory; then the same object once more with the checksums folded
+// into the pack and the unpack, a transfer gated on an event, and the checksum entry point that allocates nothing.
+// Every stage is compared with bytes built on the host.
 //
 // Build (gfx950, no GPU needed):  see __graft_entry__.build().   Run on an MI355X:  tests/cabi/_build/direct_caller <dir>
 #include "mlf_buffer.h"
@@ -9,6 +11,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
@@ -30,8 +33,8 @@ int main(int argc, char** argv) {
   REQUIRE(mlf_hip_device_count(&devices) == 0 && devices >= 1);
   REQUIRE(mlf_hip_set_device(0) == 0);
 
-  // host truth: a 300 x 70 float matrix A, and a 64 x 48 int16 matrix B that is saved through its transpose
-  const int ar = 300, ac = 70, br = 64, bc = 48;
+  // host truth: a 300 x 700 float matrix A (840 kB: it covers whole 64 KiB pieces of the image), and a 64 x 48 int16 matrix B that is saved through its transpose
+  const int ar = 300, ac = 700, br = 64, bc = 48;
   std::vector<float> a(ar * ac);
   std::vector<int16_t> b(br * bc);
   for (size_t i = 0; i < a.size(); ++i) a[i] = 0.25f * (float)i - 1000.0f;
@@ -121,6 +124,68 @@ int main(int argc, char** argv) {
   REQUIRE(hipMemcpy(a2.data(), d_a, a_bytes, hipMemcpyDeviceToHost) == hipSuccess);
   REQUIRE(hipMemcpy(b2.data(), d_b, b_bytes, hipMemcpyDeviceToHost) == hipSuccess);
   REQUIRE(std::memcmp(a2.data(), a.data(), a_bytes) == 0 && std::memcmp(b2.data(), b.data(), b_bytes) == 0);
+
+  // ---- checksums folded into the copy: one value per 64 KiB chunk of the image, from the pack and from the unpack ----
+  const uint64_t chunk = 65536, n_chunks = (image_bytes + chunk - 1) / chunk;
+  std::vector<uint32_t> chunk_want(n_chunks), chunk_got(n_chunks);
+  for (uint64_t k = 0; k < n_chunks; ++k)
+    chunk_want[k] = mlf_crc32c_host(want.data() + k * chunk, std::min(chunk, image_bytes - k * chunk));
+  mlf_plan_opts fopts;
+  std::memset(&fopts, 0, sizeof fopts);
+  fopts.crc_chunk_kib = 64;
+  mlf_plan* fused = nullptr;
+  REQUIRE(hipMemcpy(d_a, a.data(), a_bytes, hipMemcpyHostToDevice) == hipSuccess);
+  REQUIRE(hipMemcpy(d_b, b.data(), b_bytes, hipMemcpyHostToDevice) == hipSuccess);
+  REQUIRE(hipMemset(d_image, 0xCD, image_bytes + 256) == hipSuccess);
+  REQUIRE(mlf_plan_create(items.data(), items.size(), header, hdr, image_bytes, &fopts, &fused) == 0);
+  REQUIRE(mlf_plan_get_info(fused, &info) == 0 && info.crc_chunks == n_chunks && info.fused_crc_bytes >= 10 * chunk);
+  REQUIRE(mlf_pack_launch(fused, d_image, nullptr) == 0);
+  hipEvent_t packed = nullptr;  // what a transfer on another thread would wait for
+  REQUIRE(hipEventCreateWithFlags(&packed, hipEventDisableTiming) == hipSuccess && hipEventRecord(packed, nullptr) == hipSuccess);
+  REQUIRE(hipDeviceSynchronize() == hipSuccess);
+  REQUIRE(mlf_plan_crc_values(fused, chunk_got.data(), n_chunks) == 0 && chunk_got == chunk_want);
+  REQUIRE(hipMemcpy(got.data(), d_image, image_bytes + 256, hipMemcpyDeviceToHost) == hipSuccess);
+  REQUIRE(std::memcmp(got.data(), want.data(), image_bytes) == 0 && got[image_bytes] == 0xCD);
+
+  // the entry point that allocates nothing: values into caller-provided device memory
+  uint32_t* d_vals = nullptr;
+  REQUIRE(hipMalloc(reinterpret_cast<void**>(&d_vals), n_chunks * 4) == hipSuccess);
+  REQUIRE(mlf_crc32c_device_noalloc(d_image, image_bytes, chunk, d_vals, n_chunks, nullptr) == 0);
+  REQUIRE(hipDeviceSynchronize() == hipSuccess);
+  REQUIRE(hipMemcpy(chunk_got.data(), d_vals, n_chunks * 4, hipMemcpyDeviceToHost) == hipSuccess && chunk_got == chunk_want);
+
+  // a second buffer file, its pages and page-table entries made ahead; the transfer waits for the event, not the stream
+  const std::string path2 = dir + "/cabi_direct_caller_2.distcp";
+  mlf_buffer* buf2 = nullptr;
+  REQUIRE(mlf_buffer_create(path2.c_str(), 4096 + image_bytes, 1, &buf2) == 0);
+  REQUIRE(mlf_buffer_prefault(buf2, 4096, image_bytes, 2) == 0);
+  char* dst2 = static_cast<char*>(mlf_buffer_data_ptr(buf2)) + 4096;
+  landed = 0;
+  std::fill(chunk_got.begin(), chunk_got.end(), 0u);
+  REQUIRE(mlf_engine_d2h_gated(engine, d_image, dst2, image_bytes, packed, chunk, chunk_got.data(), n_chunks, &landed, &stats) == 0);
+  REQUIRE(landed == image_bytes && chunk_got == chunk_want && std::memcmp(dst2, want.data(), image_bytes) == 0);
+  double seconds = 0;
+  REQUIRE(mlf_engine_link_probe(engine, d_image, image_bytes, 1, &seconds) == 0 && seconds > 0);
+
+  // unpack with checksums: the values of the image it read, the tensors as they were
+  REQUIRE(hipMemset(d_a, 0, a_bytes) == hipSuccess && hipMemset(d_b, 0, b_bytes) == hipSuccess);
+  fopts.align_to_tensor = 1;
+  mlf_plan* fused_back = nullptr;
+  REQUIRE(mlf_plan_create(items.data(), items.size(), header, hdr, image_bytes, &fopts, &fused_back) == 0);
+  REQUIRE(mlf_unpack_launch(fused_back, d_image, nullptr) == 0);
+  REQUIRE(hipDeviceSynchronize() == hipSuccess);
+  std::fill(chunk_got.begin(), chunk_got.end(), 0u);
+  REQUIRE(mlf_plan_crc_values(fused_back, chunk_got.data(), n_chunks) == 0 && chunk_got == chunk_want);
+  REQUIRE(hipMemcpy(a2.data(), d_a, a_bytes, hipMemcpyDeviceToHost) == hipSuccess);
+  REQUIRE(hipMemcpy(b2.data(), d_b, b_bytes, hipMemcpyDeviceToHost) == hipSuccess);
+  REQUIRE(std::memcmp(a2.data(), a.data(), a_bytes) == 0 && std::memcmp(b2.data(), b.data(), b_bytes) == 0);
+  mlf_plan_destroy(fused);
+  mlf_plan_destroy(fused_back);
+  REQUIRE(mlf_buffer_close(buf2, 1, 4096 + image_bytes) == 0);
+  mlf_buffer_destroy(buf2);
+  std::remove(path2.c_str());
+  (void)hipFree(d_vals);
+  (void)hipEventDestroy(packed);
 
   // a descriptor that reaches outside the image is refused with a message, nothing is launched
   items[1].image_off = image_bytes - 4;
