@@ -27,6 +27,7 @@ import tempfile
 import threading
 import time
 import uuid
+import weakref
 from typing import Callable, Optional, Union
 
 import numpy as np
@@ -90,6 +91,8 @@ _WINDOW_PAD = 4096
 # the buffer that the windows of an image too large for HBM pass through: a quarter of the limit, at most this
 _WINDOW_BUFFER_BYTES = 8 << 30
 
+_FUSED_VALUES_LOCK = threading.Lock()
+
 _MAX_KEPT_PLANS = 64  # objects per save are few (one per writer thread); beyond this the oldest is rebuilt
 
 
@@ -101,6 +104,9 @@ class _KeptPlan:
         # the table has the device addresses and host tensors are looked up again by index: hold no tensors
         self.layout = dataclasses.replace(layout, device_tensors=[], host_tensors=[])
         self.blob = layout.blob
+        # with checksums folded into the pack: the object of the last launch, until its values have been taken (a
+        # plan holds the values of its last launch only)
+        self.last_staged: Optional[weakref.ReferenceType] = None
 
     def refreshed_blob(self, tensors, blobs) -> Optional[bytes]:
         """The blob with the current bytes of its variable parts, or None if nothing changed since last time."""
@@ -144,6 +150,7 @@ class StagedObject:
         self.data_offset: Optional[int] = None  # position of the image's first byte in the object's data section
         # an image that is held in several device buffers: [(plan, buffer, first image byte, end)], in order
         self.pieces: Optional[list] = None
+        self.fused_crcs = None  # chunk checksums out of the pack, once taken from the plan
 
     def landed_bytes(self) -> int:
         """Leading bytes of the image that are in place in the buffer file (from byte 4096 + ``data_offset`` of the
@@ -525,6 +532,11 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                 stream = torch.cuda.current_stream(device).cuda_stream
                 if kept is not None:
                     plan = kept.plan
+                    earlier = kept.last_staged() if kept.last_staged is not None else None
+                    if earlier is not None and earlier.plan is plan:
+                        # a save that is still waiting to be written: its checksums leave the plan before this
+                        # launch overwrites them
+                        self._fused_checksums(earlier)
                     if fresh_blob is not None:  # step counters, RNG state, pickled objects: new bytes, same places
                         plan.update_blob(fresh_blob, stream)
                     stats["plans_reused"] = stats.get("plans_reused", 0) + 1
@@ -554,6 +566,10 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         staged = StagedObject(layout, plan, image, device.index or 0, stream, items)
         staged.packed_event = packed if layout.image_bytes else None
         staged.owns_plan = key is None  # with a key the plan went into, or came out of, the kept plans
+        if plan is not None and plan.crc_chunk_bytes and key is not None:
+            holder = self._plan_cache.get(object_name)
+            if holder is not None and holder.plan is plan:
+                holder.last_staged = weakref.ref(staged)
         return staged
 
     # ---- plans kept from save to save ---------------------------------------------------------------------
@@ -1004,7 +1020,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                         crcs = self._transfer_in_pieces(staged, writer, start, xfer)
                     elif fd >= 0:
                         if staged.plan is not None and staged.plan.crc_chunk_bytes:
-                            crcs = staged.plan.crc_values()
+                            crcs = self._fused_checksums(staged)
                         elif self._crc_chunk_bytes:
                             crcs = hip_plan.crc32c_device(staged.image, nbytes, self._crc_chunk_bytes, staged.stream)
                         st = engine.d2h_fd(staged.image.data_ptr(), fd, METADATA_SIZE + start, nbytes, staged.stream)
@@ -1013,7 +1029,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                         # the pack folded the checksums: take them now, before the plan (kept for the next save) is
                         # launched again
                         t0 = time.perf_counter()
-                        crcs = staged.plan.crc_values()
+                        crcs = self._fused_checksums(staged)
                         xfer["crc_s"] = xfer.get("crc_s", 0.0) + time.perf_counter() - t0
                         st, _ = self._send_image(engine, staged, writer.data_address(start), nbytes, 0)
                         self._count_transfer(xfer, st, nbytes)
@@ -1036,6 +1052,15 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         else:
             integrity.remove_sidecar(str(bucket.object_id))
         return self._results_of(staged, bucket.object_name)
+
+    @staticmethod
+    def _fused_checksums(staged: StagedObject):
+        """The chunk checksums that the pack of ``staged`` left in its plan - unless a later save has launched the
+        same (kept) plan since and moved them into ``staged`` before it did."""
+        with _FUSED_VALUES_LOCK:  # the writer's thread and the next save's launch may both come for them
+            if staged.fused_crcs is None:
+                staged.fused_crcs = staged.plan.crc_values()
+        return staged.fused_crcs
 
     @staticmethod
     def _send_image(engine, staged: StagedObject, dst_host_ptr: int, nbytes: int, crc_chunk_bytes: int):

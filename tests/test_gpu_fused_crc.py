@@ -252,3 +252,54 @@ def test_saver_and_loader_checksum_modes_agree(shm_dir, background_write):
         assert isinstance(cause, integrity.ChecksumMismatchError) and "chunk(s) [5]" in str(cause), mode
         if mode == "before":  # nothing was written before the mismatch was found
             assert all(not bool(v.any()) for v in target.values() if isinstance(v, torch.Tensor))
+
+
+def test_two_saves_prepared_before_either_is_written_keep_their_own_checksums(shm_dir):
+    """A kept plan holds the checksums of its last launch only.  When the next save is prepared (and the plan launched
+    again, over changed tensors) before the previous one has been written, the previous one's values must have left
+    the plan: each object's sidecar describes that object's bytes."""
+    import ctypes
+    import os
+
+    from torch.distributed.checkpoint.planner_helpers import _create_write_items
+
+    from ml_flashpoint.checkpoint_object_manager.buffer_metadata import METADATA_SIZE
+    from ml_flashpoint.checkpoint_object_manager.checkpoint_object_manager import CheckpointObjectManager
+    from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId
+    from ml_flashpoint.core.checkpoint_saver import DefaultMLFlashpointCheckpointSaver
+    from ml_flashpoint.hip import integrity
+    from ml_flashpoint.hip import plan as P
+
+    class Resolver:
+        def __init__(self, data):
+            self.data = data
+
+        def resolve_data(self, item):
+            return self.data[item.index.fqn]
+
+    g = torch.Generator().manual_seed(3)
+    data = {f"w{i}": torch.randn(300_000, generator=g).to(DEV) for i in range(4)}  # 4.8 MB: whole 64 KiB pieces
+    items = [wi for k, v in data.items() for wi in _create_write_items(k, v)]
+    CheckpointObjectManager._worker_pool = None
+    saver = DefaultMLFlashpointCheckpointSaver(lambda: 0, lambda: 0, lambda: None, CheckpointObjectManager(), None,
+                                               initial_buffer_size_bytes=1 << 20, crc_chunk_bytes=1 << 16, crc_mode="fused")
+    cids = [CheckpointContainerId(os.path.join(shm_dir, f"step-{n}_ckpt")) for n in (1, 2)]
+    first = saver.prepare_write_data(cids[0], items, Resolver(data), "data", 1)
+    for v in data.values():
+        v.mul_(-3.0)  # the next step's values
+    second = saver.prepare_write_data(cids[1], items, Resolver(data), "data", 1)
+    assert saver.last_save_stats.get("plans_reused") == 1
+    saver.write_data(cids[0], first, replicate_after_write=False, thread_count=1)
+    saver.write_data(cids[1], second, replicate_after_write=False, thread_count=1)
+    raws = []
+    for cid in cids:
+        path = os.path.join(cid.data, "data_0_src0.distcp")
+        raw = open(path, "rb").read()
+        raws.append(raw)
+        chunk, nbytes, crcs = integrity.read_sidecar(path)
+        assert nbytes == len(raw) - METADATA_SIZE
+        for k, c in enumerate(crcs):
+            piece = raw[METADATA_SIZE + k * chunk : METADATA_SIZE + (k + 1) * chunk]
+            buf = ctypes.create_string_buffer(piece, len(piece))
+            assert P.crc32c_host(ctypes.addressof(buf), len(piece)) == int(c), (cid.data, k)
+    assert raws[0] != raws[1]
