@@ -81,6 +81,8 @@ def parse_args():
     ap.add_argument("--max-image-gb", type=float, default=0.0,
                     help="cap on the image held in HBM at once (saver and loader): smaller than the object, the save "
                          "goes window by window and blocks for the transfer; 0 = what the device has free")
+    ap.add_argument("--whole-image-restore", action="store_true",
+                    help="restore through one device buffer for the whole object instead of two alternating ones")
     ap.add_argument("--no-prefault", action="store_true", help="leave the pool file's pages to the first save, as the reference does")
     ap.add_argument("--no-link-probe", action="store_true", help="skip the bare host-link measurement")
     ap.add_argument("--no-crc-compare", action="store_true", help="skip the extra saves in the other checksum mode")
@@ -330,7 +332,8 @@ def main():
     saver = make_saver(args.save_crc)
     loader = DefaultMLFlashpointCheckpointLoader(manager, None, engine_config=engine_cfg, tile_bytes=args.tile_bytes,
                                                  block_threads=args.block_threads, use_file_io=args.restore_io == "file",
-                                                 crc_mode=args.restore_crc, max_image_bytes=max_image)
+                                                 crc_mode=args.restore_crc, max_image_bytes=max_image,
+                                                 pipelined_restore=not args.whole_image_restore)
     loader.record_kernel_events = True
     result = None
     if args.pmc_calibration:
@@ -422,6 +425,7 @@ def main():
                        "pack_ms": sv["pack_ms"], "unpack_ms": unpack_ms, "pack_bytes": sv["pack_bytes"], "unpack_bytes": unpack_bytes,
                        "r_read": ld.get("read_s", 0.0), "r_parse": ld.get("parse_s", 0.0), "r_table": ld.get("table_s", 0.0),
                        "r_crc": ld.get("crc_s", 0.0), "r_unpack_plan": ld.get("unpack_plan_s", 0.0),
+                       "r_plan_beside": ld.get("unpack_plan_beside_h2d_s", 0.0), "r_windows": ld.get("windows", 0),
                        "r_unpack": ld.get("unpack_s", 0.0), "r_commit": ld.get("commit_s", 0.0),
                        "windows": d2h.get("windows", 0), "image_pieces": d2h.get("image_pieces", 0)}
                 for k, v in row.items():
@@ -525,7 +529,8 @@ def main():
                        "engine": {"slot_mib": args.slot_mib, "slots": args.slots, "copy_threads": engine_cfg.resolved_copy_threads()},
                        "crc_chunk_mib": args.crc_chunk_mib, "save_crc": args.save_crc, "restore_crc": args.restore_crc,
                        "plan_cache": args.plan_cache, "save_io": args.save_io, "restore_io": args.restore_io,
-                       "max_image_gb": args.max_image_gb, "pool_prefault": not args.no_prefault},
+                       "max_image_gb": args.max_image_gb, "pool_prefault": not args.no_prefault,
+                       "restore": "one image" if args.whole_image_restore else "two alternating buffers"},
             **({"partial_restore": partial} if partial else {}),
             "save_GBps": round(save_gbps, 3),
             "restore_GBps": round(restore_gbps, 3),
@@ -547,6 +552,7 @@ def main():
                 "parse_headers_resolve_targets": ms("r_parse"), "descriptor_table": ms("r_table"), "h2d": ms("h2d"),
                 "of_h2d_filling_pinned_slots": ms("h2d_host"),  # pread() into the slots, overlapped with the copies
                 "checksum_pass": ms("r_crc"), "unpack_plan": ms("r_unpack_plan"),
+                "unpack_plans_built_beside_h2d": ms("r_plan_beside"), "windows": int(mean(rec["r_windows"])),
                 "unpack_and_sync": ms("r_unpack"), "commit": ms("r_commit"),
                 "other_in_read_data": round((mean(rec["r_read"]) - restore_known) * 1e3, 2)},
             "pack_GBps": round(pack_gbps, 1),

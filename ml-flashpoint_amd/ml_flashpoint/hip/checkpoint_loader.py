@@ -12,6 +12,7 @@ Items whose target lives on the host, byte-blob items, and objects in the legacy
 on the host, the way the reference serves them.
 """
 
+import concurrent.futures
 import io
 import logging
 import os
@@ -57,6 +58,15 @@ _PARTIAL_READ_MIN_SAVING = 256 << 20
 # were measured at half the link's rate)
 _SLICE_ALIGN = 2 << 20
 _PARTIAL_READ_GAP = 16 << 20
+# a restore through windows alternates between two device buffers (one is unpacked while the other is filled) when
+# each can hold at least this much
+_PIPELINED_MIN_WINDOW = 128 << 10
+# a range of at least _PIPELINED_FROM_BYTES is restored through two alternating buffers by choice: a quarter of the
+# range for both together, within these bounds (measured on the 112 GB shard: 2 x 16 GB 2.03 s, 2 x 8 GB 2.055 s,
+# 2 x 2 GB 2.095 s, one image of 112 GB 2.06-2.10 s)
+_PIPELINED_FROM_BYTES = 8 << 30
+_PIPELINED_MIN_BYTES = 2 << 30
+_PIPELINED_MAX_BYTES = 32 << 30
 _U32 = struct.Struct("<I")
 _HEADER_CACHE: dict = {}  # header pickle bytes -> (dtype, shape, stored payload bytes)
 _ESZ_CACHE: dict = {}
@@ -88,6 +98,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         use_file_io: bool = True,
         verify_on_discovery: bool = False,
         max_image_bytes: Optional[int] = None,
+        pipelined_restore: bool = True,
     ):
         """Arguments as the reference's default loader (checkpoint_loader.py:126-158), plus the copy-engine and
         kernel work-split knobs, ``verify_crc`` (check the CRC-32C sidecar of an object, when it has one, while
@@ -97,7 +108,10 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         ``verify_on_discovery`` (also check it, on the host, while choosing the checkpoint to
         recover from, so that a corrupted copy counts as missing) and ``max_image_bytes`` (largest range of an
         object that is uploaded to HBM in one piece; default: what the device has free minus 2 GiB.  A larger
-        range is restored window by window through one buffer of that size)."""
+        range is restored window by window through buffers of that size together) and ``pipelined_restore`` (a
+        range of 8 GiB or more goes through two alternating buffers - a quarter of the range together, 32 GiB at
+        most - by choice: one window is unpacked while the next crosses the link, and the restore needs that much
+        HBM instead of room for the whole range.  False: one buffer for the whole range where it fits)."""
         _lib.load()
         self._checkpoint_object_manager = checkpoint_object_manager
         self._replication_manager = replication_manager
@@ -118,6 +132,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         self._use_file_io = use_file_io
         self.verify_on_discovery = verify_on_discovery
         self._max_image_bytes = max_image_bytes
+        self._pipelined_restore = pipelined_restore
         self._engine: Optional[hip_plan.CopyEngine] = None
         self._engine_lock = threading.Lock()
         self._stats_local = threading.local()  # read_data runs on one executor thread per object
@@ -378,8 +393,17 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                     need = min(need, limit)
                 else:
                     need = hi - lo
-                    image = hip_plan.try_allocate(need, device) if need <= limit else None
-                if image is None:
+                    through = self._pipelined_limit(need, limit, rows, sidecar)
+                    if through:
+                        # a large range by choice through two modest buffers: one window is unpacked while the next
+                        # crosses the link, and the restore needs that much HBM instead of room for the whole range
+                        self._restore_windowed(object_id, stream, device, rows, through, sidecar, stats, by_choice=True)
+                        image = False
+                    else:
+                        image = hip_plan.try_allocate(need, device) if need <= limit else None
+                if image is False:
+                    pass
+                elif image is None:
                     self._restore_windowed(object_id, stream, device, rows, min(limit, need), sidecar, stats)
                 elif clusters is not None:
                     self._restore_clusters(object_id, stream, device, clusters, sidecar, stats, image)
@@ -417,15 +441,35 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         stats["h2d_host_s"] = stats.get("h2d_host_s", 0.0) + st.wait_seconds  # filling the pinned slots
         stats["h2d_bytes"] += span
 
-    def _unpack(self, items, image: torch.Tensor, span: int, cur, payload_bytes: int, crc_chunk_bytes: int = 0):
-        """Launches the unpack of ``items`` out of ``image`` and waits for it: the targets are complete, and the
-        image may be reused or freed, when this returns.  With ``crc_chunk_bytes`` the unpack kernel also folds the
-        CRC-32C of every chunk of the image; those values are returned."""
+    def _unpack_plan(self, items, span: int, crc_chunk_bytes: int = 0, booked_as: str = "unpack_plan_s") -> hip_plan.Plan:
         t0 = time.perf_counter()
         plan = hip_plan.Plan(items, b"", span, tile_bytes=self._tile_bytes, block_threads=self._block_threads,
                              align_to_tensor=True, crc_chunk_bytes=crc_chunk_bytes)
         stats = self._stats_in_progress
-        stats["unpack_plan_s"] = stats.get("unpack_plan_s", 0.0) + time.perf_counter() - t0
+        stats[booked_as] = stats.get(booked_as, 0.0) + time.perf_counter() - t0
+        return plan
+
+    def _launch_unpack(self, plan: hip_plan.Plan, image: torch.Tensor, cur, payload_bytes: int) -> torch.cuda.Event:
+        """Enqueues the unpack on ``cur`` and returns the event recorded behind it: until it has passed, the image
+        is still being read and the plan's tables are in use."""
+        if self.record_kernel_events:
+            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            begin.record(cur)
+            plan.unpack(image, cur.cuda_stream)
+            end.record(cur)
+            self.kernel_events.append((begin, end, payload_bytes))
+            return end
+        plan.unpack(image, cur.cuda_stream)
+        done = torch.cuda.Event()
+        done.record(cur)
+        return done
+
+    def _unpack(self, items, image: torch.Tensor, span: int, cur, payload_bytes: int, crc_chunk_bytes: int = 0):
+        """Launches the unpack of ``items`` out of ``image`` and waits for it: the targets are complete, and the
+        image may be reused or freed, when this returns.  With ``crc_chunk_bytes`` the unpack kernel also folds the
+        CRC-32C of every chunk of the image; those values are returned."""
+        plan = self._unpack_plan(items, span, crc_chunk_bytes)
+        stats = self._stats_in_progress
         t0 = time.perf_counter()
         try:
             if self.record_kernel_events:
@@ -524,7 +568,25 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
             self._unpack(np.concatenate(tables), image, at, cur, stats["device_payload_bytes"])
         stats["partial_read_ranges"] = stats.get("partial_read_ranges", 0) + len(clusters)
 
-    def _restore_windowed(self, object_id, stream, device, rows, limit, sidecar, stats) -> None:
+    def _pipelined_limit(self, need: int, limit: int, rows, sidecar) -> int:
+        """HBM to restore a range of ``need`` bytes through, in two alternating buffers, when that is the better way
+        (0 when one buffer for the whole range is): the range is large, the checksums can be checked window by
+        window, and no row that must stay whole is larger than a window."""
+        if need < _PIPELINED_FROM_BYTES or not self._pipelined_restore:
+            return 0
+        chunk_bytes = 0
+        if sidecar is not None:
+            chunk_bytes = sidecar[0]
+            if self._crc_mode != "fused" or chunk_bytes % 65536:
+                return 0
+        through = min(limit, max(_PIPELINED_MIN_BYTES, min(_PIPELINED_MAX_BYTES, need // 4)))
+        window = through // 2 - max(chunk_bytes, _UPLOAD_ALIGN)
+        uncut = max((r[1] - r[0] for r in rows if not r[2]), default=0)
+        if window < max(uncut, 4 * chunk_bytes, _PIPELINED_MIN_WINDOW):
+            return 0
+        return through
+
+    def _restore_windowed(self, object_id, stream, device, rows, limit, sidecar, stats, by_choice: bool = False) -> None:
         """Fallback for an object whose requested range does not fit in HBM beside the live state: the rows are
         sorted by position and restored window by window through one device buffer of at most ``limit`` bytes.  A
         contiguous row larger than a window is cut into pieces; a strided one cannot be.
@@ -535,18 +597,32 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         that no window holds completely (where the rows do not continue; those of byte blobs behind the tensors)
         are checked on the host at the end.  A mismatch raises before any tensor is committed.  With
         ``crc_mode="before"``, or a buffer too small for that, the whole object is checked on the host first."""
-        _LOGGER.warning("requested range of '%s' exceeds the HBM limit of %d bytes; restoring window by window",
-                        object_id, limit)
+        if not by_choice:
+            _LOGGER.warning("requested range of '%s' exceeds the HBM limit of %d bytes; restoring window by window",
+                            object_id, limit)
         chunk_bytes, data_bytes, want = sidecar if sidecar is not None else (0, 0, None)
-        image = None
-        while image is None:  # the largest buffer the allocator really has, at most the limit
+        # Two buffers of half the limit each, so that a window is unpacked while the next one crosses the link; one
+        # buffer of whatever the allocator still has when it cannot give two.
+        buffers = []
+        uncut = max((r[1] - r[0] for r in rows if not r[2]), default=0)  # a strided row must fit a window whole
+        while not buffers:
             if limit - _UPLOAD_ALIGN < 65536:
                 if self._max_image_bytes is not None:
                     raise ValueError(f"max_image_bytes={self._max_image_bytes} is too small to restore anything")
                 raise torch.OutOfMemoryError(f"no device buffer to restore '{object_id.data}' through")
-            image = hip_plan.try_allocate(limit, device)
-            if image is None:
-                limit //= 2
+            half = limit // 2 // _UPLOAD_ALIGN * _UPLOAD_ALIGN
+            if half - max(chunk_bytes, _UPLOAD_ALIGN) >= max(_PIPELINED_MIN_WINDOW, uncut):
+                first = hip_plan.try_allocate(half, device)
+                if first is not None:
+                    second = hip_plan.try_allocate(half, device)
+                    buffers = [first] if second is None else [first, second]
+                limit = half
+            else:
+                one = hip_plan.try_allocate(limit, device)
+                if one is not None:
+                    buffers = [one]
+                else:
+                    limit //= 2
         on_device = (sidecar is not None and self._crc_mode == "fused" and chunk_bytes % 65536 == 0
                      and limit >= 4 * chunk_bytes)
         if sidecar is not None and not on_device:
@@ -577,16 +653,59 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         windows.append((lo, current))
         cur = torch.cuda.current_stream(device)
         checked = set()
-        for lo, window_rows in windows:
-            span = max(r[1] for r in window_rows) - lo
-            self._upload(stream, lo, image, span, cur, stats)
-            got = self._unpack(self._table_of(window_rows, lo), image, span, cur,
-                               sum(r[1] - r[0] for r in window_rows if r[2]), chunk_bytes if on_device else 0)
-            if on_device:
-                first = lo // chunk_bytes
-                whole = span // chunk_bytes + (1 if lo + span == data_bytes and span % chunk_bytes else 0)
-                self._compare_checksums(object_id, got[:whole], want[first : first + whole], chunk_bytes, first, len(want))
-                checked.update(range(first, first + whole))
+        # The upload of window k+1 runs on a helper thread (the engine call returns when the bytes are in HBM) while
+        # this thread builds the tables of window k and launches its unpack; a buffer is reused once the unpack that
+        # read it has passed.  Plans stay alive until their checksums have been taken.
+        in_use = [None] * len(buffers)  # event behind the last unpack out of each buffer
+        launched = []  # (plan, first chunk, complete chunks, event)
+        stats_local = self._stats_in_progress
+
+        def upload(k):
+            self._stats_local.current = stats_local  # (the helper thread books its transfer to this restore)
+            lo_k, rows_k = windows[k]
+            span_k = max(r[1] for r in rows_k) - lo_k
+            self._upload(stream, lo_k, buffers[k % len(buffers)], span_k, cur, stats)
+            return span_k
+
+        try:
+            with concurrent.futures.ThreadPoolExecutor(max_workers=1, thread_name_prefix="mlf-upload") as helper:
+                pending = helper.submit(upload, 0)
+                for k, (lo, window_rows) in enumerate(windows):
+                    span = max(r[1] for r in window_rows) - lo
+                    # (built while the window is on its way: not a part of the restore's length)
+                    plan = self._unpack_plan(self._table_of(window_rows, lo), span, chunk_bytes if on_device else 0,
+                                             booked_as="unpack_plan_s" if len(buffers) == 1 and k else "unpack_plan_beside_h2d_s")
+                    launched.append([plan, 0, 0, None])
+                    pending.result()
+                    if k + 1 < len(windows):
+                        nxt = (k + 1) % len(buffers)
+                        if len(buffers) == 1:  # the one buffer: nothing to overlap, the unpack goes first
+                            launched[-1][3] = self._launch_unpack(plan, buffers[0], cur,
+                                                                  sum(r[1] - r[0] for r in window_rows if r[2]))
+                            launched[-1][3].synchronize()
+                        elif in_use[nxt] is not None:
+                            in_use[nxt].synchronize()
+                        pending = helper.submit(upload, k + 1)
+                    if launched[-1][3] is None:
+                        launched[-1][3] = self._launch_unpack(plan, buffers[k % len(buffers)], cur,
+                                                              sum(r[1] - r[0] for r in window_rows if r[2]))
+                    in_use[k % len(buffers)] = launched[-1][3]
+                    if on_device:
+                        first = lo // chunk_bytes
+                        whole = span // chunk_bytes + (1 if lo + span == data_bytes and span % chunk_bytes else 0)
+                        launched[-1][1:3] = [first, whole]
+            t0 = time.perf_counter()
+            cur.synchronize()
+            stats["unpack_s"] = stats.get("unpack_s", 0.0) + time.perf_counter() - t0
+            for plan, first, whole, _ in launched:
+                if on_device:
+                    got = plan.crc_values()
+                    self._compare_checksums(object_id, got[:whole], want[first : first + whole], chunk_bytes, first, len(want))
+                    checked.update(range(first, first + whole))
+        finally:
+            cur.synchronize()  # nothing reads the buffers or the tables after this
+            for entry in launched:
+                entry[0].destroy()
         if on_device:  # what no window held completely: chunks where the rows do not continue, and those of byte blobs
             self._check_on_host(object_id, stream, sidecar, sorted(set(range(len(want))) - checked))
         stats["windows"] = stats.get("windows", 0) + len(windows)

@@ -715,7 +715,8 @@ def test_restore_larger_than_the_hbm_limit_goes_window_by_window(shm_dir, manage
 
 def test_restore_goes_through_a_smaller_buffer_when_no_single_block_is_to_be_had(shm_dir, manager_future, monkeypatch):
     """The loader asks for one buffer for the whole range; when the allocator has no block of that size it halves
-    its request until it gets one and restores window by window through it - same tensors."""
+    its request until it gets one (two, to alternate between, if it can have them) and restores window by window
+    through them - same tensors."""
     from ml_flashpoint.hip import plan as P
 
     sd_cpu = {f"t{i}": torch.randn(50_000, generator=torch.Generator().manual_seed(i)) for i in range(12)}  # 2.4 MB
@@ -1064,3 +1065,48 @@ def _zero():
 
 def _none():
     return None
+
+
+def test_large_ranges_go_through_two_alternating_buffers_by_choice(shm_dir, manager_future, monkeypatch):
+    """A range from a certain size on is restored through two modest buffers even when one buffer for all of it
+    could be had: a window is unpacked while the next one is uploaded.  Same tensors, the sidecar checked window by
+    window (a flipped bit is found), and ``pipelined_restore=False`` keeps the one image."""
+    from ml_flashpoint.hip import checkpoint_loader as loader_mod
+    from ml_flashpoint.hip import integrity
+
+    monkeypatch.setattr(loader_mod, "_PIPELINED_FROM_BYTES", 1 << 20)
+    monkeypatch.setattr(loader_mod, "_PIPELINED_MIN_BYTES", 1 << 20)
+    assert loader_mod._PIPELINED_MIN_BYTES // 2 > loader_mod._PIPELINED_MIN_WINDOW
+    sd_cpu = {f"t{i:02d}": torch.randn(90_000 + 777 * i, generator=torch.Generator().manual_seed(i)) for i in range(16)}
+    sd_cpu["v.t"] = torch.arange(300 * 200, dtype=torch.int32).reshape(300, 200)
+    sd_cpu["step"] = 5
+    sd_dev = _to_dev(sd_cpu)
+    ckpt = os.path.join(shm_dir, "step-21_ckpt")
+    dcp.save(sd_dev, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(_saver(crc_chunk_bytes=1 << 16), manager_future), no_dist=True)
+
+    def targets():
+        out = {k: (torch.zeros_like(v) if isinstance(v, torch.Tensor) else None) for k, v in sd_dev.items()}
+        out["v.t"] = torch.zeros(200, 300, dtype=torch.int32, device=DEV).t()  # a strided target: its row stays whole
+        return out
+
+    loader = _loader()
+    target = targets()
+    dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), no_dist=True)
+    assert loader.last_load_stats["windows"] >= 4 and target["step"] == 5
+    assert all(torch.equal(target[k].cpu(), v) for k, v in sd_cpu.items() if isinstance(v, torch.Tensor))
+    whole = _loader(pipelined_restore=False)
+    target = targets()
+    dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, whole), no_dist=True)
+    assert "windows" not in whole.last_load_stats
+    assert all(torch.equal(target[k].cpu(), v) for k, v in sd_cpu.items() if isinstance(v, torch.Tensor))
+
+    obj = os.path.join(ckpt, "__0__0_src0.distcp")
+    with open(obj, "r+b") as f:
+        f.seek(METADATA_SIZE + 9 * (1 << 16) + 5)
+        byte = f.read(1)
+        f.seek(-1, os.SEEK_CUR)
+        f.write(bytes([byte[0] ^ 0x10]))
+    with pytest.raises(BaseException) as exc:
+        dcp.load(targets(), checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), no_dist=True)
+    cause = exc.value.failures[0][0] if hasattr(exc.value, "failures") else exc.value
+    assert isinstance(cause, integrity.ChecksumMismatchError) and "chunk(s) [9]" in str(cause)
