@@ -667,7 +667,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
 
     def _stage_windowed(self, layout, items, object_id, object_name, device, stats: dict) -> StagedObject:
         """Fallback for an object whose image does not fit in HBM beside the live state.  The records at the end of
-        the object, as many as three quarters of the limit hold, are packed into an image that stays resident, like
+        the object, as many as the limit holds beside the window buffer (a quarter of it, at most 8 GiB), are packed
+        into an image that stays resident, like
         the image of an ordinary save; the records before them are grouped into windows (a single larger record gets
         a window of its own), each packed into one reusable buffer and sent before the next is packed.  The live
         tensors of the windows are read until the last window has left, so that part runs here, inside the blocking

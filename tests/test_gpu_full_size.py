@@ -64,8 +64,11 @@ NEEDS = {"llama3-8b-shard": (240e9, 125e9), "many-small": (20e9, 10e9), "mixtral
          "strided-views": (60e9, 25e9)}
 
 
-@pytest.mark.parametrize("config", ["llama3-8b-shard", "many-small", "mixtral-expert-shard", "strided-views"])
-def test_full_size_properties(config, shm_dir, oracle_c):
+@pytest.mark.parametrize("config,limit_gb", [("llama3-8b-shard", None), ("many-small", None), ("mixtral-expert-shard", None),
+                                             ("strided-views", None),
+                                             # room for part of the image only: windows, a resident end, windowed restore
+                                             ("llama3-8b-shard", 40), ("strided-views", 3)])
+def test_full_size_properties(config, limit_gb, shm_dir, oracle_c):
     from ml_flashpoint.core.checkpoint_loader import DefaultMLFlashpointCheckpointLoader
     from ml_flashpoint.core.checkpoint_saver import DefaultMLFlashpointCheckpointSaver
     from ml_flashpoint.hip import integrity
@@ -87,12 +90,16 @@ def test_full_size_properties(config, shm_dir, oracle_c):
 
     CheckpointObjectManager._worker_pool = None
     manager = CheckpointObjectManager()
+    limit = int(limit_gb * 1e9) if limit_gb else None
     saver = DefaultMLFlashpointCheckpointSaver(lambda: 0, lambda: 0, lambda: None, manager, None,
-                                               initial_buffer_size_bytes=1 << 20, crc_chunk_bytes=CHUNK)
+                                               initial_buffer_size_bytes=1 << 20, crc_chunk_bytes=CHUNK,
+                                               max_image_bytes=limit)
     fut = concurrent.futures.Future()
     fut.set_result(_LocalManager())
     ckpt = os.path.join(shm_dir, "step-1_ckpt")
     dcp.save(sd, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(saver, fut), no_dist=True)
+    if limit:
+        assert saver.last_save_stats["windows"] >= 2 and limit // 2 < saver.last_save_stats["resident_bytes"] < limit
     saver.release_device_memory()
     obj = os.path.join(ckpt, "__0__0_src0.distcp")
     metadata = pickle.load(open(os.path.join(ckpt, ".metadata"), "rb"))
@@ -173,9 +180,11 @@ def test_full_size_properties(config, shm_dir, oracle_c):
     # -- restore into zeroed tensors: bit patterns equal the originals' ------------------------------------------
     for v in sd.values():
         v.zero_() if v.is_contiguous() else v.fill_(0)
-    loader = DefaultMLFlashpointCheckpointLoader(manager, None)
+    loader = DefaultMLFlashpointCheckpointLoader(manager, None, max_image_bytes=limit)
     dcp.load(sd, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), no_dist=True)
     torch.cuda.synchronize()
+    if limit or payload >= (8 << 30):
+        assert loader.last_load_stats["windows"] >= 2
     wrong = [k for k, v in sd.items() if workloads.fingerprint(v) != prints[k]]
     assert not wrong, wrong[:5]
     assert loader.last_load_stats["device_items"] == len(sd)
