@@ -90,6 +90,8 @@ _IMAGE_PIECE_BYTES = 8 << 30
 _WINDOW_PAD = 4096
 # the buffer that the windows of an image too large for HBM pass through: a quarter of the limit, at most this
 _WINDOW_BUFFER_BYTES = 8 << 30
+# ... in two halves that alternate (one packed while the other crosses the link) where a half is at least this large
+_WINDOW_PAIR_MIN_BYTES = 64 << 10
 
 _FUSED_VALUES_LOCK = threading.Lock()
 
@@ -667,13 +669,13 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
 
     def _stage_windowed(self, layout, items, object_id, object_name, device, stats: dict) -> StagedObject:
         """Fallback for an object whose image does not fit in HBM beside the live state.  The records at the end of
-        the object, as many as the limit holds beside the window buffer (a quarter of it, at most 8 GiB), are packed
-        into an image that stays resident, like
-        the image of an ordinary save; the records before them are grouped into windows (a single larger record gets
-        a window of its own), each packed into one reusable buffer and sent before the next is packed.  The live
-        tensors of the windows are read until the last window has left, so that part runs here, inside the blocking
-        part of the save - at the link's rate; the resident image follows on a thread of this process while the
-        training step goes on.  Blocking time: (image - resident part) / link rate."""
+        the object, as many as the limit holds beside the window buffers (a quarter of it, at most 8 GiB), are packed
+        into an image that stays resident, like the image of an ordinary save; the records before them are grouped
+        into windows (a single larger record gets a window of its own) that pass through two alternating buffers:
+        one is packed while the other crosses the link.  One thread of this process sends everything, in order -
+        windows, then the resident image - checksums what it sent and closes the buffer; this call returns when the
+        last window has been packed, i.e. when nothing reads the live tensors any more.  Blocking time: about
+        (image - resident part - two windows) / link rate."""
         _LOGGER.warning("checkpoint image of %d bytes exceeds the HBM limit; saving '%s' window by window (blocking)",
                         layout.image_bytes, object_id)
         arr = layout.items
@@ -690,7 +692,10 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         staged.consumed = True
         staged.future = concurrent.futures.Future()
         staged.done_marker = os.path.join(tempfile.gettempdir(), f"mlf_write_{os.getpid()}_{uuid.uuid4().hex}.done")
-        held = contextlib.ExitStack()  # the buffer stays open until the resident part has been written
+        held = contextlib.ExitStack()  # the buffer stays open until the last byte has been written
+        sender = concurrent.futures.ThreadPoolExecutor(max_workers=1, thread_name_prefix=f"mlf-write-{object_name}")
+        sent: list = []  # one future per window, in order
+        spent: list = []  # plans whose windows have been sent
         try:
             writer = held.enter_context(
                 self._chkpt_obj_manager.acquire_buffer(object_id, max(self._initial_buffer_size_bytes, nbytes)))
@@ -705,86 +710,92 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                 stream = torch.cuda.current_stream(device).cuda_stream
                 engine = self._get_engine()
                 sums = integrity.ChunkChecksums(self._crc_chunk_bytes, nbytes) if self._crc_chunk_bytes and nbytes else None
+                # checksum kernels get a stream of their own: the training step's kernels are queued on the pack's
+                side = torch.cuda.Stream(device=device) if sums is not None else None
 
                 def pack_rows(r0, r1, begin, end, buf):
                     """Rows [r0, r1) = image bytes [begin, end) into ``buf``.  They lie in the buffer where they lie
                     in the image modulo the pad, so that tiles and checksum chunks are cut on the same grid as in
-                    an image held whole.  Returns the plan and the pad."""
+                    an image held whole.  Returns the plan, the pad and the event recorded behind the pack."""
                     pad = begin % _WINDOW_PAD
                     sub = arr[r0:r1].copy()
                     sub["image_off"] -= begin - pad
                     plan = hip_plan.Plan(sub, layout.blob, pad + end - begin, tile_bytes=self._tile_bytes,
                                          block_threads=self._block_threads)
                     if self.record_kernel_events:
-                        t_begin, t_end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                        t_begin, packed = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                         t_begin.record()
                         plan.pack(buf, stream)
-                        t_end.record()
+                        packed.record()
                         self.kernel_events.append(
-                            (t_begin, t_end, int(sub["nbytes"][sub["kind"] == hip_plan.ITEM_DEVICE].sum())))
+                            (t_begin, packed, int(sub["nbytes"][sub["kind"] == hip_plan.ITEM_DEVICE].sum())))
                     else:
                         plan.pack(buf, stream)
-                    return plan, pad
+                        packed = torch.cuda.Event()
+                        packed.record()
+                    return plan, pad, packed
 
-                def checksum(buf, pad, begin, end, dst, on_stream):
-                    # windows end where records end, not where checksum chunks end: the parts are checksummed where
-                    # they lie in the buffer and joined per chunk
-                    t0 = time.perf_counter()
-                    sums.add(begin, end - begin,
-                             hip_plan.crc32c_device_cut(buf, pad, begin, end - begin, self._crc_chunk_bytes, dst, on_stream))
-                    xfer["crc_s"] = xfer.get("crc_s", 0.0) + time.perf_counter() - t0
+                def send(plan, buf, pad, begin, end, packed):
+                    """On the sender's thread: [begin, end) out of ``buf`` into the file, its checksums, the plan's
+                    end.  Windows end where records end, not where checksum chunks end: the parts are checksummed
+                    where they lie in the buffer and joined per chunk."""
+                    with torch.cuda.device(device):
+                        _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
+                        dst = writer.data_address(start + begin)
+                        st, _ = engine.d2h_gated(buf.data_ptr() + pad, dst, end - begin, packed.cuda_event, 0,
+                                                 ctypes.c_uint64(0))
+                        xfer["d2h_s"] += st.seconds
+                        xfer["d2h_bytes"] += end - begin
+                        if sums is not None:
+                            t0 = time.perf_counter()
+                            sums.add(begin, end - begin, hip_plan.crc32c_device_cut(
+                                buf, pad, begin, end - begin, self._crc_chunk_bytes, dst, side.cuda_stream))
+                            xfer["crc_s"] = xfer.get("crc_s", 0.0) + time.perf_counter() - t0
+                        spent.append(plan)  # (released at the end: freeing device memory waits for the whole device)
 
-                # the resident part: the longest run of records at the end that fits beside the window buffer
+                # the resident part: the longest run of records at the end that fits beside the window buffers
                 cycle = max(min(limit // 4, _WINDOW_BUFFER_BYTES), 1)
-                room = limit - cycle - 2 * _WINDOW_PAD
+                room = limit - cycle - 3 * _WINDOW_PAD
                 tail_row = len(arr)
                 while tail_row > 0 and ends[-1] - starts[tail_row - 1] <= room:
                     tail_row -= 1
-                tail = None  # (plan, image, pad, first byte, event)
+                tail = None  # arguments of its send()
                 if 0 < tail_row < len(arr):
                     tail_begin = starts[tail_row]
                     image = hip_plan.try_allocate(tail_begin % _WINDOW_PAD + nbytes - tail_begin, device)
                     if image is not None:
-                        plan, pad = pack_rows(tail_row, len(arr), tail_begin, nbytes, image)
-                        packed = torch.cuda.Event()
-                        packed.record()
-                        tail = (plan, image, pad, tail_begin, packed)
+                        plan, pad, packed = pack_rows(tail_row, len(arr), tail_begin, nbytes, image)
+                        tail = (plan, image, pad, tail_begin, nbytes, packed)
                 if tail is None:
                     tail_row, cycle = len(arr), limit
-                windows = self._windows_of(layout, cycle, tail_row)
-                buf = torch.empty(max(e - b for _, _, b, e in windows) + _WINDOW_PAD, dtype=torch.uint8, device=device)
-                for r0, r1, begin, end in windows:
-                    plan, pad = pack_rows(r0, r1, begin, end, buf)
-                    dst = writer.data_address(start + begin)
-                    st = engine.d2h(buf.data_ptr() + pad, dst, end - begin, stream)
-                    if sums is not None:
-                        checksum(buf, pad, begin, end, dst, stream)
-                    plan.destroy()
-                    xfer["d2h_s"] += st.seconds
-                    xfer["d2h_bytes"] += end - begin
-                del buf
+                # two buffers of half the size where that leaves windows worth sending, else one
+                windows = self._windows_of(layout, cycle // 2, tail_row) if cycle // 2 >= _WINDOW_PAIR_MIN_BYTES else None
+                largest = max((e - b for _, _, b, e in windows), default=0) if windows else 0
+                if windows and 2 * (largest + _WINDOW_PAD) <= cycle + 2 * _WINDOW_PAD:
+                    buffers = [torch.empty(largest + _WINDOW_PAD, dtype=torch.uint8, device=device) for _ in range(2)]
+                else:
+                    windows = self._windows_of(layout, cycle, tail_row)
+                    buffers = [torch.empty(max(e - b for _, _, b, e in windows) + _WINDOW_PAD, dtype=torch.uint8, device=device)]
+                for k, (r0, r1, begin, end) in enumerate(windows):
+                    if k >= len(buffers):
+                        sent[k - len(buffers)].result()  # the buffer's previous window has left it
+                    buf = buffers[k % len(buffers)]
+                    plan, pad, packed = pack_rows(r0, r1, begin, end, buf)
+                    sent.append(sender.submit(send, plan, buf, pad, begin, end, packed))
+                    staged.packed_event = packed  # the live tensors are not read after the last of these
         except BaseException:
+            sender.shutdown(wait=True)
             held.__exit__(*sys.exc_info())
             raise
 
         def finish():
-            """The resident part, the sidecar, the buffer's close: on the caller's thread when there is no resident
-            part, else on a thread of its own."""
+            """After the last window: the resident part, the sidecar, the buffer's close, the outcome."""
             try:
                 with held:
+                    for done in sent:
+                        done.result()
                     if tail is not None:
-                        plan, image, pad, tail_begin, packed = tail
-                        with torch.cuda.device(device):
-                            _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
-                            dst = writer.data_address(start + tail_begin)
-                            st, _ = engine.d2h_gated(image.data_ptr() + pad, dst, nbytes - tail_begin, packed.cuda_event, 0,
-                                                     ctypes.c_uint64(0))
-                            xfer["d2h_s"] += st.seconds
-                            xfer["d2h_bytes"] += nbytes - tail_begin
-                            if sums is not None:
-                                # on a stream of its own: the training step's kernels are queued on the pack's
-                                checksum(image, pad, tail_begin, nbytes, dst, torch.cuda.Stream(device=device).cuda_stream)
-                            plan.destroy()
+                        send(*tail)
                 if sums is not None:
                     integrity.write_sidecar(str(object_id), self._crc_chunk_bytes, nbytes, sums.result())
                 else:
@@ -792,14 +803,14 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                 outcome = (True, self._results_of(staged, object_name))
             except BaseException as e:  # reported to whoever waits; a thread must not die silently
                 _LOGGER.exception("Windowed write of '%s' failed", object_id)
-                outcome = (False, f"{type(e).__name__}: {e}", e)
+                outcome = (False, f"{type(e).__name__}: {e}")
+            for plan in spent:
+                plan.destroy()
             stats.update({k: stats.get(k, 0) + v for k, v in xfer.items()})  # (the dict last_save_stats refers to)
-            if tail is None and not outcome[0]:
-                raise outcome[2]
             try:
                 tmp = staged.done_marker + ".tmp"
                 with open(tmp, "wb") as f:
-                    pickle.dump(outcome[:2], f)
+                    pickle.dump(outcome, f)
                 os.rename(tmp, staged.done_marker)
             finally:
                 if outcome[0]:
@@ -809,13 +820,13 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
 
         stats["objects"] += 1
         stats["windows"] = stats.get("windows", 0) + len(windows)
+        stats["window_buffers"] = len(buffers)
         stats["device_payload_bytes"] += layout.device_payload_bytes
         stats["image_bytes"] += nbytes
-        if tail is None:
-            finish()
-        else:
+        if tail is not None:
             stats["resident_bytes"] = stats.get("resident_bytes", 0) + nbytes - tail[3]
-            threading.Thread(target=finish, name=f"mlf-write-{object_name}", daemon=True).start()
+        sender.submit(finish)
+        sender.shutdown(wait=False)  # the thread ends when finish() has run
         return staged
 
     @staticmethod
