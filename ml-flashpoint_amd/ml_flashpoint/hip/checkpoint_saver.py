@@ -273,8 +273,9 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         ``background_write`` (True: ``prepare_write_data`` also starts the transfer into the buffer object on a
         background thread of this process; ``write_data`` - here or in a worker process that received the buckets -
         then only waits for it, for at most ``remote_wait_timeout_s`` across processes), ``max_image_bytes`` (largest
-        image to hold in HBM at once; default: what is free on the device.  A larger object is packed and sent window
-        by window inside ``prepare_write_data``, which then blocks for the whole transfer), ``reuse_plans`` (keep
+        image to hold in HBM at once; default: what is free on the device.  Of a larger object the end stays resident
+        and follows on a thread, the rest is packed and sent window by window inside ``prepare_write_data``, which
+        blocks for that part of the transfer), ``reuse_plans`` (keep
         the layout and the device-resident tables of every object from one save to the next and use them again
         when the tensors' addresses, shapes, strides and dtypes are the same; only the bytes of host-resident items
         are refreshed.  With 20 000 tensors this takes 60 ms out of the blocking part of each save after the first),
