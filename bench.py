@@ -57,7 +57,7 @@ def parse_args():
     ap.add_argument("--tile-bytes", type=int, default=0)
     ap.add_argument("--block-threads", type=int, default=0)
     ap.add_argument("--slot-mib", type=int, default=32)
-    ap.add_argument("--slots", type=int, default=4)
+    ap.add_argument("--slots", type=int, default=3)
     ap.add_argument("--copy-threads", type=int, default=0, help="0 = the engine's default (CPUs available, at most 16)")
     ap.add_argument("--crc-chunk-mib", type=int, default=32,
                     help="CRC-32C per chunk of this size, computed on the GPU during the save and verified on the GPU during "

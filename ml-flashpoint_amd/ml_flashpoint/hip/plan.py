@@ -357,7 +357,7 @@ class Plan:
 class CopyEngine:
     """Ring of pinned slots + copy streams + host threads between device images and pageable host memory."""
 
-    def __init__(self, slot_bytes: int = 32 << 20, n_slots: int = 4, n_threads: int = 8):
+    def __init__(self, slot_bytes: int = 32 << 20, n_slots: int = 3, n_threads: int = 8):
         handle = ctypes.c_void_p()
         _lib.check(_lib.load().mlf_engine_create(slot_bytes, n_slots, n_threads, ctypes.byref(handle)), "mlf_engine_create")
         self._handle = handle
