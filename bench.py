@@ -456,6 +456,22 @@ def main():
         mean = lambda xs: sum(xs) / len(xs)  # noqa: E731
         pack_s = mean(rec["pack_ms"]) * 1e-3
         algorithmic = 2 * mean(rec["pack_bytes"])
+        # ---- the unpack kernels by themselves: one more restore through one image, nothing beside them ----
+        clean_unpack = None
+        if not args.whole_image_restore and max_image is None and mean(rec["r_windows"]) > 0:
+            whole = DefaultMLFlashpointCheckpointLoader(manager, None, engine_config=engine_cfg, tile_bytes=args.tile_bytes,
+                                                        block_threads=args.block_threads, use_file_io=args.restore_io == "file",
+                                                        crc_mode=args.restore_crc, pipelined_restore=False)
+            whole.record_kernel_events = True
+            dcp.load(sd, checkpoint_id=prev.data, storage_reader=MemoryStorageReader(prev.data, whole), no_dist=True)
+            torch.cuda.synchronize()
+            clean_unpack = (sum(b.elapsed_time(e) for b, e, _ in whole.kernel_events) * 1e-3,
+                            sum(n for _, _, n in whole.kernel_events))
+            whole_engine = getattr(whole, "_engine", None)
+            if whole_engine is not None:
+                whole_engine.destroy()
+            del whole
+
         # ---- the other way to the checksums, for comparison: two more saves (the first builds its plan) ----
         crc_modes = None
         if args.crc_chunk_mib and not args.no_crc_compare and max_image is None:
@@ -567,7 +583,11 @@ def main():
                 "unpack_and_sync": ms("r_unpack"), "commit": ms("r_commit"),
                 "other_in_read_data": round((mean(rec["r_read"]) - restore_known) * 1e3, 2)},
             "pack_GBps": round(pack_gbps, 1),
-            "unpack_GBps": round(2 * mean(rec["unpack_bytes"]) / 1e9 / unpack_s, 1) if unpack_s > 0 else None,
+            # the unpack kernels on an otherwise idle device; in the default restore of a large object they run window by
+            # window beside the copies that fill the other buffer (and hide behind them): that sum is the second figure
+            "unpack_GBps": round(2 * clean_unpack[1] / 1e9 / clean_unpack[0], 1) if clean_unpack and clean_unpack[0] > 0 else (
+                round(2 * mean(rec["unpack_bytes"]) / 1e9 / unpack_s, 1) if unpack_s > 0 else None),
+            **({"unpack_GBps_beside_h2d": round(2 * mean(rec["unpack_bytes"]) / 1e9 / unpack_s, 1)} if clean_unpack and unpack_s > 0 else {}),
             "d2h_GBps": round(mean(rec["d2h_bytes"]) / 1e9 / mean(rec["d2h"]), 2) if mean(rec["d2h"]) > 0 else None,
             **({"host_copy_GBps": round(mean(rec["host_copy_bytes"]) / 1e9 / mean(rec["host_copy_s"]), 2),
                 "host_copy_bytes": int(mean(rec["host_copy_bytes"]))} if mean(rec["host_copy_s"]) > 0 else {}),
