@@ -303,3 +303,32 @@ def test_two_saves_prepared_before_either_is_written_keep_their_own_checksums(sh
             buf = ctypes.create_string_buffer(piece, len(piece))
             assert P.crc32c_host(ctypes.addressof(buf), len(piece)) == int(c), (cid.data, k)
     assert raws[0] != raws[1]
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_checksums_of_a_piece_cut_on_the_sections_chunk_grid(seed, oracle_c):
+    """``crc32c_device_cut``: a piece of a data section lies somewhere in a device buffer (same position modulo 16 as in
+    the section) and, already, in host memory; its checksums come back cut where the section's chunks end - the
+    first part may start off the 16-byte grid the kernels read on, its leading bytes are then taken on the host."""
+    import ctypes
+
+    from ml_flashpoint.hip import integrity
+    from ml_flashpoint.hip import plan as P
+
+    rng = np.random.default_rng(seed)
+    chunk = 65536
+    for _ in range(6):
+        data_off = int(rng.integers(0, 5 * chunk))
+        nbytes = int(rng.integers(1, 4 * chunk))
+        if seed == 3:
+            nbytes = int(rng.integers(1, 40))  # pieces shorter than a vector
+        buf_off = data_off % 16 + 16 * int(rng.integers(0, 300))
+        host = rng.integers(0, 256, nbytes, dtype=np.uint8)
+        buf = torch.zeros(buf_off + nbytes + 64, dtype=torch.uint8, device=DEV)
+        buf[buf_off : buf_off + nbytes] = torch.from_numpy(host).to(DEV)
+        got = P.crc32c_device_cut(buf, buf_off, data_off, nbytes, chunk, host.ctypes.data)
+        parts = integrity.ChunkChecksums.cuts(data_off, nbytes, chunk)
+        want = [oracle_c.oracle_crc32c(host[first - data_off : first - data_off + n].tobytes(), n) for first, n in parts]
+        assert got == want, (data_off, nbytes, buf_off)
+    with pytest.raises(ValueError, match="modulo 16"):
+        P.crc32c_device_cut(torch.zeros(256, dtype=torch.uint8, device=DEV), 1, 0, 100, chunk, 0)
