@@ -121,6 +121,31 @@ def test_worker_process_waits_for_the_gpu_owning_process(shm_dir, manager_future
     _check_files(cid, snapshot)
 
 
+def test_worker_process_waits_for_a_save_that_had_room_for_part_of_the_image_only(shm_dir, manager_future):
+    """With room for part of the image the blocking part sends windows and a thread of the parent sends the resident
+    end; a spawned worker that received the buckets waits for that thread's outcome like for any background write."""
+    saver = _make_saver(max_image_bytes=4 << 20, crc_chunk_bytes=1 << 16)  # the object holds 8 MiB
+    dist = _DistWrapper(None, False, 0)
+    sd = _state_dict()
+    cid = CheckpointContainerId(os.path.join(shm_dir, "step-4_ckpt"))
+    saver.initialize_checkpoint(cid)
+    writer = MemoryStorageWriter(saver, manager_future)
+    writer.reset(cid.data)
+    buckets, metadata, *_ = statedictsaver.generate_plan(cid, sd, writer, DefaultSavePlanner(), dist)
+    assert saver.last_save_stats["windows"] >= 2 and saver.last_save_stats["resident_bytes"] > 0
+    staged = MemoryStorageWriter.stage_write_data_buckets(cid, buckets, non_blocking=True)
+    snapshot = {k: v.cpu() for k, v in sd.items()}
+    for v in sd.values():
+        v.zero_()
+    ctx = torch_mp.get_context("spawn")
+    with concurrent.futures.ProcessPoolExecutor(max_workers=1, mp_context=ctx) as pool:
+        worker_results = pool.submit(worker_write, cid, writer, staged).result(timeout=120)
+    assert len(worker_results) == len(sd)
+    statedictsaver.finish_write(cid, writer, metadata, dist)
+    saver.finalize_checkpoint(cid)
+    _check_files(cid, snapshot)
+
+
 def test_failure_in_the_background_write_reaches_the_waiter(shm_dir, manager_future, monkeypatch):
     saver = _make_saver(background_write=True)
     cid = CheckpointContainerId(os.path.join(shm_dir, "step-4_ckpt"))
