@@ -85,6 +85,9 @@ def parse_args():
                     help="restore through one device buffer for the whole object instead of two alternating ones")
     ap.add_argument("--no-prefault", action="store_true", help="leave the pool file's pages to the first save, as the reference does")
     ap.add_argument("--no-link-probe", action="store_true", help="skip the bare host-link measurement")
+    ap.add_argument("--busy-gpu-probe", action="store_true",
+                    help="also time a save whose transfer runs on a background thread while bf16 GEMMs, then HBM copies, "
+                         "keep the device busy: what the transfer costs them, and what they cost the transfer")
     ap.add_argument("--no-crc-compare", action="store_true", help="skip the extra saves in the other checksum mode")
     ap.add_argument("--root", default=None, help="directory on tmpfs for the pool and checkpoints")
     return ap.parse_args()
@@ -243,6 +246,64 @@ def _rewrite_warm(path, tensors):
     return spans
 
 
+def _busy_gpu_probe(device, saver, sd, root, manager):
+    """One save with ``background_write=True`` (the transfer starts inside ``prepare_write_data`` on a thread) while
+    this thread keeps the device busy the way a training step would: 8192^3 bf16 GEMMs for the first half of the
+    transfer, 4 GiB device-to-device copies for the second.  Returns their rates alone and beside the transfer, and
+    how long the save took."""
+    import torch
+    from torch.distributed.checkpoint.planner_helpers import _create_write_items
+
+    from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId
+
+    torch.cuda.empty_cache()  # (or the operands below would be cut out of the block the images of the steps lay in)
+    a = torch.randn(8192, 8192, device=device, dtype=torch.bfloat16)
+    b = torch.randn(8192, 8192, device=device, dtype=torch.bfloat16)
+    x = torch.empty(1 << 30, dtype=torch.float32, device=device)
+    y = torch.empty_like(x)
+
+    def gemms(seconds):
+        torch.cuda.synchronize()
+        n, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(20):
+                torch.matmul(a, b)
+            torch.cuda.synchronize()
+            n += 20
+        return n * 2 * 8192 ** 3 / (time.perf_counter() - t0) / 1e12
+
+    def copies(seconds):
+        torch.cuda.synchronize()
+        n, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(10):
+                y.copy_(x)
+            torch.cuda.synchronize()
+            n += 10
+        return n * 2 * x.numel() * 4 / (time.perf_counter() - t0) / 1e12
+
+    class Resolver:
+        def resolve_data(self, item):
+            return sd[item.index.fqn]
+
+    gemms(0.5)  # clocks up
+    alone = (gemms(1.0), copies(1.0))
+    items = [wi for k, v in sd.items() if isinstance(v, torch.Tensor) for wi in _create_write_items(k, v)]
+    out = None
+    for step in range(2):  # the second runs on the kept plan
+        cid = CheckpointContainerId(os.path.join(root, "run", f"step-{3000 + step}_ckpt"))
+        t0 = time.perf_counter()
+        buckets = saver.prepare_write_data(cid, items, Resolver(), "busy", 1)
+        beside = (gemms(0.8), copies(0.8))
+        saver.write_data(cid, buckets, replicate_after_write=False, thread_count=1)
+        out = {"save_s": round(time.perf_counter() - t0, 3),
+               "gemm_TFLOPs": {"alone": round(alone[0], 1), "beside_the_transfer": round(beside[0], 1)},
+               "hbm_copy_TBps": {"alone": round(alone[1], 3), "beside_the_transfer": round(beside[1], 3)}}
+        manager.delete_container(cid)
+    saver.release_device_memory()
+    return out
+
+
 class _LocalManager:
     """In-process stand-in for ``torch.multiprocessing.Manager()``: ``dict()`` and ``Event()`` only."""
 
@@ -320,16 +381,17 @@ def main():
     manager.warm_up_pool()
     max_image = int(args.max_image_gb * 1e9) if args.max_image_gb > 0 else None
 
-    def make_saver(crc_mode):
+    def make_saver(crc_mode, **more):
         made = DefaultMLFlashpointCheckpointSaver(
             lambda: 0, lambda: 0, lambda: None, manager, None, initial_buffer_size_bytes=1 << 20,
             engine_config=engine_cfg, tile_bytes=args.tile_bytes, block_threads=args.block_threads,
             crc_chunk_bytes=args.crc_chunk_mib << 20, crc_mode=crc_mode, use_file_io=args.save_io == "file",
-            max_image_bytes=max_image)
+            max_image_bytes=max_image, **more)
         made.record_kernel_events = True
         return made
 
     saver = make_saver(args.save_crc)
+    saver.warm_up(device)  # at start-up, like the pool: pinned slots, streams clear of the training stream's queue
     loader = DefaultMLFlashpointCheckpointLoader(manager, None, engine_config=engine_cfg, tile_bytes=args.tile_bytes,
                                                  block_threads=args.block_threads, use_file_io=args.restore_io == "file",
                                                  crc_mode=args.restore_crc, max_image_bytes=max_image,
@@ -507,6 +569,11 @@ def main():
                           "save_s": round(runs[-1]["save"], 4)}
         manager.delete_container(prev)
 
+        # ---- a save whose transfer runs on a thread while the device is kept busy, as by a training step ----
+        busy = None
+        if args.busy_gpu_probe and max_image is None:
+            busy = _busy_gpu_probe(device, make_saver(args.save_crc, background_write=True), sd, root, manager)
+
         # ---- the host link by itself: device <-> the engine's pinned slots, nothing behind them ----
         link = None
         if not args.no_link_probe:
@@ -597,6 +664,7 @@ def main():
             **({"link_roofline": link} if link else {}),
             **({"crc_modes": crc_modes} if crc_modes else {}),
             **({"with_dcp_plan_cache": with_cache} if with_cache else {}),
+            **({"beside_a_busy_gpu": busy} if busy else {}),
             "parity": "restored tensors bit-identical to originals (fingerprints)",
             "roofline": {"bound": "hbm",
                          "kernel": "mlf_fused_crc_kernel<pack> (copy + CRC-32C)" if args.save_crc == "fused" else "mlf_flat_kernel<pack>",

@@ -230,6 +230,22 @@ int mlf_engine_h2d(mlf_engine* engine, const void* src_host, void* dst_dev, uint
  * reference counterpart. */
 int mlf_engine_link_probe(mlf_engine* engine, void* dev_buf, uint64_t nbytes, int to_host, double* seconds);
 
+/* Moves the engine's streams off the hardware queue of `busy_stream` - the stream the training step runs on.  The HIP
+ * runtime spreads a process's streams over a few hardware queues (GPU_MAX_HW_QUEUES, 4 unless the environment says
+ * otherwise), and a queue runs its commands in order: a copy stream that shares its queue with a stream that is kept
+ * full waits behind that stream's kernels - measured 10-13 GB/s instead of 53-56 beside back-to-back GEMMs.  Which
+ * streams share is decided when they are created and cannot be asked for, so it is measured: both streams idle, a
+ * 2 ms kernel of one wavefront on `busy_stream`, an empty kernel on the engine's stream; if that one has to wait, the
+ * stream is replaced by a new one that does not.  Waits for `busy_stream` to drain (several times): call it at
+ * set-up, or in the blocking part of the first save.  `still_shared` (may be null) receives the number of the
+ * engine's three streams for which no free queue was found.  No reference counterpart. */
+int mlf_engine_avoid_stream(mlf_engine* engine, void* busy_stream, uint32_t* still_shared);
+
+/* The stream the engine runs its checksum kernels on (a raw hipStream_t), for checksum calls a caller makes between
+ * the engine's transfers (mlf_crc32c_device on pieces of an image): a stream that mlf_engine_avoid_stream has
+ * already moved out of the training stream's way. */
+void* mlf_engine_checksum_stream(mlf_engine* engine);
+
 /* Host -> host on the engine's threads: `nbytes` from `src_host` to `dst_host` (ranges must not overlap).  For
  * checkpoint items that are resident in host memory - the reference copies those into the mapping with torch's
  * intra-op threads (checkpoint_saver.py:443-450,797-800); they do not visit the device here either. */

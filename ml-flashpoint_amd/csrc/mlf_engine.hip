@@ -150,6 +150,39 @@ struct mlf_engine {
   std::mutex busy;  // one transfer at a time per engine
 };
 
+namespace {
+
+// The two kernels of the hardware-queue test (mlf_engine_avoid_stream).  The first keeps one wavefront busy for a
+// stated time by the device's constant-rate clock (100 MHz) - bounded by a count as well, so that it ends whatever
+// that clock does; the second does nothing but exist.
+__global__ void mlf_queue_test_hold(uint64_t ticks, uint32_t* out) {
+  const uint64_t t0 = wall_clock64();
+  uint32_t n = 0;
+  while (wall_clock64() - t0 < ticks && n < (1u << 22)) ++n;
+  if (threadIdx.x == 0) *out = n;
+}
+
+__global__ void mlf_queue_test_touch(uint32_t* out) {
+  if (threadIdx.x == 0) *out = 1u;
+}
+
+// Whether work on `s` waits for work enqueued earlier on `busy`: both idle, a 2 ms kernel on `busy`, an empty kernel
+// on `s`; on a hardware queue of its own the empty kernel is done in microseconds, behind the 2 ms kernel it is not.
+int shares_hardware_queue(hipStream_t s, hipStream_t busy, uint32_t* d_flags, bool* shared) {
+  HIP_TRY(hipStreamSynchronize(busy));
+  HIP_TRY(hipStreamSynchronize(s));
+  hipLaunchKernelGGL(mlf_queue_test_hold, dim3(1), dim3(64), 0, busy, 200000ull, d_flags);
+  hipLaunchKernelGGL(mlf_queue_test_touch, dim3(1), dim3(64), 0, s, d_flags + 16);
+  HIP_TRY(hipGetLastError());
+  const double t0 = now_s();
+  HIP_TRY(hipStreamSynchronize(s));
+  *shared = now_s() - t0 > 1e-3;
+  HIP_TRY(hipStreamSynchronize(busy));
+  return MLF_HIP_OK;
+}
+
+}  // namespace
+
 extern "C" {
 
 int mlf_engine_destroy(mlf_engine* e) {
@@ -419,6 +452,50 @@ int mlf_engine_d2h_gated(mlf_engine* e, const void* src_dev, void* dst_host, uin
   gate.by_event = true;
   return engine_d2h(e, src_dev, host, nbytes, gate, stats, crc);
 }
+
+int mlf_engine_avoid_stream(mlf_engine* e, void* busy_stream, uint32_t* still_shared) {
+  if (!e) return fail(MLF_HIP_BAD_ARG, "null engine");
+  std::lock_guard<std::mutex> g(e->busy);
+  HIP_TRY(hipSetDevice(e->device));
+  hipStream_t busy = static_cast<hipStream_t>(busy_stream);
+  uint32_t* d_flags = nullptr;
+  HIP_TRY(hipMalloc(reinterpret_cast<void**>(&d_flags), 128));
+  std::vector<hipStream_t> rejected;  // kept until the end: a destroyed stream's queue would be handed out again
+  uint32_t left = 0;
+  int rc = MLF_HIP_OK;
+  hipStream_t* mine[3] = {&e->streams[0], &e->streams[1], &e->crc_stream};
+  for (hipStream_t* slot : mine) {
+    bool shared = false;
+    if ((rc = shares_hardware_queue(*slot, busy, d_flags, &shared))) break;
+    for (int attempt = 0; shared && attempt < 8 && rc == MLF_HIP_OK; ++attempt) {
+      hipStream_t candidate = nullptr;
+      if (hipStreamCreateWithFlags(&candidate, hipStreamNonBlocking) != hipSuccess) {
+        rc = fail(MLF_HIP_RUNTIME, "hipStreamCreateWithFlags failed");
+        break;
+      }
+      bool also = false;
+      if ((rc = shares_hardware_queue(candidate, busy, d_flags, &also))) {
+        rejected.push_back(candidate);
+        break;
+      }
+      if (also) {
+        rejected.push_back(candidate);
+      } else {
+        rejected.push_back(*slot);
+        *slot = candidate;
+        shared = false;
+      }
+    }
+    if (rc != MLF_HIP_OK) break;
+    left += shared ? 1u : 0u;
+  }
+  for (hipStream_t s : rejected) (void)hipStreamDestroy(s);
+  (void)hipFree(d_flags);
+  if (rc == MLF_HIP_OK && still_shared) *still_shared = left;
+  return rc;
+}
+
+void* mlf_engine_checksum_stream(mlf_engine* e) { return e ? e->crc_stream : nullptr; }
 
 int mlf_engine_link_probe(mlf_engine* e, void* dev_buf, uint64_t nbytes, int to_host, double* seconds) {
   if (!e || !dev_buf || !seconds) return fail(MLF_HIP_BAD_ARG, "null argument");

@@ -134,6 +134,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         self._max_image_bytes = max_image_bytes
         self._pipelined_restore = pipelined_restore
         self._engine: Optional[hip_plan.CopyEngine] = None
+        self._engine_clear_of: Optional[int] = None
         self._engine_lock = threading.Lock()
         self._stats_local = threading.local()  # read_data runs on one executor thread per object
         self._init_discovery()
@@ -155,6 +156,18 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                 cfg = self._engine_config
                 self._engine = hip_plan.CopyEngine(cfg.slot_bytes, cfg.n_slots, cfg.resolved_copy_threads())
             return self._engine
+
+    def _keep_clear_of(self, device: torch.device) -> None:
+        """Once per engine: its streams off the hardware queue of the stream that is current on ``device`` (the one the
+        unpack runs on, and whatever else the process keeps busy there); see the saver's ``warm_up``."""
+        engine = self._get_engine()
+        with self._engine_lock:
+            if self._engine_clear_of is not None:
+                return
+            self._engine_clear_of = torch.cuda.current_stream(device).cuda_stream
+        left = engine.avoid_stream(self._engine_clear_of)
+        if left:
+            _LOGGER.warning("%d of the copy engine's streams share a hardware queue with the current stream", left)
 
     @override
     @log_execution_time(logger=_LOGGER, name="read_metadata")
@@ -378,6 +391,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                     clusters = None
             with torch.cuda.device(device):
                 _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
+                self._keep_clear_of(device)
                 limit = self._image_limit(device)
                 # one buffer for the range (or for the largest neighbourhood of a partial read) if the allocator
                 # has a block of that size; through a smaller buffer, window by window, if it has not

@@ -315,6 +315,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
 
     def _init_runtime_state(self):
         self._engine: Optional[hip_plan.CopyEngine] = None
+        self._engine_clear_of: Optional[int] = None  # the stream whose hardware queue the engine's streams avoid
         self._engine_lock = threading.Lock()
         self.last_save_stats: dict = {}
         # set to True to bracket every pack launch with timing events on its stream; (start, end, payload bytes)
@@ -326,7 +327,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
     # ---- pickling: only configuration crosses a process boundary --------------------------------------
     def __getstate__(self):
         state = self.__dict__.copy()
-        for key in ("_replication_manager", "_engine", "_engine_lock", "last_save_stats", "kernel_events", "_plan_cache"):
+        for key in ("_replication_manager", "_engine", "_engine_clear_of", "_engine_lock", "last_save_stats", "kernel_events",
+                    "_plan_cache"):
             state.pop(key, None)
         return state
 
@@ -341,6 +343,27 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                 cfg = self._engine_config
                 self._engine = hip_plan.CopyEngine(cfg.slot_bytes, cfg.n_slots, cfg.resolved_copy_threads())
             return self._engine
+
+    def warm_up(self, device: Optional[torch.device] = None) -> None:
+        """Creates the copy engine (pinned slots, streams, threads) and moves its streams off the hardware queue of
+        the stream that is current on ``device`` now - the one the training step runs on: HIP spreads a process's
+        streams over a few hardware queues, and a copy stream that shares its queue with a stream that is kept full
+        waits behind that stream's kernels (measured: 10-13 GB/s instead of 53-56 beside back-to-back GEMMs).  The
+        first ``prepare_write_data`` does this by itself, inside its blocking part (30-50 ms, once, and it waits for
+        the stream to drain); a job that calls ``warm_up`` at start-up spares its first save that."""
+        with self._engine_lock:
+            if self._engine_clear_of is not None:
+                return
+        device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+        with torch.cuda.device(device):
+            _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
+            engine = self._get_engine()
+            stream = torch.cuda.current_stream(device).cuda_stream
+            left = engine.avoid_stream(stream)
+        if left:
+            _LOGGER.warning("%d of the copy engine's streams share a hardware queue with the current stream: transfers "
+                            "beside a busy device will be slow (more queues: GPU_MAX_HW_QUEUES)", left)
+        self._engine_clear_of = stream
 
     # ---- dirty marker / directory ----------------------------------------------------------------------
     @override
@@ -517,6 +540,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         items = [item for item, _ in tensor_data] + [item for item, _ in bytes_data]
         plan = image = packed = None
         stream = 0
+        if layout.image_bytes and self._engine_clear_of is None:
+            self.warm_up(device)  # once: the engine's streams off the hardware queue of the stream the pack runs on
         if layout.image_bytes and object_id is not None:
             if layout.image_bytes <= self._image_limit(device):
                 with torch.cuda.device(device):
@@ -713,8 +738,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                 stream = torch.cuda.current_stream(device).cuda_stream
                 engine = self._get_engine()
                 sums = integrity.ChunkChecksums(self._crc_chunk_bytes, nbytes) if self._crc_chunk_bytes and nbytes else None
-                # checksum kernels get a stream of their own: the training step's kernels are queued on the pack's
-                side = torch.cuda.Stream(device=device) if sums is not None else None
+                # checksum kernels go to the engine's checksum stream: the training step's kernels are queued on the pack's
+                side = engine.checksum_stream
 
                 def pack_rows(r0, r1, begin, end, buf):
                     """Rows [r0, r1) = image bytes [begin, end) into ``buf``.  They lie in the buffer where they lie
@@ -752,7 +777,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                         if sums is not None:
                             t0 = time.perf_counter()
                             sums.add(begin, end - begin, hip_plan.crc32c_device_cut(
-                                buf, pad, begin, end - begin, self._crc_chunk_bytes, dst, side.cuda_stream))
+                                buf, pad, begin, end - begin, self._crc_chunk_bytes, dst, side))
                             xfer["crc_s"] = xfer.get("crc_s", 0.0) + time.perf_counter() - t0
                         spent.append(plan)  # (released at the end: freeing device memory waits for the whole device)
 
@@ -1108,9 +1133,10 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         engine = self._get_engine()
         nbytes = staged.layout.data_bytes
         sums = integrity.ChunkChecksums(self._crc_chunk_bytes, nbytes) if self._crc_chunk_bytes and nbytes else None
-        # the checksum kernels get a stream of their own: this may be a background thread, and the training step's
-        # kernels are queued on the stream the pack ran on
-        side = torch.cuda.Stream(device=staged.device_index) if sums is not None else None
+        # the checksum kernels go to the engine's checksum stream: this may be a background thread, and the training
+        # step's kernels are queued on the stream the pack ran on
+        side = engine.checksum_stream
+        spent = []
         for k, (plan, buf, begin, end) in enumerate(staged.pieces):
             pad = begin % _WINDOW_PAD
             dst = writer.data_address(start + begin)
@@ -1124,13 +1150,15 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                 # the piece has left the device, so its pack is over: the side stream may read it at once
                 t0 = time.perf_counter()
                 sums.add(begin, end - begin, hip_plan.crc32c_device_cut(buf, pad, begin, end - begin,
-                                                                         self._crc_chunk_bytes, dst, side.cuda_stream))
+                                                                         self._crc_chunk_bytes, dst, side))
                 xfer["crc_s"] = xfer.get("crc_s", 0.0) + time.perf_counter() - t0
             staged._landed.value = end
             staged.pieces[k] = None
-            plan.destroy()
-            del buf
+            spent.append(plan)
+            del buf  # back to the allocator now: the training step may want the room
         staged.pieces = None
+        for plan in spent:  # at the end: releasing device memory waits for the whole device, busy as it may be
+            plan.destroy()
         return sums.result() if sums is not None else None
 
     def _transfer_in_pieces(self, staged: StagedObject, writer, start: int, xfer: dict):
@@ -1255,3 +1283,4 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             if self._engine is not None:
                 self._engine.destroy()
                 self._engine = None
+                self._engine_clear_of = None

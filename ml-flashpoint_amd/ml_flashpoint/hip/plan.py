@@ -426,6 +426,19 @@ class CopyEngine:
         """Host memory to host memory on the engine's threads (checkpoint items that are resident on the host)."""
         _lib.check(_lib.load().mlf_engine_host_copy(self._handle, dst_host_ptr, src_host_ptr, nbytes), "mlf_engine_host_copy")
 
+    def avoid_stream(self, busy_stream: int) -> int:
+        """Moves the engine's streams off the hardware queue of ``busy_stream`` (a raw ``hipStream_t``: the stream the
+        training step runs on), where they would wait behind its kernels; waits for that stream to drain while it
+        tests.  Returns how many of the engine's three streams could not be moved."""
+        left = ctypes.c_uint32(0)
+        _lib.check(_lib.load().mlf_engine_avoid_stream(self._handle, busy_stream, ctypes.byref(left)), "mlf_engine_avoid_stream")
+        return int(left.value)
+
+    @property
+    def checksum_stream(self) -> int:
+        """The engine's checksum stream (raw ``hipStream_t``), for checksum calls between its transfers."""
+        return int(_lib.load().mlf_engine_checksum_stream(self._handle) or 0)
+
     def h2d(self, src_host_ptr: int, dst_dev_ptr: int, nbytes: int, consumer_stream: int = 0) -> _lib.XferStats:
         stats = _lib.XferStats()
         _lib.check(

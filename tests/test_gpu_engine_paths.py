@@ -134,3 +134,43 @@ def test_gated_transfer_waits_for_its_event_and_not_for_the_stream():
     engine.d2h_gated(dev2.data_ptr(), arena.data_ptr(), nbytes, None, 0, landed)
     assert torch.equal(arena, host)
     engine.destroy()
+
+
+def test_engines_keep_their_streams_off_the_hardware_queue_of_the_training_stream():
+    """HIP spreads a process's streams over a few hardware queues; a copy stream that shares its queue with a stream
+    that is kept full crawls.  Several engines are created (so that some of their streams land on the default
+    stream's queue), each is told to avoid the default stream, and each must then move data at a sane rate while
+    kernels are queued back to back on the default stream - without the call at least one of them would not."""
+    import threading
+
+    from ml_flashpoint.hip import plan as P
+
+    n = 2 << 30
+    buf = torch.zeros(n, dtype=torch.uint8, device=DEV)
+    a = torch.randn(4096, 4096, device=DEV, dtype=torch.bfloat16)
+    stop = threading.Event()
+
+    def busy():  # kernels back to back on the default stream, ~10 ms queued at any time
+        while not stop.is_set():
+            for _ in range(40):
+                torch.matmul(a, a)
+            torch.cuda.synchronize()
+
+    engines = [P.CopyEngine(slot_bytes=8 << 20, n_slots=3, n_threads=4) for _ in range(5)]
+    try:
+        idle = n / engines[0].link_probe(buf.data_ptr(), n, True)
+        left = [engine.avoid_stream(torch.cuda.current_stream().cuda_stream) for engine in engines]
+        assert left == [0] * len(engines)
+        worker = threading.Thread(target=busy)
+        worker.start()
+        try:
+            time.sleep(0.1)
+            rates = [n / engine.link_probe(buf.data_ptr(), n, True) for engine in engines]
+        finally:
+            stop.set()
+            worker.join()
+        assert min(rates) > 0.6 * idle, (idle, rates)
+        assert all(engine.checksum_stream for engine in engines)
+    finally:
+        for engine in engines:
+            engine.destroy()
