@@ -230,19 +230,20 @@ int mlf_engine_h2d(mlf_engine* engine, const void* src_host, void* dst_dev, uint
  * reference counterpart. */
 int mlf_engine_link_probe(mlf_engine* engine, void* dev_buf, uint64_t nbytes, int to_host, double* seconds);
 
-/* Moves the engine's streams off the hardware queue of `busy_stream` - the stream the training step runs on.  The HIP
+/* Moves the engine's streams off the hardware queues of `busy_streams` - the streams the training step runs on.  The HIP
  * runtime spreads a process's streams over a few hardware queues (GPU_MAX_HW_QUEUES, 4 unless the environment says
  * otherwise), and a queue runs its commands in order: a copy stream that shares its queue with a stream that is kept
  * full waits behind that stream's kernels - measured 10-13 GB/s instead of 53-56 beside back-to-back GEMMs.  Which
  * streams share is decided when they are created and cannot be asked for, so it is measured: both streams idle, a
- * 2 ms kernel of one wavefront on `busy_stream`, an empty kernel on the engine's stream; if that one has to wait, the
- * stream is replaced by a new one that does not.  Waits for `busy_stream` to drain (several times): call it at
- * set-up, or in the blocking part of the first save.  `still_shared` (may be null) receives the number of the
- * engine's three streams for which no free queue was found.  No reference counterpart. */
-int mlf_engine_avoid_stream(mlf_engine* engine, void* busy_stream, uint32_t* still_shared);
+ * 2 ms kernel of one wavefront on a busy stream, an empty kernel on the engine's stream; if that one has to wait, the
+ * stream is replaced by a new one that waits for none of them.  Waits for the busy streams to drain (several times):
+ * call it at set-up, or in the blocking part of the first save.  `busy_streams` holds `n_busy` raw hipStream_t values
+ * (a null entry is the default stream); `still_shared` (may be null) receives the number of the engine's three
+ * streams for which no free queue was found.  No reference counterpart. */
+int mlf_engine_avoid_streams(mlf_engine* engine, void* const* busy_streams, uint32_t n_busy, uint32_t* still_shared);
 
 /* The stream the engine runs its checksum kernels on (a raw hipStream_t), for checksum calls a caller makes between
- * the engine's transfers (mlf_crc32c_device on pieces of an image): a stream that mlf_engine_avoid_stream has
+ * the engine's transfers (mlf_crc32c_device on pieces of an image): a stream that mlf_engine_avoid_streams has
  * already moved out of the training stream's way. */
 void* mlf_engine_checksum_stream(mlf_engine* engine);
 

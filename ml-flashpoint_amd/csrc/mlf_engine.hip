@@ -168,7 +168,7 @@ __global__ void mlf_queue_test_touch(uint32_t* out) {
 
 // Whether work on `s` waits for work enqueued earlier on `busy`: both idle, a 2 ms kernel on `busy`, an empty kernel
 // on `s`; on a hardware queue of its own the empty kernel is done in microseconds, behind the 2 ms kernel it is not.
-int shares_hardware_queue(hipStream_t s, hipStream_t busy, uint32_t* d_flags, bool* shared) {
+int waits_behind(hipStream_t s, hipStream_t busy, uint32_t* d_flags, bool* shared) {
   HIP_TRY(hipStreamSynchronize(busy));
   HIP_TRY(hipStreamSynchronize(s));
   hipLaunchKernelGGL(mlf_queue_test_hold, dim3(1), dim3(64), 0, busy, 200000ull, d_flags);
@@ -453,11 +453,18 @@ int mlf_engine_d2h_gated(mlf_engine* e, const void* src_dev, void* dst_host, uin
   return engine_d2h(e, src_dev, host, nbytes, gate, stats, crc);
 }
 
-int mlf_engine_avoid_stream(mlf_engine* e, void* busy_stream, uint32_t* still_shared) {
+int mlf_engine_avoid_streams(mlf_engine* e, void* const* busy_streams, uint32_t n_busy, uint32_t* still_shared) {
   if (!e) return fail(MLF_HIP_BAD_ARG, "null engine");
+  if (n_busy == 0 || !busy_streams) return fail(MLF_HIP_BAD_ARG, "no stream to avoid");
   std::lock_guard<std::mutex> g(e->busy);
   HIP_TRY(hipSetDevice(e->device));
-  hipStream_t busy = static_cast<hipStream_t>(busy_stream);
+  // shares a queue with any of the busy streams?
+  auto shares_hardware_queue = [&](hipStream_t s, uint32_t* flags, bool* shared) -> int {
+    *shared = false;
+    for (uint32_t k = 0; k < n_busy && !*shared; ++k)
+      if (int err = waits_behind(s, static_cast<hipStream_t>(busy_streams[k]), flags, shared)) return err;
+    return MLF_HIP_OK;
+  };
   uint32_t* d_flags = nullptr;
   HIP_TRY(hipMalloc(reinterpret_cast<void**>(&d_flags), 128));
   std::vector<hipStream_t> rejected;  // kept until the end: a destroyed stream's queue would be handed out again
@@ -466,7 +473,7 @@ int mlf_engine_avoid_stream(mlf_engine* e, void* busy_stream, uint32_t* still_sh
   hipStream_t* mine[3] = {&e->streams[0], &e->streams[1], &e->crc_stream};
   for (hipStream_t* slot : mine) {
     bool shared = false;
-    if ((rc = shares_hardware_queue(*slot, busy, d_flags, &shared))) break;
+    if ((rc = shares_hardware_queue(*slot, d_flags, &shared))) break;
     for (int attempt = 0; shared && attempt < 8 && rc == MLF_HIP_OK; ++attempt) {
       hipStream_t candidate = nullptr;
       if (hipStreamCreateWithFlags(&candidate, hipStreamNonBlocking) != hipSuccess) {
@@ -474,7 +481,7 @@ int mlf_engine_avoid_stream(mlf_engine* e, void* busy_stream, uint32_t* still_sh
         break;
       }
       bool also = false;
-      if ((rc = shares_hardware_queue(candidate, busy, d_flags, &also))) {
+      if ((rc = shares_hardware_queue(candidate, d_flags, &also))) {
         rejected.push_back(candidate);
         break;
       }

@@ -344,13 +344,14 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                 self._engine = hip_plan.CopyEngine(cfg.slot_bytes, cfg.n_slots, cfg.resolved_copy_threads())
             return self._engine
 
-    def warm_up(self, device: Optional[torch.device] = None) -> None:
+    def warm_up(self, device: Optional[torch.device] = None, also_avoid: tuple = ()) -> None:
         """Creates the copy engine (pinned slots, streams, threads) and moves its streams off the hardware queue of
         the stream that is current on ``device`` now - the one the training step runs on: HIP spreads a process's
         streams over a few hardware queues, and a copy stream that shares its queue with a stream that is kept full
         waits behind that stream's kernels (measured: 10-13 GB/s instead of 53-56 beside back-to-back GEMMs).  The
         first ``prepare_write_data`` does this by itself, inside its blocking part (30-50 ms, once, and it waits for
-        the stream to drain); a job that calls ``warm_up`` at start-up spares its first save that."""
+        the stream to drain); a job that calls ``warm_up`` at start-up spares its first save that.  ``also_avoid``:
+        other streams of the job that are kept busy (``torch.cuda.Stream`` objects or raw handles)."""
         with self._engine_lock:
             if self._engine_clear_of is not None:
                 return
@@ -359,7 +360,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
             engine = self._get_engine()
             stream = torch.cuda.current_stream(device).cuda_stream
-            left = engine.avoid_stream(stream)
+            left = engine.avoid_stream(stream, *[getattr(other, "cuda_stream", other) for other in also_avoid])
         if left:
             _LOGGER.warning("%d of the copy engine's streams share a hardware queue with the current stream: transfers "
                             "beside a busy device will be slow (more queues: GPU_MAX_HW_QUEUES)", left)

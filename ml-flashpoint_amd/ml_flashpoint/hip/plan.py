@@ -426,12 +426,14 @@ class CopyEngine:
         """Host memory to host memory on the engine's threads (checkpoint items that are resident on the host)."""
         _lib.check(_lib.load().mlf_engine_host_copy(self._handle, dst_host_ptr, src_host_ptr, nbytes), "mlf_engine_host_copy")
 
-    def avoid_stream(self, busy_stream: int) -> int:
-        """Moves the engine's streams off the hardware queue of ``busy_stream`` (a raw ``hipStream_t``: the stream the
-        training step runs on), where they would wait behind its kernels; waits for that stream to drain while it
-        tests.  Returns how many of the engine's three streams could not be moved."""
+    def avoid_stream(self, *busy_streams: int) -> int:
+        """Moves the engine's streams off the hardware queues of ``busy_streams`` (raw ``hipStream_t`` values: the
+        streams the training step runs on), where they would wait behind those streams' kernels; waits for them to
+        drain while it tests.  Returns how many of the engine's three streams could not be moved."""
         left = ctypes.c_uint32(0)
-        _lib.check(_lib.load().mlf_engine_avoid_stream(self._handle, busy_stream, ctypes.byref(left)), "mlf_engine_avoid_stream")
+        handles = (ctypes.c_void_p * len(busy_streams))(*busy_streams)
+        _lib.check(_lib.load().mlf_engine_avoid_streams(self._handle, handles, len(busy_streams), ctypes.byref(left)),
+                   "mlf_engine_avoid_streams")
         return int(left.value)
 
     @property
