@@ -95,6 +95,10 @@ int main(int argc, char** argv) {
   REQUIRE(mlf_buffer_reserve(buf, 4096, image_bytes) == 0);
   mlf_engine* engine = nullptr;
   REQUIRE(mlf_engine_create(1 << 20, 2, 2, &engine) == 0);
+  void* busy_streams[1] = {nullptr};  // the default stream: the engine's streams move off its hardware queue
+  uint32_t still_shared = 9;
+  REQUIRE(mlf_engine_avoid_streams(engine, busy_streams, 1, &still_shared) == 0 && still_shared == 0);
+  REQUIRE(mlf_engine_checksum_stream(engine) != nullptr);
   uint64_t landed = 7;
   uint32_t crc_sent = 0;
   mlf_xfer_stats stats;
