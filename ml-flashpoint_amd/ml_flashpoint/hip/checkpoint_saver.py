@@ -315,7 +315,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
 
     def _init_runtime_state(self):
         self._engine: Optional[hip_plan.CopyEngine] = None
-        self._engine_clear_of: Optional[int] = None  # the stream whose hardware queue the engine's streams avoid
+        self._engine_clear_of: Optional[set] = None  # the streams whose hardware queues the engine's streams avoid
         self._engine_lock = threading.Lock()
         self.last_save_stats: dict = {}
         # set to True to bracket every pack launch with timing events on its stream; (start, end, payload bytes)
@@ -349,22 +349,23 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         the stream that is current on ``device`` now - the one the training step runs on: HIP spreads a process's
         streams over a few hardware queues, and a copy stream that shares its queue with a stream that is kept full
         waits behind that stream's kernels (measured: 10-13 GB/s instead of 53-56 beside back-to-back GEMMs).  The
-        first ``prepare_write_data`` does this by itself, inside its blocking part (30-50 ms, once, and it waits for
-        the stream to drain); a job that calls ``warm_up`` at start-up spares its first save that.  ``also_avoid``:
-        other streams of the job that are kept busy (``torch.cuda.Stream`` objects or raw handles)."""
-        with self._engine_lock:
-            if self._engine_clear_of is not None:
-                return
+        first ``prepare_write_data`` does this by itself, inside its blocking part (30-50 ms, once - again if a
+        later save finds another stream current - and it waits for the stream to drain); a job that calls
+        ``warm_up`` at start-up spares its first save that.  ``also_avoid``: other streams of the job that are kept
+        busy (``torch.cuda.Stream`` objects or raw handles)."""
         device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+        wanted = {torch.cuda.current_stream(device).cuda_stream} | {getattr(s, "cuda_stream", s) for s in also_avoid}
+        with self._engine_lock:
+            if self._engine_clear_of is not None and wanted <= self._engine_clear_of:
+                return
+            wanted |= self._engine_clear_of or set()
         with torch.cuda.device(device):
             _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
-            engine = self._get_engine()
-            stream = torch.cuda.current_stream(device).cuda_stream
-            left = engine.avoid_stream(stream, *[getattr(other, "cuda_stream", other) for other in also_avoid])
+            left = self._get_engine().avoid_stream(*sorted(wanted))
         if left:
-            _LOGGER.warning("%d of the copy engine's streams share a hardware queue with the current stream: transfers "
-                            "beside a busy device will be slow (more queues: GPU_MAX_HW_QUEUES)", left)
-        self._engine_clear_of = stream
+            _LOGGER.warning("%d of the copy engine's streams share a hardware queue with a stream of the training step: "
+                            "transfers beside a busy device will be slow (more queues: GPU_MAX_HW_QUEUES)", left)
+        self._engine_clear_of = wanted
 
     # ---- dirty marker / directory ----------------------------------------------------------------------
     @override
@@ -541,8 +542,9 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         items = [item for item, _ in tensor_data] + [item for item, _ in bytes_data]
         plan = image = packed = None
         stream = 0
-        if layout.image_bytes and self._engine_clear_of is None:
-            self.warm_up(device)  # once: the engine's streams off the hardware queue of the stream the pack runs on
+        if layout.image_bytes and (self._engine_clear_of is None
+                                   or torch.cuda.current_stream(device).cuda_stream not in self._engine_clear_of):
+            self.warm_up(device)  # the engine's streams off the hardware queue of the stream the pack runs on
         if layout.image_bytes and object_id is not None:
             if layout.image_bytes <= self._image_limit(device):
                 with torch.cuda.device(device):

@@ -146,6 +146,32 @@ def test_worker_process_waits_for_a_save_that_had_room_for_part_of_the_image_onl
     _check_files(cid, snapshot)
 
 
+def test_engine_streams_follow_the_stream_the_save_runs_on(shm_dir, manager_future):
+    """``warm_up`` moves the copy engine's streams off the hardware queue of the stream that is current then; a save
+    that later runs on another stream adds that one - and writes the same bytes."""
+    saver = _make_saver(background_write=True)
+    saver.warm_up()
+    assert saver._engine_clear_of == {torch.cuda.current_stream().cuda_stream}
+    saver.warm_up()  # nothing to do twice
+    dist = _DistWrapper(None, False, 0)
+    sd = _state_dict()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    cid = CheckpointContainerId(os.path.join(shm_dir, "step-5_ckpt"))
+    saver.initialize_checkpoint(cid)
+    writer = MemoryStorageWriter(saver, manager_future)
+    writer.reset(cid.data)
+    with torch.cuda.stream(side):
+        buckets, metadata, *_ = statedictsaver.generate_plan(cid, sd, writer, DefaultSavePlanner(), dist)
+        staged = MemoryStorageWriter.stage_write_data_buckets(cid, buckets, non_blocking=True)
+    assert saver._engine_clear_of == {torch.cuda.current_stream().cuda_stream, side.cuda_stream}
+    snapshot = {k: v.cpu() for k, v in sd.items()}
+    statedictsaver.write_data(cid, writer, staged, replicate_after_write=False)
+    statedictsaver.finish_write(cid, writer, metadata, dist)
+    saver.finalize_checkpoint(cid)
+    _check_files(cid, snapshot)
+
+
 def test_failure_in_the_background_write_reaches_the_waiter(shm_dir, manager_future, monkeypatch):
     saver = _make_saver(background_write=True)
     cid = CheckpointContainerId(os.path.join(shm_dir, "step-4_ckpt"))
