@@ -473,8 +473,9 @@ def main():
             file_bytes = os.path.getsize(os.path.join(cid.data, "__0__0_src0.distcp"))
             prev = cid
             line = (f"[bench] it {it} {'timed ' if timed else ('prime ' if it == 0 else 'warmup')} save {sv['save']:.3f}s (blocking "
-                    f"{sv['blocking'] * 1e3:.1f} ms, pack kernel {sv['pack_ms']:.2f} ms, d2h {d2h.get('d2h_s', 0):.3f}s) "
-                    f"restore {t2 - t1:.3f}s (h2d {ld.get('h2d_s', 0):.3f}s, unpack {unpack_ms:.2f} ms)")
+                    f"{sv['blocking'] * 1e3:.1f} ms, pack kernel {sv['pack_ms']:.2f} ms, d2h {d2h.get('d2h_s', 0):.3f}s, of which "
+                    f"{d2h.get('d2h_wait_s', 0):.3f}s waiting for the pack) restore {t2 - t1:.3f}s (h2d {ld.get('h2d_s', 0):.3f}s, "
+                    f"of which {ld.get('h2d_host_s', 0):.3f}s filling slots, unpack {unpack_ms:.2f} ms)")
             print(line, file=sys.stderr, flush=True)
             if it == 0:
                 first = {"save": sv["save"], "restore": t2 - t1, "blocking": sv["blocking"]}
