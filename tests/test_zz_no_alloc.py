@@ -5,8 +5,6 @@ fixed device array that every call on the device shares and that keeps the last 
 made on two calls in a row, the second on a smaller input, and once more after an unrelated call in between.
 """
 
-import ctypes
-
 import numpy as np
 import pytest
 import torch
