@@ -1110,3 +1110,49 @@ def test_large_ranges_go_through_two_alternating_buffers_by_choice(shm_dir, mana
         dcp.load(targets(), checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), no_dist=True)
     cause = exc.value.failures[0][0] if hasattr(exc.value, "failures") else exc.value
     assert isinstance(cause, integrity.ChecksumMismatchError) and "chunk(s) [9]" in str(cause)
+
+
+def test_a_failed_upload_in_a_pipelined_restore_is_reported_and_the_loader_stays_usable(shm_dir, manager_future, monkeypatch):
+    """The upload of a later window fails on the helper thread (forced from the host; every kernel that was launched
+    still runs to its end): the restore raises that error, commits nothing, and the same loader restores the object
+    correctly afterwards."""
+    from ml_flashpoint.hip import checkpoint_loader as loader_mod
+
+    monkeypatch.setattr(loader_mod, "_PIPELINED_FROM_BYTES", 1 << 20)
+    monkeypatch.setattr(loader_mod, "_PIPELINED_MIN_BYTES", 1 << 20)
+    sd_cpu = {f"t{i:02d}": torch.randn(90_000 + 777 * i, generator=torch.Generator().manual_seed(100 + i)) for i in range(16)}
+    sd_dev = _to_dev(sd_cpu)
+    ckpt = os.path.join(shm_dir, "step-22_ckpt")
+    dcp.save(sd_dev, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(_saver(crc_chunk_bytes=1 << 16), manager_future), no_dist=True)
+
+    loader = _loader()
+    real_upload = loader._upload
+    calls = []
+
+    def failing_upload(*args, **kwargs):
+        calls.append(1)
+        if len(calls) == 3:
+            raise OSError("injected: the third window could not be read")
+        return real_upload(*args, **kwargs)
+
+    committed = []
+
+    class Planner(dcp.DefaultLoadPlanner):
+        def commit_tensor(self, read_item, tensor):
+            committed.append(read_item.dest_index.fqn)
+            return super().commit_tensor(read_item, tensor)
+
+    monkeypatch.setattr(loader, "_upload", failing_upload)
+    target = {k: torch.zeros_like(v) for k, v in sd_dev.items()}
+    with pytest.raises(BaseException) as exc:
+        dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), planner=Planner(), no_dist=True)
+    cause = exc.value.failures[0][0] if hasattr(exc.value, "failures") else exc.value
+    assert isinstance(cause, OSError) and "injected" in str(cause)
+    assert len(calls) >= 3 and committed == []
+    torch.cuda.synchronize()
+
+    monkeypatch.setattr(loader, "_upload", real_upload)
+    target = {k: torch.zeros_like(v) for k, v in sd_dev.items()}
+    dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), planner=Planner(), no_dist=True)
+    assert loader.last_load_stats["windows"] >= 4 and sorted(committed) == sorted(sd_cpu)
+    assert all(torch.equal(target[k].cpu(), v) for k, v in sd_cpu.items())
