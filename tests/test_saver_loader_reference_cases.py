@@ -580,12 +580,6 @@ def test_read_a_missing_object(backend, tmp_path):
 
 
 # ---- read_tensor on the host (loader :223-380) ---------------------------------------------------------------------------------
-def _host_loader():
-    from ml_flashpoint.hip.checkpoint_loader import HipMLFlashpointCheckpointLoader
-
-    return HipMLFlashpointCheckpointLoader(CheckpointObjectManager(), None)  # no kernel is launched by read_tensor
-
-
 def _torch_saved(tensor):
     stream = io.BytesIO()
     torch.save(tensor, stream)
@@ -608,7 +602,7 @@ def _torch_saved(tensor):
 def test_read_tensor_known_slices_of_a_torch_saved_record(stored, offsets, lengths, expected, optimized):
     """A ``torch.save`` record is read by either loader setting: its first four bytes give a length far above the
     limit for a header, so the optimized loader falls back (loader tests :223-302, :359-380)."""
-    got = _host_loader().read_tensor(_torch_saved(stored), _read_item(LoadItemType.TENSOR, 0, offsets, lengths),
+    got = _host_loader("hip").read_tensor(_torch_saved(stored), _read_item(LoadItemType.TENSOR, 0, offsets, lengths),
                                      use_optimized_loader=optimized)
     assert got.dtype == expected.dtype and torch.equal(got, expected)
 
@@ -621,17 +615,17 @@ def test_read_tensor_of_a_header_record():
     stream.write(TensorHeader(dtype=tensor.dtype, shape=tensor.shape).to_bytes())
     stream.write(tensor.numpy().tobytes())
     stream.seek(len(b"skipped"))
-    got = _host_loader().read_tensor(stream, _read_item(LoadItemType.TENSOR, 0, (0,), (3,)), use_optimized_loader=True)
+    got = _host_loader("hip").read_tensor(stream, _read_item(LoadItemType.TENSOR, 0, (0,), (3,)), use_optimized_loader=True)
     assert got.dtype == torch.int32 and torch.equal(got, tensor)
     stream.seek(len(b"skipped"))
     with pytest.raises(Exception):  # without the optimized loader the record is handed to torch.load, which rejects it
-        _host_loader().read_tensor(stream, _read_item(LoadItemType.TENSOR, 0, (0,), (3,)))
+        _host_loader("hip").read_tensor(stream, _read_item(LoadItemType.TENSOR, 0, (0,), (3,)))
 
 
 def test_read_tensor_of_bytes_that_are_no_record():
     with pytest.raises(IndexError):  # what torch.load raises for this text (loader test :304-320)
-        _host_loader().read_tensor(io.BytesIO(b"this is not a valid tensor"), _read_item(LoadItemType.TENSOR, 0, (0,), (1,)))
+        _host_loader("hip").read_tensor(io.BytesIO(b"this is not a valid tensor"), _read_item(LoadItemType.TENSOR, 0, (0,), (1,)))
     header = TensorHeader(dtype=torch.float32, shape=torch.Size([4])).to_bytes()
     with pytest.raises(Exception):  # a header whose payload is cut short
-        _host_loader().read_tensor(io.BytesIO(header + b"\0" * 15), _read_item(LoadItemType.TENSOR, 0, (0,), (4,)),
+        _host_loader("hip").read_tensor(io.BytesIO(header + b"\0" * 15), _read_item(LoadItemType.TENSOR, 0, (0,), (4,)),
                                    use_optimized_loader=True)
