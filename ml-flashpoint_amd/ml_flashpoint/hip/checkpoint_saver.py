@@ -726,7 +726,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         held = contextlib.ExitStack()  # the buffer stays open until the last byte has been written
         sender = concurrent.futures.ThreadPoolExecutor(max_workers=1, thread_name_prefix=f"mlf-write-{object_name}")
         sent: list = []  # one future per window, in order
-        spent: list = []  # plans whose windows have been sent
+        made: list = []  # every plan built here; released at the end (freeing device memory waits for the whole device)
         try:
             writer = held.enter_context(
                 self._chkpt_obj_manager.acquire_buffer(object_id, max(self._initial_buffer_size_bytes, nbytes)))
@@ -753,6 +753,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                     sub["image_off"] -= begin - pad
                     plan = hip_plan.Plan(sub, layout.blob, pad + end - begin, tile_bytes=self._tile_bytes,
                                          block_threads=self._block_threads)
+                    made.append(plan)
                     if self.record_kernel_events:
                         t_begin, packed = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                         t_begin.record()
@@ -782,7 +783,6 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                             sums.add(begin, end - begin, hip_plan.crc32c_device_cut(
                                 buf, pad, begin, end - begin, self._crc_chunk_bytes, dst, side))
                             xfer["crc_s"] = xfer.get("crc_s", 0.0) + time.perf_counter() - t0
-                        spent.append(plan)  # (released at the end: freeing device memory waits for the whole device)
 
                 # the resident part: the longest run of records at the end that fits beside the window buffers
                 cycle = max(min(limit // 4, _WINDOW_BUFFER_BYTES), 1)
@@ -816,6 +816,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                     staged.packed_event = packed  # the live tensors are not read after the last of these
         except BaseException:
             sender.shutdown(wait=True)
+            for plan in made:
+                plan.destroy()
             held.__exit__(*sys.exc_info())
             raise
 
@@ -835,7 +837,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             except BaseException as e:  # reported to whoever waits; a thread must not die silently
                 _LOGGER.exception("Windowed write of '%s' failed", object_id)
                 outcome = (False, f"{type(e).__name__}: {e}")
-            for plan in spent:
+            for plan in made:
                 plan.destroy()
             stats.update({k: stats.get(k, 0) + v for k, v in xfer.items()})  # (the dict last_save_stats refers to)
             try:
