@@ -152,7 +152,7 @@ struct mlf_engine {
 
 namespace {
 
-// The two kernels of the hardware-queue test (mlf_engine_avoid_stream).  The first keeps one wavefront busy for a
+// The two kernels of the hardware-queue test (mlf_engine_avoid_streams).  The first keeps one wavefront busy for a
 // stated time by the device's constant-rate clock (100 MHz) - bounded by a count as well, so that it ends whatever
 // that clock does; the second does nothing but exist.
 __global__ void mlf_queue_test_hold(uint64_t ticks, uint32_t* out) {
