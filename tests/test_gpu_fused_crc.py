@@ -116,6 +116,49 @@ def test_pack_with_checksums_small_images(nbytes, oracle_c):
         assert fused.crc_values().tolist() == _oracle_chunks(oracle_c, raw, chunk).tolist()
 
 
+def test_one_item_beyond_4_gib_with_checksums():
+    """A single tensor of 5 GiB + 12 345 bytes at a byte-misaligned address: positions inside the item pass 2^32.
+    The fused pack moves what the plain pack moves, its per-chunk values equal the stand-alone pass over the image
+    (itself held to the host's CRC at 8.5 GiB elsewhere), and the fused unpack brings the tensor back and reports
+    the same values."""
+    from ml_flashpoint.hip import plan as P
+
+    need = 4 * (5 << 30) + (2 << 30)
+    if torch.cuda.mem_get_info()[0] < need:
+        pytest.skip("not enough free device memory")
+    n = 5 * (1 << 30) + 12345
+    gen = torch.Generator(device=DEV).manual_seed(41)
+    parent = torch.randint(0, 256, (n + 64,), dtype=torch.uint8, device=DEV, generator=gen)
+    tensor = parent[3 : 3 + n]
+    layout = P.build_save_layout([tensor])
+    chunk = 32 << 20
+    plain = P.Plan(layout.items, layout.blob, layout.image_bytes)
+    fused = P.Plan(layout.items, layout.blob, layout.image_bytes, crc_chunk_bytes=chunk)
+    assert fused.info.fused_crc_bytes > (1 << 32)
+    image_a = torch.zeros(layout.image_bytes, dtype=torch.uint8, device=DEV)
+    image_b = torch.full((layout.image_bytes + 512,), 0xCD, dtype=torch.uint8, device=DEV)
+    plain.pack(image_a)
+    fused.pack(image_b)
+    got = fused.crc_values()
+    torch.cuda.synchronize()
+    assert torch.equal(image_a, image_b[: layout.image_bytes])
+    assert bool((image_b[layout.image_bytes :] == 0xCD).all()), "pack wrote past the end of the image"
+    want = P.crc32c_device(image_b, layout.image_bytes, chunk)
+    assert len(got) == -(-layout.image_bytes // chunk) and got.tolist() == want.tolist()
+    del image_a, plain, fused
+    back = torch.full((n + 64,), 0x5A, dtype=torch.uint8, device=DEV)
+    table = P.ItemTable()
+    (offset, length), = layout.spans
+    table.add_contiguous(back.data_ptr() + 7, offset + length - n, 1, n)
+    unpacker = P.Plan(table.to_array(), b"", layout.image_bytes, align_to_tensor=True, crc_chunk_bytes=chunk)
+    unpacker.unpack(image_b)
+    got = unpacker.crc_values()
+    torch.cuda.synchronize()
+    assert got.tolist() == want.tolist()
+    assert torch.equal(back[7 : 7 + n], tensor)
+    assert bool((back[:7] == 0x5A).all()) and bool((back[7 + n :] == 0x5A).all()), "guard bytes"
+
+
 @pytest.mark.parametrize("chunk", [65536, 1 << 20, 32 << 20])
 def test_unpack_with_checksums_restores_and_reports_the_images_values(chunk, oracle_c):
     from ml_flashpoint.hip import plan as P
