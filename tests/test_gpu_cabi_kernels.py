@@ -154,6 +154,33 @@ def test_pack_strided_views_match_bruteforce_oracle(dtype):
     assert plan.info.n_strided_items > 0
 
 
+def _broadcast_views(base):
+    """Views with stride-0 dimensions (``expand``): every element of the logical tensor is written out, as
+    ``copy_`` into a contiguous buffer does."""
+    m = base[0]
+    return [
+        m[5].expand(64, 96),  # one row, repeated: strides (0, 1)
+        m[:, 5:6].expand(64, 96),  # one column, repeated along the fast dimension: strides (96, 0)
+        m[3, 7].expand(40, 50),  # one element: strides (0, 0)
+        base[:, 2:3, ::2].expand(3, 33, 48),  # a broadcast dimension between two real ones, the last one strided
+        m.t()[:, None, :].expand(96, 4, 64),  # transposed and broadcast
+    ]
+
+
+@pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.bfloat16, torch.float32, torch.int64])
+def test_pack_views_with_broadcast_dimensions(dtype):
+    gen = torch.Generator().manual_seed(15)
+    base_cpu = _rand_tensor(gen, (3, 64, 96), dtype)
+    cpu, dev = _broadcast_views(base_cpu), _broadcast_views(base_cpu.to(DEV))
+    assert all(0 in t.stride() for t in dev)
+    _, _, _, got = _pack_image(dev)
+    assert got == b"".join(
+        oracle_fmt.header_bytes(oracle_fmt.dtype_name(t.dtype), tuple(t.shape)) + oracle_fmt.payload_bytes_bruteforce(t)
+        for t in cpu
+    )
+    assert got == oracle_fmt.data_section(cpu)[0]
+
+
 TRANSPOSE_SHAPES = [(16, 16), (17, 130), (128, 128), (129, 257), (300, 31), (64, 1000), (5, 40, 70)]
 
 
