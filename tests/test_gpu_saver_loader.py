@@ -1156,3 +1156,34 @@ def test_a_failed_upload_in_a_pipelined_restore_is_reported_and_the_loader_stays
     dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), planner=Planner(), no_dist=True)
     assert loader.last_load_stats["windows"] >= 4 and sorted(committed) == sorted(sd_cpu)
     assert all(torch.equal(target[k].cpu(), v) for k, v in sd_cpu.items())
+
+
+def test_tied_and_overlapping_tensors_are_saved_once_per_name_and_restored_into_shared_storage(shm_dir, manager_future):
+    """Tied weights (one tensor under two names), a slice of it under a third and a view of its transpose: every
+    name gets its own record, as the reference's per-item loop writes them (checkpoint_saver.py:667-698); restoring
+    into targets that share storage the same way writes the same bytes through every alias."""
+    g = torch.Generator().manual_seed(7)
+    w_cpu = torch.randn(96, 160, generator=g)
+    other_cpu = torch.randn(50_000, generator=g)
+
+    def tied(w, other):
+        return {"embed.weight": w, "lm_head.weight": w, "embed.first_rows": w[:40], "embed.transposed": w.t(),
+                "other": other, "step": 9}
+
+    sd_cpu, sd_dev = tied(w_cpu, other_cpu), tied(w_cpu.to(DEV), other_cpu.to(DEV))
+    ckpt = os.path.join(shm_dir, "step-31_ckpt")
+    dcp.save(sd_dev, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(_saver(crc_chunk_bytes=1 << 16), manager_future),
+             no_dist=True)
+    raw = open(os.path.join(ckpt, "__0__0_src0.distcp"), "rb").read()
+    metadata = pickle.load(open(os.path.join(ckpt, ".metadata"), "rb"))
+    image, spans, got_spans = _expected_file(sd_cpu, metadata, raw)
+    assert raw == image and got_spans == spans
+    assert len([i for i in metadata.storage_data if i.fqn.startswith(("embed", "lm_head"))]) == 4
+
+    target = tied(torch.zeros(96, 160, device=DEV), torch.zeros(50_000, device=DEV))
+    target["step"] = None
+    dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, _loader()), no_dist=True)
+    assert target["step"] == 9 and target["lm_head.weight"].data_ptr() == target["embed.weight"].data_ptr()
+    for k, v in sd_cpu.items():
+        if isinstance(v, torch.Tensor):
+            assert torch.equal(_bits(target[k]), _bits(v)), k
