@@ -1187,3 +1187,56 @@ def test_tied_and_overlapping_tensors_are_saved_once_per_name_and_restored_into_
     for k, v in sd_cpu.items():
         if isinstance(v, torch.Tensor):
             assert torch.equal(_bits(target[k]), _bits(v)), k
+
+
+def test_a_real_module_and_optimizer_state_round_trip(shm_dir, manager_future):
+    """What a training script hands over: ``module.state_dict(keep_vars=True)`` (Parameters that require grad, a
+    channels-last convolution weight, buffers, an integer counter) and ``optimizer.state_dict()`` (nested dicts, lists
+    of hyper-parameters, per-parameter moments, 0-dim step tensors).  The object equals the oracle's image of the same
+    state on the host, and a second model and optimizer loaded from it hold the same bits: weights, buffers, moments,
+    step counts, hyper-parameters."""
+    torch.manual_seed(3)
+
+    def build():
+        model = torch.nn.Sequential(
+            torch.nn.Conv2d(3, 8, 3, padding=1), torch.nn.BatchNorm2d(8), torch.nn.Flatten(), torch.nn.Linear(8 * 6 * 6, 10)
+        ).to(DEV).to(memory_format=torch.channels_last)
+        return model, torch.optim.AdamW(model.parameters(), lr=1e-2)
+
+    def step(model, optim, seed):
+        x = torch.randn(4, 3, 6, 6, generator=torch.Generator().manual_seed(seed)).to(DEV)
+        optim.zero_grad()
+        model(x).square().mean().backward()
+        optim.step()
+
+    model, optim = build()
+    for seed in (1, 2):
+        step(model, optim, seed)
+    sd = {"model": model.state_dict(keep_vars=True), "optim": optim.state_dict()}
+    assert sd["model"]["0.weight"].requires_grad and not sd["model"]["0.weight"].is_contiguous()
+    ckpt = os.path.join(shm_dir, "step-41_ckpt")
+    dcp.save(sd, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(_saver(crc_chunk_bytes=1 << 16), manager_future),
+             no_dist=True)
+    raw = open(os.path.join(ckpt, "__0__0_src0.distcp"), "rb").read()
+    metadata = pickle.load(open(os.path.join(ckpt, ".metadata"), "rb"))
+    from torch.distributed.checkpoint._nested_dict import flatten_state_dict
+
+    flat, _ = flatten_state_dict(sd)
+    flat_cpu = {k: (v.detach().cpu() if isinstance(v, torch.Tensor) else v) for k, v in flat.items()}
+    image, spans, got_spans = _expected_file(flat_cpu, metadata, raw)
+    assert raw == image and got_spans == spans
+
+    model2, optim2 = build()
+    step(model2, optim2, 77)  # gives the second optimizer its state entries (other values)
+    sd2 = {"model": model2.state_dict(keep_vars=True), "optim": optim2.state_dict()}
+    dcp.load(sd2, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, _loader()), no_dist=True)
+    optim2.load_state_dict(sd2["optim"])
+    for (k, a), b in zip(model.state_dict().items(), model2.state_dict().values()):
+        assert torch.equal(_bits(a), _bits(b)), k
+    want, got = optim.state_dict(), optim2.state_dict()
+    assert got["param_groups"] == want["param_groups"] and got["state"].keys() == want["state"].keys()
+    for index, moments in want["state"].items():
+        assert moments.keys() == got["state"][index].keys()
+        for name, value in moments.items():
+            assert torch.equal(_bits(value), _bits(got["state"][index][name])), (index, name)
+    assert int(got["state"][0]["step"]) == 2  # (the second optimizer had taken one step of its own)
