@@ -60,6 +60,8 @@ MIXED = [
     ((129, 3), torch.float8_e5m2),
     ((4099,), torch.float8_e4m3fnuz),
     ((2, 515), torch.float8_e5m2fnuz),
+    ((4097,), torch.float8_e8m0fnu),  # the block scales of the MX formats
+    ((96, 1040), torch.float4_e2m1fn_x2),  # two fp4 values per byte
     ((1 << 20,), torch.float32),
     ((777, 513), torch.float64),
 ]
@@ -470,7 +472,8 @@ def test_unpack_restores_full_tensors_bit_exact():
     cpu = [_rand_tensor(gen, s, d) for s, d in MIXED]
     data, spans = oracle_fmt.data_section(cpu)
     image = torch.frombuffer(bytearray(data), dtype=torch.uint8).to(DEV)
-    targets = [torch.zeros_like(t, device=DEV) for t in cpu]
+    # (zeroed as bytes: torch has no fill kernel for some of the dtypes, the packed fp4 pairs among them)
+    targets = [torch.zeros(t.numel() * t.element_size(), dtype=torch.uint8, device=DEV).view(t.dtype).reshape(t.shape) for t in cpu]
     table = P.ItemTable()
     for t, tgt, (off, length) in zip(cpu, targets, spans):
         nbytes = t.numel() * t.element_size()
