@@ -279,3 +279,13 @@ def test_a_forked_child_starts_with_free_locks_and_a_running_collector():
             CheckpointObjectManager._worker_pool_lock.release()
     assert os.WIFEXITED(status) and os.WEXITSTATUS(status) == 0
     assert gc.isenabled()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The benchmark measures one GPU's share of the path; asked for more it says so and exits, before any GPU work."""
+    import sys
+
+    bench = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bench.py")
+    done = subprocess.run([sys.executable, bench, "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert done.returncode == 2
+    assert "one GPU" in done.stderr + done.stdout
