@@ -84,7 +84,7 @@ def parse_args():
     ap.add_argument("--whole-image-restore", action="store_true",
                     help="restore through one device buffer for the whole object instead of two alternating ones")
     ap.add_argument("--no-prefault", action="store_true", help="leave the pool file's pages to the first save, as the reference does")
-    ap.add_argument("--no-link-probe", action="store_true", help="skip the bare host-link measurement")
+    ap.add_argument("--no-link-probe", action="store_true", help="skip the bare host-link and device-copy measurements")
     ap.add_argument("--busy-gpu-probe", action="store_true",
                     help="also time a save whose transfer runs on a background thread while bf16 GEMMs, then HBM copies, "
                          "keep the device busy: what the transfer costs them, and what they cost the transfer")
@@ -244,6 +244,43 @@ def _rewrite_warm(path, tensors):
         mv.release()
         mm.close()
     return spans
+
+
+def _hbm_copy_probe(device, tile_bytes, block_threads, nbytes=8 << 30, reps=5):
+    """What this device's memory gives a plain copy, measured in the same run as the pack: torch's device-to-device
+    ``copy_`` of ``nbytes``, and this library's flat kernel packing one contiguous tensor of that size (one record
+    header, one span, no other tables).  Both move 2 x ``nbytes``; the best of ``reps`` launches counts."""
+    import torch
+
+    from ml_flashpoint.hip import plan as hip_plan
+
+    src = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+    layout = hip_plan.build_save_layout([src])
+    image = torch.empty(layout.image_bytes, dtype=torch.uint8, device=device)
+    plan = hip_plan.Plan(layout.items, layout.blob, layout.image_bytes, tile_bytes=tile_bytes, block_threads=block_threads)
+    stream = torch.cuda.current_stream(device)
+
+    def best_ms(launch):
+        launch()  # untimed first launch
+        times = []
+        for _ in range(reps):
+            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            begin.record(stream)
+            launch()
+            end.record(stream)
+            end.synchronize()
+            times.append(begin.elapsed_time(end))
+        return min(times)
+
+    try:
+        torch_ms = best_ms(lambda: image[:nbytes].copy_(src))
+        flat_ms = best_ms(lambda: plan.pack(image, stream.cuda_stream))
+    finally:
+        plan.destroy()
+    return {"bytes": nbytes, "torch_copy_GBps": round(2 * nbytes / 1e6 / torch_ms, 1),
+            "flat_kernel_one_tensor_GBps": round(2 * nbytes / 1e6 / flat_ms, 1),
+            "what": "read + write rate of a device-to-device copy of one contiguous tensor: torch's copy_ and this "
+                    "library's pack kernel, best of %d launches each" % reps}
 
 
 def _busy_gpu_probe(device, saver, sd, root, manager):
@@ -595,6 +632,11 @@ def main():
                     "bytes": probe_bytes, "slot_mib": args.slot_mib, "streams": 2,
                     "what": "pinned hipMemcpyAsync between HBM and the copy engine's own slots, no host-side copy"}
 
+        # ---- the device's own copy rate, beside which the pack's figure is to be read ----
+        copy_probe = None
+        if not args.no_link_probe and max_image is None:
+            copy_probe = _hbm_copy_probe(device, args.tile_bytes, args.block_threads)
+
         step_s = mean(rec["step"])
         gb = file_bytes / 1e9
         unpack_s = mean(rec["unpack_ms"]) * 1e-3
@@ -663,6 +705,7 @@ def main():
             **({"save_windows": int(mean(rec["windows"])), "save_image_pieces": int(mean(rec["image_pieces"]))}
                if mean(rec["windows"]) or mean(rec["image_pieces"]) else {}),
             **({"link_roofline": link} if link else {}),
+            **({"hbm_copy_probe": copy_probe} if copy_probe else {}),
             **({"crc_modes": crc_modes} if crc_modes else {}),
             **({"with_dcp_plan_cache": with_cache} if with_cache else {}),
             **({"beside_a_busy_gpu": busy} if busy else {}),
