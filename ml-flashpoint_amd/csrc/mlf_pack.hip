@@ -78,10 +78,6 @@ struct StridedDesc {
   int64_t tstride[MLF_MAX_DIMS];  // bytes
   int64_t istride[MLF_MAX_DIMS];  // bytes
   int64_t step[MLF_MAX_DIMS];     // 256 written in the mixed radix of `shape`: what one loop trip adds to the index
-  // > 0: the image side is contiguous along the last dimension and the tensor side takes every gather_k-th element
-  // (2..4) of long rows; work items then never cross a row, and packing reads whole vectors and keeps what it needs
-  uint32_t gather_k;
-  uint32_t pad;
 };
 
 struct StridedWork {  // one workgroup's work: elements [start, start+count) of descriptor `desc`
@@ -90,10 +86,21 @@ struct StridedWork {  // one workgroup's work: elements [start, start+count) of 
   uint32_t desc;
 };
 
+// A piece of one row of an item whose image side is contiguous along the last dimension while the tensor side takes
+// every k-th element (k = 2..4) of long rows: `count` elements, consecutive in the image, k * esz bytes apart in the
+// tensor.  Packing reads whole vectors and keeps what it needs; unpacking hands image vectors out through LDS.
+struct GatherWork {
+  uint64_t tensor;  // device address of the piece's first element
+  uint64_t image;   // its byte offset in the image
+  uint32_t count;
+  uint16_t k, esz;
+};
+
 constexpr int kMaxBatchDims = MLF_MAX_DIMS - 2;
-constexpr uint32_t kTransTilesPerEntry = 256;
 
 // A 2-D transposition (plus outer "batch" dims): dim a is contiguous on the tensor side, dim b on the image side.
+// The tile grid starts a_lead elements before element 0 along a and b_lead before it along b, so that tile cuts fall
+// on 128-byte lines of the tensor side (a) and of the image side (b) in every row whose pitch is a multiple of 128.
 struct TransDesc {
   uint64_t tensor;  // device address of element 0
   uint64_t image;   // byte offset of element 0 in the image
@@ -102,18 +109,19 @@ struct TransDesc {
   int64_t na, nb;   // extents of a and b
   int64_t ld_t;     // tensor-side byte stride of dim b (dim a has byte stride esz there)
   int64_t ld_i;     // image-side byte stride of dim a  (dim b has byte stride esz there)
-  uint32_t tiles_a, tiles_b;
-  uint64_t n_tiles;  // batch count * tiles_a * tiles_b
+  uint32_t a_lead, b_lead;
   int64_t bshape[kMaxBatchDims];
   int64_t bts[kMaxBatchDims];  // bytes
   int64_t bis[kMaxBatchDims];  // bytes
 };
 
-struct TransWork {  // kTransTilesPerEntry consecutive tiles of descriptor `desc`, starting at `first_tile`
-  uint64_t first_tile;
+struct TransTile {  // one workgroup's tile: (ta, tb) of batch `batch` of descriptor `desc`; desc == kNoTile: none
   uint32_t desc;
-  uint32_t pad;
+  uint32_t ta, tb;
+  uint32_t batch;
 };
+constexpr uint32_t kNoTile = 0xFFFFFFFFu;
+constexpr int kTransClasses = 5;  // element sizes 1, 2, 4, 8, 16
 
 
 // ---------------------------------------------------------------------------------------------------------
@@ -345,82 +353,127 @@ __device__ __forceinline__ void strided_walk(const StridedDesc* __restrict__ d, 
 }
 
 // Packing `x[..., ::k]` (k = 2, 3, 4) out of long rows.  Element-sized accesses top out near 0.45 T elements/s on
-// this part whatever the loop around them looks like, so a thread reads the 16 k source bytes that hold its 16 output
-// bytes as k whole vectors, keeps every k-th element with compile-time shuffles, and writes one vector.
+// this part whatever the loop around them looks like, so the kept elements are cut out of whole 16-byte vectors with
+// compile-time shuffles and written as whole vectors.  A work item (a piece of one row, at most kGatherUnitsPerBlock
+// output vectors) is shared by kGatherSplit workgroups that make one trip each: short-lived workgroups that follow
+// each other through the rows keep the traffic a compact window on both sides, as in the flat kernel.
+constexpr uint32_t kGatherSplit = 4;
+
 template <int K, typename T>
-__device__ __forceinline__ void strided_gather(const StridedDesc* __restrict__ d, const StridedWork& w,
-                                               char* __restrict__ image) {
-  typedef T elem_u __attribute__((aligned(1)));
+__device__ __forceinline__ void gather_units(const char* __restrict__ sp, char* __restrict__ dp, uint32_t u0,
+                                             uint32_t u1) {
   constexpr int EPV = 16 / (int)sizeof(T);
-  const int last = (int)d->ndim - 1;
-  const uint64_t len = (uint64_t)d->shape[last];
-  uint64_t row = w.start / len;  // uniform over the workgroup: scalar arithmetic
-  const uint64_t j0 = w.start - row * len;
-  int64_t toff = (int64_t)j0 * d->tstride[last], ioff = (int64_t)j0 * d->istride[last];
-#pragma unroll
-  for (int dim = MLF_MAX_DIMS - 2; dim >= 0; --dim) {
-    if (dim < last) {
-      const uint64_t extent = (uint64_t)d->shape[dim];
-      const uint64_t q = row / extent;
-      const int64_t at = (int64_t)(row - q * extent);
-      toff += at * d->tstride[dim];
-      ioff += at * d->istride[dim];
-      row = q;
-    }
-  }
-  const char* sp = reinterpret_cast<const char*>(d->tensor) + toff;
-  char* dp = image + d->image + ioff;
-  // whole units only where all 16 K source bytes lie at or before the item's last element: a vector load must not
-  // run past the end of the row (the storage may end there)
-  const uint32_t n_units = (uint32_t)((((uint64_t)w.count - 1) * K + 1) / (uint64_t)(EPV * K));
-  for (uint32_t u = threadIdx.x; u < n_units; u += 256) {
-    union {
-      u32x4 v[K];
-      T e[K * EPV];
-    } in;
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t w0 = u0 + (threadIdx.x & ~63u);  // this wavefront's 64 units
+  if (K == 2 && w0 + 64u <= u1) {
+    // k = 2, a whole block of 64 units: 2 KiB in, 1 KiB out.  Every lane loads one vector of the block's first KiB
+    // and one of its second (two loads that each cover a KiB of consecutive bytes, instead of 64 pieces of 16 bytes
+    // 32 apart), keeps the even elements of both - 8 bytes for output position 8 * lane, 8 bytes for 512 + 8 * lane -
+    // and trades one half with its neighbour, so that the even lane stores the pair's 16 bytes of the first half of
+    // the output block and the odd lane those of the second.
+    const char* s = sp + (size_t)w0 * 32;
     union {
       u32x4 v;
       T e[EPV];
-    } out;
-    const char* s = sp + (size_t)u * (16 * K);
+    } a, b;
+    a.v = __builtin_nontemporal_load(gload<u32x4_u>(s + lane * 16u));
+    b.v = __builtin_nontemporal_load(gload<u32x4_u>(s + 1024u + lane * 16u));
+    union {
+      uint32_t w[2];
+      T e[EPV / 2];
+    } ca, cb;
 #pragma unroll
-    for (int j = 0; j < K; ++j) in.v[j] = __builtin_nontemporal_load(gload<u32x4_u>(s + 16 * j));
-#pragma unroll
-    for (int j = 0; j < EPV; ++j) out.e[j] = in.e[j * K];
-    __builtin_nontemporal_store(out.v, gstore<u32x4_u>(dp + (size_t)u * 16));
+    for (int j = 0; j < EPV / 2; ++j) {
+      ca.e[j] = a.e[2 * j];
+      cb.e[j] = b.e[2 * j];
+    }
+    const bool odd = lane & 1u;
+    const uint32_t give0 = odd ? ca.w[0] : cb.w[0], give1 = odd ? ca.w[1] : cb.w[1];
+    // quad_perm [1, 0, 3, 2]: every lane reads its neighbour in the pair
+    const uint32_t take0 = (uint32_t)__builtin_amdgcn_mov_dpp((int)give0, 0xB1, 0xF, 0xF, true);
+    const uint32_t take1 = (uint32_t)__builtin_amdgcn_mov_dpp((int)give1, 0xB1, 0xF, 0xF, true);
+    u32x4 out;
+    out.x = odd ? take0 : ca.w[0];
+    out.y = odd ? take1 : ca.w[1];
+    out.z = odd ? cb.w[0] : take0;
+    out.w = odd ? cb.w[1] : take1;
+    char* o = dp + (size_t)w0 * 16 + (odd ? 512u + (lane - 1u) * 8u : lane * 8u);
+    __builtin_nontemporal_store(out, gstore<u32x4_u>(o));
+    return;
   }
-  // the elements after the last whole unit (fewer than 2 EPV): one each for the first threads
+  const uint32_t u = w0 + lane;
+  if (u >= u1) return;
+  union {
+    u32x4 v[K];
+    T e[K * EPV];
+  } in;
+  union {
+    u32x4 v;
+    T e[EPV];
+  } out;
+  const char* s = sp + (size_t)u * (16 * K);
+#pragma unroll
+  for (int j = 0; j < K; ++j) in.v[j] = __builtin_nontemporal_load(gload<u32x4_u>(s + 16 * j));
+#pragma unroll
+  for (int j = 0; j < EPV; ++j) out.e[j] = in.e[j * K];
+  __builtin_nontemporal_store(out.v, gstore<u32x4_u>(dp + (size_t)u * 16));
+}
+
+template <typename T>
+__device__ __forceinline__ void gather_piece(const GatherWork& w, uint32_t sub, char* __restrict__ image) {
+  typedef T elem_u __attribute__((aligned(1)));
+  constexpr uint32_t EPV = 16 / (uint32_t)sizeof(T);
+  const uint32_t K = w.k;
+  const char* sp = reinterpret_cast<const char*>(w.tensor);
+  char* dp = image + w.image;
+  // whole units only where all 16 K source bytes lie at or before the piece's last element: a vector load must not
+  // run past the end of the row (the storage may end there)
+  const uint32_t n_units = (uint32_t)((((uint64_t)w.count - 1) * K + 1) / (uint64_t)(EPV * K));
+  const uint32_t u0 = sub * 256u, u1 = n_units < u0 + 256u ? n_units : u0 + 256u;
+  if (u0 < u1) {
+    switch (K) {
+      case 2: gather_units<2, T>(sp, dp, u0, u1); break;
+      case 3: gather_units<3, T>(sp, dp, u0, u1); break;
+      default: gather_units<4, T>(sp, dp, u0, u1); break;
+    }
+  }
+  // the elements after the last whole unit (fewer than 2 EPV): one each for the first threads of the last workgroup
   const uint32_t j = n_units * EPV + threadIdx.x;
-  if (j < w.count) *gstore<elem_u>(dp + (size_t)j * sizeof(T)) = *gload<elem_u>(sp + (size_t)j * (K * sizeof(T)));
+  if (sub == kGatherSplit - 1u && j < w.count)
+    *gstore<elem_u>(dp + (size_t)j * sizeof(T)) = *gload<elem_u>(sp + (size_t)j * (K * sizeof(T)));
+}
+
+__global__ void __launch_bounds__(256) mlf_gather_kernel(const GatherWork* __restrict__ work, uint32_t n_wgs,
+                                                         char* __restrict__ image) {
+  // Workgroups reach the eight XCDs round-robin; the image side of neighbouring workgroups meets in partly written
+  // lines (image offsets are arbitrary), which should meet in one L2: of every 8 * kRun workgroups each XCD takes
+  // kRun consecutive ones.  Measured on 667 `[r0:r1, ::2]` bands of 2-16 MB (TB/s of 2 x payload; 4.3 is the ceiling
+  // of a kernel that must fetch the skipped elements too): runs of 1 / 4 / 16 / 64 / 256 workgroups 3.88 / 3.92 /
+  // 4.09 / 4.23 / 4.25; one workgroup per work item making four trips, lanes reading 16 bytes 32 apart: 3.37.
+  constexpr uint32_t kRun = 64, G = 8u * kRun;
+  uint32_t wg = blockIdx.x;
+  const uint32_t g0 = wg / G * G;
+  if (g0 + G <= n_wgs) wg = g0 + (wg & 7u) * kRun + ((wg - g0) >> 3);
+  const GatherWork w = work[wg / kGatherSplit];
+  const uint32_t sub = wg % kGatherSplit;
+  switch (w.esz) {
+    case 1: gather_piece<uint8_t>(w, sub, image); break;
+    case 2: gather_piece<uint16_t>(w, sub, image); break;
+    case 4: gather_piece<uint32_t>(w, sub, image); break;
+    default: gather_piece<uint64_t>(w, sub, image); break;
+  }
 }
 
 // The way back, unpacking into `x[..., ::k]`: the gaps must not be written, so the stores stay element-sized, but
 // the image side is read as whole vectors and handed out through LDS so that neighbouring lanes store neighbouring
 // elements.  That removes almost half of the element-sized accesses (all the loads).
 template <typename T>
-__device__ __forceinline__ void strided_scatter(const StridedDesc* __restrict__ d, const StridedWork& w,
-                                                char* __restrict__ image, u32x4* __restrict__ lds) {
+__device__ __forceinline__ void scatter_piece(const GatherWork& w, char* __restrict__ image, u32x4* __restrict__ lds) {
   typedef T elem_u __attribute__((aligned(1)));
   constexpr uint32_t EPV = 16 / (uint32_t)sizeof(T);
-  const int last = (int)d->ndim - 1;
-  const uint64_t len = (uint64_t)d->shape[last];
-  uint64_t row = w.start / len;  // uniform over the workgroup: scalar arithmetic
-  const uint64_t j0 = w.start - row * len;
-  const int64_t ts = d->tstride[last];
-  int64_t toff = (int64_t)j0 * ts, ioff = (int64_t)j0 * d->istride[last];
-#pragma unroll
-  for (int dim = MLF_MAX_DIMS - 2; dim >= 0; --dim) {
-    if (dim < last) {
-      const uint64_t extent = (uint64_t)d->shape[dim];
-      const uint64_t q = row / extent;
-      const int64_t at = (int64_t)(row - q * extent);
-      toff += at * d->tstride[dim];
-      ioff += at * d->istride[dim];
-      row = q;
-    }
-  }
-  const char* sp = image + d->image + ioff;
-  char* dp = reinterpret_cast<char*>(d->tensor) + toff;
+  const int64_t ts = (int64_t)w.k * (int64_t)sizeof(T);
+  const char* sp = image + w.image;
+  char* dp = reinterpret_cast<char*>(w.tensor);
   const uint32_t n_units = w.count / EPV;
   const T* __restrict__ lds_elems = reinterpret_cast<const T*>(lds);
   for (uint32_t base = 0; base < n_units; base += 256) {  // uniform trip count: every thread reaches the barriers
@@ -437,13 +490,14 @@ __device__ __forceinline__ void strided_scatter(const StridedDesc* __restrict__ 
   if (j < w.count) *gstore<elem_u>(dp + (int64_t)j * ts) = *gload<elem_u>(sp + (size_t)j * sizeof(T));
 }
 
-template <typename T>
-__device__ __forceinline__ void strided_gather_k(const StridedDesc* __restrict__ d, const StridedWork& w,
-                                                 char* __restrict__ image) {
-  switch (d->gather_k) {
-    case 2: strided_gather<2, T>(d, w, image); break;
-    case 3: strided_gather<3, T>(d, w, image); break;
-    default: strided_gather<4, T>(d, w, image); break;
+__global__ void __launch_bounds__(256) mlf_scatter_kernel(const GatherWork* __restrict__ work, char* __restrict__ image) {
+  __shared__ u32x4 lds[256];
+  const GatherWork w = work[blockIdx.x];
+  switch (w.esz) {
+    case 1: scatter_piece<uint8_t>(w, image, lds); break;
+    case 2: scatter_piece<uint16_t>(w, image, lds); break;
+    case 4: scatter_piece<uint32_t>(w, image, lds); break;
+    default: scatter_piece<uint64_t>(w, image, lds); break;
   }
 }
 
@@ -453,25 +507,6 @@ __global__ void __launch_bounds__(256) mlf_strided_kernel(const StridedDesc* __r
                                                           char* __restrict__ image) {
   const StridedWork w = work[blockIdx.x];
   const StridedDesc* __restrict__ d = descs + w.desc;
-  if (PACK && d->gather_k) {
-    switch (d->esz) {
-      case 1: strided_gather_k<uint8_t>(d, w, image); break;
-      case 2: strided_gather_k<uint16_t>(d, w, image); break;
-      case 4: strided_gather_k<uint32_t>(d, w, image); break;
-      default: strided_gather_k<uint64_t>(d, w, image); break;
-    }
-    return;
-  }
-  if (!PACK && d->gather_k) {
-    __shared__ u32x4 lds[256];
-    switch (d->esz) {
-      case 1: strided_scatter<uint8_t>(d, w, image, lds); break;
-      case 2: strided_scatter<uint16_t>(d, w, image, lds); break;
-      case 4: strided_scatter<uint32_t>(d, w, image, lds); break;
-      default: strided_scatter<uint64_t>(d, w, image, lds); break;
-    }
-    return;
-  }
   switch (d->esz) {
     case 1: strided_walk<PACK, uint8_t>(d, w, image); break;
     case 2: strided_walk<PACK, uint16_t>(d, w, image); break;
@@ -484,63 +519,43 @@ __global__ void __launch_bounds__(256) mlf_strided_kernel(const StridedDesc* __r
 // ---------------------------------------------------------------------------------------------------------
 // transpose kernel (LDS-tiled)
 // ---------------------------------------------------------------------------------------------------------
-// One workgroup moves one T x T tile of a 2-D transposition through LDS so that both the read (along the source's
-// contiguous dimension) and the write (along the destination's) are made of whole, consecutive >= 128-byte runs.
-// Global accesses are 16-byte vectors on both sides (hardware-unaligned where the view starts off a boundary; narrower
-// accesses are bound by the number of lane accesses, not by bytes); LDS is addressed per element on the transposed side.  T = 128 / 64 / 64 / 32 / 16 elements for esz = 1 / 2 / 4 / 8 / 16;
-// rows of the LDS tile are padded so that a column walk does not stay in one bank.
+// One workgroup moves one tile of A x B elements of a 2-D transposition through LDS so that both the read (along
+// the source's contiguous dimension) and the write (along the destination's) are made of whole 16-byte vectors in
+// runs of at least 128 consecutive bytes (narrower accesses are bound by the number of lane accesses, not by
+// bytes).  The tile lies in LDS as it is read, rows along the source's contiguous dimension, and the 16-byte columns
+// of row y are permuted by xor with (y / elements-per-vector): vector writes stay aligned and conflict-free, and
+// the column walk that assembles a destination vector from EPV rows meets a different bank group in every lane.
 constexpr uint32_t kTransThreads = 256;
-constexpr uint32_t kTransPatch = 8;  // neighbouring tile-rows per XCD where 64 tile-rows are left (then 4, 2, 1)
-constexpr uint32_t kTransLdsBytes = 128 * (128 + 16);
 
-__host__ __device__ inline uint32_t trans_tile_dim(uint32_t esz) {
-  return esz == 1 ? 128u : esz <= 4 ? 64u : esz == 8 ? 32u : 16u;
+// Tile extents in elements along the side that is read (x) and the side that is written (y): 128 bytes by 256 for
+// elements of up to 8 bytes (the tile then holds 32 / 16 / 8 / 4 KiB for 1 / 2 / 4 / 8-byte elements), 16 x 16
+// elements of 16 bytes.  Measured on 667 transposed blocks of 2-16 MB with pitches off the 128-byte lines (TB/s of
+// 2 x payload, pack / unpack): 128 x 128 bytes 4.20 / 4.41, 128 x 256 4.47 / 4.50, 256 x 256 4.02 / 3.89,
+// 64 x 256 4.30 / 4.32, 128 x 512 3.83 / 4.10: longer runs on the written side pay (partly written lines cost more
+// than partly used fetched ones) until the tile's LDS footprint cuts the number of resident workgroups.
+__host__ __device__ constexpr uint32_t trans_tile_x(uint32_t esz) { return esz == 16 ? 16u : 128u / esz; }
+__host__ __device__ constexpr uint32_t trans_tile_y(uint32_t esz) { return esz == 16 ? 16u : 256u / esz; }
+// tile extents in elements along a (contiguous on the tensor side) and b (contiguous on the image side)
+__host__ __device__ constexpr uint32_t trans_tile_a(uint32_t esz, bool pack) {
+  return pack ? trans_tile_x(esz) : trans_tile_y(esz);
 }
-
-template <bool PACK, typename E, typename V>
-__device__ __forceinline__ void trans_tile(const TransDesc* __restrict__ d, uint64_t tile, char* __restrict__ image,
-                                           char* __restrict__ lds) {
-  constexpr uint32_t ESZ = sizeof(E), VEC = sizeof(V), EPV = VEC / ESZ;
-  const uint32_t T = trans_tile_dim(ESZ);
-  // LDS rows are padded by one dword (two for 8-byte elements): a column walk of one vector per lane then spreads
-  // over the banks (lane stride EPV * pitch = 8, 16, 4, 4 banks modulo 64 for 2-, 1-, 4-, 8-byte elements)
-  const uint32_t pitch = T * ESZ + (ESZ == 16 ? 16u : ESZ == 8 ? 8u : 4u);
+__host__ __device__ constexpr uint32_t trans_tile_b(uint32_t esz, bool pack) {
+  return pack ? trans_tile_y(esz) : trans_tile_x(esz);
+}
+template <bool PACK, typename E, uint32_t A, uint32_t B>
+__device__ __forceinline__ void trans_tile(const TransDesc* __restrict__ d, uint64_t batch, uint32_t ta, uint32_t tb,
+                                           char* __restrict__ image, char* __restrict__ lds) {
+  typedef u32x4 V;
+  constexpr uint32_t ESZ = sizeof(E), EPV = 16 / ESZ;
+  // x: the source's contiguous dimension, y: the destination's
+  constexpr uint32_t TX = PACK ? A : B, TY = PACK ? B : A;
+  constexpr uint32_t VX = TX / EPV, VY = TY / EPV;  // vectors per source row / per destination row
+  constexpr uint32_t pitch = TX * ESZ;
+  static_assert((VX & (VX - 1)) == 0 && (VY & (VY - 1)) == 0, "tile extents are powers of two");
+  static_assert((TY * VX) % kTransThreads == 0 && (TX * VY) % kTransThreads == 0, "whole trips over a tile");
   typedef V vec_u __attribute__((aligned(1)));
-  typedef V vec_lds __attribute__((aligned(ESZ < 4 ? 4 : ESZ)));  // as aligned as an LDS row start is
   typedef E elem_u __attribute__((aligned(1)));
 
-  // which tile: batch index, then tile row (a) and tile column (b); b runs fastest
-  const uint64_t per_batch = (uint64_t)d->tiles_a * d->tiles_b;
-  uint64_t batch = tile / per_batch;
-  const uint32_t rem = (uint32_t)(tile - batch * per_batch);
-  // Visiting order.  Workgroups reach the eight XCDs round-robin, and every XCD has its own L2, so the order decides
-  // which L2 sees which lines.  Tile-rows are taken in bands; within a band the tile-column advances slowly and
-  // eight consecutive workgroups take eight different tile-rows, so that the tiles next to each other along b (they
-  // share destination lines when packing) are always eight workgroups apart: same XCD.  Where 8 * kTransPatch
-  // tile-rows are left, XCD k takes the kTransPatch neighbouring tile-rows [k * kTransPatch, (k + 1) * kTransPatch)
-  // of the band, so that tiles next to each other along a (they share source lines) are on one XCD too; fewer rows
-  // are covered with patches of 4, then 2, then plain bands of eight.  (Full 8192 x 16384 transposes, TB/s: bands of
-  // 8: 2.9-3.9; patches of 8: 3.8-5.2.)
-  uint32_t ta = 0, tb = 0, row0 = 0, left = rem;
-#pragma unroll
-  for (uint32_t patch = kTransPatch; patch >= 1; patch >>= 1) {
-    // rows [row0, row0 + rows) are visited in bands of 8 * patch tile-rows; the last pass (patch == 1) takes all
-    // that is left, its last band possibly short of eight rows
-    const uint32_t band_h = 8u * patch;
-    const uint32_t rows = patch > 1 ? (d->tiles_a - row0) / band_h * band_h : d->tiles_a - row0;
-    const uint32_t tiles = rows * d->tiles_b;
-    if (left < tiles) {
-      const uint32_t band = left / (band_h * d->tiles_b);
-      const uint32_t in_band = left - band * (band_h * d->tiles_b);
-      const uint32_t rows_here = rows - band * band_h < band_h ? rows - band * band_h : band_h;
-      tb = in_band / rows_here;
-      const uint32_t j = in_band - tb * rows_here;
-      ta = row0 + band * band_h + (rows_here == band_h ? (j & 7u) * patch + (j >> 3) : j);
-      break;
-    }
-    left -= tiles;
-    row0 += rows;
-  }
   int64_t toff = 0, ioff = 0;
   for (int k = (int)d->nbatch - 1; k >= 0; --k) {
     const uint64_t extent = (uint64_t)d->bshape[k];
@@ -550,62 +565,93 @@ __device__ __forceinline__ void trans_tile(const TransDesc* __restrict__ d, uint
     toff += i * d->bts[k];
     ioff += i * d->bis[k];
   }
-  const int64_t a0 = (int64_t)ta * T, b0 = (int64_t)tb * T;
-  // x: the source's contiguous dimension, y: the destination's
+  // the tile's first element; negative in the first tile row / column when the grid starts before element 0
+  const int64_t a0 = (int64_t)ta * A - (int64_t)d->a_lead, b0 = (int64_t)tb * B - (int64_t)d->b_lead;
   const int64_t nx = PACK ? d->na : d->nb, ny = PACK ? d->nb : d->na;
   const int64_t x0 = PACK ? a0 : b0, y0 = PACK ? b0 : a0;
   const int64_t ld_src = PACK ? d->ld_t : d->ld_i, ld_dst = PACK ? d->ld_i : d->ld_t;
   const char* src = (PACK ? reinterpret_cast<const char*>(d->tensor) + toff : image + d->image + ioff) + x0 * ESZ + y0 * ld_src;
   char* dst = (PACK ? image + d->image + ioff : reinterpret_cast<char*>(d->tensor) + toff) + x0 * ld_dst + y0 * ESZ;
-  const uint32_t xn = (uint32_t)(nx - x0 < (int64_t)T ? nx - x0 : T);  // valid extent of this tile
-  const uint32_t yn = (uint32_t)(ny - y0 < (int64_t)T ? ny - y0 : T);
-  const uint32_t vec_per_row = T / EPV, n_vec = T * vec_per_row;
+  // the part of the tile that belongs to the item: [xlo, xhi) x [ylo, yhi)
+  const uint32_t xlo = x0 < 0 ? (uint32_t)(-x0) : 0u, ylo = y0 < 0 ? (uint32_t)(-y0) : 0u;
+  const uint32_t xhi = (uint32_t)(nx - x0 < (int64_t)TX ? nx - x0 : TX);
+  const uint32_t yhi = (uint32_t)(ny - y0 < (int64_t)TY ? ny - y0 : TY);
+  const uint32_t tid = threadIdx.x;
 
-  for (uint32_t v = threadIdx.x; v < n_vec; v += kTransThreads) {
-    const uint32_t y = v / vec_per_row, x = (v - y * vec_per_row) * EPV;
-    if (y >= yn || x >= xn) continue;
-    const char* g = src + (int64_t)y * ld_src + (int64_t)x * ESZ;
-    char* l = lds + y * pitch + x * ESZ;
-    if (x + EPV <= xn) {
-      *reinterpret_cast<vec_lds*>(l) = *gload<vec_u>(g);
+  if (xlo == 0u && ylo == 0u && xhi == TX && yhi == TY) {
+    // a whole tile: every load is issued before the first LDS access
+    constexpr uint32_t N1 = TY * VX / kTransThreads, N2 = TX * VY / kTransThreads;
+    V in[N1];
+#pragma unroll
+    for (uint32_t i = 0; i < N1; ++i) {
+      const uint32_t v = tid + i * kTransThreads, y = v / VX, xv = v % VX;
+      in[i] = *gload<vec_u>(src + (int64_t)y * ld_src + xv * 16u);
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < N1; ++i) {
+      const uint32_t v = tid + i * kTransThreads, y = v / VX, xv = v % VX;
+      *reinterpret_cast<V*>(lds + y * pitch + ((xv ^ ((y / EPV) & (VX - 1u))) << 4)) = in[i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t i = 0; i < N2; ++i) {
+      const uint32_t v = tid + i * kTransThreads, x = v / VY, yv = v % VY;
+      const char* l = lds + yv * EPV * pitch + (((x / EPV) ^ (yv & (VX - 1u))) << 4) + (x % EPV) * ESZ;
+      V out;
+      E* parts = reinterpret_cast<E*>(&out);
+#pragma unroll
+      for (uint32_t k = 0; k < EPV; ++k) parts[k] = *reinterpret_cast<const E*>(l + k * pitch);
+      *gstore<vec_u>(dst + (int64_t)x * ld_dst + yv * 16u) = out;
+    }
+    return;
+  }
+  // a tile on the item's edge: the same walk, element by element where a vector is not wholly inside
+  for (uint32_t v = tid; v < TY * VX; v += kTransThreads) {
+    const uint32_t y = v / VX, xv = v % VX, x = xv * EPV;
+    if (y < ylo || y >= yhi || x + EPV <= xlo || x >= xhi) continue;
+    const char* g = src + (int64_t)y * ld_src + xv * 16u;
+    char* l = lds + y * pitch + ((xv ^ ((y / EPV) & (VX - 1u))) << 4);
+    if (x >= xlo && x + EPV <= xhi) {
+      *reinterpret_cast<V*>(l) = *gload<vec_u>(g);
     } else {
-      for (uint32_t k = 0; x + k < xn; ++k) reinterpret_cast<E*>(l)[k] = reinterpret_cast<const elem_u*>(g)[k];
+      for (uint32_t k = 0; k < EPV; ++k)
+        if (x + k >= xlo && x + k < xhi) reinterpret_cast<E*>(l)[k] = *gload<elem_u>(g + k * ESZ);
     }
   }
   __syncthreads();
-  for (uint32_t v = threadIdx.x; v < n_vec; v += kTransThreads) {
-    const uint32_t x = v / vec_per_row, y = (v - x * vec_per_row) * EPV;
-    if (x >= xn || y >= yn) continue;
-    char* g = dst + (int64_t)x * ld_dst + (int64_t)y * ESZ;
-    const char* l = lds + y * pitch + x * ESZ;
-    if (y + EPV <= yn) {
+  for (uint32_t v = tid; v < TX * VY; v += kTransThreads) {
+    const uint32_t x = v / VY, yv = v % VY, y = yv * EPV;
+    if (x < xlo || x >= xhi || y + EPV <= ylo || y >= yhi) continue;
+    char* g = dst + (int64_t)x * ld_dst + yv * 16u;
+    const char* l = lds + y * pitch + (((x / EPV) ^ (yv & (VX - 1u))) << 4) + (x % EPV) * ESZ;
+    if (y >= ylo && y + EPV <= yhi) {
       V out;
       E* parts = reinterpret_cast<E*>(&out);
 #pragma unroll
       for (uint32_t k = 0; k < EPV; ++k) parts[k] = *reinterpret_cast<const E*>(l + k * pitch);
       *gstore<vec_u>(g) = out;
     } else {
-      for (uint32_t k = 0; y + k < yn; ++k) reinterpret_cast<elem_u*>(g)[k] = *reinterpret_cast<const E*>(l + k * pitch);
+      for (uint32_t k = 0; k < EPV; ++k)
+        if (y + k >= ylo && y + k < yhi) *gstore<elem_u>(g + k * ESZ) = *reinterpret_cast<const E*>(l + k * pitch);
     }
   }
 }
 
-template <bool PACK>
+// Which tile a workgroup takes comes from a table the plan builds on the host, one entry per workgroup, because the
+// order matters.  Workgroups reach the eight XCDs round-robin, and every XCD has its own L2: tiles next to each other
+// along a share lines of the tensor side, tiles next to each other along b lines of the image side, wherever a tile
+// row does not start on a line.  The table gives XCD x (entries x, x + 8, x + 16 ...) compact patches of
+// neighbouring tiles, one after the other: lines that two of its tiles share are fetched from HBM once and merged in
+// that L2 before they are written; only the patches' rims meet another L2.
+template <bool PACK, typename E>
 __global__ void __launch_bounds__(kTransThreads) mlf_transpose_kernel(const TransDesc* __restrict__ descs,
-                                                            const TransWork* __restrict__ work,
+                                                            const TransTile* __restrict__ tiles,
                                                             char* __restrict__ image) {
-  __shared__ __attribute__((aligned(16))) char lds[kTransLdsBytes];
-  const TransWork w = work[blockIdx.x / kTransTilesPerEntry];
-  const TransDesc* __restrict__ d = descs + w.desc;
-  const uint64_t tile = w.first_tile + (blockIdx.x % kTransTilesPerEntry);
-  if (tile >= d->n_tiles) return;  // uniform per workgroup: nobody reaches the barrier
-  switch (d->esz) {
-    case 1: trans_tile<PACK, uint8_t, u32x4>(d, tile, image, lds); break;
-    case 2: trans_tile<PACK, uint16_t, u32x4>(d, tile, image, lds); break;
-    case 4: trans_tile<PACK, uint32_t, u32x4>(d, tile, image, lds); break;
-    case 8: trans_tile<PACK, uint64_t, u32x4>(d, tile, image, lds); break;
-    default: trans_tile<PACK, u32x4, u32x4>(d, tile, image, lds); break;  // 16
-  }
+  constexpr uint32_t A = trans_tile_a(sizeof(E), PACK), B = trans_tile_b(sizeof(E), PACK);
+  __shared__ __attribute__((aligned(16))) char lds[A * B * sizeof(E)];
+  const TransTile t = tiles[blockIdx.x];
+  if (t.desc == kNoTile) return;  // uniform: nobody reaches the barrier
+  trans_tile<PACK, E, A, B>(descs + t.desc, t.batch, t.ta, t.tb, image, lds);
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -752,9 +798,13 @@ struct mlf_plan {
   uint64_t n_spans[kSpanClasses] = {0, 0, 0, 0};
   uint32_t tile_bytes = 4096;
   StridedDesc* d_descs = nullptr;
-  StridedWork* d_work = nullptr;
+  StridedWork* d_work = nullptr;   // work of the generic walk
+  GatherWork* d_gwork = nullptr;  // row pieces of the `[..., ::k]` items: vector gather when packing, LDS scatter when unpacking
+  uint64_t n_work = 0, n_gwork = 0;
   TransDesc* d_tdescs = nullptr;
-  TransWork* d_twork = nullptr;
+  // the transpose kernel's tile table when packing [0] and unpacking [1]: one range per element size 1, 2, 4, 8, 16
+  TransTile* d_ttiles[2] = {nullptr, nullptr};
+  uint64_t ttiles_first[2][kTransClasses + 1] = {{0}, {0}};
   char* d_blob = nullptr;
   uint64_t blob_size = 0;
   char* h_blob = nullptr;            // pinned staging of mlf_plan_update_blob, allocated on first use
@@ -778,8 +828,10 @@ struct mlf_plan {
     for (Span* t : d_spans) (void)hipFree(t);
     (void)hipFree(d_descs);
     (void)hipFree(d_work);
+    (void)hipFree(d_gwork);
     (void)hipFree(d_tdescs);
-    (void)hipFree(d_twork);
+    (void)hipFree(d_ttiles[0]);
+    (void)hipFree(d_ttiles[1]);
     (void)hipFree(d_blob);
     if (h_blob) (void)hipHostFree(h_blob);
     if (blob_copied) (void)hipEventDestroy(blob_copied);
@@ -793,7 +845,7 @@ namespace {
 constexpr uint32_t kDefaultTileBytes = 4096;
 constexpr uint32_t kStridedElemsPerBlock = 32 * 1024;
 constexpr uint32_t kGatherMinRow = 256;         // `[..., ::k]` rows at least this long take the vector gather
-constexpr uint32_t kGatherUnitsPerBlock = 1024;  // 16-byte output vectors per work item (four per thread)
+constexpr uint32_t kGatherUnitsPerBlock = 256 * kGatherSplit;  // 16-byte output vectors per work item: one per thread of each of its workgroups
 
 struct SpanTables {
   std::vector<Span> cls[kSpanClasses];
@@ -844,11 +896,19 @@ struct FlatSink {
       const uint64_t e0 = (image_off + kEntryBytes - 1) / kEntryBytes;
       const uint64_t e1 = std::min<uint64_t>((image_off + n) / kEntryBytes, fused_entries);
       if (e1 > e0) {
-        for (uint64_t e = e0; e < e1; ++e) (*ent)[e] = tensor_addr + (e * kEntryBytes - image_off);
-        fused_bytes += (e1 - e0) * kEntryBytes;
-        const uint64_t head = e0 * kEntryBytes - image_off, tail_at = e1 * kEntryBytes - image_off;
-        if (head) cut_spans(*tables, tensor_addr, image_off, head, tile, align_to_tensor, cut_mask);
-        if (tail_at < n) cut_spans(*tables, tensor_addr + tail_at, image_off + tail_at, n - tail_at, tile, align_to_tensor, cut_mask);
+        // An entry has one address: when two runs cover the same image range (an unpack that restores one record
+        // into two targets), the first keeps the entry and the later run's share of it goes to the span tables
+        // like any edge, so both targets are written and every byte of the image is checksummed once.
+        uint64_t at = 0;  // bytes of the run handed out so far
+        for (uint64_t e = e0; e < e1; ++e) {
+          if ((*ent)[e]) continue;
+          const uint64_t from = e * kEntryBytes - image_off;
+          if (from > at) cut_spans(*tables, tensor_addr + at, image_off + at, from - at, tile, align_to_tensor, cut_mask);
+          (*ent)[e] = tensor_addr + from;
+          fused_bytes += kEntryBytes;
+          at = from + kEntryBytes;
+        }
+        if (at < n) cut_spans(*tables, tensor_addr + at, image_off + at, n - at, tile, align_to_tensor, cut_mask);
         return;
       }
     }
@@ -881,6 +941,42 @@ Collapsed collapse_dims(const mlf_item& it) {
   c.ndim = n;
   return c;
 }
+
+// The transpose kernel's tile table.  Every transposed item's tile grid is cut into patches of patch_a x patch_b
+// neighbouring tiles (the grid's rim: what is left); a patch goes, whole, to the XCD whose list is shortest so far,
+// which keeps the eight lists level and neighbouring patches in flight at about the same time.  The table interleaves
+// the lists - entry 8 s + x is the s-th tile of XCD x - and pads the shorter ones with empty entries.
+// Patches are long along the side that is written - partly written lines then meet in one L2, which matters more
+// than partly used fetched lines meeting there.  Same 667 blocks, patches of (tiles along the read side) x (along
+// the written side): 1 x 64 4.17 / 3.93 with 128 x 128-byte tiles, 64 x 1 3.13 / 4.39 (the written side is a for an
+// unpack), 8 x 8 4.10 / 4.41; with 128 x 256-byte tiles 2 x 16 4.34 / 4.49, 4 x 16 4.47 / 4.50, 8 x 8 4.36 / 4.44.
+constexpr uint32_t kTransPatchRead = 4, kTransPatchWritten = 16;
+struct TransOrder {
+  uint32_t patch_a = 1, patch_b = 1;
+  std::vector<TransTile> list[8];
+  uint32_t next = 0;  // where the search for the shortest list starts: ties go round
+  void add(uint32_t desc, uint32_t tiles_a, uint32_t tiles_b, uint32_t batches) {
+    for (uint32_t batch = 0; batch < batches; ++batch)
+      for (uint32_t a0 = 0; a0 < tiles_a; a0 += patch_a)
+        for (uint32_t b0 = 0; b0 < tiles_b; b0 += patch_b) {
+          uint32_t x = next;
+          for (uint32_t k = 1; k < 8; ++k)
+            if (list[(next + k) & 7].size() < list[x].size()) x = (next + k) & 7;
+          next = (x + 1) & 7;
+          const uint32_t a1 = std::min(tiles_a, a0 + patch_a), b1 = std::min(tiles_b, b0 + patch_b);
+          for (uint32_t tb = b0; tb < b1; ++tb)
+            for (uint32_t ta = a0; ta < a1; ++ta) list[x].push_back(TransTile{desc, ta, tb, batch});
+        }
+  }
+  std::vector<TransTile> interleaved() const {
+    size_t longest = 0;
+    for (const auto& l : list) longest = std::max(longest, l.size());
+    std::vector<TransTile> out(longest * 8, TransTile{kNoTile, 0, 0, 0});
+    for (uint32_t x = 0; x < 8; ++x)
+      for (size_t s = 0; s < list[x].size(); ++s) out[s * 8 + x] = list[x][s];
+    return out;
+  }
+};
 
 template <typename T>
 int upload(const std::vector<T>& host, T** dev) {
@@ -978,8 +1074,11 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
   FlatSink flat{&tiles, plan->has_crc ? &ent : nullptr, fused_entries, 0, tile, align_to_tensor, plan->cut_mask};
   std::vector<StridedDesc> descs;
   std::vector<StridedWork> work;
+  std::vector<GatherWork> gwork;
   std::vector<TransDesc> tdescs;
-  std::vector<TransWork> twork;
+  TransOrder torder[2][kTransClasses];
+  for (auto& o : torder[0]) o.patch_a = kTransPatchRead, o.patch_b = kTransPatchWritten;
+  for (auto& o : torder[1]) o.patch_a = kTransPatchWritten, o.patch_b = kTransPatchRead;
   mlf_plan_info& info = plan->info;
   info.n_items = n_items;
   info.image_bytes = image_bytes;
@@ -1075,9 +1174,9 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
         td.nb = c.shape[last];
         td.ld_t = c.ts[last] * (int64_t)esz;
         td.ld_i = c.is[a] * (int64_t)esz;
-        const uint32_t T = trans_tile_dim(esz);
-        td.tiles_a = (uint32_t)((td.na + T - 1) / T);
-        td.tiles_b = (uint32_t)((td.nb + T - 1) / T);
+        // tile cuts on the 128-byte lines of both sides (where the addresses are multiples of the element size)
+        if (it.ptr % esz == 0) td.a_lead = (uint32_t)(it.ptr % 128u) / esz;
+        if (it.image_off % esz == 0) td.b_lead = (uint32_t)(it.image_off % 128u) / esz;
         uint64_t batches = 1;
         for (int d = 0; d < last; ++d) {
           if (d == a) continue;
@@ -1087,13 +1186,48 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
           ++td.nbatch;
           batches *= (uint64_t)c.shape[d];
         }
-        td.n_tiles = batches * td.tiles_a * td.tiles_b;
-        const uint32_t tdesc_idx = (uint32_t)tdescs.size();
+        if (batches >> 32 || td.na >> 35 || td.nb >> 35 || tdescs.size() >= kNoTile) {
+          rc = fail(MLF_HIP_BAD_ARG, "item " + std::to_string(k) + ": too many tiles in a transposed view");
+          break;
+        }
+        for (int dir = 0; dir < 2; ++dir) {
+          const uint32_t A = trans_tile_a(esz, dir == 0), B = trans_tile_b(esz, dir == 0);
+          torder[dir][__builtin_ctz(esz)].add((uint32_t)tdescs.size(), (uint32_t)((td.na + td.a_lead + A - 1) / A),
+                          (uint32_t)((td.nb + td.b_lead + B - 1) / B), (uint32_t)batches);
+        }
         tdescs.push_back(td);
-        for (uint64_t first = 0; first < td.n_tiles; first += kTransTilesPerEntry) twork.push_back(TransWork{first, tdesc_idx, 0});
         ++info.n_transposed_items;
         continue;
       }
+    }
+    const int lastd = c.ndim - 1;
+    // `[..., ::k]` of long rows.  Measured on `[:, ::k]` of 8192 x 16384 parents (TB/s of 2 x payload, element walk ->
+    // vector gather): k = 2: 1.0 -> 3.2 (1-byte), 1.7 -> 3.5 (2), 3.2 -> 3.6 (4), 3.3 -> 3.6 (8); k = 3: 1.0 -> 2.1 (1),
+    // 1.6 -> 2.2 (2), but 2.3 -> 1.7 (4): wider elements keep the element walk unless k = 2
+    if (esz <= 8 && c.is[lastd] == 1 && c.ts[lastd] >= 2 && c.ts[lastd] <= 4 && (esz <= 2 || c.ts[lastd] == 2) &&
+        c.shape[lastd] >= (int64_t)kGatherMinRow && numel / (uint64_t)c.shape[lastd] <= (1u << 24)) {
+      // row by row: a work item never crosses a row, so its elements are evenly spaced on both sides
+      const uint64_t row_len = (uint64_t)c.shape[lastd], rows = numel / row_len;
+      const uint64_t piece = (uint64_t)kGatherUnitsPerBlock * (16 / esz);
+      const uint64_t k = (uint64_t)c.ts[lastd];
+      int64_t idx[MLF_MAX_DIMS] = {0};
+      for (uint64_t r = 0; r < rows; ++r) {
+        int64_t toff = 0, ioff = 0;
+        for (int d = 0; d < lastd; ++d) {
+          toff += idx[d] * c.ts[d];
+          ioff += idx[d] * c.is[d];
+        }
+        const uint64_t trow = it.ptr + (uint64_t)(toff * (int64_t)esz), irow = it.image_off + (uint64_t)(ioff * (int64_t)esz);
+        for (uint64_t j = 0; j < row_len; j += piece)
+          gwork.push_back(GatherWork{trow + j * k * esz, irow + j * esz, (uint32_t)std::min<uint64_t>(piece, row_len - j),
+                                     (uint16_t)k, (uint16_t)esz});
+        for (int d = lastd - 1; d >= 0; --d) {
+          if (++idx[d] < c.shape[d]) break;
+          idx[d] = 0;
+        }
+      }
+      ++info.n_strided_items;
+      continue;
     }
     StridedDesc sd{};
     sd.tensor = it.ptr;
@@ -1112,26 +1246,10 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
         rest /= (uint64_t)c.shape[d];
       }
     }
-    const int lastd = c.ndim - 1;
-    // measured on `[:, ::k]` of 8192 x 16384 parents (TB/s of 2 x payload, element walk -> vector gather): k = 2:
-    // 1.0 -> 3.2 (1-byte), 1.7 -> 3.5 (2), 3.2 -> 3.6 (4), 3.3 -> 3.6 (8); k = 3: 1.0 -> 2.1 (1), 1.6 -> 2.2 (2), but
-    // 2.3 -> 1.7 (4): wider elements keep the element walk unless k = 2
-    if (lastd >= 0 && esz <= 8 && c.is[lastd] == 1 && c.ts[lastd] >= 2 && c.ts[lastd] <= 4 &&
-        (esz <= 2 || c.ts[lastd] == 2) && c.shape[lastd] >= (int64_t)kGatherMinRow)
-      sd.gather_k = (uint32_t)c.ts[lastd];
     const uint32_t desc_idx = (uint32_t)descs.size();
     descs.push_back(sd);
-    if (sd.gather_k) {
-      // row by row: a work item never crosses a row, so its elements are evenly spaced on both sides
-      const uint64_t row_len = (uint64_t)c.shape[lastd], rows = numel / row_len;
-      const uint64_t piece = (uint64_t)kGatherUnitsPerBlock * (16 / esz);
-      for (uint64_t r = 0; r < rows; ++r)
-        for (uint64_t j = 0; j < row_len; j += piece)
-          work.push_back(StridedWork{r * row_len + j, (uint32_t)std::min<uint64_t>(piece, row_len - j), desc_idx});
-    } else {
-      for (uint64_t s0 = 0; s0 < numel; s0 += kStridedElemsPerBlock)
-        work.push_back(StridedWork{s0, (uint32_t)std::min<uint64_t>(kStridedElemsPerBlock, numel - s0), desc_idx});
-    }
+    for (uint64_t s0 = 0; s0 < numel; s0 += kStridedElemsPerBlock)
+      work.push_back(StridedWork{s0, (uint32_t)std::min<uint64_t>(kStridedElemsPerBlock, numel - s0), desc_idx});
     ++info.n_strided_items;
   }
   for (int c = 0; c < kSpanClasses && rc == MLF_HIP_OK; ++c) {
@@ -1140,8 +1258,19 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
   }
   if (rc == MLF_HIP_OK) rc = upload(descs, &plan->d_descs);
   if (rc == MLF_HIP_OK) rc = upload(work, &plan->d_work);
+  if (rc == MLF_HIP_OK) rc = upload(gwork, &plan->d_gwork);
+  plan->n_work = work.size();
+  plan->n_gwork = gwork.size();
   if (rc == MLF_HIP_OK) rc = upload(tdescs, &plan->d_tdescs);
-  if (rc == MLF_HIP_OK) rc = upload(twork, &plan->d_twork);
+  for (int dir = 0; dir < 2; ++dir) {
+    std::vector<TransTile> ttiles;
+    for (int cls = 0; cls < kTransClasses; ++cls) {
+      const std::vector<TransTile> part = torder[dir][cls].interleaved();
+      ttiles.insert(ttiles.end(), part.begin(), part.end());
+      plan->ttiles_first[dir][cls + 1] = ttiles.size();
+    }
+    if (rc == MLF_HIP_OK) rc = upload(ttiles, &plan->d_ttiles[dir]);
+  }
   if (rc == MLF_HIP_OK && plan->has_crc) {
     // entries the fused kernel does not serve are checksummed from the finished image
     std::vector<uint32_t> slow;
@@ -1161,9 +1290,9 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
     return rc;
   }
   info.n_flat_tiles = 0;
-  info.table_bytes = descs.size() * sizeof(StridedDesc) + work.size() * sizeof(StridedWork) +
-                     tdescs.size() * sizeof(TransDesc) + twork.size() * sizeof(TransWork) + blob_bytes;
-  info.n_transposed_work = twork.size();
+  info.table_bytes = descs.size() * sizeof(StridedDesc) + work.size() * sizeof(StridedWork) + gwork.size() * sizeof(GatherWork) +
+                     tdescs.size() * sizeof(TransDesc) + (plan->ttiles_first[0][kTransClasses] + plan->ttiles_first[1][kTransClasses]) * sizeof(TransTile) + blob_bytes;
+  info.n_transposed_work = std::max(plan->ttiles_first[0][kTransClasses], plan->ttiles_first[1][kTransClasses]);
   for (int c = 0; c < kSpanClasses; ++c) {
     if (c != kSmallClass) info.n_flat_tiles += plan->n_spans[c] << kSpanShift[c];
     info.table_bytes += plan->n_spans[c] * sizeof(Span);
@@ -1181,7 +1310,7 @@ int mlf_plan_create(const mlf_item* items, uint64_t n_items, const void* host_bl
     }
     plan->flat_total = (uint32_t)wgs;
   }
-  info.n_strided_work = work.size();
+  info.n_strided_work = work.size() + gwork.size();
   *out = plan.release();
   return MLF_HIP_OK;
 }
@@ -1261,17 +1390,34 @@ int launch_plan(const mlf_plan* plan, char* image, hipStream_t stream) {
                        plan->d_spans[kSmallClass] + first, count, image);
     HIP_TRY(hipGetLastError());
   }
-  const uint64_t trans_per_launch = std::max<uint64_t>(1, 0xFFFFFFFFull / ((uint64_t)kTransTilesPerEntry * kTransThreads));
-  for (uint64_t first = 0; first < plan->info.n_transposed_work; first += trans_per_launch) {
-    const uint64_t count = std::min<uint64_t>(trans_per_launch, plan->info.n_transposed_work - first);
-    hipLaunchKernelGGL((mlf_transpose_kernel<PACK>), dim3((uint32_t)(count * kTransTilesPerEntry)), dim3(kTransThreads), 0, stream,
-                       plan->d_tdescs, plan->d_twork + first, image);
-    HIP_TRY(hipGetLastError());
+  for (int cls = 0; cls < kTransClasses; ++cls) {
+    const uint64_t* range = plan->ttiles_first[PACK ? 0 : 1] + cls;
+    for (uint64_t first = range[0]; first < range[1]; first += (1u << 23)) {  // whole sets of eight
+      const dim3 grid((uint32_t)std::min<uint64_t>(1u << 23, range[1] - first)), block(kTransThreads);
+      const TransTile* tiles = plan->d_ttiles[PACK ? 0 : 1] + first;
+      switch (cls) {
+        case 0: hipLaunchKernelGGL((mlf_transpose_kernel<PACK, uint8_t>), grid, block, 0, stream, plan->d_tdescs, tiles, image); break;
+        case 1: hipLaunchKernelGGL((mlf_transpose_kernel<PACK, uint16_t>), grid, block, 0, stream, plan->d_tdescs, tiles, image); break;
+        case 2: hipLaunchKernelGGL((mlf_transpose_kernel<PACK, uint32_t>), grid, block, 0, stream, plan->d_tdescs, tiles, image); break;
+        case 3: hipLaunchKernelGGL((mlf_transpose_kernel<PACK, uint64_t>), grid, block, 0, stream, plan->d_tdescs, tiles, image); break;
+        default: hipLaunchKernelGGL((mlf_transpose_kernel<PACK, u32x4>), grid, block, 0, stream, plan->d_tdescs, tiles, image); break;
+      }
+      HIP_TRY(hipGetLastError());
+    }
   }
-  for (uint64_t first = 0; first < plan->info.n_strided_work; first += (1u << 23)) {
-    const uint64_t count = std::min<uint64_t>(1u << 23, plan->info.n_strided_work - first);
+  for (uint64_t first = 0; first < plan->n_work; first += (1u << 23)) {
+    const uint64_t count = std::min<uint64_t>(1u << 23, plan->n_work - first);
     hipLaunchKernelGGL((mlf_strided_kernel<PACK>), dim3((uint32_t)count), dim3(256), 0, stream, plan->d_descs,
                        plan->d_work + first, image);
+    HIP_TRY(hipGetLastError());
+  }
+  for (uint64_t first = 0; first < plan->n_gwork; first += (1u << 21)) {
+    const uint64_t count = std::min<uint64_t>(1u << 21, plan->n_gwork - first);
+    if (PACK)
+      hipLaunchKernelGGL(mlf_gather_kernel, dim3((uint32_t)(count * kGatherSplit)), dim3(256), 0, stream,
+                         plan->d_gwork + first, (uint32_t)(count * kGatherSplit), image);
+    else
+      hipLaunchKernelGGL(mlf_scatter_kernel, dim3((uint32_t)count), dim3(256), 0, stream, plan->d_gwork + first, image);
     HIP_TRY(hipGetLastError());
   }
   if (plan->blob_size) {

@@ -201,6 +201,41 @@ def test_unpack_with_checksums_restores_and_reports_the_images_values(chunk, ora
     assert (bad != want).nonzero()[0].tolist() == [at // chunk]
 
 
+@pytest.mark.parametrize("align_to_tensor", [True, False])
+def test_unpack_with_checksums_one_record_into_two_targets(align_to_tensor, oracle_c):
+    """Two items of an unpack plan may read the same range of the image (one stored tensor restored into two targets,
+    wholly or in part).  With checksums on, every target is written and the chunk values are those of the image."""
+    from ml_flashpoint.hip import plan as P
+
+    sizes = [(1 << 20) + 77, (3 << 20) + 5, 600_001]
+    source = _misaligned_tensors(sizes, seed=23)
+    layout = P.build_save_layout(source)
+    image = torch.zeros(layout.image_bytes, dtype=torch.uint8, device=DEV)
+    P.Plan(layout.items, layout.blob, layout.image_bytes).pack(image)
+    torch.cuda.synchronize()
+    chunk = 1 << 20
+    want = _oracle_chunks(oracle_c, image.cpu().numpy().tobytes(), chunk)
+    payload_at = [offset + length - n for (offset, length), n in zip(layout.spans, sizes)]
+    # (record, first byte of the record's payload, length): the whole of record 1 twice, then a part of it that
+    # starts inside a 64 KiB piece another target already owns, then records 0 and 2 once each
+    wanted = [(1, 0, sizes[1]), (1, 0, sizes[1]), (1, 70_001, 2 << 20), (0, 0, sizes[0]), (2, 0, sizes[2])]
+    parents = [torch.full((n + 96,), 0x5A, dtype=torch.uint8, device=DEV) for _, _, n in wanted]
+    targets = [p[32 + (3 * k) % 16 :][:n] for k, (p, (_, _, n)) in enumerate(zip(parents, wanted))]
+    table = P.ItemTable()
+    for t, (rec, first, n) in zip(targets, wanted):
+        table.add_contiguous(t.data_ptr(), payload_at[rec] + first, 1, n)
+    plan = P.Plan(table.to_array(), b"", layout.image_bytes, align_to_tensor=align_to_tensor, crc_chunk_bytes=chunk)
+    assert plan.info.fused_crc_bytes <= layout.image_bytes  # no piece of the image is counted twice
+    plan.unpack(image)
+    got = plan.crc_values()
+    torch.cuda.synchronize()
+    assert got.tolist() == want.tolist()
+    for k, (p, t, (rec, first, n)) in enumerate(zip(parents, targets, wanted)):
+        assert torch.equal(t, source[rec][first : first + n]), k
+        lo = 32 + (3 * k) % 16
+        assert bool((p[:lo] == 0x5A).all()) and bool((p[lo + n :] == 0x5A).all()), f"guard bytes of {k}"
+
+
 def test_checksum_option_argument_checks():
     from ml_flashpoint.hip import _lib
     from ml_flashpoint.hip import plan as P
