@@ -46,7 +46,7 @@ class CheckpointObjectManager:
                     wanted = self._pool_config
                     owner._worker_pool = BufferPool(pool_dir_path=wanted.pool_dir_path, rank=wanted.rank,
                                                     num_buffers=wanted.num_buffers, buffer_size=wanted.buffer_size)
-                    if getattr(wanted, "prefault", True):
+                    if getattr(wanted, "prefault", False):
                         owner._worker_pool.start_prefault()
                 except Exception:
                     _LOGGER.exception("Failed to initialize BufferPool")

@@ -9,8 +9,10 @@ back: the pool notices on its next ``acquire``.
 Behaviour, names and messages are the reference's (src/ml_flashpoint/core/buffer_pool.py:35-342); ``ensure_capacity``
 is an addition for writers that know the total size up front, and so is ``prefault``: the reference creates its pool
 files sparse (buffer_pool.py:324-342) and the first checkpoint into each pays for its pages - 10 s for a 112 GB
-object against 2 s from then on.  With ``prefault`` a background thread allocates and maps the pages of every pool
-file right after the pool is created; a buffer is not lent out before its own file is done.
+object against 2 s from then on.  With ``prefault`` (off unless asked for: it commits ``num_buffers x buffer_size``
+of host memory, where sparse files only ever hold what was written) a background thread allocates and maps the
+pages of every pool file right after the pool is created; a buffer is not lent out before its own file is done.
+The step is skipped, with a warning, when the file system or the host does not have that much memory to spare.
 """
 
 from __future__ import annotations
@@ -103,7 +105,9 @@ class BufferPoolConfig:
     rank: int
     num_buffers: int
     buffer_size: int
-    prefault: bool = True  # allocate and map the pool files' pages in the background, right after creating them
+    # allocate and map the pool files' pages in the background, right after creating them: num_buffers x buffer_size
+    # of host memory from then on, so it is for the caller to ask for
+    prefault: bool = False
 
     def __post_init__(self):
         if not self.pool_dir_path:
@@ -121,6 +125,22 @@ class _Loan(NamedTuple):
 
 # pool files smaller than this are not worth a background thread: their pages cost microseconds
 _PREFAULT_MIN_BYTES = 64 << 20
+
+
+def _spare_bytes(directory: str) -> int:
+    """What a prefault may commit: the smaller of the file system's free space and the host's available memory (a
+    tmpfs reports its size limit, not what the host can still back), less a tenth of either for everybody else."""
+    stat = os.statvfs(directory)
+    spare = stat.f_bavail * stat.f_frsize
+    try:
+        with open("/proc/meminfo") as f:
+            for line in f:
+                if line.startswith("MemAvailable:"):
+                    spare = min(spare, int(line.split()[1]) * 1024)
+                    break
+    except OSError:
+        pass
+    return spare - spare // 10
 
 
 class BufferPool:
@@ -161,6 +181,12 @@ class BufferPool:
         if self.buffer_size < _PREFAULT_MIN_BYTES or self._prefault_worker is not None:
             return
         order = list(reversed(self.free_buffers))  # acquire() pops from the end
+        wanted = sum(stream.buffer_obj.get_capacity() for stream in order)
+        spare = _spare_bytes(self.pool_dir)
+        if wanted > spare:
+            _LOGGER.warning("BufferPool: not prefaulting %d bytes of pool files in '%s': only %d bytes to spare; "
+                            "their pages are left to the saves that fill them.", wanted, self.pool_dir, spare)
+            return
         for stream in order:
             self._prefaulted[stream.buffer_obj.get_id()] = threading.Event()
 
@@ -201,13 +227,18 @@ class BufferPool:
             if not self.free_buffers:
                 raise RuntimeError(f"BufferPool exhausted. All {self.num_buffers} buffers are in use.")
             stream = self.free_buffers.pop()
-            ready = self._prefaulted.get(stream.buffer_obj.get_id())
-            if ready is not None:
-                ready.wait()  # the background thread is still mapping this file's pages: it may not be resized yet
+            pool_file = stream.buffer_obj.get_id()
+            self.active_buffers[pool_file] = _Loan(stream, None)  # taken; without a name it is never reclaimed
+        ready = self._prefaulted.get(pool_file)
+        if ready is not None:
+            # the background thread is still mapping this file's pages: it may not be resized yet.  Waited for
+            # outside the lock, so that other acquires and the reclaiming of deleted objects go on meanwhile.
+            ready.wait()
+        with self._lock:
             try:
                 self._reuse_buffer(stream, associated_symlink)
             except Exception:
-                self.active_buffers.pop(stream.buffer_obj.get_id(), None)
+                self.active_buffers.pop(pool_file, None)
                 self.free_buffers.append(stream)
                 raise
             return PooledBufferIO(stream)

@@ -398,10 +398,71 @@ def test_pool_prefaults_its_files_in_the_background(shm_dir):
     lazy.teardown()
     # through the manager: the pool can be created, and waited for, before the first save
     CheckpointObjectManager._worker_pool = None
-    manager = CheckpointObjectManager(BufferPoolConfig(os.path.join(shm_dir, "managed"), 0, 1, size))
+    manager = CheckpointObjectManager(BufferPoolConfig(os.path.join(shm_dir, "managed"), 0, 1, size, prefault=True))
     assert manager.warm_up_pool(wait=True) > 0.0
     with manager.acquire_buffer(CheckpointObjectId(os.path.join(shm_dir, "ckpt", "a.distcp")), 1 << 20) as writer:
         writer.write(b"abc")
     assert open(os.path.join(shm_dir, "ckpt", "a.distcp"), "rb").read()[METADATA_SIZE:] == b"abc"
     manager.teardown_pool()
     assert CheckpointObjectManager(None).warm_up_pool() == 0.0
+    # the default is the reference's: sparse pool files, nothing committed before a save writes it
+    assert BufferPoolConfig(os.path.join(shm_dir, "sparse"), 0, 1, size).prefault is False
+    manager = CheckpointObjectManager(BufferPoolConfig(os.path.join(shm_dir, "sparse"), 0, 1, size))
+    assert manager.warm_up_pool(wait=True) == 0.0
+    pool_file = os.path.join(shm_dir, "sparse", "buffer_0_0.dist")
+    assert os.path.getsize(pool_file) == size and os.stat(pool_file).st_blocks * 512 < size
+    manager.teardown_pool()
+
+
+def test_pool_prefault_is_skipped_when_memory_is_short(shm_dir, monkeypatch):
+    """Prefaulting commits the whole pool; with less than that to spare (file system or host) it does not start."""
+    import logging
+    import os
+
+    from ml_flashpoint.core import buffer_pool
+
+    monkeypatch.setattr(buffer_pool, "_spare_bytes", lambda directory: 100 << 20)
+    size = 96 << 20
+    seen = []
+    handler = logging.Handler()
+    handler.emit = lambda record: seen.append(record.getMessage())
+    buffer_pool._LOGGER.addHandler(handler)
+    try:
+        pool = buffer_pool.BufferPool(os.path.join(shm_dir, "tight"), num_buffers=2, buffer_size=size, prefault=True)
+    finally:
+        buffer_pool._LOGGER.removeHandler(handler)
+    assert pool._prefault_worker is None and any("not prefaulting" in m for m in seen)
+    path = pool.free_buffers[0].buffer_obj.get_id()
+    assert os.stat(path).st_blocks * 512 < size
+    with pool.acquire(os.path.join(shm_dir, "o.distcp")) as stream:  # still usable, pages on demand
+        stream.write(b"x" * 1000)
+    pool.teardown()
+    monkeypatch.undo()
+    spare = buffer_pool._spare_bytes(shm_dir)
+    stat = os.statvfs(shm_dir)
+    assert 0 < spare <= stat.f_bavail * stat.f_frsize
+
+
+def test_pool_waits_for_a_prefault_outside_its_lock(shm_dir):
+    """While one acquire waits for its file's pages, the pool's lock is free: another acquire gets the other buffer."""
+    import os
+    import threading
+
+    from ml_flashpoint.core.buffer_pool import BufferPool
+
+    pool = BufferPool(os.path.join(shm_dir, "pool"), num_buffers=2, buffer_size=1 << 20)
+    slow = pool.free_buffers[-1].buffer_obj.get_id()  # the buffer the next acquire takes
+    pool._prefaulted[slow] = threading.Event()        # as if its pages were still being mapped
+    got = {}
+    first = threading.Thread(target=lambda: got.setdefault("first", pool.acquire(os.path.join(shm_dir, "a.distcp"))))
+    first.start()
+    while slow not in pool.active_buffers:  # taken, and now waiting
+        pass
+    second = pool.acquire(os.path.join(shm_dir, "b.distcp"))  # would deadlock if the wait held the lock
+    assert second.buffer_obj.get_id() != slow and "first" not in got
+    with __import__("pytest").raises(RuntimeError, match="exhausted"):
+        pool.acquire(os.path.join(shm_dir, "c.distcp"))
+    pool._prefaulted[slow].set()
+    first.join(5)
+    assert got["first"].buffer_obj.get_id() == slow and os.path.islink(os.path.join(shm_dir, "a.distcp"))
+    pool.teardown()
