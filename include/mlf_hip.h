@@ -152,7 +152,10 @@ int mlf_crc32c_device(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes
  * Limit: at most 262 144 segment values per call (segments are 64 KiB to 512 KiB by the size of the buffer and are
  * doubled, while they still divide `chunk_bytes`, until their count fits); more than that, e.g. 16 GiB in 64 KiB
  * chunks, is refused with a message.  All calls on one device share that device's array and every call
- * overwrites it: calls that overlap in time on one device race; calls ordered on one stream do not. */
+ * overwrites it: calls that overlap in time on one device race; calls ordered on one stream do not (replays of a
+ * captured graph that holds the call count as calls: the array's address is part of the graph).  Where the array
+ * lies on a device is looked up once, by mlf_hip_set_device(device) or else by the first call on that device; that
+ * lookup is not for a stream under capture, so call mlf_hip_set_device first (or make one call) before capturing. */
 int mlf_crc32c_device_noalloc(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint32_t* out_dev,
                               uint64_t n_out, void* stream);
 /* Same function on host memory (SSE4.2), and the combine law crc(A||B) from crc(A), crc(B), len(B). */
@@ -244,7 +247,8 @@ int mlf_engine_avoid_streams(mlf_engine* engine, void* const* busy_streams, uint
 
 /* The stream the engine runs its checksum kernels on (a raw hipStream_t), for checksum calls a caller makes between
  * the engine's transfers (mlf_crc32c_device on pieces of an image): a stream that mlf_engine_avoid_streams has
- * already moved out of the training stream's way. */
+ * already moved out of the training stream's way.  A later mlf_engine_avoid_streams may give the engine another
+ * one; a handle returned earlier stays a valid stream until mlf_engine_destroy. */
 void* mlf_engine_checksum_stream(mlf_engine* engine);
 
 /* Host -> host on the engine's threads: `nbytes` from `src_host` to `dst_host` (ranges must not overlap).  For

@@ -209,6 +209,21 @@ constexpr int kNoAllocMaxDevices = 64;
 std::mutex g_scratch_mu;
 void* g_scratch_ptr[kNoAllocMaxDevices];  // device address of `scratch` on each device, looked up on first use there
 
+// The device address of `scratch` on `device`, which must be the current device.  Looked up once per device (the
+// lookup may load the code object there: not something to do while a stream is being captured) and kept.
+int noalloc_scratch_of(int device, void** out) {
+  if (device < 0 || device >= kNoAllocMaxDevices) return fail(MLF_HIP_BAD_ARG, "device index beyond the per-device table");
+  std::lock_guard<std::mutex> g(g_scratch_mu);
+  if (!g_scratch_ptr[device]) {
+    void* p = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return fail(MLF_HIP_RUNTIME, "hipGetSymbolAddress returned a null address for the scratch array");
+    g_scratch_ptr[device] = p;
+  }
+  *out = g_scratch_ptr[device];
+  return MLF_HIP_OK;
+}
+
 struct CrcFoldConsts {
   uint32_t xrow, x4, x16, x32, x64, x128, x256, x512;
 };
@@ -254,6 +269,12 @@ void crc_init_host() {
 }  // namespace
 
 namespace mlf {
+
+int crc_noalloc_prime(int device) {
+  void* unused = nullptr;
+  return noalloc_scratch_of(device, &unused);
+}
+
 
 
 void crc_fused_destroy(FusedCrc* f) {
@@ -521,19 +542,8 @@ int mlf_crc32c_device_noalloc(const void* dev_ptr, uint64_t nbytes, uint64_t chu
                     std::to_string(kNoAllocMaxSegs) + " (use larger chunks, several calls, or mlf_crc32c_device)");
   int device = 0;
   HIP_TRY(hipGetDevice(&device));
-  if (device < 0 || device >= kNoAllocMaxDevices) return fail(MLF_HIP_BAD_ARG, "device index beyond the per-device table");
   void* base = nullptr;
-  {
-    // once per device, with that device current: every device holds its own copy of the array at its own address
-    std::lock_guard<std::mutex> g(g_scratch_mu);
-    if (!g_scratch_ptr[device]) {
-      void* p = nullptr;
-      HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
-      if (!p) return fail(MLF_HIP_RUNTIME, "hipGetSymbolAddress returned a null address for the scratch array");
-      g_scratch_ptr[device] = p;
-    }
-    base = g_scratch_ptr[device];
-  }
+  if (int rc = noalloc_scratch_of(device, &base)) return rc;  // looked up on the first call on a device, kept since
   CrcConsts* consts = static_cast<CrcConsts*>(base);
   uint32_t* seg = reinterpret_cast<uint32_t*>(static_cast<char*>(base) + kNoAllocConstsBytes);
   hipStream_t stream = static_cast<hipStream_t>(stream_);

@@ -144,6 +144,9 @@ struct mlf_engine {
   std::vector<hipEvent_t> slot_done;
   hipStream_t streams[2] = {nullptr, nullptr};
   hipStream_t crc_stream = nullptr;  // checksum kernels run beside the copies, not before them
+  // streams that mlf_engine_avoid_streams replaced: handles to them may still be in a caller's hands (the checksum
+  // stream is handed out), so they live as long as the engine does
+  std::vector<hipStream_t> retired;
   hipEvent_t gate = nullptr;
   CrcScratch crc;  // of the checksum passes that run beside transfers; allocated on first use, grown when too small
   std::unique_ptr<WorkerPool> pool;
@@ -167,16 +170,21 @@ __global__ void mlf_queue_test_touch(uint32_t* out) {
 }
 
 // Whether work on `s` waits for work enqueued earlier on `busy`: both idle, a 2 ms kernel on `busy`, an empty kernel
-// on `s`; on a hardware queue of its own the empty kernel is done in microseconds, behind the 2 ms kernel it is not.
+// on `s`.  On a hardware queue of its own the empty kernel is done while the 2 ms kernel is still running; behind that
+// kernel it is done after it, and `busy` is idle by then.  Decided by that order, not by a clock: a host thread that
+// loses the processor between the two calls can only make an independent stream look dependent, which costs a
+// replacement stream and nothing else.
 int waits_behind(hipStream_t s, hipStream_t busy, uint32_t* d_flags, bool* shared) {
   HIP_TRY(hipStreamSynchronize(busy));
   HIP_TRY(hipStreamSynchronize(s));
   hipLaunchKernelGGL(mlf_queue_test_hold, dim3(1), dim3(64), 0, busy, 200000ull, d_flags);
   hipLaunchKernelGGL(mlf_queue_test_touch, dim3(1), dim3(64), 0, s, d_flags + 16);
   HIP_TRY(hipGetLastError());
-  const double t0 = now_s();
   HIP_TRY(hipStreamSynchronize(s));
-  *shared = now_s() - t0 > 1e-3;
+  const hipError_t other = hipStreamQuery(busy);
+  if (other != hipSuccess && other != hipErrorNotReady) HIP_TRY(other);
+  (void)hipGetLastError();  // "not ready" is an answer, not a failure to report later
+  *shared = other == hipSuccess;
   HIP_TRY(hipStreamSynchronize(busy));
   return MLF_HIP_OK;
 }
@@ -195,6 +203,10 @@ int mlf_engine_destroy(mlf_engine* e) {
   if (e->crc_stream) {
     (void)hipStreamSynchronize(e->crc_stream);
     (void)hipStreamDestroy(e->crc_stream);
+  }
+  for (hipStream_t s : e->retired) {
+    (void)hipStreamSynchronize(s);
+    (void)hipStreamDestroy(s);
   }
   crc_scratch_free(&e->crc);
   delete e;
@@ -467,7 +479,8 @@ int mlf_engine_avoid_streams(mlf_engine* e, void* const* busy_streams, uint32_t 
   };
   uint32_t* d_flags = nullptr;
   HIP_TRY(hipMalloc(reinterpret_cast<void**>(&d_flags), 128));
-  std::vector<hipStream_t> rejected;  // kept until the end: a destroyed stream's queue would be handed out again
+  std::vector<hipStream_t> rejected;  // candidates that were no better; kept until the end: a destroyed stream's
+                                      // queue would be handed out again
   uint32_t left = 0;
   int rc = MLF_HIP_OK;
   hipStream_t* mine[3] = {&e->streams[0], &e->streams[1], &e->crc_stream};
@@ -488,7 +501,7 @@ int mlf_engine_avoid_streams(mlf_engine* e, void* const* busy_streams, uint32_t 
       if (also) {
         rejected.push_back(candidate);
       } else {
-        rejected.push_back(*slot);
+        e->retired.push_back(*slot);  // not destroyed: somebody may still hold its handle, or have work on it
         *slot = candidate;
         shared = false;
       }

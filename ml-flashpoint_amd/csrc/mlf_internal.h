@@ -139,6 +139,9 @@ int crc_enqueue(const void* dev_ptr, uint64_t nbytes, uint64_t chunk_bytes, uint
 int crc_finish(CrcScratch* scratch, hipStream_t stream, uint64_t n_chunks, uint32_t* out_host);
 // Frees the scratch (its stream must be idle).
 void crc_scratch_free(CrcScratch* scratch);
+// Looks up, once, where the fixed scratch array of mlf_crc32c_device_noalloc lies on `device` (the current device), so
+// that the entry point's first call there has nothing left to resolve - it may be made while a stream is captured.
+int crc_noalloc_prime(int device);
 
 }  // namespace mlf
 

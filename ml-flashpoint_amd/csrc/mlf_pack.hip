@@ -1001,7 +1001,9 @@ int mlf_hip_device_count(int* out) {
 
 int mlf_hip_set_device(int device) {
   HIP_TRY(hipSetDevice(device));
-  return MLF_HIP_OK;
+  // set-up of the library on this device: the address of mlf_crc32c_device_noalloc's scratch array is resolved here,
+  // so that the entry point itself may be called while a stream is being captured
+  return crc_noalloc_prime(device);
 }
 
 int mlf_hip_mem_info(uint64_t* free_bytes, uint64_t* total_bytes) {

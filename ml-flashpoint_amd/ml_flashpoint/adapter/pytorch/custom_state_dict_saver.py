@@ -66,11 +66,24 @@ def generate_plan(
             central_plan, global_metadata = _agree_on_plan(local_plan, storage_writer, planner, world_dist_wrapper)
         buckets = storage_writer.prepare_write_data_buckets(checkpoint_id, planner.finish_plan(central_plan), planner)
         expect = getattr(storage_writer, "expect_metadata", None)
-        if expect is not None:
-            # one process on its own: the metadata object that finish_write will be given is known now, and the
-            # writer may pickle it while the data is on its way (with several ranks it depends on everyone's results)
-            expect(global_metadata if not world_dist_wrapper.use_dist else None)
+        if expect is not None and torchdist.get_node_local_rank(fallback_rank=0) == 0:
+            # This process is going to write the metadata object in finish_write, and which object that is, is known
+            # now (a validated cache: the one the last planning save produced, which the caller was handed then and
+            # hands back to finish_write): the writer may pickle it while the data is on its way.  With several
+            # ranks the others' write results are predicted to be those of the previous save.
+            saver = getattr(storage_writer, "checkpoint_saver", None)
+            if global_metadata is not None:
+                _remember(saver, "last_global_metadata", global_metadata)
+            expect(global_metadata if global_metadata is not None else getattr(saver, "last_global_metadata", None),
+                   others_as_before=bool(world_dist_wrapper.use_dist))
         return buckets, global_metadata, central_plan, local_plan, cache.central_plan == central_plan
+
+
+def _remember(holder, name: str, value) -> None:
+    try:
+        setattr(holder, name, value)
+    except AttributeError:
+        pass
 
 
 def _agree_on_plan(local_plan, storage_writer, planner, dist: _DistWrapper):

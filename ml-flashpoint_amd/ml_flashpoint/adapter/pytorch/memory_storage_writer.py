@@ -104,10 +104,12 @@ class _WriteLedger:
 class _EarlyMetadata:
     """The checkpoint's metadata object pickled while its data is still on the way to the buffer.
 
-    Where every item ends up is decided when the object is laid out, long before the last byte is written, so when
-    one process plans, writes and finishes a save (no other rank's results to wait for) the metadata object - whose
-    pickling takes 150 ms for 20 000 tensors - need not wait for the write.  ``finish_checkpoint`` uses the bytes
-    only if they describe exactly what the write then reported; otherwise it pickles again, as without this."""
+    Where every item ends up is decided when the object is laid out, long before the last byte is written, so the
+    metadata object - whose pickling takes 150 ms for 20 000 tensors - need not wait for the write.  This rank's
+    part of it is predicted from the layout; with several ranks the others' parts are taken to be what they were in
+    the previous save (the same plan puts the same items at the same offsets of objects of the same names), which
+    the rank that writes the metadata object saw when it finished that save.  ``finish_checkpoint`` uses the bytes
+    only if they describe exactly what all ranks then reported; otherwise it pickles again, as without this."""
 
     def __init__(self, checkpoint_id, metadata: Metadata, where: dict, storage_meta):
         self.checkpoint_id, self.metadata, self.where, self.storage_meta = checkpoint_id, metadata, where, storage_meta
@@ -150,7 +152,9 @@ class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
         self._current_checkpoint_id: CheckpointContainerId | None = None
         self._current_save_id: str | None = None
         self._expected_metadata: Metadata | None = None  # see expect_metadata
+        self._others_as_before = False
         self._early_metadata: _EarlyMetadata | None = None
+        self.early_metadata_used = False  # the last finish_checkpoint wrote bytes that were pickled ahead of time
 
     # the ledger's two dicts under the names other code (and the reference's tests) know them by
     @property
@@ -170,19 +174,26 @@ class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
         self._ledger.results = value
 
     def __getstate__(self):
-        left_behind = ("_main_process_torchmp_manager_future", "_expected_metadata", "_early_metadata")
+        left_behind = ("_main_process_torchmp_manager_future", "_expected_metadata", "_early_metadata")  # (re-set below)
         return {k: v for k, v in self.__dict__.items() if k not in left_behind}
 
     def __setstate__(self, state):
         self.__dict__.update(state, _main_process_torchmp_manager_future=None, _expected_metadata=None,
                              _early_metadata=None)
+        self._others_as_before = False
 
-    def expect_metadata(self, metadata: Metadata | None) -> None:
-        """Tells the writer which metadata object ``finish_checkpoint`` is going to be called with, for a save that
-        this one process plans, writes and finishes alone: the writer may then pickle it while the data is still
-        being written (see ``_EarlyMetadata``).  Optional; without it, or in a process that received the writer by
-        pickling, nothing changes."""
+    def expect_metadata(self, metadata: Metadata | None, others_as_before: bool | None = None) -> None:
+        """Tells the writer which metadata object ``finish_checkpoint`` is going to be called with, in the process
+        that is going to call it: the writer may then pickle it while the data is still being written (see
+        ``_EarlyMetadata``).  ``others_as_before``: other ranks contribute write results too, and they are predicted
+        to be what the previous ``finish_checkpoint`` of this writer's saver saw (default: whether the process group
+        has more than one rank); no prediction, and no early pickling, on the first save.  Optional; without it, or
+        in a process that received the writer by pickling, nothing changes."""
         self._expected_metadata = metadata
+        if others_as_before is None:
+            dist = torch.distributed
+            others_as_before = dist.is_available() and dist.is_initialized() and dist.get_world_size() > 1
+        self._others_as_before = bool(others_as_before)
 
     # ---- identity of the save in progress ------------------------------------------------------------------------
     def _require_reset(self) -> CheckpointContainerId:
@@ -337,6 +348,11 @@ class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
             return
         if predicted is not None:
             where = {result.index: result.storage_data for result in predicted}
+            if self._others_as_before:
+                before = getattr(self._checkpoint_saver, "last_write_locations", None)
+                if not before:
+                    return  # nothing to go by yet
+                where = {**before, **where}
             self._early_metadata = _EarlyMetadata(checkpoint_id, metadata, where, self.storage_meta())
 
     @_timed(logger=_LOGGER, name="get_write_results")
@@ -379,9 +395,14 @@ class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
         early, self._early_metadata = self._early_metadata, None
         ready = early.result_for(checkpoint_id, metadata, where, metadata.storage_meta) if early is not None else None
         write_bytes = getattr(self._checkpoint_saver, "write_metadata_bytes", None)
-        if ready is not None and write_bytes is not None:
+        self.early_metadata_used = ready is not None and write_bytes is not None
+        if self.early_metadata_used:
             write_bytes(checkpoint_id, ready)  # pickled while the data was being written: same bytes, no wait
         else:
             self._checkpoint_saver.write_metadata(checkpoint_id, metadata)
+        try:  # what the next save's prediction of the other ranks' results goes by (writers come and go, savers stay)
+            self._checkpoint_saver.last_write_locations = where
+        except AttributeError:
+            pass
         if self._ledger.results is not None:
             self._ledger.results.pop(checkpoint_id, None)

@@ -94,7 +94,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         tile_bytes: int = 0,
         block_threads: int = 0,
         verify_crc: bool = True,
-        crc_mode: str = "fused",
+        crc_mode: str = "before",
         use_file_io: bool = True,
         verify_on_discovery: bool = False,
         max_image_bytes: Optional[int] = None,
@@ -102,9 +102,13 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
     ):
         """Arguments as the reference's default loader (checkpoint_loader.py:126-158), plus the copy-engine and
         kernel work-split knobs, ``verify_crc`` (check the CRC-32C sidecar of an object, when it has one, while
-        restoring it), ``crc_mode`` (how a whole-object restore checks it: ``"fused"`` - the unpack kernel folds the
-        checksums of the image it reads, so the image is read once and a mismatch is reported after the targets were
-        written; ``"before"`` - a checksum pass over the image first, and nothing is written on a mismatch) and
+        restoring it), ``crc_mode`` (when it is checked.  ``"before"``, the default: no byte reaches a target, or the
+        planner, before the chunk it lies in has been checked - a checksum pass over every uploaded range or window
+        ahead of its unpack, a host-side check ahead of every item that is served on the host; after a
+        ``ChecksumMismatchError`` the targets hold what they held before, or, where earlier windows of the object
+        had already passed, verified bytes of this checkpoint - never corrupt ones.  ``"fused"``: the unpack kernel
+        folds the checksums of the image it scatters, so the image is read once, and a mismatch is reported after
+        the targets were written - for callers that discard the targets on any error) and
         ``verify_on_discovery`` (also check it, on the host, while choosing the checkpoint to
         recover from, so that a corrupted copy counts as missing) and ``max_image_bytes`` (largest range of an
         object that is uploaded to HBM in one piece; default: what the device has free minus 2 GiB.  A larger
@@ -265,10 +269,26 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
             optimized = stream.format_signature == CheckpointFormat.MLF_FORMAT
             device_reqs = []  # (req, target, dtype, shape, payload_off, stored payload bytes)
             whole = stream.raw_view()
+            sidecar = integrity.read_sidecar(checkpoint_object_id.data) if self._verify_crc else None
+            if sidecar is not None and sidecar[1] != recorded:
+                raise integrity.ChecksumMismatchError(
+                    f"'{checkpoint_object_id.data}': sidecar covers {sidecar[1]} bytes, object holds {recorded}")
+            host_checked: set = set()  # chunks already checked on the host for items served there
+
+            def check_on_host_first(offset: int, length: int) -> None:
+                """crc_mode "before": the chunks an item lies in are checked before the item is handed out."""
+                if sidecar is None or self._crc_mode != "before" or length <= 0:
+                    return
+                chunk = sidecar[0]
+                todo = sorted(set(range(offset // chunk, (offset + length - 1) // chunk + 1)) - host_checked)
+                self._check_on_host(checkpoint_object_id, stream, sidecar, todo)
+                host_checked.update(todo)
+
             t_parse = time.perf_counter()
             for req in read_items:
                 item_md = storage_data[req.storage_index]
                 if req.type == LoadItemType.BYTE_IO:
+                    check_on_host_first(item_md.offset, item_md.length)
                     view = cast(IO[bytes], _create_file_view(stream, item_md.offset, item_md.length))
                     data = io.BytesIO(view.read(item_md.length))
                     data.seek(0)
@@ -280,6 +300,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                     # host-resident target: one copy, from a tensor laid over the record's payload in the mapping
                     # into the target (the reference reads the record into a bytes object first,
                     # checkpoint_loader.py:195-208)
+                    check_on_host_first(item_md.offset, item_md.length)
                     tensor = self._payload_view(whole, recorded, checkpoint_object_id, req, *parsed)
                     tensor = narrow_tensor_by_index(tensor, req.storage_offsets, req.lengths)
                     assert target.size() == tensor.size(), (
@@ -290,6 +311,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                     stats["host_items"] += 1
                     continue
                 if parsed is None:
+                    check_on_host_first(item_md.offset, item_md.length)
                     view = cast(IO[bytes], _create_file_view(stream, item_md.offset, item_md.length))
                     tensor = self.read_tensor(view, req, use_optimized_loader=optimized)
                     assert target.size() == tensor.size(), (
@@ -302,7 +324,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                 device_reqs.append((req, target) + parsed)
             stats["parse_s"] = time.perf_counter() - t_parse  # headers parsed, targets resolved, host items served
             if device_reqs:
-                self._read_device_items(checkpoint_object_id, stream, device_reqs, planner, stats)
+                self._read_device_items(checkpoint_object_id, stream, device_reqs, planner, stats, sidecar)
         stats["read_s"] = time.perf_counter() - t_start
         self.last_load_stats = stats
 
@@ -315,16 +337,12 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         cached = torch.cuda.memory_reserved(device) - torch.cuda.memory_allocated(device)
         return max(free + cached - (2 << 30), 64 << 20)
 
-    def _read_device_items(self, object_id, stream, device_reqs, planner, stats) -> None:
+    def _read_device_items(self, object_id, stream, device_reqs, planner, stats, sidecar) -> None:
         devices = {t.device for _, t, *_ in device_reqs}
         if len(devices) != 1:
             raise ValueError("all device targets of one checkpoint object must live on the same device")
         device = devices.pop()
         written = stream.len_written_data
-        sidecar = integrity.read_sidecar(object_id.data) if self._verify_crc else None
-        if sidecar is not None and sidecar[1] != written:
-            raise integrity.ChecksumMismatchError(
-                f"'{object_id.data}': sidecar covers {sidecar[1]} bytes, object holds {written}")
 
         # Every request becomes one row: where its bytes lie in the data section ([first, last), absolute for now)
         # and how to add it to a descriptor table once the offset of the uploaded range is known.  A request for a
@@ -591,10 +609,10 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         chunk_bytes = 0
         if sidecar is not None:
             chunk_bytes = sidecar[0]
-            if self._crc_mode != "fused" or chunk_bytes % 65536:
+            if chunk_bytes % (65536 if self._crc_mode == "fused" else _UPLOAD_ALIGN):
                 return 0
         through = min(limit, max(_PIPELINED_MIN_BYTES, min(_PIPELINED_MAX_BYTES, need // 4)))
-        window = through // 2 - max(chunk_bytes, _UPLOAD_ALIGN)
+        window = through // 2 - 2 * max(chunk_bytes, _UPLOAD_ALIGN)
         uncut = max((r[1] - r[0] for r in rows if not r[2]), default=0)
         if window < max(uncut, 4 * chunk_bytes, _PIPELINED_MIN_WINDOW):
             return 0
@@ -605,12 +623,15 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         sorted by position and restored window by window through one device buffer of at most ``limit`` bytes.  A
         contiguous row larger than a window is cut into pieces; a strided one cannot be.
 
-        With a sidecar and ``crc_mode="fused"`` every window starts on a checksum chunk, so the unpack of a window
-        yields the checksums of the chunks it holds completely; a chunk that a window ends in is held completely by
-        the next window when the rows continue there (it starts on that chunk: a few MiB are uploaded twice); chunks
-        that no window holds completely (where the rows do not continue; those of byte blobs behind the tensors)
-        are checked on the host at the end.  A mismatch raises before any tensor is committed.  With
-        ``crc_mode="before"``, or a buffer too small for that, the whole object is checked on the host first."""
+        With a sidecar every window starts on a checksum chunk.  ``crc_mode="before"``: a window is uploaded up to the
+        end of the last chunk its rows touch, a checksum pass over the window runs first, and the window is unpacked
+        only if every chunk matches - the next window is already crossing the link meanwhile; a chunk that two
+        windows share is uploaded and checked twice.  ``crc_mode="fused"``: the unpack of a window yields the
+        checksums of the chunks it holds completely; a chunk that a window ends in is held completely by the next
+        window when the rows continue there; chunks that no window holds completely (where the rows do not continue;
+        those of byte blobs behind the tensors) are checked on the host at the end, and a mismatch raises before any
+        tensor is committed, after targets were written.  With a buffer too small for either, the whole object is
+        checked on the host first."""
         if not by_choice:
             _LOGGER.warning("requested range of '%s' exceeds the HBM limit of %d bytes; restoring window by window",
                             object_id, limit)
@@ -637,16 +658,26 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                     buffers = [one]
                 else:
                     limit //= 2
-        on_device = (sidecar is not None and self._crc_mode == "fused" and chunk_bytes % 65536 == 0
+        fused = self._crc_mode == "fused"
+        on_device = (sidecar is not None and chunk_bytes % (65536 if fused else _UPLOAD_ALIGN) == 0
                      and limit >= 4 * chunk_bytes)
+        check_first = on_device and not fused  # a checksum pass over every window ahead of its unpack
         if sidecar is not None and not on_device:
             self._check_on_host(object_id, stream, sidecar, range(len(want)))
         align = chunk_bytes if on_device else _UPLOAD_ALIGN
-        usable = limit - align  # a window starts on an upload boundary at or below its first row
-        piece = usable // 65536 * 65536  # a multiple of every element size
+
+        # a window starts on an upload boundary at or below its first row and, where it is checked before it is
+        # unpacked, ends on the chunk boundary at or above its last row (or where the data section ends)
+        def start_of(first: int) -> int:
+            return first // align * align
+
+        def end_of(last: int) -> int:
+            return min(-(-last // chunk_bytes) * chunk_bytes, data_bytes) if check_first else last
+
+        piece = (limit - (2 if check_first else 1) * align) // 65536 * 65536  # a multiple of every element size
         pieces = []
         for first, last, contiguous, args in sorted(rows, key=lambda r: r[0]):
-            if last - first <= usable:
+            if end_of(last) - start_of(first) <= limit:
                 pieces.append((first, last, contiguous, args))
             elif contiguous:
                 ptr, esz = args
@@ -658,11 +689,11 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                     f"HBM limit of {limit} bytes")
         windows, current, lo = [], [], 0
         for row in pieces:
-            if current and row[1] - lo > limit:
+            if current and end_of(row[1]) - lo > limit:
                 windows.append((lo, current))
                 current = []
             if not current:
-                lo = row[0] // align * align
+                lo = start_of(row[0])
             current.append(row)
         windows.append((lo, current))
         cur = torch.cuda.current_stream(device)
@@ -674,23 +705,26 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         launched = []  # (plan, first chunk, complete chunks, event)
         stats_local = self._stats_in_progress
 
+        def span_of(k):
+            lo_k, rows_k = windows[k]
+            return end_of(max(r[1] for r in rows_k)) - lo_k
+
         def upload(k):
             self._stats_local.current = stats_local  # (the helper thread books its transfer to this restore)
-            lo_k, rows_k = windows[k]
-            span_k = max(r[1] for r in rows_k) - lo_k
-            self._upload(stream, lo_k, buffers[k % len(buffers)], span_k, cur, stats)
-            return span_k
+            self._upload(stream, windows[k][0], buffers[k % len(buffers)], span_of(k), cur, stats)
 
         try:
             with concurrent.futures.ThreadPoolExecutor(max_workers=1, thread_name_prefix="mlf-upload") as helper:
                 pending = helper.submit(upload, 0)
                 for k, (lo, window_rows) in enumerate(windows):
-                    span = max(r[1] for r in window_rows) - lo
+                    span = span_of(k)
                     # (built while the window is on its way: not a part of the restore's length)
-                    plan = self._unpack_plan(self._table_of(window_rows, lo), span, chunk_bytes if on_device else 0,
+                    plan = self._unpack_plan(self._table_of(window_rows, lo), span, chunk_bytes if on_device and fused else 0,
                                              booked_as="unpack_plan_s" if len(buffers) == 1 and k else "unpack_plan_beside_h2d_s")
                     launched.append([plan, 0, 0, None])
                     pending.result()
+                    if check_first and len(buffers) == 1:
+                        self._check_window(object_id, buffers[0], lo, span, sidecar, cur, checked)
                     if k + 1 < len(windows):
                         nxt = (k + 1) % len(buffers)
                         if len(buffers) == 1:  # the one buffer: nothing to overlap, the unpack goes first
@@ -700,11 +734,13 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                         elif in_use[nxt] is not None:
                             in_use[nxt].synchronize()
                         pending = helper.submit(upload, k + 1)
+                    if check_first and len(buffers) > 1:  # while the next window is on its way
+                        self._check_window(object_id, buffers[k % len(buffers)], lo, span, sidecar, cur, checked)
                     if launched[-1][3] is None:
                         launched[-1][3] = self._launch_unpack(plan, buffers[k % len(buffers)], cur,
                                                               sum(r[1] - r[0] for r in window_rows if r[2]))
                     in_use[k % len(buffers)] = launched[-1][3]
-                    if on_device:
+                    if on_device and fused:
                         first = lo // chunk_bytes
                         whole = span // chunk_bytes + (1 if lo + span == data_bytes and span % chunk_bytes else 0)
                         launched[-1][1:3] = [first, whole]
@@ -712,7 +748,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
             cur.synchronize()
             stats["unpack_s"] = stats.get("unpack_s", 0.0) + time.perf_counter() - t0
             for plan, first, whole, _ in launched:
-                if on_device:
+                if on_device and fused:
                     got = plan.crc_values()
                     self._compare_checksums(object_id, got[:whole], want[first : first + whole], chunk_bytes, first, len(want))
                     checked.update(range(first, first + whole))
@@ -723,6 +759,18 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         if on_device:  # what no window held completely: chunks where the rows do not continue, and those of byte blobs
             self._check_on_host(object_id, stream, sidecar, sorted(set(range(len(want))) - checked))
         stats["windows"] = stats.get("windows", 0) + len(windows)
+
+    def _check_window(self, object_id, buffer: torch.Tensor, lo: int, span: int, sidecar, cur, checked: set) -> None:
+        """Checksum pass over a window that starts on a chunk boundary and ends on one (or where the data section
+        ends), compared with the sidecar before anything is unpacked from it."""
+        chunk_bytes, _, want = sidecar
+        t0 = time.perf_counter()
+        got = hip_plan.crc32c_device(buffer, span, chunk_bytes, cur.cuda_stream)
+        stats = self._stats_in_progress
+        stats["crc_s"] = stats.get("crc_s", 0.0) + time.perf_counter() - t0
+        first = lo // chunk_bytes
+        self._compare_checksums(object_id, got, want[first : first + len(got)], chunk_bytes, first, len(want))
+        checked.update(range(first, first + len(got)))
 
     def _check_on_host(self, object_id, stream, sidecar, chunks) -> None:
         """Compares the given chunks of an object's data section with its sidecar, reading them on the host."""

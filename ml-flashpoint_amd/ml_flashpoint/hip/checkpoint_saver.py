@@ -323,12 +323,17 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         self.record_kernel_events = False
         self.kernel_events: list = []
         self._plan_cache: dict = {}  # object name -> _KeptPlan
+        # Kept for the adapter from save to save (writers are made anew for every save, the saver stays): where every
+        # rank's items went in the last save that this process finished, and the metadata object of the last planning
+        # save - what the next save's metadata object is pickled from while its data is still in flight.
+        self.last_write_locations: Optional[dict] = None
+        self.last_global_metadata = None
 
     # ---- pickling: only configuration crosses a process boundary --------------------------------------
     def __getstate__(self):
         state = self.__dict__.copy()
         for key in ("_replication_manager", "_engine", "_engine_clear_of", "_engine_lock", "last_save_stats", "kernel_events",
-                    "_plan_cache"):
+                    "_plan_cache", "last_write_locations", "last_global_metadata"):
             state.pop(key, None)
         return state
 
@@ -365,7 +370,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         if left:
             _LOGGER.warning("%d of the copy engine's streams share a hardware queue with a stream of the training step: "
                             "transfers beside a busy device will be slow (more queues: GPU_MAX_HW_QUEUES)", left)
-        self._engine_clear_of = wanted
+        with self._engine_lock:
+            self._engine_clear_of = wanted | (self._engine_clear_of or set())
 
     # ---- dirty marker / directory ----------------------------------------------------------------------
     @override
@@ -542,8 +548,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         items = [item for item, _ in tensor_data] + [item for item, _ in bytes_data]
         plan = image = packed = None
         stream = 0
-        if layout.image_bytes and (self._engine_clear_of is None
-                                   or torch.cuda.current_stream(device).cuda_stream not in self._engine_clear_of):
+        clear_of = self._engine_clear_of  # (one read: warm_up replaces the set, it never changes one in place)
+        if layout.image_bytes and (clear_of is None or torch.cuda.current_stream(device).cuda_stream not in clear_of):
             self.warm_up(device)  # the engine's streams off the hardware queue of the stream the pack runs on
         if layout.image_bytes and object_id is not None:
             if layout.image_bytes <= self._image_limit(device):

@@ -209,11 +209,9 @@ def test_next_save_does_not_wait_for_the_previous_transfer(shm_dir, manager_futu
 
     first = begin(10, big)
     first_transfer = saver._staged_of(first[3][0]).future
-    t0 = time.perf_counter()
     second = begin(11, small)
-    blocked_s = time.perf_counter() - t0
+    # order, not a duration: the second save was planned, packed and staged while the first was still on the link
     assert not first_transfer.done(), "the second save's blocking part outlasted the first save's transfer"
-    assert blocked_s < 0.25
     snapshot = {k: v.cpu() for k, v in small.items()}
     for v in small.values():
         v.add_(1.0)

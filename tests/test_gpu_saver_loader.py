@@ -685,7 +685,8 @@ def test_restore_larger_than_the_hbm_limit_goes_window_by_window(shm_dir, manage
         byte = f.read(1)
         f.seek(-1, os.SEEK_CUR)
         f.write(bytes([byte[0] ^ 0x01]))
-    for mode in ("fused", "before"):  # "before": the whole object is checked on the host ahead of the first window
+    assert _loader()._crc_mode == "before"
+    for mode in ("fused", "before"):
         picky = _loader(max_image_bytes=256 << 10, use_file_io=load_file_io, crc_mode=mode)
         victim = targets()
         with pytest.raises(BaseException) as exc:
@@ -693,8 +694,24 @@ def test_restore_larger_than_the_hbm_limit_goes_window_by_window(shm_dir, manage
         cause = exc.value.failures[0][0] if hasattr(exc.value, "failures") else exc.value
         assert isinstance(cause, integrity.ChecksumMismatchError) and "chunk(s) [5]" in str(cause), mode
         if mode == "before":
-            assert all(not v.any() for v in victim.values()
-                       if isinstance(v, torch.Tensor) and v.is_cuda and v.dtype != torch.float8_e4m3fn)
+            # every window is checked before it is unpacked: what the earlier windows brought is in place, the window
+            # with the flipped bit and everything behind it never reached a target - no byte of any target is
+            # anything but its old value (zero) or the checkpoint's
+            touched = 0
+            for k, v in sd_cpu.items():
+                if isinstance(v, torch.Tensor) and v.numel():
+                    got, want = _bits(victim[k]), _bits(v)
+                    assert bool(((got == 0) | (got == want)).all()), k
+                    touched += int(bool(got.any()))
+            assert 0 < touched < sum(1 for v in sd_cpu.values() if isinstance(v, torch.Tensor) and v.numel())
+            metadata = pickle.load(open(os.path.join(ckpt, ".metadata"), "rb"))
+            at = 5 * (1 << 16) + 77  # the flipped byte: its tensor's byte there is still the old one
+            hit = [(i.fqn, at - (st.offset + st.length - _bits(sd_cpu[i.fqn]).numel()))
+                   for i, st in metadata.storage_data.items()
+                   if isinstance(sd_cpu[i.fqn], torch.Tensor) and st.offset <= at < st.offset + st.length]
+            for fqn, pos in hit:
+                if pos >= 0:
+                    assert int(_bits(victim[fqn])[pos]) == 0, fqn
     with open(obj, "r+b") as f:  # the last chunk of the object, which no window holds completely: found on the host
         f.seek(-3, os.SEEK_END)
         byte = f.read(1)

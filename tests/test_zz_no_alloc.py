@@ -107,3 +107,43 @@ def test_noalloc_crc_refuses_what_does_not_fit_and_bad_arguments():
     assert lib.mlf_crc32c_device_noalloc(buf.data_ptr(), 1 << 20, 65536, None, 16, stream) != 0
     assert lib.mlf_crc32c_device_noalloc(buf.data_ptr(), 0, 65536, None, 0, stream) == 0  # nothing to do
     torch.cuda.synchronize()
+
+
+def test_noalloc_crc_inside_a_captured_graph_replayed_over_changing_data():
+    """The entry point enqueues kernels and nothing else, so it may be recorded into a HIP graph - once
+    ``mlf_hip_set_device`` (or an earlier call) has resolved where the scratch array lies on the device.  Every replay,
+    with other work of the program and synchronizations in between, yields what the allocating entry point yields
+    for the data the buffer holds at that moment."""
+    from ml_flashpoint.hip import _lib
+    from ml_flashpoint.hip import plan as P
+
+    lib = _lib.load()
+    _lib.check(lib.mlf_hip_set_device(torch.cuda.current_device()), "mlf_hip_set_device")  # resolves the array's address
+    nbytes, chunk = (24 << 20) + 4096, 2 << 20
+    n_chunks = -(-nbytes // chunk)
+    data = _random_bytes(nbytes, 7)
+    out = torch.full((n_chunks + 2,), _FILL, dtype=torch.int32, device=DEV)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    free_before, _ = torch.cuda.mem_get_info()
+    with torch.cuda.graph(graph, stream=side):
+        rc = lib.mlf_crc32c_device_noalloc(data.data_ptr(), nbytes, chunk, out.data_ptr(), out.numel(),
+                                           torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "mlf_crc32c_device_noalloc under capture")
+    assert (_u32(out) == 0xDEADBEEF).all(), "capturing must not run anything"
+    other = _random_bytes((3 << 20) + 5, 9)
+    for replay in range(4):
+        if replay:
+            data.copy_(_random_bytes(nbytes, 100 + replay))  # the program's own eager work between the replays ...
+            P.crc32c_device(other, other.numel(), 1 << 20)    # ... including a call that uses other scratch
+        out.fill_(_FILL)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = P.crc32c_device(data, nbytes, chunk)
+        got = _u32(out)
+        assert got[:n_chunks].tolist() == want.tolist(), f"replay {replay}"
+        assert (got[n_chunks:] == 0xDEADBEEF).all()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after >= free_before - (8 << 20)  # the graph object itself is all that was added
