@@ -299,10 +299,14 @@ int crc_fused_setup(FusedCrc* f) {
   f->n_groups = (f->image_bytes + group_bytes - 1) / group_bytes;
   f->n_chunks = (f->image_bytes + f->chunk_bytes - 1) / f->chunk_bytes;
   // state advanced by one row of the fused kernel's walk (its cells are wgs_per_group cells apart), sliced by byte
-  std::vector<uint32_t> row_tab(1024);
-  const uint32_t x_row = x_pow_bytes((uint64_t)kCellBytes * f->wgs_per_group);
+  // and, behind it, advanced by four bytes: joins the remainders of a lane's four neighbouring dwords
+  std::vector<uint32_t> row_tab(2048);
+  const uint32_t x_row = x_pow_bytes((uint64_t)kCellBytes * f->wgs_per_group), x_dword = x_pow_bytes(4);
   for (int b = 0; b < 4; ++b)
-    for (uint32_t v = 0; v < 256; ++v) row_tab[b * 256 + v] = gf_mul(x_row, v << (8 * b));
+    for (uint32_t v = 0; v < 256; ++v) {
+      row_tab[b * 256 + v] = gf_mul(x_row, v << (8 * b));
+      row_tab[1024 + b * 256 + v] = gf_mul(x_dword, v << (8 * b));
+    }
   // dword j of lane t's vector lies 4096 - 16 t - 4 j bytes in front of its cell's end (its own four bytes included)
   std::vector<uint32_t> lane_w(1024);
   for (uint32_t t = 0; t < 256; ++t)
@@ -312,8 +316,8 @@ int crc_fused_setup(FusedCrc* f) {
   HIP_TRY(hipMemset(f->d_ent_val, 0, std::max<uint64_t>(f->n_ent, 1) * sizeof(uint32_t)));
   HIP_TRY(hipMalloc(reinterpret_cast<void**>(&f->d_fast_val), std::max<uint64_t>(n_fast, 1) * sizeof(uint32_t)));
   HIP_TRY(hipMalloc(reinterpret_cast<void**>(&f->d_group_val), std::max<uint64_t>(f->n_groups, 1) * sizeof(uint32_t)));
-  HIP_TRY(hipMalloc(reinterpret_cast<void**>(&f->d_row_tab), 4096));
-  HIP_TRY(hipMemcpy(f->d_row_tab, row_tab.data(), 4096, hipMemcpyHostToDevice));
+  HIP_TRY(hipMalloc(reinterpret_cast<void**>(&f->d_row_tab), 8192));
+  HIP_TRY(hipMemcpy(f->d_row_tab, row_tab.data(), 8192, hipMemcpyHostToDevice));
   HIP_TRY(hipMalloc(reinterpret_cast<void**>(&f->d_lane_w), 4096));
   HIP_TRY(hipMemcpy(f->d_lane_w, lane_w.data(), 4096, hipMemcpyHostToDevice));
   HIP_TRY(hipMalloc(reinterpret_cast<void**>(&f->d_sink), 4096));

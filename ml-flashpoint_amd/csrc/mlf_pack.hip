@@ -668,13 +668,17 @@ __global__ void __launch_bounds__(kTransThreads) mlf_transpose_kernel(const Tran
 // workgroup: the remainder, relative to the end of the workgroup's last cell, of its cells laid G apart - one
 // value per workgroup, chained by mlf_crc_groups_kernel.  Cells of entries without an address (record headers, item
 // edges, strided items ...) are skipped here; the other kernels move them and their remainders are taken from the
-// finished image.  The checksum arithmetic hides behind the memory traffic (measured on 16 GiB: copy alone in this
-// order 4.7-5.6 TB/s, with the checksum 5.7-5.8; one 4 KiB tile per workgroup without checksum 6.2): what the kernel
-// gives up against the flat kernel - 39.3 against 34.3 ms on the 112 GB shard - is the price of workgroups that live
-// for sixteen rows instead of one, not of the arithmetic.  Eight or four rows per workgroup do not amortise the
-// closing multiplications (5.0 and 3.7 TB/s), thirty-two gain nothing.
+// finished image.  The checksum arithmetic hides behind the memory traffic completely: with the table lookups and
+// the closing multiplications taken out (values then wrong, timing only) a 51.5 GB pack takes 17.9 ms against 17.8
+// with them, where the flat kernel takes 15.8; without the LDS tables and the barrier as well: 18.1; 4 / 8 / 16 / 32
+// rows per workgroup with the arithmetic: 17.7 / 17.8 / 17.8 / 18.7; 2 / 3 / 4 / 6 / 8 rows requested ahead: 17.9 /
+// 17.8 / 17.8 / 18.0 / 17.7; aligned granules realigned across lanes instead of byte-misaligned loads: 18.5.  What
+// the kernel gives up against the flat kernel (about 11 %) is in how its workgroups walk the image, not in what
+// they compute.  The closing joins a lane's four accumulators with three four-byte advances (table lookups) and
+// multiplies once by the lane's weight; four general products there made 40 % of the kernel's vector instructions.
 constexpr uint32_t kFusedRows = 16;   // cells per workgroup; FusedCrc::rows
 constexpr uint32_t kFusedAhead = 4;   // rows requested before the first is used
+constexpr uint32_t kFusedGridLog2 = 16;  // workgroups per grid row, as in the flat kernel's launch (one long row: 3 % slower)
 // workgroups per group: 64 (groups of 4 MiB) and 512 (32 MiB) move the 112 GB shard equally fast when packing; unpacking
 // into byte-misaligned tensors is faster with 64 (5.5 against 4.7 TB/s), and chaining 64 values per group takes 0.05 ms
 // where 512 take 0.6
@@ -688,28 +692,31 @@ constexpr uint32_t kCellsPerEntryLog2 = 4;
 
 template <bool PACK>
 __global__ void __launch_bounds__(256) mlf_fused_crc_kernel(const uint64_t* __restrict__ ent, char* __restrict__ image,
-                                                            uint32_t G, uint32_t xcd_sets,
+                                                            uint32_t G, uint32_t xcd_sets, uint32_t n_wgs,
                                                             const uint32_t* __restrict__ row_tab,
                                                             const u32x4* __restrict__ lane_w,
                                                             uint32_t* __restrict__ fast_val, char* __restrict__ sink) {
   // kFusedTabCopies copies of the table, entry v of copy c at word v * copies + c, lane l reads copy l % copies:
   // lookups with random v then spread over that many times more banks
   __shared__ uint32_t tab[1024 * kFusedTabCopies];
+  __shared__ uint32_t tab4[1024];  // state advanced by four bytes, sliced by state byte
   __shared__ uint32_t part[4];
   const uint32_t tid = threadIdx.x, lane = tid & 63u;
-  uint32_t group = blockIdx.x / G;
-  uint32_t w = blockIdx.x - group * G;
+  const uint32_t wg = (blockIdx.y << kFusedGridLog2) + blockIdx.x;
+  if (wg >= n_wgs) return;  // padding of the last grid row
+  uint32_t group = wg / G;
+  uint32_t w = wg - group * G;
   // Workgroups reach the eight XCDs round-robin, and a source line that straddles a cell cut should be served by one
   // L2, not fetched from HBM by two: neighbouring cells go to the same XCD.
   if ((G & 511u) == 0) {
     // within every 512 workgroups XCD x takes 64 consecutive cells of a row
     const uint32_t lo = w & 511u;
     w = (w & ~511u) + (lo & 7u) * 64u + (lo >> 3);
-  } else if (blockIdx.x < xcd_sets * 8u * G) {
+  } else if (wg < xcd_sets * 8u * G) {
     // smaller groups: of every eight consecutive groups XCD x takes group x whole (measured on the 112 GB shard with
     // groups of 64: fetched bytes 1.047 -> 1.030 x the payload, same time; what is left is one extra 128-byte line
     // per misaligned cell, fetched again because the neighbour's row passed through that L2 some microseconds earlier)
-    const uint32_t set = blockIdx.x / (8u * G), lo = blockIdx.x - set * 8u * G;
+    const uint32_t set = wg / (8u * G), lo = wg - set * 8u * G;
     group = set * 8u + (lo & 7u);
     w = lo >> 3;
   }
@@ -742,13 +749,15 @@ __global__ void __launch_bounds__(256) mlf_fused_crc_kernel(const uint64_t* __re
             : spare_src) + tid * 16u)
 #define MLF_FUSED_DST(k)                                                                          \
   ((base[k] ? (PACK ? image + ((cell0 + (uint64_t)(k) * G) << 12) : reinterpret_cast<char*>(base[k])) : sink) + tid * 16u)
+#define MLF_FUSED_LOAD(slot, k) raw[slot] = __builtin_nontemporal_load(gload<u32x4_u>(MLF_FUSED_SRC(k)))
 #pragma unroll
-  for (uint32_t k = 0; k < kFusedAhead; ++k) raw[k] = __builtin_nontemporal_load(gload<u32x4_u>(MLF_FUSED_SRC(k)));
+  for (uint32_t k = 0; k < kFusedAhead; ++k) MLF_FUSED_LOAD(k, k);
 #pragma unroll
   for (uint32_t k = 0; k < 4; ++k) {
     const uint32_t t = row_tab[tid + 256u * k];
 #pragma unroll
     for (uint32_t c = 0; c < kFusedTabCopies; ++c) tab[(tid + 256u * k) * kFusedTabCopies + c] = t;
+    tab4[tid + 256u * k] = row_tab[1024u + tid + 256u * k];
   }
   __syncthreads();
   const uint32_t* my = tab + (lane & (kFusedTabCopies - 1u));
@@ -760,7 +769,7 @@ __global__ void __launch_bounds__(256) mlf_fused_crc_kernel(const uint64_t* __re
   for (uint32_t k = 0; k < kFusedRows; ++k) {
     const u32x4 v = raw[k % kFusedAhead];  // the cell's vector as it lies in the image
     if (k + kFusedAhead < kFusedRows)      // the slot just read is free again
-      raw[k % kFusedAhead] = __builtin_nontemporal_load(gload<u32x4_u>(MLF_FUSED_SRC(k + kFusedAhead)));
+      MLF_FUSED_LOAD(k % kFusedAhead, k + kFusedAhead);
     __builtin_nontemporal_store(v, gstore<u32x4_u>(MLF_FUSED_DST(k)));
     const uint32_t ours = base[k] ? 0xFFFFFFFFu : 0u;
     a0 = MLF_FUSED_ADV(a0) ^ (v.x & ours);
@@ -773,8 +782,17 @@ __global__ void __launch_bounds__(256) mlf_fused_crc_kernel(const uint64_t* __re
 #undef MLF_FUSED_SRC
 #undef MLF_FUSED_DST
 #undef MLF_FUSED_ADV
-  const u32x4 wts = lane_w[tid];
-  uint32_t acc = gf_mul(a0, wts.x) ^ gf_mul(a1, wts.y) ^ gf_mul(a2, wts.z) ^ gf_mul(a3, wts.w);
+#undef MLF_FUSED_LOAD
+  // The lane's four dwords lie next to each other, so their remainders are joined by three advances of four bytes
+  // (table lookups), and only the joined value needs a general multiplication by the lane's weight: one bitwise
+  // product per lane and workgroup instead of four.
+#define MLF_FUSED_ADV4(a) \
+  (tab4[(a) & 255u] ^ tab4[256u + (((a) >> 8) & 255u)] ^ tab4[512u + (((a) >> 16) & 255u)] ^ tab4[768u + ((a) >> 24)])
+  uint32_t joined = MLF_FUSED_ADV4(a0) ^ a1;
+  joined = MLF_FUSED_ADV4(joined) ^ a2;
+  joined = MLF_FUSED_ADV4(joined) ^ a3;
+#undef MLF_FUSED_ADV4
+  uint32_t acc = gf_mul(joined, lane_w[tid].w);
 #pragma unroll
   for (int s = 1; s < 64; s <<= 1) acc ^= (uint32_t)__shfl_xor((int)acc, s, 64);
   if (lane == 0u) part[tid >> 6] = acc;
@@ -1364,8 +1382,11 @@ int launch_plan(const mlf_plan* plan, char* image, hipStream_t stream) {
     const FusedCrc& f = plan->crc;
     const uint64_t n_wg = f.fused_groups * f.wgs_per_group;
     if (n_wg) {
-      hipLaunchKernelGGL((mlf_fused_crc_kernel<PACK>), dim3((uint32_t)n_wg), dim3(256), 0, stream, f.d_ent, image,
-                         f.wgs_per_group, (uint32_t)(f.fused_groups / 8), f.d_row_tab, f.d_lane_w, f.d_fast_val, f.d_sink);
+      const dim3 grid(std::min<uint32_t>((uint32_t)n_wg, 1u << kFusedGridLog2),
+                      (uint32_t)((n_wg + (1u << kFusedGridLog2) - 1) >> kFusedGridLog2));
+      hipLaunchKernelGGL((mlf_fused_crc_kernel<PACK>), grid, dim3(256), 0, stream, f.d_ent, image,
+                         f.wgs_per_group, (uint32_t)(f.fused_groups / 8), (uint32_t)n_wg, f.d_row_tab, f.d_lane_w,
+                         f.d_fast_val, f.d_sink);
       HIP_TRY(hipGetLastError());
     }
   }

@@ -352,9 +352,11 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         rows = []  # (first, last, contiguous?, table arguments)
         conversions = []  # (target, buffer of the stored dtype): the reference's `copy_` converts, so this does too
         for req, target, dtype, shape, payload_off, stored_bytes in device_reqs:
-            if target.dtype != dtype:
-                # restored bit-exact into a buffer of the stored dtype; torch converts on the device afterwards,
-                # on the stream the unpack runs on (checkpoint_loader.py:335 does the same conversion on the host)
+            if target.dtype != dtype or (target.dim() > _lib.MAX_DIMS and not target.is_contiguous()
+                                         and not hip_plan.describable(tuple(target.shape), tuple(target.stride()))):
+                # restored bit-exact into a contiguous buffer of the stored dtype; torch's ``copy_`` converts, or
+                # scatters into a view of more dimensions than a descriptor holds, on the device afterwards, on the
+                # stream the unpack runs on (checkpoint_loader.py:335 does the same ``copy_`` on the host)
                 stored_as = torch.empty(target.size(), dtype=dtype, device=device)
                 conversions.append((target, stored_as))
                 target = stored_as
@@ -372,10 +374,8 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                 first, last = payload_off, payload_off + stored_bytes
                 if target.is_contiguous():
                     rows.append((first, last, True, (target.data_ptr(), esz)))
-                elif ndim <= _lib.MAX_DIMS:
+                else:  # (a view of too many dimensions was replaced by a contiguous stand-in above)
                     rows.append((first, last, False, (target.data_ptr(), esz, tuple(shape), tuple(target.stride()), None)))
-                else:
-                    raise NotImplementedError(f"rank > {_lib.MAX_DIMS} targets must be contiguous")
             else:
                 stored_strides = hip_plan._contiguous_strides(tuple(shape))
                 lengths = [l if l < sz else sz for l, sz in zip(req_lengths, shape)]
@@ -387,12 +387,22 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                 numel = box_shape.numel()
                 if numel == 0:
                     continue
+                box = (tuple(lengths), tuple(target.stride()), tuple(stored_strides))
                 if ndim > _lib.MAX_DIMS:
-                    raise NotImplementedError(f"sub-box reads of rank > {_lib.MAX_DIMS} tensors are not supported")
+                    box = hip_plan.collapse_dims(*box)
+                    if len(box[0]) > _lib.MAX_DIMS:
+                        # a box that is narrowed in so many dimensions that no merging helps: into a contiguous
+                        # stand-in of the box's shape first (its strides merge wherever the stored ones do)
+                        stored_as = torch.empty(box_shape, dtype=dtype, device=device)
+                        conversions.append((target, stored_as))
+                        target = stored_as
+                        box = hip_plan.collapse_dims(tuple(lengths), tuple(target.stride()), tuple(stored_strides))
+                        if len(box[0]) > _lib.MAX_DIMS:
+                            raise ValueError(f"req {req.storage_index}: a sub-box of {len(box[0])} dimensions after merging "
+                                             f"does not fit the descriptor table's {_lib.MAX_DIMS}")
                 first = payload_off + sum(o * st for o, st in zip(offsets, stored_strides)) * esz
                 last = first + (sum((l - 1) * st for l, st in zip(lengths, stored_strides)) + 1) * esz
-                rows.append((first, last, False,
-                             (target.data_ptr(), esz, tuple(lengths), tuple(target.stride()), tuple(stored_strides))))
+                rows.append((first, last, False, (target.data_ptr(), esz) + box))
                 stored_bytes = numel * esz
             stats["device_payload_bytes"] += stored_bytes
         stats["table_s"] = time.perf_counter() - t_rows
@@ -621,7 +631,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
     def _restore_windowed(self, object_id, stream, device, rows, limit, sidecar, stats, by_choice: bool = False) -> None:
         """Fallback for an object whose requested range does not fit in HBM beside the live state: the rows are
         sorted by position and restored window by window through one device buffer of at most ``limit`` bytes.  A
-        contiguous row larger than a window is cut into pieces; a strided one cannot be.
+        contiguous row larger than a window is cut into pieces, a strided one or a sub-box into smaller boxes.
 
         With a sidecar every window starts on a checksum chunk.  ``crc_mode="before"``: a window is uploaded up to the
         end of the last chunk its rows touch, a checksum pass over the window runs first, and the window is unpacked
@@ -684,9 +694,9 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                 for begin in range(first, last, piece):
                     pieces.append((begin, min(begin + piece, last), True, (ptr + (begin - first), esz)))
             else:
-                raise NotImplementedError(
-                    f"'{object_id.data}': a strided or partial read spanning {last - first} bytes does not fit the "
-                    f"HBM limit of {limit} bytes")
+                # a strided target or a sub-box whose bytes span more of the image than a window holds: cut along its
+                # outermost dimension (then the next one) into boxes that do
+                pieces.extend(self._cut_box(first, args, piece))
         windows, current, lo = [], [], 0
         for row in pieces:
             if current and end_of(row[1]) - lo > limit:
@@ -759,6 +769,31 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         if on_device:  # what no window held completely: chunks where the rows do not continue, and those of byte blobs
             self._check_on_host(object_id, stream, sidecar, sorted(set(range(len(want))) - checked))
         stats["windows"] = stats.get("windows", 0) + len(windows)
+
+    @staticmethod
+    def _cut_box(first: int, args, usable: int):
+        """Cuts a strided row - (target address, element size, shape, target strides, image strides or None), whose
+        element 0 lies at data-section byte ``first`` - into rows of the same kind that each span at most ``usable``
+        bytes of the image: slabs along the first dimension that has more than one index, and slabs of those along
+        the next one where a single index is still too much.  Down to single elements if it must be."""
+        ptr, esz, shape, strides, image_strides = args
+        if image_strides is None:
+            image_strides = tuple(hip_plan._contiguous_strides(shape))
+
+        def span(box_shape):
+            return (sum((n - 1) * st for n, st in zip(box_shape, image_strides)) + 1) * esz
+
+        if span(shape) <= usable:
+            return [(first, first + span(shape), False, (ptr, esz, tuple(shape), tuple(strides), tuple(image_strides)))]
+        d = next(i for i, n in enumerate(shape) if n > 1)  # (a single element never exceeds a window)
+        one = span(shape[:d] + (1,) + shape[d + 1:])
+        per = (usable - one) // (image_strides[d] * esz) + 1 if one <= usable else 1
+        out = []
+        for i0 in range(0, shape[d], per):
+            sub = shape[:d] + (min(per, shape[d] - i0),) + shape[d + 1:]
+            out.extend(HipMLFlashpointCheckpointLoader._cut_box(
+                first + i0 * image_strides[d] * esz, (ptr + i0 * strides[d] * esz, esz, sub, strides, image_strides), usable))
+        return out
 
     def _check_window(self, object_id, buffer: torch.Tensor, lo: int, span: int, sidecar, cur, checked: set) -> None:
         """Checksum pass over a window that starts on a chunk boundary and ends on one (or where the data section

@@ -520,6 +520,14 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             blobs.append(data.read())
         tensors = [t for _, t in tensor_data]
         t0 = time.perf_counter()
+        for i, t in enumerate(tensors):
+            if t.dim() > _lib.MAX_DIMS and t.device.type != "cpu" and not t.is_contiguous() \
+                    and not hip_plan.describable(tuple(t.shape), tuple(t.stride())):
+                # A view of more dimensions than a descriptor holds, also after merging neighbours: made contiguous
+                # on the device, on the stream the pack follows on, and packed from there as one run - what the
+                # reference's ``copy_`` into the buffer does on the host (checkpoint_saver.py:797-800).  The copy is
+                # a new tensor at every save, so such an object's plan is rebuilt every time.
+                tensors[i] = t.contiguous()
         key = self._plan_key(tensors, blobs) if self._reuse_plans and object_name is not None else None
         kept = self._plan_cache.get(object_name) if key is not None else None
         if kept is not None and kept.key != key:

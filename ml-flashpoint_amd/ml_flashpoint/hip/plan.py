@@ -38,6 +38,29 @@ def _contiguous_strides(shape: Sequence[int]) -> List[int]:
     return strides
 
 
+def collapse_dims(shape: Sequence[int], stride: Sequence[int],
+                  image_stride: Optional[Sequence[int]] = None) -> Tuple[tuple, tuple, tuple]:
+    """The same elements at the same places described with as few dimensions as possible: dimensions of extent 1
+    dropped, neighbours merged where stepping the outer one equals walking off the end of the inner one on both
+    sides.  ``image_stride`` None: the C-contiguous strides of ``shape``.  Strides in elements."""
+    if image_stride is None:
+        image_stride = _contiguous_strides(shape)
+    out: List[List[int]] = []
+    for n, ts, im in zip(shape, stride, image_stride):
+        if n == 1:
+            continue
+        if out and out[-1][1] == ts * n and out[-1][2] == im * n:
+            out[-1] = [out[-1][0] * n, ts, im]
+        else:
+            out.append([n, ts, im])
+    return tuple(d[0] for d in out), tuple(d[1] for d in out), tuple(d[2] for d in out)
+
+
+def describable(shape: Sequence[int], stride: Sequence[int], image_stride: Optional[Sequence[int]] = None) -> bool:
+    """Whether a strided item fits the descriptor table's ``MAX_DIMS`` dimensions (after ``collapse_dims``)."""
+    return len(shape) <= MAX_DIMS or len(collapse_dims(shape, stride, image_stride)[0]) <= MAX_DIMS
+
+
 class ItemTable:
     """Column-wise builder of an ``mlf_item`` array.
 
@@ -79,13 +102,18 @@ class ItemTable:
         stride: Sequence[int],
         image_stride: Optional[Sequence[int]] = None,
     ) -> None:
-        if len(shape) > MAX_DIMS:
-            raise NotImplementedError(f"tensors of rank > {MAX_DIMS} that are not contiguous are not supported")
         numel = 1
         for s in shape:
             numel *= s
         if image_stride is None:
             image_stride = _contiguous_strides(shape)
+        if len(shape) > MAX_DIMS:
+            # more dimensions than a table row holds: most such views are fewer once neighbours are merged; callers
+            # stage the rest through a contiguous copy (see ``describable``)
+            shape, stride, image_stride = collapse_dims(shape, stride, image_stride)
+            if len(shape) > MAX_DIMS:
+                raise ValueError(f"a strided item of {len(shape)} dimensions after merging does not fit the descriptor "
+                                 f"table's {MAX_DIMS}; stage it through a contiguous copy")
         self._strided.append((len(self.ptr), tuple(shape), tuple(stride), tuple(image_stride)))
         self.add_contiguous(ptr, image_off, elem_size, numel * elem_size)
 

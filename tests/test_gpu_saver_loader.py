@@ -633,8 +633,8 @@ def test_image_is_held_in_pieces_when_no_single_block_is_to_be_had(shm_dir, mana
 def test_restore_larger_than_the_hbm_limit_goes_window_by_window(shm_dir, manager_future, load_file_io):
     """With ``max_image_bytes`` far below the object size the loader uploads and unpacks windows of rows through
     one small device buffer (contiguous rows larger than a window are cut); the restored bits are the same, the
-    CRC sidecar is still honoured (windows start on checksum chunks and the unpack kernel checks what it scatters),
-    and a strided read that cannot be cut says so."""
+    CRC sidecar is still honoured (windows start on checksum chunks and are checked before they are unpacked), and a
+    strided target that spans more than a window is restored through boxes that fit."""
     from ml_flashpoint.hip import integrity
 
     sd_cpu = dict(_mixed_state_dict())
@@ -672,11 +672,13 @@ def test_restore_larger_than_the_hbm_limit_goes_window_by_window(shm_dir, manage
     roomy = _loader(max_image_bytes=700 << 10, use_file_io=load_file_io)
     dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, roomy), no_dist=True)
     assert roomy.last_load_stats["windows"] >= 2 and torch.equal(target["wide"].cpu(), sd_cpu["wide"])
-    # ... one that is larger than a window is refused, not mangled
-    with pytest.raises(BaseException) as exc:
-        dcp.load(targets(transposed_wide=True), checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), no_dist=True)
-    cause = exc.value.failures[0][0] if hasattr(exc.value, "failures") else exc.value
-    assert isinstance(cause, NotImplementedError) and "does not fit the HBM limit" in str(cause)
+    # ... one that is larger than a window is cut into boxes that fit, as torch's ``copy_`` would take any target
+    target = targets(transposed_wide=True)
+    dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), no_dist=True)
+    assert loader.last_load_stats["windows"] >= 5 and torch.equal(target["wide"].cpu(), sd_cpu["wide"])
+    for k, v in sd_cpu.items():
+        if isinstance(v, torch.Tensor):
+            assert torch.equal(_bits(target[k]), _bits(v)), k
 
     obj = os.path.join(ckpt, "__0__0_src0.distcp")
     assert loader.last_load_stats.get("crc_s", 0.0) >= 0.0
@@ -1288,3 +1290,41 @@ def test_mx_quantized_weights_round_trip(shm_dir, manager_future):
     for k, v in sd_cpu.items():
         if isinstance(v, torch.Tensor):
             assert target[k].dtype == v.dtype and torch.equal(target[k].cpu().view(torch.uint8), v.view(torch.uint8)), k
+
+
+def test_views_of_more_dimensions_than_a_descriptor_holds(shm_dir, manager_future):
+    """Sources and targets of rank 9 that are not contiguous: a permutation that merges into fewer dimensions goes
+    through the kernels as it is, one that does not is staged through a contiguous copy on the device (the saver) or
+    restored into a contiguous stand-in and scattered by ``copy_`` (the loader) - as the reference's ``copy_`` takes
+    any view (checkpoint_saver.py:797-800, checkpoint_loader.py:331-336).  Bytes against the oracle's index walk."""
+    g = torch.Generator().manual_seed(21)
+    base = torch.randint(-(2**15), 2**15, (2, 3, 2, 2, 3, 2, 2, 3, 2), dtype=torch.int16, generator=g)
+    scattered = base.permute(8, 7, 6, 5, 4, 3, 2, 1, 0)       # nine dimensions, none of which merge
+    mergeable = base.permute(0, 1, 2, 3, 4, 5, 6, 8, 7)       # the first seven merge into one
+    wide = torch.randint(0, 255, (2, 2, 2, 2, 2, 2, 2, 2, 2, 2, 3), dtype=torch.uint8, generator=g)[..., ::2]  # rank 11
+    sd_cpu = {"scattered": scattered, "mergeable": mergeable, "wide": wide, "plain": torch.arange(10.0)}
+    sd_dev = _to_dev(sd_cpu)
+    assert not sd_dev["scattered"].is_contiguous() and sd_dev["scattered"].dim() == 9
+    ckpt = os.path.join(shm_dir, "step-3_ckpt")
+    saver = _saver()
+    for _ in range(2):  # the second save rebuilds the plan of an object that holds a staged copy
+        dcp.save(sd_dev, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(saver, manager_future), no_dist=True)
+    raw = open(os.path.join(ckpt, "__0__0_src0.distcp"), "rb").read()
+    metadata = pickle.load(open(os.path.join(ckpt, ".metadata"), "rb"))
+    for index, where in metadata.storage_data.items():
+        want = fmt.payload_bytes_bruteforce(sd_cpu[index.fqn])
+        got = raw[METADATA_SIZE + where.offset + where.length - len(want) : METADATA_SIZE + where.offset + where.length]
+        assert got == want, index.fqn
+    image, _, _ = _expected_file(sd_cpu, metadata, raw)
+    assert raw == image
+    # back into views of the same kinds (over zeroed storage), and into plain tensors
+    zero = torch.zeros(base.shape, dtype=torch.int16, device=DEV)
+    wide_zero = torch.zeros(wide.shape[:-1] + (3,), dtype=torch.uint8, device=DEV)
+    target = {"scattered": zero.permute(8, 7, 6, 5, 4, 3, 2, 1, 0),
+              "mergeable": torch.zeros(base.shape, dtype=torch.int16, device=DEV).permute(0, 1, 2, 3, 4, 5, 6, 8, 7),
+              "wide": wide_zero[..., ::2], "plain": torch.zeros(10, device=DEV)}
+    dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, _loader()), no_dist=True)
+    for k, v in sd_cpu.items():
+        assert torch.equal(target[k].cpu(), v), k
+    assert torch.equal(zero.cpu(), base), "the scatter went through the view into its storage"
+    assert not bool(wide_zero[..., 1].any()), "the columns the view skips stay untouched"

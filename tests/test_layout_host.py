@@ -160,5 +160,73 @@ def test_device_rows_carry_address_and_strides_and_headers_stay_in_the_blob():
 def test_rank_limit_of_strided_rows():
     nine = torch.zeros((2,) * 9)
     P.build_save_layout([_FakeDeviceTensor(nine, 4096)])                    # contiguous: a run of bytes, any rank
-    with pytest.raises(NotImplementedError, match="rank > 8"):
-        P.build_save_layout([_FakeDeviceTensor(nine.transpose(0, 8), 4096)])
+    # a view whose neighbouring dimensions merge fits a descriptor whatever its rank ...
+    layout = P.build_save_layout([_FakeDeviceTensor(nine.transpose(7, 8), 4096)])
+    row = layout.items[-1]
+    assert int(row["ndim"]) == 3 and row["shape"][:3].tolist() == [128, 2, 2] and row["stride"][:3].tolist() == [4, 1, 2]
+    # ... one that stays above eight dimensions is for the caller to stage through a contiguous copy
+    assert P.describable(tuple(nine.transpose(7, 8).shape), tuple(nine.transpose(7, 8).stride()))
+    reversed_dims = nine.permute(*range(8, -1, -1))
+    assert not P.describable(tuple(reversed_dims.shape), tuple(reversed_dims.stride()))
+    with pytest.raises(ValueError, match="contiguous copy"):
+        P.build_save_layout([_FakeDeviceTensor(reversed_dims, 4096)])
+
+
+@settings(max_examples=60, deadline=None)
+@given(st.data())
+def test_merged_dimensions_address_the_same_elements(data):
+    """``collapse_dims``: the merged description visits the same (tensor element, image element) pairs in the same
+    order as the original one."""
+    ndim = data.draw(st.integers(1, 10))
+    shape = tuple(data.draw(st.integers(1, 3)) for _ in range(ndim))
+    parent = torch.zeros(tuple(n + data.draw(st.integers(0, 1)) for n in shape))
+    view = parent[tuple(slice(0, n) for n in shape)].permute(*data.draw(st.permutations(range(ndim))))
+    shape, stride = tuple(view.shape), tuple(view.stride())
+    image = tuple(P._contiguous_strides(shape))
+    if data.draw(st.booleans()):  # the stored side of a sub-box read: strides of a larger C-contiguous tensor
+        image = tuple(P._contiguous_strides(tuple(n + 1 for n in shape)))
+
+    def pairs(shape, stride, image):
+        out = []
+        for idx in np.ndindex(*shape) if shape else [()]:
+            out.append((sum(i * s for i, s in zip(idx, stride)), sum(i * s for i, s in zip(idx, image))))
+        return out
+
+    merged = P.collapse_dims(shape, stride, image)
+    assert len(merged[0]) <= len(shape) and all(n > 1 for n in merged[0])
+    assert pairs(*merged) == pairs(shape, stride, image)
+
+
+@settings(max_examples=60, deadline=None)
+@given(st.data())
+def test_oversize_strided_rows_are_cut_into_boxes_that_cover_them_exactly(data):
+    """The loader's ``_cut_box``: every piece spans at most the given number of image bytes, and together the pieces
+    map exactly the original row's image bytes to the original target addresses."""
+    from ml_flashpoint.hip.checkpoint_loader import HipMLFlashpointCheckpointLoader as Loader
+
+    ndim = data.draw(st.integers(1, 4))
+    shape = tuple(data.draw(st.integers(1, 5)) for _ in range(ndim))
+    esz = data.draw(st.sampled_from([1, 2, 4]))
+    target = torch.zeros(tuple(n + 1 for n in shape)).permute(*data.draw(st.permutations(range(ndim))))
+    strides = tuple(target.stride())[:ndim]
+    stored = tuple(P._contiguous_strides(tuple(n + data.draw(st.integers(0, 2)) for n in shape)))
+    image_strides = data.draw(st.sampled_from([None, stored]))
+    first, ptr = data.draw(st.integers(0, 1000)), 1 << 20
+    usable = data.draw(st.integers(esz, 64 * esz))
+
+    def mapping(row):
+        begin, end, contiguous, (p, e, shp, st_t, st_i) = row
+        st_i = st_i if st_i is not None else tuple(P._contiguous_strides(shp))
+        assert not contiguous and end - begin == (sum((n - 1) * s for n, s in zip(shp, st_i)) + 1) * e
+        return {begin + sum(i * s for i, s in zip(idx, st_i)) * e: p + sum(i * s for i, s in zip(idx, st_t)) * e
+                for idx in np.ndindex(*shp)}
+
+    whole = mapping(Loader._cut_box(first, (ptr, esz, shape, strides, image_strides), 1 << 40)[0])
+    pieces = Loader._cut_box(first, (ptr, esz, shape, strides, image_strides), usable)
+    got = {}
+    for piece in pieces:
+        assert piece[1] - piece[0] <= usable
+        part = mapping(piece)
+        assert not set(part) & set(got)
+        got.update(part)
+    assert got == whole
