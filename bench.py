@@ -64,8 +64,9 @@ def parse_args():
                          "the restore (0 = off)")
     ap.add_argument("--save-crc", choices=["beside", "fused"], default="beside",
                     help="where the save's checksums are computed: a pass of its own beside the transfer, or inside the pack kernel")
-    ap.add_argument("--restore-crc", choices=["fused", "before"], default="fused",
-                    help="how the restore verifies them: inside the unpack kernel, or a pass of its own before it")
+    ap.add_argument("--restore-crc", choices=["fused", "before"], default="before",
+                    help="how the restore verifies them: a pass over every uploaded window before it is unpacked (the "
+                         "loader's default), or inside the unpack kernel")
     ap.add_argument("--cpu-baseline-gb", type=float, default=12.0, help="size of the CPU baseline's sample (0 = skip)")
     ap.add_argument("--plan-cache", action="store_true",
                     help="reuse the save plan across steps once two consecutive plans compared equal, as the reference's "
@@ -85,10 +86,14 @@ def parse_args():
                     help="restore through one device buffer for the whole object instead of two alternating ones")
     ap.add_argument("--no-prefault", action="store_true", help="leave the pool file's pages to the first save, as the reference does")
     ap.add_argument("--no-link-probe", action="store_true", help="skip the bare host-link and device-copy measurements")
-    ap.add_argument("--busy-gpu-probe", action="store_true",
-                    help="also time a save whose transfer runs on a background thread while bf16 GEMMs, then HBM copies, "
-                         "keep the device busy: what the transfer costs them, and what they cost the transfer")
+    ap.add_argument("--no-busy-gpu-probe", action="store_true",
+                    help="skip the save whose transfer runs on a background thread while bf16 GEMMs, then HBM copies, keep "
+                         "the device busy (what the transfer costs them, and what they cost the transfer)")
     ap.add_argument("--no-crc-compare", action="store_true", help="skip the extra saves in the other checksum mode")
+    ap.add_argument("--no-plan-cache-compare", action="store_true", help="skip the extra saves on a reused DCP plan")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="the default run (llama3-8b-shard at full scale) also measures the many-small and strided-views "
+                         "configurations, one warm-up and three timed steps each, and reports them under other_workloads")
     ap.add_argument("--root", default=None, help="directory on tmpfs for the pool and checkpoints")
     return ap.parse_args()
 
@@ -122,8 +127,9 @@ def build_workload(name, device, scale):
     return sd, label, parents
 
 
-def cpu_baseline(sd, sample_bytes, root, device):
-    """The reference's CPU path, restated by the oracle, on a prefix of the state dict of about ``sample_bytes``."""
+def cpu_baseline(sd, sample_bytes, root, device, passes=5):
+    """The reference's CPU path, restated by the oracle, on a prefix of the state dict of about ``sample_bytes``
+    (the whole of it when that is larger)."""
     import torch
 
     from ml_flashpoint.core.checkpoint_id_types import CheckpointContainerId
@@ -142,7 +148,6 @@ def cpu_baseline(sd, sample_bytes, root, device):
     path = os.path.join(cid.data, "sample.distcp")
     tensors = list(sample.values())
     times = {"stage": [], "write": [], "restore": []}
-    passes = 5
     for rep in range(1 + passes):  # the first pass faults the tmpfs pages in, like the GPU path's prime iteration
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -193,8 +198,12 @@ def cpu_baseline(sd, sample_bytes, root, device):
         "unit": "GB/s",
         "cores": threads,
         "kind": "port",
-        "sample": f"first {len(sample)} tensors ({gb:.2f} GB) of the same state dict; one warm-up pass, then the median of {passes} "
-                  "(warm tmpfs pages)",
+        "sample": (f"all {len(sample)} tensors" if len(sample) == len(sd) else f"first {len(sample)} tensors") +
+                  f" ({gb:.2f} GB) of the same state dict; one warm-up pass, then the median of {passes} (warm tmpfs pages)",
+        "tensors": len(sample),
+        # the reference's per-tensor loops: stage (.to("cpu")), write (header + copy_ into the mapping), restore
+        "us_per_tensor": {"stage": round(stage * 1e6 / len(sample), 1), "write": round(write * 1e6 / len(sample), 1),
+                          "restore": round(restore * 1e6 / len(sample), 1)},
         "passes": passes,
         "spread": {k: [round(min(v), 3), round(max(v), 3)] for k, v in times.items()},
         "save_GBps": round(gb / (stage + write), 3),
@@ -362,7 +371,34 @@ def main():
         print("bench.py measures one GPU's share of the save/restore path; runs with --gpus > 1 are not part of this "
               "build (each rank would run this same pipeline independently on its own shard).", file=sys.stderr)
         sys.exit(2)
+    result = run_workload(args)
+    if args.workload == "llama3-8b-shard" and args.scale >= 1.0 and args.max_image_gb <= 0 and not args.no_other_workloads:
+        # the configurations whose cost is not in the bytes: 20 000 small tensors (host time per tensor) and 2 000
+        # non-contiguous views (gather / transpose / scatter kernels); same pipeline, fewer steps, no side probes
+        keep = ("save_GBps", "restore_GBps", "blocking_save_ms", "blocking_breakdown_ms", "blocking_host_us_per_tensor",
+                "save_tail_ms", "pack_GBps", "unpack_GBps", "unpack_GBps_beside_h2d", "d2h_GBps", "h2d_GBps",
+                "restore_breakdown_ms", "with_dcp_plan_cache", "cpu_baseline", "parity", "ms_per_step", "value")
+        others = {}
+        for name in ("many-small", "strided-views"):
+            sub = argparse.Namespace(**vars(args))
+            sub.workload, sub.steps, sub.warmup = name, 3, 1
+            sub.no_link_probe = sub.no_crc_compare = sub.no_busy_gpu_probe = True
+            sub.partial_restore_prefix, sub.pmc_calibration = None, False
+            sub.no_plan_cache_compare = name != "many-small"  # where the DCP planner is most of the blocking time
+            sub.cpu_baseline_gb = 1e3 if name == "many-small" and args.cpu_baseline_gb > 0 else 0.0  # the whole dict
+            sub.cpu_baseline_passes = 3
+            full = run_workload(sub)
+            others[name] = {"workload": full["config"]["workload"], "tensors": full["config"]["tensors"],
+                            "payload_bytes": full["config"]["payload_bytes"], "steps": sub.steps, "warmup": sub.warmup,
+                            **{k: full[k] for k in keep if k in full},
+                            "pack_frac_of_hbm_peak": full["roofline"]["frac"], "pack_ms": full["roofline"]["avg_launch_ms"]}
+        result["other_workloads"] = others
+    print(json.dumps(result), flush=True)
 
+
+def run_workload(args):
+    """Builds the workload, runs the prime, warm-up and timed steps and the side measurements the arguments ask for,
+    gives the device memory back and returns the result line as a dict."""
     import torch
     import torch.distributed.checkpoint as dcp
     from torch.distributed.checkpoint import DefaultSavePlanner
@@ -473,7 +509,7 @@ def main():
         stats = dict(the_saver.last_save_stats)
         del buckets, staged, results
         return {"save": t_saved - t0, "blocking": t_block - t0, "plan": t_launch - prepare_s - t0, "pack_launch": prepare_s,
-                "tail": t_saved - t_written, "stats": stats,
+                "tail": t_saved - t_written, "write": t_written - t_block, "stats": stats,
                 "pack_ms": sum(b.elapsed_time(e) for b, e, _ in the_saver.kernel_events),
                 "pack_bytes": sum(n for _, _, n in the_saver.kernel_events)}
 
@@ -596,20 +632,36 @@ def main():
             other.release_device_memory()
         # ---- the same save once the plan of the previous one is reused (the reference's cached_ckpt_structure) ----
         with_cache = None
-        if not args.plan_cache and not args.no_crc_compare and max_image is None:
+        if not args.plan_cache and not args.no_plan_cache_compare and max_image is None:
             state["use_cache"], runs = True, []
             for k in range(3):  # the first compares its plan with the last one's, the next ones skip the planning
                 manager.delete_container(prev)
                 prev = CheckpointContainerId(os.path.join(root, "run", f"step-{2000 + k}_ckpt"))
                 runs.append(one_save(saver, prev))
             state["use_cache"] = False
-            with_cache = {"blocking_save_ms": round(runs[-1]["blocking"] * 1e3, 2), "dcp_plan_ms": round(runs[-1]["plan"] * 1e3, 2),
-                          "save_s": round(runs[-1]["save"], 4)}
+            last, st = runs[-1], runs[-1]["stats"]
+            part = lambda key: round(st.get(key, 0.0) * 1e3, 2)  # noqa: E731
+            with_cache = {"blocking_save_ms": round(last["blocking"] * 1e3, 2), "dcp_plan_ms": round(last["plan"] * 1e3, 2),
+                          "save_s": round(last["save"], 4),
+                          # where the save's time goes: the blocking part (plan, layout + pack launch, the wait for the
+                          # pack), then write_data (buffer acquired and sized, the transfer, close + truncate, the
+                          # checksum sidecar, one WriteResult per item; the rest is the writer's own bookkeeping and
+                          # the prediction of the results for the early metadata), then the tail (finish_write,
+                          # finalize)
+                          "save_breakdown_ms": {
+                              "dcp_plan": round(last["plan"] * 1e3, 2), "layout_and_pack_launch": round(last["pack_launch"] * 1e3, 2),
+                              "wait_for_pack": round((last["blocking"] - last["plan"] - last["pack_launch"]) * 1e3, 2),
+                              "write_data": round(last["write"] * 1e3, 2), "of_write_acquire_buffer": part("acquire_s"),
+                              "of_write_transfer": part("d2h_s"), "of_write_close_buffer": part("close_s"),
+                              "of_write_sidecar": part("sidecar_s"), "of_write_results": part("results_s"),
+                              "of_write_other": round((last["write"] - sum(st.get(k, 0.0) for k in (
+                                  "acquire_s", "d2h_s", "close_s", "sidecar_s", "results_s"))) * 1e3, 2),
+                              "tail_finish_and_finalize": round(last["tail"] * 1e3, 2)}}
         manager.delete_container(prev)
 
         # ---- a save whose transfer runs on a thread while the device is kept busy, as by a training step ----
         busy = None
-        if args.busy_gpu_probe and max_image is None:
+        if not args.no_busy_gpu_probe and max_image is None:
             busy = _busy_gpu_probe(device, make_saver(args.save_crc, background_write=True), sd, root, manager)
 
         # ---- the host link by itself: device <-> the engine's pinned slots, nothing behind them ----
@@ -628,9 +680,12 @@ def main():
                 up.append(engine.link_probe(scratch.data_ptr(), probe_bytes, False))
             down, up = min(down), min(up)
             del scratch
-            link = {"d2h_peak_GBps": round(probe_bytes / 1e9 / down, 2), "h2d_peak_GBps": round(probe_bytes / 1e9 / up, 2),
+            link = {"d2h_probe_GBps": round(probe_bytes / 1e9 / down, 2), "h2d_probe_GBps": round(probe_bytes / 1e9 / up, 2),
+                    "pcie_gen5_x16_GBps": 64.0,
                     "bytes": probe_bytes, "slot_mib": args.slot_mib, "streams": 2,
-                    "what": "pinned hipMemcpyAsync between HBM and the copy engine's own slots, no host-side copy"}
+                    "what": "probe: pinned hipMemcpyAsync between HBM and the copy engine's own slots, no host-side copy, "
+                            "best of three per direction - a measurement of the link on this box in this run, not a "
+                            "ceiling (a transfer can come out a little above it); 64 GB/s is the link's nominal rate"}
 
         # ---- the device's own copy rate, beside which the pack's figure is to be read ----
         copy_probe = None
@@ -643,8 +698,10 @@ def main():
         pack_gbps = algorithmic / 1e9 / pack_s if pack_s > 0 else 0.0
         save_gbps, restore_gbps = gb / mean(rec["save"]), gb / mean(rec["restore"])
         if link:
-            link["save_frac"] = round(save_gbps / link["d2h_peak_GBps"], 4)
-            link["restore_frac"] = round(restore_gbps / link["h2d_peak_GBps"], 4)
+            link["save_frac_of_probe"] = round(save_gbps / link["d2h_probe_GBps"], 4)
+            link["restore_frac_of_probe"] = round(restore_gbps / link["h2d_probe_GBps"], 4)
+            link["save_frac_of_pcie"] = round(save_gbps / link["pcie_gen5_x16_GBps"], 4)
+            link["restore_frac_of_pcie"] = round(restore_gbps / link["pcie_gen5_x16_GBps"], 4)
         ratio = PACK_TRAFFIC_RATIO.get((args.workload, args.save_crc)) if args.scale >= 1.0 and max_image is None else None
         ms = lambda key: round(mean(rec[key]) * 1e3, 2)  # noqa: E731
         restore_known = sum(mean(rec[k]) for k in ("r_parse", "r_table", "h2d", "r_crc", "r_unpack_plan", "r_unpack", "r_commit"))
@@ -667,6 +724,7 @@ def main():
                        "crc_chunk_mib": args.crc_chunk_mib, "save_crc": args.save_crc, "restore_crc": args.restore_crc,
                        "plan_cache": args.plan_cache, "save_io": args.save_io, "restore_io": args.restore_io,
                        "max_image_gb": args.max_image_gb, "pool_prefault": not args.no_prefault,
+                       "busy_gpu_probe": not args.no_busy_gpu_probe,
                        "restore": "one image" if args.whole_image_restore else "two alternating buffers"},
             **({"partial_restore": partial} if partial else {}),
             "save_GBps": round(save_gbps, 3),
@@ -721,7 +779,8 @@ def main():
                          "avg_launch_ms": round(pack_s * 1e3, 3)},
         }
         if args.cpu_baseline_gb > 0:
-            result["cpu_baseline"] = cpu_baseline(sd, args.cpu_baseline_gb * 1e9, root, device)
+            result["cpu_baseline"] = cpu_baseline(sd, args.cpu_baseline_gb * 1e9, root, device,
+                                                  passes=getattr(args, "cpu_baseline_passes", 5))
     finally:
         try:
             manager.teardown_pool()
@@ -729,7 +788,20 @@ def main():
             pass
         mgr.shutdown()
         shutil.rmtree(root, ignore_errors=True)
-    print(json.dumps(result), flush=True)
+        # the next workload of this process starts from an empty device
+        try:
+            saver.release_device_memory()
+            loader_engine = getattr(loader, "_engine", None)
+            if loader_engine is not None:
+                loader_engine.destroy()
+                loader._engine = None
+        except Exception:
+            pass
+        sd.clear()
+        del parents
+        gc.collect()
+        torch.cuda.empty_cache()
+    return result
 
 
 if __name__ == "__main__":

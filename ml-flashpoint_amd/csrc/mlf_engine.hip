@@ -169,23 +169,25 @@ __global__ void mlf_queue_test_touch(uint32_t* out) {
   if (threadIdx.x == 0) *out = 1u;
 }
 
-// Whether work on `s` waits for work enqueued earlier on `busy`: both idle, a 2 ms kernel on `busy`, an empty kernel
-// on `s`.  On a hardware queue of its own the empty kernel is done while the 2 ms kernel is still running; behind that
-// kernel it is done after it, and `busy` is idle by then.  Decided by that order, not by a clock: a host thread that
-// loses the processor between the two calls can only make an independent stream look dependent, which costs a
-// replacement stream and nothing else.
-int waits_behind(hipStream_t s, hipStream_t busy, uint32_t* d_flags, bool* shared) {
+// Whether work on `s` waits for work enqueued earlier on `busy`: both idle, an event, a 2 ms kernel and another event
+// on `busy`, an empty kernel and an event on `s`.  On a hardware queue of its own the empty kernel is done long before
+// the 2 ms kernel, behind that kernel it is done after it.  Decided by the device's own time stamps of the three
+// events - the empty kernel's completion lies before or after the long kernel's - not by a host clock or a constant.
+int waits_behind(hipStream_t s, hipStream_t busy, uint32_t* d_flags, hipEvent_t* ev, bool* shared) {
   HIP_TRY(hipStreamSynchronize(busy));
   HIP_TRY(hipStreamSynchronize(s));
+  HIP_TRY(hipEventRecord(ev[0], busy));
   hipLaunchKernelGGL(mlf_queue_test_hold, dim3(1), dim3(64), 0, busy, 200000ull, d_flags);
+  HIP_TRY(hipEventRecord(ev[1], busy));
   hipLaunchKernelGGL(mlf_queue_test_touch, dim3(1), dim3(64), 0, s, d_flags + 16);
+  HIP_TRY(hipEventRecord(ev[2], s));
   HIP_TRY(hipGetLastError());
-  HIP_TRY(hipStreamSynchronize(s));
-  const hipError_t other = hipStreamQuery(busy);
-  if (other != hipSuccess && other != hipErrorNotReady) HIP_TRY(other);
-  (void)hipGetLastError();  // "not ready" is an answer, not a failure to report later
-  *shared = other == hipSuccess;
-  HIP_TRY(hipStreamSynchronize(busy));
+  HIP_TRY(hipEventSynchronize(ev[2]));
+  HIP_TRY(hipEventSynchronize(ev[1]));
+  float held_ms = 0.0f, touched_ms = 0.0f;
+  HIP_TRY(hipEventElapsedTime(&held_ms, ev[0], ev[1]));
+  HIP_TRY(hipEventElapsedTime(&touched_ms, ev[0], ev[2]));
+  *shared = touched_ms >= held_ms;
   return MLF_HIP_OK;
 }
 
@@ -471,14 +473,22 @@ int mlf_engine_avoid_streams(mlf_engine* e, void* const* busy_streams, uint32_t 
   std::lock_guard<std::mutex> g(e->busy);
   HIP_TRY(hipSetDevice(e->device));
   // shares a queue with any of the busy streams?
+  hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
   auto shares_hardware_queue = [&](hipStream_t s, uint32_t* flags, bool* shared) -> int {
     *shared = false;
     for (uint32_t k = 0; k < n_busy && !*shared; ++k)
-      if (int err = waits_behind(s, static_cast<hipStream_t>(busy_streams[k]), flags, shared)) return err;
+      if (int err = waits_behind(s, static_cast<hipStream_t>(busy_streams[k]), flags, ev, shared)) return err;
     return MLF_HIP_OK;
   };
   uint32_t* d_flags = nullptr;
   HIP_TRY(hipMalloc(reinterpret_cast<void**>(&d_flags), 128));
+  for (hipEvent_t& e1 : ev)
+    if (hipEventCreate(&e1) != hipSuccess) {  // (timing enabled: their time stamps are what is compared)
+      for (hipEvent_t e2 : ev)
+        if (e2) (void)hipEventDestroy(e2);
+      (void)hipFree(d_flags);
+      return fail(MLF_HIP_RUNTIME, "hipEventCreate failed");
+    }
   std::vector<hipStream_t> rejected;  // candidates that were no better; kept until the end: a destroyed stream's
                                       // queue would be handed out again
   uint32_t left = 0;
@@ -510,6 +520,7 @@ int mlf_engine_avoid_streams(mlf_engine* e, void* const* busy_streams, uint32_t 
     left += shared ? 1u : 0u;
   }
   for (hipStream_t s : rejected) (void)hipStreamDestroy(s);
+  for (hipEvent_t e1 : ev) (void)hipEventDestroy(e1);
   (void)hipFree(d_flags);
   if (rc == MLF_HIP_OK && still_shared) *still_shared = left;
   return rc;

@@ -238,6 +238,40 @@ class StagedTensorRef:
         return torch.empty((), dtype=self.dtype).element_size()
 
 
+_MARKER_PREFIX, _MARKER_SUFFIXES = "mlf_write_", (".done", ".done.tmp")
+
+
+def _sweep_stale_markers() -> int:
+    """Removes the result markers (``mlf_write_<pid>_<id>.done`` in the temporary directory) of writer processes that
+    no longer exist: a writer that crashed between writing its marker and its waiter reading it leaves the file
+    behind, and nothing else would ever take it away.  Markers of live processes are left alone, whoever they
+    belong to.  Returns the number of files removed."""
+    removed = 0
+    try:
+        names = os.listdir(tempfile.gettempdir())
+    except OSError:
+        return 0
+    for name in names:
+        if not (name.startswith(_MARKER_PREFIX) and name.endswith(_MARKER_SUFFIXES)):
+            continue
+        pid = name[len(_MARKER_PREFIX):].split("_", 1)[0]
+        if not pid.isdigit() or int(pid) == os.getpid():
+            continue
+        try:
+            os.kill(int(pid), 0)  # signal 0: existence check only
+            continue
+        except ProcessLookupError:
+            pass
+        except OSError:  # it exists but is not ours to signal: not ours to clean up after either
+            continue
+        try:
+            os.remove(os.path.join(tempfile.gettempdir(), name))
+            removed += 1
+        except OSError:
+            pass
+    return removed
+
+
 class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
     def __init__(
         self,
@@ -286,6 +320,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         ``prepare_write_data`` instead, for training loops that update them before the transfer has ended).
         """
         _lib.load()  # fail now, loudly, if the native library is not there
+        _sweep_stale_markers()
         self._global_rank_getter = global_rank_getter
         self._local_rank_getter = local_rank_getter
         self._barrier_func = global_barrier_func
@@ -1052,6 +1087,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         layout = staged.layout
         nbytes = layout.data_bytes
         crcs = None
+        marks = [time.perf_counter()]  # -> buffer ready -> bytes in place -> buffer closed -> sidecar -> results
         with self._chkpt_obj_manager.acquire_buffer(
             bucket.object_id, max(self._initial_buffer_size_bytes, nbytes, 1)
         ) as writer:
@@ -1063,6 +1099,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                 reserve = getattr(writer, "reserve", None)
                 if reserve is not None:
                     reserve(nbytes)  # pages allocated ahead of the copy threads (first use of a buffer file only)
+                marks.append(time.perf_counter())
                 with torch.cuda.device(staged.device_index):
                     _lib.check(_lib.load().mlf_hip_set_device(staged.device_index), "mlf_hip_set_device")
                     start = writer.tell()
@@ -1099,6 +1136,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                                                     self._crc_chunk_bytes)
                         self._count_transfer(xfer, st, nbytes)
                     staged._landed.value = nbytes
+                marks.append(time.perf_counter())
             elif streaming is not None:  # an object without data: nothing to follow, but it is to be replicated
                 self._announce_transfer(streaming, bucket, staged, 0, 0, outcome)
         staged.consumed = True
@@ -1106,11 +1144,18 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         if staged.plan is not None and staged.owns_plan:
             staged.plan.destroy()
         staged.plan = None
+        marks.append(time.perf_counter())
         if crcs is not None:
             integrity.write_sidecar(str(bucket.object_id), self._crc_chunk_bytes, nbytes, crcs)
         else:
             integrity.remove_sidecar(str(bucket.object_id))
-        return self._results_of(staged, bucket.object_name)
+        marks.append(time.perf_counter())
+        results = self._results_of(staged, bucket.object_name)
+        marks.append(time.perf_counter())
+        if len(marks) == 6:  # host time of a write around the transfer itself, for whoever reads last_save_stats
+            for name, a, b in (("acquire_s", 0, 1), ("close_s", 2, 3), ("sidecar_s", 3, 4), ("results_s", 4, 5)):
+                xfer[name] = xfer.get(name, 0.0) + marks[b] - marks[a]
+        return results
 
     @staticmethod
     def _fused_checksums(staged: StagedObject):

@@ -158,23 +158,30 @@ def test_engines_keep_their_streams_off_the_hardware_queue_of_the_training_strea
             torch.cuda.synchronize()
 
     engines = [P.CopyEngine(slot_bytes=8 << 20, n_slots=3, n_threads=4) for _ in range(5)]
-    try:
-        idle = n / engines[0].link_probe(buf.data_ptr(), n, True)
-        left = [engine.avoid_stream(torch.cuda.current_stream().cuda_stream) for engine in engines]
-        assert left == [0] * len(engines)
+
+    def rates_beside_a_busy_default_stream():
+        stop.clear()
         worker = threading.Thread(target=busy)
         worker.start()
         try:
             time.sleep(0.1)
-            rates = [n / engine.link_probe(buf.data_ptr(), n, True) for engine in engines]
+            return [n / engine.link_probe(buf.data_ptr(), n, True) for engine in engines]
         finally:
             stop.set()
             worker.join()
-        # reported, not judged: what an engine moves beside a busy stream depends on the box; that no stream of any
-        # engine is left on the busy stream's hardware queue is what the call promises, and was asserted above
-        print(f"link rate idle {idle / 1e9:.1f} GB/s; beside a busy default stream: "
+
+    try:
+        idle = n / engines[0].link_probe(buf.data_ptr(), n, True)
+        before = rates_beside_a_busy_default_stream()
+        left = [engine.avoid_stream(torch.cuda.current_stream().cuda_stream) for engine in engines]
+        assert left == [0] * len(engines)
+        rates = rates_beside_a_busy_default_stream()
+        print(f"link rate idle {idle / 1e9:.1f} GB/s; beside a busy default stream, as created: "
+              + ", ".join(f"{r / 1e9:.1f}" for r in before) + " GB/s; after avoid_stream: "
               + ", ".join(f"{r / 1e9:.1f}" for r in rates) + " GB/s")
-        assert all(r > 0 for r in rates)
+        # One engine against the others in the same run, not against a figure: an engine with a stream left on the
+        # busy stream's hardware queue moves a quarter of what the others move (measured: 12.7 against 52-53 GB/s).
+        assert min(rates) > 0.5 * max(rates), (idle, before, rates)
         assert all(engine.checksum_stream for engine in engines)
     finally:
         for engine in engines:

@@ -289,3 +289,26 @@ def test_bench_refuses_more_than_one_gpu():
     done = subprocess.run([sys.executable, bench, "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert done.returncode == 2
     assert "one GPU" in done.stderr + done.stdout
+
+
+def test_result_markers_of_dead_writer_processes_are_swept(tmp_path, monkeypatch):
+    """A background writer hands its results to a waiter in another process through a marker file in the temporary
+    directory; a writer that died leaves it behind.  Markers whose process no longer exists go when a saver is
+    made; those of live processes stay."""
+    import os
+    import subprocess
+    import sys
+    import tempfile
+
+    from ml_flashpoint.hip import checkpoint_saver as hip_saver
+
+    monkeypatch.setattr(tempfile, "tempdir", str(tmp_path))
+    gone = subprocess.Popen([sys.executable, "-c", "pass"])
+    gone.wait()
+    dead = [tmp_path / f"mlf_write_{gone.pid}_abc.done", tmp_path / f"mlf_write_{gone.pid}_abc.done.tmp"]
+    alive = [tmp_path / f"mlf_write_{os.getpid()}_own.done", tmp_path / f"mlf_write_{os.getppid()}_parent.done",
+             tmp_path / "mlf_write_notapid_x.done", tmp_path / "unrelated.done"]
+    for path in dead + alive:
+        path.write_bytes(b"x")
+    assert hip_saver._sweep_stale_markers() == 2
+    assert not any(p.exists() for p in dead) and all(p.exists() for p in alive)
