@@ -41,7 +41,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, vendor figure
 PACK_TRAFFIC_RATIO = {
     ("llama3-8b-shard", "beside"): 1.0008,
     ("llama3-8b-shard", "fused"): 1.0158,
-    ("strided-views", "beside"): 1.253,
+    ("strided-views", "beside"): 1.214,
 }
 
 

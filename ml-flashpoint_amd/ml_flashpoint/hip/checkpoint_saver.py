@@ -913,7 +913,13 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
 
     @staticmethod
     def _results_of(staged: StagedObject, object_name: str) -> list[WriteResult]:
-        return [
+        """One WriteResult per item of the object, from its layout.  Made once per staged object: the prediction that
+        lets the metadata object be pickled early and the write itself ask for the same list (20 ms apiece at
+        20 000 items)."""
+        made = getattr(staged, "_results", None)
+        if made is not None and made[0] == object_name:
+            return made[1]
+        results = [
             WriteResult(
                 index=item.index,
                 size_in_bytes=length,
@@ -921,6 +927,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             )
             for item, (offset, length) in zip(staged.items, staged.layout.spans)
         ]
+        staged._results = (object_name, results)
+        return results
 
     # ---- write_data -----------------------------------------------------------------------------
     @override
