@@ -510,6 +510,8 @@ def run_workload(args):
         del buckets, staged, results
         return {"save": t_saved - t0, "blocking": t_block - t0, "plan": t_launch - prepare_s - t0, "pack_launch": prepare_s,
                 "tail": t_saved - t_written, "write": t_written - t_block, "stats": stats,
+                "metadata": ("previous bytes, storage_meta exchanged" if writer.early_metadata_respliced else
+                             "pickled beside the transfer" if writer.early_metadata_used else "pickled in finish_write"),
                 "pack_ms": sum(b.elapsed_time(e) for b, e, _ in the_saver.kernel_events),
                 "pack_bytes": sum(n for _, _, n in the_saver.kernel_events)}
 
@@ -634,7 +636,7 @@ def run_workload(args):
         with_cache = None
         if not args.plan_cache and not args.no_plan_cache_compare and max_image is None:
             state["use_cache"], runs = True, []
-            for k in range(3):  # the first compares its plan with the last one's, the next ones skip the planning
+            for k in range(4):  # the first compares its plan with the last one's, the next ones skip the planning
                 manager.delete_container(prev)
                 prev = CheckpointContainerId(os.path.join(root, "run", f"step-{2000 + k}_ckpt"))
                 runs.append(one_save(saver, prev))
@@ -642,7 +644,7 @@ def run_workload(args):
             last, st = runs[-1], runs[-1]["stats"]
             part = lambda key: round(st.get(key, 0.0) * 1e3, 2)  # noqa: E731
             with_cache = {"blocking_save_ms": round(last["blocking"] * 1e3, 2), "dcp_plan_ms": round(last["plan"] * 1e3, 2),
-                          "save_s": round(last["save"], 4),
+                          "save_s": round(last["save"], 4), "metadata_object": last["metadata"],
                           # where the save's time goes: the blocking part (plan, layout + pack launch, the wait for the
                           # pack), then write_data (buffer acquired and sized, the transfer, close + truncate, the
                           # checksum sidecar, one WriteResult per item; the rest is the writer's own bookkeeping and

@@ -101,6 +101,53 @@ class _WriteLedger:
         return self.events[checkpoint_id].wait(timeout=timeout_s)
 
 
+_STORAGE_META_KEY = b"\x8c\x0cstorage_meta"  # SHORT_BINUNICODE, length 12: the field's name as a key of the state dict
+
+
+def _last_frame(pickled: bytes) -> int | None:
+    """Offset of the FRAME opcode (protocol 4: 0x95 + eight bytes of length) that runs to the end of ``pickled``."""
+    at = len(pickled)
+    while True:
+        at = pickled.rfind(b"\x95", 0, at)
+        if at < 0:
+            return None
+        if at + 9 <= len(pickled) and int.from_bytes(pickled[at + 1 : at + 9], "little") == len(pickled) - at - 9:
+            return at
+
+
+def repickled_with_storage_meta(pickled: bytes, metadata: Metadata, old: StorageMeta, new: StorageMeta) -> bytes | None:
+    """``pickle.dumps`` of a metadata object that differs from the one ``pickled`` was made from in ``storage_meta``
+    only (``old`` there, ``new`` now) - without pickling its tens of thousands of entries again - or None where that
+    cannot be done safely.
+
+    A dataclass is pickled field by field in declaration order, and ``storage_meta`` comes after the two big
+    dictionaries, so everything up to its key is the same stream of opcodes for both objects.  What follows the key
+    is taken from the pickle of a stand-in with empty dictionaries, once with ``old`` and once with ``new``.  A tail
+    may only be moved from one pickle into another if it does not depend on how many objects were memoized before it
+    (back-references carry explicit memo numbers).  For ``old`` that is shown by the stand-in's tail being byte for
+    byte the tail of ``pickled``; for ``new`` by a second stand-in, with some hundred more memo entries in front,
+    giving the same tail.  Anything else - a tail that refers back into the dictionaries or to an object of its own,
+    another field order - ends in None, never in wrong bytes.  The length of the last frame is corrected."""
+    try:
+        stand_in = dataclasses.replace(metadata, state_dict_metadata={}, planner_data=None, storage_data={})
+        shifted = dataclasses.replace(stand_in, state_dict_metadata={f"k{i}": i for i in range(300)})
+        tail_old, tail_new, tail_new_shifted = (
+            pickle.dumps(dataclasses.replace(base, storage_meta=meta), protocol=pickle.DEFAULT_PROTOCOL)
+            for base, meta in ((stand_in, old), (stand_in, new), (shifted, new)))
+    except Exception:
+        return None
+    cut, cut_old, cut_new, cut_shifted = (b.rfind(_STORAGE_META_KEY) for b in (pickled, tail_old, tail_new, tail_new_shifted))
+    if min(cut, cut_old, cut_new, cut_shifted) < 0 or pickled[cut:] != tail_old[cut_old:] \
+            or tail_new[cut_new:] != tail_new_shifted[cut_shifted:]:
+        return None
+    frame = _last_frame(pickled)
+    if frame is None or frame + 9 > cut:
+        return None  # unframed, or the tail is spread over two frames
+    tail = tail_new[cut_new:]
+    length = len(pickled) - frame - 9 + len(tail) - (len(pickled) - cut)
+    return b"".join((pickled[:frame], b"\x95", length.to_bytes(8, "little"), pickled[frame + 9 : cut], tail))
+
+
 class _EarlyMetadata:
     """The checkpoint's metadata object pickled while its data is still on the way to the buffer.
 
@@ -109,19 +156,32 @@ class _EarlyMetadata:
     part of it is predicted from the layout; with several ranks the others' parts are taken to be what they were in
     the previous save (the same plan puts the same items at the same offsets of objects of the same names), which
     the rank that writes the metadata object saw when it finished that save.  ``finish_checkpoint`` uses the bytes
-    only if they describe exactly what all ranks then reported; otherwise it pickles again, as without this."""
+    only if they describe exactly what all ranks then reported; otherwise it pickles again, as without this.
 
-    def __init__(self, checkpoint_id, metadata: Metadata, where: dict, storage_meta):
+    ``before``: ``(metadata, where, storage_meta, bytes)`` of the last metadata object this process wrote.  When it
+    was the same metadata object with every item in the same place - the steady state of a run that keeps its DCP
+    plan - the new bytes are the old ones with the ``storage_meta`` part exchanged
+    (``repickled_with_storage_meta``), which takes a millisecond instead of the pickling."""
+
+    def __init__(self, checkpoint_id, metadata: Metadata, where: dict, storage_meta, before=None):
         self.checkpoint_id, self.metadata, self.where, self.storage_meta = checkpoint_id, metadata, where, storage_meta
         self.payload: bytes | None = None
+        self.respliced = False
+        self.predicted, self.others_as_before = None, False  # what `where` was made from (set by whoever made it)
+        self._before = before
         self._thread = threading.Thread(target=self._run, name="mlf-early-metadata", daemon=True)
         self._thread.start()
 
     def _run(self):
         try:
             with utils.gc_paused():
-                filled = dataclasses.replace(self.metadata, storage_data=self.where, storage_meta=self.storage_meta)
-                self.payload = pickle.dumps(filled)
+                before, self._before = self._before, None
+                if before is not None and before[0] is self.metadata and (before[1] is self.where or before[1] == self.where):
+                    self.payload = repickled_with_storage_meta(before[3], self.metadata, before[2], self.storage_meta)
+                    self.respliced = self.payload is not None
+                if self.payload is None:
+                    filled = dataclasses.replace(self.metadata, storage_data=self.where, storage_meta=self.storage_meta)
+                    self.payload = pickle.dumps(filled)
         except Exception:  # the ordinary path takes over
             _LOGGER.warning("could not pickle the metadata object ahead of time", exc_info=True)
 
@@ -155,6 +215,7 @@ class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
         self._others_as_before = False
         self._early_metadata: _EarlyMetadata | None = None
         self.early_metadata_used = False  # the last finish_checkpoint wrote bytes that were pickled ahead of time
+        self.early_metadata_respliced = False  # ... and those were the previous save's with storage_meta exchanged
 
     # the ledger's two dicts under the names other code (and the reference's tests) know them by
     @property
@@ -346,14 +407,26 @@ class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
         except Exception:
             _LOGGER.warning("could not predict the write results", exc_info=True)
             return
-        if predicted is not None:
+        if predicted is None:
+            return
+        others = None
+        if self._others_as_before:
+            others = getattr(self._checkpoint_saver, "last_write_locations", None)
+            if not others:
+                return  # nothing to go by yet
+        # (metadata, where, storage_meta, bytes, the predicted results and the other ranks' part that `where` was
+        # made from) of the last metadata object written: a saver that keeps its plans predicts the same result
+        # objects again, and then `where` need not be built anew either
+        before = getattr(self._checkpoint_saver, "last_metadata_pickle", None)
+        if before is not None and before[5] is others and len(before[4]) == len(predicted) \
+                and all(a is b for a, b in zip(before[4], predicted)):
+            where = before[1]
+        else:
             where = {result.index: result.storage_data for result in predicted}
-            if self._others_as_before:
-                before = getattr(self._checkpoint_saver, "last_write_locations", None)
-                if not before:
-                    return  # nothing to go by yet
-                where = {**before, **where}
-            self._early_metadata = _EarlyMetadata(checkpoint_id, metadata, where, self.storage_meta())
+            if others is not None:
+                where = {**others, **where}
+        self._early_metadata = _EarlyMetadata(checkpoint_id, metadata, where, self.storage_meta(), before)
+        self._early_metadata.predicted, self._early_metadata.others_as_before = predicted, others is not None
 
     @_timed(logger=_LOGGER, name="get_write_results")
     def get_write_results(
@@ -396,11 +469,19 @@ class MemoryStorageWriter(StorageWriter, staging.BlockingAsyncStager):
         ready = early.result_for(checkpoint_id, metadata, where, metadata.storage_meta) if early is not None else None
         write_bytes = getattr(self._checkpoint_saver, "write_metadata_bytes", None)
         self.early_metadata_used = ready is not None and write_bytes is not None
+        self.early_metadata_respliced = self.early_metadata_used and early.respliced
         if self.early_metadata_used:
             write_bytes(checkpoint_id, ready)  # pickled while the data was being written: same bytes, no wait
         else:
             self._checkpoint_saver.write_metadata(checkpoint_id, metadata)
         try:  # what the next save's prediction of the other ranks' results goes by (writers come and go, savers stay)
+            if self.early_metadata_used and hasattr(self._checkpoint_saver, "last_metadata_pickle"):
+                # the early bytes were right, so early.where says what `where` says: kept as the record of where
+                # everything went, it is also the very dict the next save's prediction starts from, and that save
+                # can tell by identity that nothing has moved
+                where = early.where
+                self._checkpoint_saver.last_metadata_pickle = (
+                    metadata, where, metadata.storage_meta, ready, early.predicted, where if early.others_as_before else None)
             self._checkpoint_saver.last_write_locations = where
         except AttributeError:
             pass

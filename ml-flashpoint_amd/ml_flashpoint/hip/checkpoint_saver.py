@@ -111,6 +111,9 @@ class _KeptPlan:
         # with checksums folded into the pack: the object of the last launch, until its values have been taken (a
         # plan holds the values of its last launch only)
         self.last_staged: Optional[weakref.ReferenceType] = None
+        # (object name, the save's items, their WriteResults): a save planned from a kept DCP plan brings the very
+        # same items again, and the layout is this one's, so the results are the same objects from save to save
+        self.results: Optional[tuple] = None
 
     def refreshed_blob(self, tensors, blobs) -> Optional[bytes]:
         """The blob with the current bytes of its variable parts, or None if nothing changed since last time."""
@@ -155,6 +158,8 @@ class StagedObject:
         # an image that is held in several device buffers: [(plan, buffer, first image byte, end)], in order
         self.pieces: Optional[list] = None
         self.fused_crcs = None  # chunk checksums out of the pack, once taken from the plan
+        self.kept: Optional[_KeptPlan] = None  # the kept plan this object was packed with, if any
+        self._results: Optional[tuple] = None  # (object name, WriteResults), once made
 
     def landed_bytes(self) -> int:
         """Leading bytes of the image that are in place in the buffer file (from byte 4096 + ``data_offset`` of the
@@ -363,12 +368,13 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         # save - what the next save's metadata object is pickled from while its data is still in flight.
         self.last_write_locations: Optional[dict] = None
         self.last_global_metadata = None
+        self.last_metadata_pickle = None  # (see MemoryStorageWriter: the bytes of the last metadata object written)
 
     # ---- pickling: only configuration crosses a process boundary --------------------------------------
     def __getstate__(self):
         state = self.__dict__.copy()
         for key in ("_replication_manager", "_engine", "_engine_clear_of", "_engine_lock", "last_save_stats", "kernel_events",
-                    "_plan_cache", "last_write_locations", "last_global_metadata"):
+                    "_plan_cache", "last_write_locations", "last_global_metadata", "last_metadata_pickle"):
             state.pop(key, None)
         return state
 
@@ -648,6 +654,9 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         staged = StagedObject(layout, plan, image, device.index or 0, stream, items)
         staged.packed_event = packed if layout.image_bytes else None
         staged.owns_plan = key is None  # with a key the plan went into, or came out of, the kept plans
+        staged.kept = self._plan_cache.get(object_name) if key is not None and plan is not None else None
+        if staged.kept is not None and staged.kept.plan is not plan:
+            staged.kept = None
         if plan is not None and plan.crc_chunk_bytes and key is not None:
             holder = self._plan_cache.get(object_name)
             if holder is not None and holder.plan is plan:
@@ -915,10 +924,17 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
     def _results_of(staged: StagedObject, object_name: str) -> list[WriteResult]:
         """One WriteResult per item of the object, from its layout.  Made once per staged object: the prediction that
         lets the metadata object be pickled early and the write itself ask for the same list (20 ms apiece at
-        20 000 items)."""
-        made = getattr(staged, "_results", None)
+        20 000 items) - and once per kept plan while the saves bring the same items (a kept DCP plan): callers get
+        the same list and the same result objects again and must not change them."""
+        made = staged._results
         if made is not None and made[0] == object_name:
             return made[1]
+        kept = staged.kept
+        before = kept.results if kept is not None else None
+        if before is not None and before[0] == object_name and len(before[1]) == len(staged.items) \
+                and all(a is b for a, b in zip(before[1], staged.items)):
+            staged._results = (object_name, before[2])
+            return before[2]
         results = [
             WriteResult(
                 index=item.index,
@@ -928,6 +944,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             for item, (offset, length) in zip(staged.items, staged.layout.spans)
         ]
         staged._results = (object_name, results)
+        if kept is not None:
+            kept.results = (object_name, list(staged.items), results)
         return results
 
     # ---- write_data -----------------------------------------------------------------------------
