@@ -267,7 +267,6 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                 raise ValueError(f"'{checkpoint_object_id.data}' is truncated: its metadata block records {recorded} "
                                  f"bytes of data, the file holds {held}")
             optimized = stream.format_signature == CheckpointFormat.MLF_FORMAT
-            device_reqs = []  # (req, target, dtype, shape, payload_off, stored payload bytes)
             whole = stream.raw_view()
             sidecar = integrity.read_sidecar(checkpoint_object_id.data) if self._verify_crc else None
             if sidecar is not None and sidecar[1] != recorded:
@@ -284,49 +283,112 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                 self._check_on_host(checkpoint_object_id, stream, sidecar, todo)
                 host_checked.update(todo)
 
-            t_parse = time.perf_counter()
-            for req in read_items:
-                item_md = storage_data[req.storage_index]
-                if req.type == LoadItemType.BYTE_IO:
-                    check_on_host_first(item_md.offset, item_md.length)
-                    view = cast(IO[bytes], _create_file_view(stream, item_md.offset, item_md.length))
-                    data = io.BytesIO(view.read(item_md.length))
-                    data.seek(0)
-                    planner.load_bytes(req, data)
-                    continue
-                target = planner.resolve_tensor(req).detach()
-                parsed = self._parse_header(whole, item_md.offset, item_md.length) if optimized else None
-                if parsed is not None and target.device.type == "cpu":
-                    # host-resident target: one copy, from a tensor laid over the record's payload in the mapping
-                    # into the target (the reference reads the record into a bytes object first,
-                    # checkpoint_loader.py:195-208)
-                    check_on_host_first(item_md.offset, item_md.length)
-                    tensor = self._payload_view(whole, recorded, checkpoint_object_id, req, *parsed)
-                    tensor = narrow_tensor_by_index(tensor, req.storage_offsets, req.lengths)
-                    assert target.size() == tensor.size(), (
-                        f"req {req.storage_index} mismatch sizes {target.size()} vs {tensor.size()}"
-                    )
-                    target.copy_(tensor)
-                    planner.commit_tensor(req, target)
-                    stats["host_items"] += 1
-                    continue
-                if parsed is None:
-                    check_on_host_first(item_md.offset, item_md.length)
-                    view = cast(IO[bytes], _create_file_view(stream, item_md.offset, item_md.length))
-                    tensor = self.read_tensor(view, req, use_optimized_loader=optimized)
-                    assert target.size() == tensor.size(), (
-                        f"req {req.storage_index} mismatch sizes {target.size()} vs {tensor.size()}"
-                    )
-                    target.copy_(tensor)
-                    planner.commit_tensor(req, target)
-                    stats["host_items"] += 1
-                    continue
-                device_reqs.append((req, target) + parsed)
-            stats["parse_s"] = time.perf_counter() - t_parse  # headers parsed, targets resolved, host items served
-            if device_reqs:
-                self._read_device_items(checkpoint_object_id, stream, device_reqs, planner, stats, sidecar)
+            early = self._start_early_upload(stream, read_items, planner, storage_data, recorded, sidecar, stats) \
+                if optimized else None
+            try:
+                self._serve_items(checkpoint_object_id, stream, read_items, planner, storage_data, optimized, whole,
+                                  recorded, sidecar, check_on_host_first, stats, early)
+            finally:
+                if early is not None:  # the file and its mapping are closed below: nothing may still be reading them
+                    concurrent.futures.wait([early[1]])
         stats["read_s"] = time.perf_counter() - t_start
         self.last_load_stats = stats
+
+    def _start_early_upload(self, stream, read_items, planner, storage_data, recorded: int, sidecar, stats):
+        """Where the records that are asked for lie in the object is known from the checkpoint's metadata, so when
+        they are going to be read through one device buffer in one piece - the whole data section if the object has
+        checksums - the upload can begin before the record headers are parsed and the targets resolved (5 us per
+        item on the host: 110 ms for 20 000 items, beside an upload of 150 ms).  Returns ``(buffer, future of the
+        upload, device, first byte, end)`` when the read is certain to be of that kind, else None."""
+        asked = {req.storage_index: storage_data[req.storage_index]
+                 for req in read_items if req.type != LoadItemType.BYTE_IO}
+        if not asked or recorded <= 0:
+            return None
+        if sidecar is not None:
+            lo, hi = 0, recorded  # checksums cover the whole data section
+        else:
+            lo = min(info.offset for info in asked.values()) // _UPLOAD_ALIGN * _UPLOAD_ALIGN
+            hi = min(max(info.offset + info.length for info in asked.values()), recorded)
+        span = hi - lo
+        if span <= 0 or (span >= _PIPELINED_FROM_BYTES and self._pipelined_restore):
+            return None
+        # a read that leaves out enough of the range to be worth several smaller uploads is decided on later
+        if span - sum(info.length for info in asked.values()) + 256 * len(asked) >= _PARTIAL_READ_MIN_SAVING:
+            return None
+        # the device the targets live on: the first few requests say (an object all of whose first targets are
+        # host-resident is taken to be one for the host)
+        device = None
+        for req in [req for req in read_items[:64] if req.type != LoadItemType.BYTE_IO][:8]:
+            device = planner.resolve_tensor(req).device
+            if device.type != "cpu":
+                break
+        if device is None or device.type == "cpu":
+            return None
+        with torch.cuda.device(device):
+            _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
+            self._keep_clear_of(device)
+            image = hip_plan.try_allocate(span, device) if span <= self._image_limit(device) else None
+            if image is None:
+                return None
+            cur = torch.cuda.current_stream(device)
+        done: concurrent.futures.Future = concurrent.futures.Future()
+
+        def run():
+            try:
+                self._upload(stream, lo, image, span, cur, stats)
+                done.set_result(None)
+            except BaseException as e:  # handed to whoever waits for the bytes
+                done.set_exception(e)
+
+        threading.Thread(target=run, name="mlf-early-upload", daemon=True).start()
+        stats["upload_began_before_parse"] = 1
+        return image, done, device, lo, hi
+
+    def _serve_items(self, checkpoint_object_id, stream, read_items, planner, storage_data, optimized, whole, recorded,
+                     sidecar, check_on_host_first, stats, early) -> None:
+        """Items for the host are served one by one; those for the device are collected and restored together."""
+        device_reqs = []  # (req, target, dtype, shape, payload_off, stored payload bytes)
+        t_parse = time.perf_counter()
+        for req in read_items:
+            item_md = storage_data[req.storage_index]
+            if req.type == LoadItemType.BYTE_IO:
+                check_on_host_first(item_md.offset, item_md.length)
+                view = cast(IO[bytes], _create_file_view(stream, item_md.offset, item_md.length))
+                data = io.BytesIO(view.read(item_md.length))
+                data.seek(0)
+                planner.load_bytes(req, data)
+                continue
+            target = planner.resolve_tensor(req).detach()
+            parsed = self._parse_header(whole, item_md.offset, item_md.length) if optimized else None
+            if parsed is not None and target.device.type == "cpu":
+                # host-resident target: one copy, from a tensor laid over the record's payload in the mapping
+                # into the target (the reference reads the record into a bytes object first,
+                # checkpoint_loader.py:195-208)
+                check_on_host_first(item_md.offset, item_md.length)
+                tensor = self._payload_view(whole, recorded, checkpoint_object_id, req, *parsed)
+                tensor = narrow_tensor_by_index(tensor, req.storage_offsets, req.lengths)
+                assert target.size() == tensor.size(), (
+                    f"req {req.storage_index} mismatch sizes {target.size()} vs {tensor.size()}"
+                )
+                target.copy_(tensor)
+                planner.commit_tensor(req, target)
+                stats["host_items"] += 1
+                continue
+            if parsed is None:
+                check_on_host_first(item_md.offset, item_md.length)
+                view = cast(IO[bytes], _create_file_view(stream, item_md.offset, item_md.length))
+                tensor = self.read_tensor(view, req, use_optimized_loader=optimized)
+                assert target.size() == tensor.size(), (
+                    f"req {req.storage_index} mismatch sizes {target.size()} vs {tensor.size()}"
+                )
+                target.copy_(tensor)
+                planner.commit_tensor(req, target)
+                stats["host_items"] += 1
+                continue
+            device_reqs.append((req, target) + parsed)
+        stats["parse_s"] = time.perf_counter() - t_parse  # headers parsed, targets resolved, host items served
+        if device_reqs:
+            self._read_device_items(checkpoint_object_id, stream, device_reqs, planner, stats, sidecar, early)
 
     def _image_limit(self, device: torch.device) -> int:
         """Bytes of HBM one uploaded range may take: the explicit limit, or what the device and torch's allocator
@@ -337,9 +399,9 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         cached = torch.cuda.memory_reserved(device) - torch.cuda.memory_allocated(device)
         return max(free + cached - (2 << 30), 64 << 20)
 
-    def _read_device_items(self, object_id, stream, device_reqs, planner, stats, sidecar) -> None:
+    def _read_device_items(self, object_id, stream, device_reqs, planner, stats, sidecar, early=None) -> None:
         devices = {t.device for _, t, *_ in device_reqs}
-        if len(devices) != 1:
+        if len(devices) != 1 or (early is not None and early[2] not in devices):
             raise ValueError("all device targets of one checkpoint object must live on the same device")
         device = devices.pop()
         written = stream.len_written_data
@@ -413,10 +475,17 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                 lo, hi = 0, written  # checksums cover the whole data section
             lo = lo // _UPLOAD_ALIGN * _UPLOAD_ALIGN
             clusters = None
-            if (hi - lo) - sum(r[1] - r[0] for r in rows) >= _PARTIAL_READ_MIN_SAVING:
+            if early is not None and early[3] <= lo and hi <= early[4]:  # the range is already on its way into a buffer
+                with torch.cuda.device(device):
+                    self._restore_range(object_id, stream, device, rows, early[3], early[4], sidecar, stats, early[0], early[1])
+                    for target, stored_as in conversions:
+                        target.copy_(stored_as)
+                rows = []
+            elif (hi - lo) - sum(r[1] - r[0] for r in rows) >= _PARTIAL_READ_MIN_SAVING:
                 clusters = self._clusters_of(rows, sidecar[0] if sidecar is not None else None, written)
                 if (hi - lo) - sum(c_hi - c_lo for c_lo, c_hi, _ in clusters) < _PARTIAL_READ_MIN_SAVING:
                     clusters = None
+        if rows:
             with torch.cuda.device(device):
                 _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
                 self._keep_clear_of(device)
@@ -528,11 +597,15 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         finally:
             plan.destroy()
 
-    def _restore_range(self, object_id, stream, device, rows, lo, hi, sidecar, stats, image) -> None:
-        """One upload of [lo, hi) into ``image``, checksum on the GPU if the object has a sidecar, one unpack."""
+    def _restore_range(self, object_id, stream, device, rows, lo, hi, sidecar, stats, image, uploaded=None) -> None:
+        """One upload of [lo, hi) into ``image`` (``uploaded``: the future of one that was started earlier),
+        checksum on the GPU if the object has a sidecar, one unpack."""
         span = hi - lo
         cur = torch.cuda.current_stream(device)
-        self._upload(stream, lo, image, span, cur, stats)
+        if uploaded is not None:
+            uploaded.result()
+        else:
+            self._upload(stream, lo, image, span, cur, stats)
         if sidecar is not None:
             chunk_bytes, data_bytes, want = sidecar
             if self._crc_mode == "fused" and chunk_bytes % 65536 == 0 and data_bytes == span:

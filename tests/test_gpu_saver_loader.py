@@ -149,6 +149,9 @@ def test_dcp_save_bytes_equal_oracle_and_load_is_bit_exact(shm_dir, manager_futu
             if isinstance(v, torch.Tensor):
                 assert torch.equal(_bits(target[k]), _bits(v)), k
         assert loader.last_load_stats["device_items"] >= 8 and loader.last_load_stats["host_items"] == 1
+        # where the records lie is in the checkpoint's metadata: the range that holds them is on its way to the
+        # device before their headers are parsed
+        assert loader.last_load_stats.get("upload_began_before_parse", 0) == 1
 
     # and the oracle's CPU loader restores our file
     target = {k: (torch.zeros_like(v) if isinstance(v, torch.Tensor) else None) for k, v in sd_cpu.items()}
@@ -970,7 +973,7 @@ def test_a_partial_read_uploads_only_what_it_needs(shm_dir, monkeypatch, with_si
 
     targets, stats = read()
     assert all(torch.equal(targets[k].cpu(), data_cpu[k]) for k in wanted)
-    assert stats["partial_read_ranges"] == 2
+    assert stats["partial_read_ranges"] == 2 and "upload_began_before_parse" not in stats
     assert stats["h2d_bytes"] <= 2 * ((1 << 18) + (3 << 16))  # two tensors and at most a chunk or two around each
     untouched = info[by_offset[7]]
     with open(oid.data, "r+b") as f:  # damage in a tensor nobody asked for
