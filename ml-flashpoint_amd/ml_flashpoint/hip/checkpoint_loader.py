@@ -283,23 +283,26 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                 self._check_on_host(checkpoint_object_id, stream, sidecar, todo)
                 host_checked.update(todo)
 
-            early = self._start_early_upload(stream, read_items, planner, storage_data, recorded, sidecar, stats) \
-                if optimized else None
+            resolved: dict = {}  # id(request) -> target, for the requests whose target was looked at ahead of time
+            early = self._start_early_upload(stream, read_items, planner, storage_data, recorded, sidecar, stats,
+                                             resolved) if optimized else None
             try:
                 self._serve_items(checkpoint_object_id, stream, read_items, planner, storage_data, optimized, whole,
-                                  recorded, sidecar, check_on_host_first, stats, early)
+                                  recorded, sidecar, check_on_host_first, stats, early, resolved)
             finally:
                 if early is not None:  # the file and its mapping are closed below: nothing may still be reading them
                     concurrent.futures.wait([early[1]])
         stats["read_s"] = time.perf_counter() - t_start
         self.last_load_stats = stats
 
-    def _start_early_upload(self, stream, read_items, planner, storage_data, recorded: int, sidecar, stats):
+    def _start_early_upload(self, stream, read_items, planner, storage_data, recorded: int, sidecar, stats,
+                            resolved: dict):
         """Where the records that are asked for lie in the object is known from the checkpoint's metadata, so when
         they are going to be read through one device buffer in one piece - the whole data section if the object has
         checksums - the upload can begin before the record headers are parsed and the targets resolved (5 us per
         item on the host: 110 ms for 20 000 items, beside an upload of 150 ms).  Returns ``(buffer, future of the
-        upload, device, first byte, end)`` when the read is certain to be of that kind, else None."""
+        upload, device, first byte, end)`` when the read is certain to be of that kind, else None.  Targets it had to
+        resolve to learn the device are left in ``resolved`` (a planner is asked for every target once)."""
         asked = {req.storage_index: storage_data[req.storage_index]
                  for req in read_items if req.type != LoadItemType.BYTE_IO}
         if not asked or recorded <= 0:
@@ -319,7 +322,8 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         # host-resident is taken to be one for the host)
         device = None
         for req in [req for req in read_items[:64] if req.type != LoadItemType.BYTE_IO][:8]:
-            device = planner.resolve_tensor(req).device
+            resolved[id(req)] = planner.resolve_tensor(req).detach()
+            device = resolved[id(req)].device
             if device.type != "cpu":
                 break
         if device is None or device.type == "cpu":
@@ -345,7 +349,7 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         return image, done, device, lo, hi
 
     def _serve_items(self, checkpoint_object_id, stream, read_items, planner, storage_data, optimized, whole, recorded,
-                     sidecar, check_on_host_first, stats, early) -> None:
+                     sidecar, check_on_host_first, stats, early, resolved: dict) -> None:
         """Items for the host are served one by one; those for the device are collected and restored together."""
         device_reqs = []  # (req, target, dtype, shape, payload_off, stored payload bytes)
         t_parse = time.perf_counter()
@@ -358,7 +362,9 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                 data.seek(0)
                 planner.load_bytes(req, data)
                 continue
-            target = planner.resolve_tensor(req).detach()
+            target = resolved.pop(id(req), None)
+            if target is None:
+                target = planner.resolve_tensor(req).detach()
             parsed = self._parse_header(whole, item_md.offset, item_md.length) if optimized else None
             if parsed is not None and target.device.type == "cpu":
                 # host-resident target: one copy, from a tensor laid over the record's payload in the mapping
