@@ -6,6 +6,7 @@ import ctypes
 import io
 import os
 import pickle
+import threading
 
 import pytest
 import torch
@@ -1177,6 +1178,64 @@ def test_a_failed_upload_in_a_pipelined_restore_is_reported_and_the_loader_stays
     dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), planner=Planner(), no_dist=True)
     assert loader.last_load_stats["windows"] >= 4 and sorted(committed) == sorted(sd_cpu)
     assert all(torch.equal(target[k].cpu(), v) for k, v in sd_cpu.items())
+
+
+@pytest.mark.parametrize("with_sidecar", [True, False])
+def test_an_upload_that_began_before_the_headers_were_parsed_and_fails_is_reported(shm_dir, manager_future, monkeypatch,
+                                                                                  with_sidecar):
+    """The range that holds the requested records is uploaded on a thread while the headers are parsed.  If that
+    upload fails (forced from the host), the restore raises its error, commits nothing and leaves nothing running
+    that still reads the object; a corrupt object is found before a target is touched; the loader stays usable."""
+    from ml_flashpoint.hip import integrity
+
+    sd_cpu = {f"t{i:02d}": torch.randn(40_000 + 333 * i, generator=torch.Generator().manual_seed(7 + i)) for i in range(12)}
+    sd_dev = _to_dev(sd_cpu)
+    ckpt = os.path.join(shm_dir, "step-31_ckpt")
+    dcp.save(sd_dev, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(
+        _saver(crc_chunk_bytes=(1 << 16) if with_sidecar else 0), manager_future), no_dist=True)
+    loader = _loader()
+    real_upload = loader._upload
+    threads = []
+
+    def failing_upload(*args, **kwargs):
+        threads.append(threading.current_thread().name)
+        raise OSError("injected: the object could not be read")
+
+    committed = []
+
+    class Planner(dcp.DefaultLoadPlanner):
+        def commit_tensor(self, read_item, tensor):
+            committed.append(read_item.dest_index.fqn)
+            return super().commit_tensor(read_item, tensor)
+
+    monkeypatch.setattr(loader, "_upload", failing_upload)
+    target = {k: torch.full_like(v, 5.0) for k, v in sd_dev.items()}
+    with pytest.raises(BaseException) as exc:
+        dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), planner=Planner(), no_dist=True)
+    cause = exc.value.failures[0][0] if hasattr(exc.value, "failures") else exc.value
+    assert isinstance(cause, OSError) and "injected" in str(cause)
+    assert threads == ["mlf-early-upload"] and committed == []
+    assert not any(t.name == "mlf-early-upload" for t in threading.enumerate())
+    assert all(bool((v == 5.0).all()) for v in target.values())
+
+    monkeypatch.setattr(loader, "_upload", real_upload)
+    dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), planner=Planner(), no_dist=True)
+    assert loader.last_load_stats["upload_began_before_parse"] == 1 and sorted(committed) == sorted(sd_cpu)
+    assert all(torch.equal(target[k].cpu(), v) for k, v in sd_cpu.items())
+    if with_sidecar:  # one flipped bit: found by the pass over the uploaded range, before any target is written
+        obj = os.path.join(ckpt, "__0__0_src0.distcp")
+        with open(obj, "r+b") as f:
+            f.seek(METADATA_SIZE + 100_000)
+            byte = f.read(1)
+            f.seek(-1, os.SEEK_CUR)
+            f.write(bytes([byte[0] ^ 0x04]))
+        target = {k: torch.full_like(v, 5.0) for k, v in sd_dev.items()}
+        with pytest.raises(BaseException) as exc:
+            dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, loader), no_dist=True)
+        cause = exc.value.failures[0][0] if hasattr(exc.value, "failures") else exc.value
+        assert isinstance(cause, integrity.ChecksumMismatchError)
+        torch.cuda.synchronize()
+        assert all(bool((v == 5.0).all()) for v in target.values())
 
 
 def test_tied_and_overlapping_tensors_are_saved_once_per_name_and_restored_into_shared_storage(shm_dir, manager_future):
