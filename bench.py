@@ -42,6 +42,7 @@ PACK_TRAFFIC_RATIO = {
     ("llama3-8b-shard", "beside"): 1.0008,
     ("llama3-8b-shard", "fused"): 1.0158,
     ("strided-views", "beside"): 1.214,
+    ("mixtral-expert-shard", "beside"): 1.0008,
 }
 
 
@@ -91,6 +92,8 @@ def parse_args():
                          "the device busy (what the transfer costs them, and what they cost the transfer)")
     ap.add_argument("--no-crc-compare", action="store_true", help="skip the extra saves in the other checksum mode")
     ap.add_argument("--no-plan-cache-compare", action="store_true", help="skip the extra saves on a reused DCP plan")
+    ap.add_argument("--no-limited-hbm-compare", dest="limited_hbm_compare", action="store_false",
+                    help="skip the extra save + restore with room in HBM for 57 %% and for 14 %% of the image")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="the default run (llama3-8b-shard at full scale) also measures the many-small and strided-views "
                          "configurations, one warm-up and three timed steps each, and reports them under other_workloads")
@@ -383,6 +386,7 @@ def main():
             sub = argparse.Namespace(**vars(args))
             sub.workload, sub.steps, sub.warmup = name, 3, 1
             sub.no_link_probe = sub.no_crc_compare = sub.no_busy_gpu_probe = True
+            sub.limited_hbm_compare = False
             sub.partial_restore_prefix, sub.pmc_calibration = None, False
             sub.no_plan_cache_compare = name != "many-small"  # where the DCP planner is most of the blocking time
             sub.cpu_baseline_gb = 1e3 if name == "many-small" and args.cpu_baseline_gb > 0 else 0.0  # the whole dict
@@ -459,7 +463,7 @@ def run_workload(args):
             lambda: 0, lambda: 0, lambda: None, manager, None, initial_buffer_size_bytes=1 << 20,
             engine_config=engine_cfg, tile_bytes=args.tile_bytes, block_threads=args.block_threads,
             crc_chunk_bytes=args.crc_chunk_mib << 20, crc_mode=crc_mode, use_file_io=args.save_io == "file",
-            max_image_bytes=max_image, **more)
+            max_image_bytes=more.pop("max_image_bytes", max_image), **more)
         made.record_kernel_events = True
         return made
 
@@ -662,6 +666,44 @@ def run_workload(args):
                               "tail_finish_and_finalize": round(last["tail"] * 1e3, 2)}}
         manager.delete_container(prev)
 
+        # ---- the same object with room in HBM for part of its image only: the end of the object stays resident, the
+        # rest goes window by window inside the blocking part; the restore goes through windows of that size ----
+        limited = None
+        if args.limited_hbm_compare and max_image is None and payload >= (8 << 30):
+            limited = {}
+            for share in (0.57, 0.14):  # 64 GB and 16 GB of room for the 112 GB shard
+                room = int(payload * share)
+                tight = make_saver(args.save_crc, max_image_bytes=room)
+                tight_loader = DefaultMLFlashpointCheckpointLoader(
+                    manager, None, engine_config=engine_cfg, tile_bytes=args.tile_bytes, block_threads=args.block_threads,
+                    use_file_io=args.restore_io == "file", crc_mode=args.restore_crc, max_image_bytes=room)
+                for again in range(2):  # the first creates the engines, their pinned slots and the window buffers
+                    cid = CheckpointContainerId(os.path.join(root, "run", f"step-{4000 + int(share * 100) + again}_ckpt"))
+                    sv = one_save(tight, cid)
+                    for v in sd.values():
+                        v.zero_() if v.is_contiguous() else v.fill_(0)
+                    gc.collect()
+                    torch.cuda.synchronize()
+                    t1 = time.perf_counter()
+                    dcp.load(sd, checkpoint_id=cid.data, storage_reader=MemoryStorageReader(cid.data, tight_loader), no_dist=True)
+                    torch.cuda.synchronize()
+                    t2 = time.perf_counter()
+                    wrong = [k for k, v in sd.items() if workloads.fingerprint(v) != prints[k]]
+                    manager.delete_container(cid)
+                    if wrong:
+                        break
+                tight.release_device_memory()
+                limited[f"{room / 1e9:.0f}_GB_of_room"] = {
+                    "save_s": round(sv["save"], 3), "blocking_save_ms": round(sv["blocking"] * 1e3, 1),
+                    "save_windows": sv["stats"].get("windows", 0), "restore_s": round(t2 - t1, 3),
+                    "restore_windows": tight_loader.last_load_stats.get("windows", 0),
+                    "restored_bit_identical": not wrong}
+                for made in (getattr(tight, "_engine", None), getattr(tight_loader, "_engine", None)):
+                    if made is not None:
+                        made.destroy()
+                del tight, tight_loader
+                torch.cuda.empty_cache()
+
         # ---- a save whose transfer runs on a thread while the device is kept busy, as by a training step ----
         busy = None
         if not args.no_busy_gpu_probe and max_image is None:
@@ -779,6 +821,7 @@ def run_workload(args):
             **({"crc_modes": crc_modes} if crc_modes else {}),
             **({"with_dcp_plan_cache": with_cache} if with_cache else {}),
             **({"beside_a_busy_gpu": busy} if busy else {}),
+            **({"with_room_for_part_of_the_image": limited} if limited else {}),
             "parity": "restored tensors bit-identical to originals (fingerprints)",
             "roofline": {"bound": "hbm",
                          "kernel": "mlf_fused_crc_kernel<pack> (copy + CRC-32C)" if args.save_crc == "fused" else "mlf_flat_kernel<pack>",
