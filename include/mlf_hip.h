@@ -251,6 +251,14 @@ int mlf_engine_avoid_streams(mlf_engine* engine, void* const* busy_streams, uint
  * one; a handle returned earlier stays a valid stream until mlf_engine_destroy. */
 void* mlf_engine_checksum_stream(mlf_engine* engine);
 
+/* Who takes the per-chunk CRC-32C of a device-to-host transfer that asks for one (mlf_engine_d2h_crc, _watched,
+ * _gated).  on = 0 (the state of a new engine): kernels on the engine's checksum stream read the image once more
+ * while it crosses the link.  on != 0: the host threads that move the pinned slots into the destination take the
+ * checksums of what they move (crc32 instructions beside the copy loop, three interleaved chains per thread) - no
+ * kernel, no second read of the image from device memory; the values are the same.  Takes effect with the next
+ * transfer.  No reference counterpart (the reference keeps no checksums). */
+int mlf_engine_set_host_checksums(mlf_engine* engine, int on);
+
 /* Host -> host on the engine's threads: `nbytes` from `src_host` to `dst_host` (ranges must not overlap).  For
  * checkpoint items that are resident in host memory - the reference copies those into the mapping with torch's
  * intra-op threads (checkpoint_saver.py:443-450,797-800); they do not visit the device here either. */

@@ -3,6 +3,8 @@
 // include/mlf_hip.h.
 #include "mlf_internal.h"
 
+#include <immintrin.h>
+
 #include <algorithm>
 #include <atomic>
 #include <condition_variable>
@@ -101,6 +103,102 @@ void pool_memcpy(WorkerPool& pool, char* dst, const char* src, size_t n) {
   });
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// copy + CRC-32C on the host threads
+// ---------------------------------------------------------------------------------------------------------
+// The threads that move a pinned slot into the buffer touch every byte of the image anyway, and the crc32
+// instruction retires eight bytes per cycle when three independent chains keep it busy: a piece is cut into three
+// lanes that are copied (32-byte loads, streaming stores: the destination is written once and not read soon) and
+// checksummed side by side, and the lanes' states are joined with two multiplications.  Measured on the MI355X host
+// (16 threads, 2 MiB pieces, 24 GiB into a tmpfs mapping): memcpy 190 GB/s, this loop 212 GB/s - against the 56 GB/s
+// the link delivers.
+
+// CRC state after `n` more bytes (state in, state out; no initial or final inversion)
+inline uint64_t crc_advance(uint64_t s, const char* p, size_t n) {
+  for (; n >= 8; n -= 8, p += 8) {
+    uint64_t w;
+    memcpy(&w, p, 8);
+    s = _mm_crc32_u64(s, w);
+  }
+  while (n--) s = _mm_crc32_u8((uint32_t)s, (unsigned char)*p++);
+  return s;
+}
+
+// x^(8 * n) for the lane length in use (pieces are of one size but for the last one: looked up once per thread)
+inline uint32_t lane_weight(size_t n) {
+  thread_local size_t known_n = 0;
+  thread_local uint32_t known_x = 0;
+  if (n != known_n) {
+    known_x = x_pow_bytes(n);
+    known_n = n;
+  }
+  return known_x;
+}
+
+// Copies [src, src + n) to dst (dst == nullptr: only reads it) and returns its CRC-32C.
+__attribute__((target("avx2,sse4.2"))) uint32_t copy_crc_avx2(char* dst, const char* src, size_t n) {
+  const size_t lane = (n / 3) & ~(size_t)63;
+  uint64_t c0 = 0xFFFFFFFFu, c1 = 0, c2 = 0;
+  if (lane >= 1024) {
+    const char *p0 = src, *p1 = src + lane, *p2 = src + 2 * lane;
+    const bool copy = dst != nullptr;
+    const bool stream = copy && (reinterpret_cast<uintptr_t>(dst) & 31u) == 0;  // (lanes are multiples of 64 bytes)
+    char *q0 = dst, *q1 = dst + lane, *q2 = dst + 2 * lane;
+#define MLF_LANE(p, q, c)                                                                \
+  {                                                                                      \
+    if (copy) {                                                                          \
+      const __m256i a = _mm256_loadu_si256(reinterpret_cast<const __m256i*>(p + i));      \
+      const __m256i b = _mm256_loadu_si256(reinterpret_cast<const __m256i*>(p + i + 32)); \
+      if (stream) {                                                                      \
+        _mm256_stream_si256(reinterpret_cast<__m256i*>(q + i), a);                       \
+        _mm256_stream_si256(reinterpret_cast<__m256i*>(q + i + 32), b);                  \
+      } else {                                                                           \
+        _mm256_storeu_si256(reinterpret_cast<__m256i*>(q + i), a);                       \
+        _mm256_storeu_si256(reinterpret_cast<__m256i*>(q + i + 32), b);                  \
+      }                                                                                  \
+    }                                                                                    \
+    uint64_t w[8];                                                                       \
+    memcpy(w, p + i, 64);                                                                \
+    c = _mm_crc32_u64(c, w[0]);                                                          \
+    c = _mm_crc32_u64(c, w[1]);                                                          \
+    c = _mm_crc32_u64(c, w[2]);                                                          \
+    c = _mm_crc32_u64(c, w[3]);                                                          \
+    c = _mm_crc32_u64(c, w[4]);                                                          \
+    c = _mm_crc32_u64(c, w[5]);                                                          \
+    c = _mm_crc32_u64(c, w[6]);                                                          \
+    c = _mm_crc32_u64(c, w[7]);                                                          \
+  }
+    for (size_t i = 0; i < lane; i += 64) {
+      MLF_LANE(p0, q0, c0)
+      MLF_LANE(p1, q1, c1)
+      MLF_LANE(p2, q2, c2)
+    }
+#undef MLF_LANE
+    if (stream) _mm_sfence();  // streaming stores are ordered before whatever announces the piece
+    const uint32_t x = lane_weight(lane);
+    c0 = gf_mul(x, (uint32_t)c0) ^ (uint32_t)c1;
+    c0 = gf_mul(x, (uint32_t)c0) ^ (uint32_t)c2;
+    src += 3 * lane;
+    if (dst) dst += 3 * lane;
+    n -= 3 * lane;
+  }
+  if (dst && n) memcpy(dst, src, n);
+  return (uint32_t)crc_advance(c0, src, n) ^ 0xFFFFFFFFu;
+}
+
+uint32_t copy_crc(char* dst, const char* src, size_t n) {
+  static const bool avx2 = __builtin_cpu_supports("avx2") && __builtin_cpu_supports("sse4.2");
+  if (avx2) return copy_crc_avx2(dst, src, n);
+  if (dst && n) memcpy(dst, src, n);
+  return (uint32_t)crc_advance(0xFFFFFFFFu, src, n) ^ 0xFFFFFFFFu;
+}
+
+// A piece of the image that one thread has copied and checksummed
+struct CheckedPiece {
+  uint64_t image_off, len;
+  uint32_t crc;
+};
+
 // The pageable end of a transfer: a plain pointer, or a byte range of an open file (pread/pwrite).  Going
 // through the file descriptor moves the same page-cache pages as a MAP_SHARED mapping would, without building
 // (and later tearing down) one page-table entry per 4 KiB of a buffer that can be 100+ GB.
@@ -132,6 +230,38 @@ int pool_host_copy(WorkerPool& pool, const HostEnd& host, uint64_t host_off, cha
   return err.load();
 }
 
+// slot -> host end like pool_host_copy, every thread also taking the CRC-32C of what it moves.  The pieces are cut
+// where checksum chunks end (chunk k covers image bytes [k * chunk_bytes, (k + 1) * chunk_bytes)), and `out` gets
+// them in image order.
+int pool_host_copy_checked(WorkerPool& pool, const HostEnd& host, uint64_t image_off, char* slot, size_t n,
+                           uint64_t chunk_bytes, std::vector<CheckedPiece>* out) {
+  const unsigned parts = std::max<unsigned>(1, std::min<size_t>(pool.width(), n / ((size_t)1 << 20)));
+  size_t per = (n + parts - 1) / parts;
+  per = (per + 4095) & ~(size_t)4095;
+  std::vector<std::vector<CheckedPiece>> found(parts);
+  std::atomic<int> err{0};
+  pool.run(parts, [&](unsigned i) {
+    size_t off = (size_t)i * per;
+    if (off >= n) return;
+    const size_t end = std::min(off + per, n);
+    while (off < end) {
+      const uint64_t at = image_off + off;
+      const size_t len = (size_t)std::min<uint64_t>(end - off, chunk_bytes - at % chunk_bytes);
+      uint32_t crc;
+      if (host.fd < 0) {
+        crc = copy_crc(host.ptr + at, slot + off, len);
+      } else {
+        crc = copy_crc(nullptr, slot + off, len);
+        if (int e = full_pwrite(host.fd, slot + off, len, host.file_off + at)) err.store(e);
+      }
+      found[i].push_back({at, len, crc});
+      off += len;
+    }
+  });
+  for (const auto& list : found) out->insert(out->end(), list.begin(), list.end());
+  return err.load();
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------------------------------------
@@ -151,6 +281,9 @@ struct mlf_engine {
   CrcScratch crc;  // of the checksum passes that run beside transfers; allocated on first use, grown when too small
   std::unique_ptr<WorkerPool> pool;
   std::mutex busy;  // one transfer at a time per engine
+  // checksums of a device-to-host transfer: taken by the host threads as they move the slots (true), or by kernels
+  // on crc_stream that read the image once more while it crosses the link (false)
+  std::atomic<bool> host_checksums{false};
 };
 
 namespace {
@@ -302,6 +435,11 @@ int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t
   if (crc.landed) __atomic_store_n(crc.landed, (uint64_t)0, __ATOMIC_RELEASE);
   const bool want_crc = crc.chunk_bytes != 0 && nbytes != 0;
   const uint64_t n_crc = want_crc ? (nbytes + crc.chunk_bytes - 1) / crc.chunk_bytes : 0;
+  if (want_crc && crc.n_out < n_crc) return fail(MLF_HIP_BAD_ARG, "checksum output too small");
+  const bool on_host = want_crc && e->host_checksums.load();
+  std::vector<CheckedPiece> pieces;
+  std::vector<uint32_t> chunk_crc(on_host ? n_crc : 0);
+  std::vector<uint64_t> chunk_len(on_host ? n_crc : 0, 0);
   struct CrcGuard {  // on every exit path the checksum kernels have finished before the scratch can be used again
     hipStream_t stream;
     bool armed;
@@ -309,7 +447,7 @@ int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t
       if (armed) (void)hipStreamSynchronize(stream);
     }
   } crc_guard{e->crc_stream, false};
-  if (want_crc) {
+  if (want_crc && !on_host) {
     // the image is complete once the gate has passed and is not modified afterwards, so its checksum can be
     // computed while the link-bound copies run: it costs neither blocking time nor transfer time
     if (ready) HIP_TRY(hipStreamWaitEvent(e->crc_stream, ready, 0));
@@ -337,14 +475,26 @@ int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t
     const double w0 = now_s();
     HIP_TRY(hipEventSynchronize(e->slot_done[s]));
     if (c == 0) wait = now_s() - w0;
-    if (int err = pool_host_copy(*e->pool, host, off, e->slots[s], len, true))
+    if (on_host) {
+      pieces.clear();
+      if (int err = pool_host_copy_checked(*e->pool, host, off, e->slots[s], len, crc.chunk_bytes, &pieces))
+        return fail(MLF_HIP_RUNTIME, std::string("pwrite() to the buffer file failed: ") + strerror(err));
+      for (const CheckedPiece& p : pieces) {  // in image order: crc(A || B) = crc(A) * x^(8 |B|) + crc(B)
+        const uint64_t k = p.image_off / crc.chunk_bytes;
+        chunk_crc[k] = chunk_len[k] ? mlf_crc32c_combine(chunk_crc[k], p.crc, p.len) : p.crc;
+        chunk_len[k] += p.len;
+      }
+    } else if (int err = pool_host_copy(*e->pool, host, off, e->slots[s], len, true)) {
       return fail(MLF_HIP_RUNTIME, std::string("pwrite() to the buffer file failed: ") + strerror(err));
+    }
     if (crc.landed) __atomic_store_n(crc.landed, off + len, __ATOMIC_RELEASE);  // the host threads' stores come first
     if (c + n_slots < n_chunks)
       if (int rc = issue(c + n_slots)) return rc;
   }
   drain.armed = false;  // every chunk's event has been waited for
-  if (want_crc) {
+  if (on_host) {
+    std::copy(chunk_crc.begin(), chunk_crc.end(), crc.out_host);
+  } else if (want_crc) {
     crc_guard.armed = false;
     if (int rc = crc_finish(&e->crc, e->crc_stream, n_crc, crc.out_host)) return rc;
   }
@@ -527,6 +677,12 @@ int mlf_engine_avoid_streams(mlf_engine* e, void* const* busy_streams, uint32_t 
 }
 
 void* mlf_engine_checksum_stream(mlf_engine* e) { return e ? e->crc_stream : nullptr; }
+
+int mlf_engine_set_host_checksums(mlf_engine* e, int on) {
+  if (!e) return fail(MLF_HIP_BAD_ARG, "null engine");
+  e->host_checksums.store(on != 0);
+  return MLF_HIP_OK;
+}
 
 int mlf_engine_link_probe(mlf_engine* e, void* dev_buf, uint64_t nbytes, int to_host, double* seconds) {
   if (!e || !dev_buf || !seconds) return fail(MLF_HIP_BAD_ARG, "null argument");

@@ -292,7 +292,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         tile_bytes: int = 0,
         block_threads: int = 0,
         crc_chunk_bytes: int = 0,
-        crc_mode: str = "beside",
+        crc_mode: str = "host",
         use_file_io: bool = False,
         background_write: bool = False,
         remote_wait_timeout_s: float = 1800.0,
@@ -305,10 +305,14 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
 
         Keyword-only extras: ``engine_config`` (pinned ring), ``tile_bytes`` / ``block_threads`` (pack kernel work
         split, 0 = library default), ``crc_chunk_bytes`` (> 0: compute a CRC-32C per chunk of every object on the
-        GPU and keep it beside the object), ``crc_mode`` (where those checksums are computed: ``"beside"`` - a pass
-        of its own over the finished image, on the copy engine's third stream while the image crosses the link, so it
-        adds nothing to the blocking part but reads the image a second time; ``"fused"`` - inside the pack kernel,
-        which then moves 2 x payload bytes through HBM instead of 3 x and runs about 10 % longer), ``use_file_io`` (False, the default: the host threads memcpy the
+        GPU and keep it beside the object), ``crc_mode`` (where those checksums are computed: ``"host"``, the default - by the
+        copy engine's host threads as they move the pinned slots into the buffer, crc32 instructions beside the
+        copy loop: no kernel, no second read of the image, nothing added to the blocking part, and on the hosts
+        measured no slower than the plain copy; objects that are sent in pieces or through windows are checksummed
+        as with ``"beside"``; ``"beside"`` - a pass of kernels over the finished image, on the copy engine's third
+        stream while the image crosses the link: nothing added to the blocking part either, but the image is read
+        from device memory a second time; ``"fused"`` - inside the pack kernel, which then runs about 12 % longer),
+        ``use_file_io`` (False, the default: the host threads memcpy the
         pinned slots into the mapping, whose page-table entries a pooled buffer keeps from save to save; True: they
         pwrite() through the file descriptor, which tmpfs serialises on the inode lock - measured 5x slower),
         ``background_write`` (True: ``prepare_write_data`` also starts the transfer into the buffer object on a
@@ -339,8 +343,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         self._engine_config = engine_config or EngineConfig()
         self._tile_bytes = tile_bytes
         self._block_threads = block_threads
-        if crc_mode not in ("beside", "fused"):
-            raise ValueError("crc_mode must be 'beside' or 'fused'")
+        if crc_mode not in ("beside", "fused", "host"):
+            raise ValueError("crc_mode must be 'beside', 'fused' or 'host'")
         if crc_chunk_bytes % 65536:
             raise ValueError("crc_chunk_bytes must be a multiple of 65536")
         self._crc_chunk_bytes = crc_chunk_bytes
@@ -388,6 +392,7 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             if self._engine is None:
                 cfg = self._engine_config
                 self._engine = hip_plan.CopyEngine(cfg.slot_bytes, cfg.n_slots, cfg.resolved_copy_threads())
+                self._engine.set_host_checksums(self._crc_mode == "host")
             return self._engine
 
     def warm_up(self, device: Optional[torch.device] = None, also_avoid: tuple = ()) -> None:

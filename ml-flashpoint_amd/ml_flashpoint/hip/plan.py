@@ -391,6 +391,11 @@ class CopyEngine:
         self._handle = handle
         self.slot_bytes, self.n_slots, self.n_threads = slot_bytes, n_slots, n_threads
 
+    def set_host_checksums(self, on: bool) -> None:
+        """Who takes the checksums of the ``d2h_*`` calls that ask for them: the host threads as they move the
+        slots (True), or kernels that read the image once more beside the copies (False, the state of a new engine)."""
+        _lib.check(_lib.load().mlf_engine_set_host_checksums(self._handle, 1 if on else 0), "mlf_engine_set_host_checksums")
+
     def d2h(self, src_dev_ptr: int, dst_host_ptr: int, nbytes: int, producer_stream: int = 0) -> _lib.XferStats:
         stats = _lib.XferStats()
         _lib.check(

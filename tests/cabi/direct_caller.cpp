@@ -168,6 +168,13 @@ int main(int argc, char** argv) {
   std::fill(chunk_got.begin(), chunk_got.end(), 0u);
   REQUIRE(mlf_engine_d2h_gated(engine, d_image, dst2, image_bytes, packed, chunk, chunk_got.data(), n_chunks, &landed, &stats) == 0);
   REQUIRE(landed == image_bytes && chunk_got == chunk_want && std::memcmp(dst2, want.data(), image_bytes) == 0);
+  // the same transfer with the checksums taken by the host threads that copy the slots: same bytes, same values
+  REQUIRE(mlf_engine_set_host_checksums(engine, 1) == 0);
+  std::memset(dst2, 0, image_bytes);
+  std::fill(chunk_got.begin(), chunk_got.end(), 0u);
+  REQUIRE(mlf_engine_d2h_gated(engine, d_image, dst2, image_bytes, packed, chunk, chunk_got.data(), n_chunks, &landed, &stats) == 0);
+  REQUIRE(landed == image_bytes && chunk_got == chunk_want && std::memcmp(dst2, want.data(), image_bytes) == 0);
+  REQUIRE(mlf_engine_set_host_checksums(engine, 0) == 0 && mlf_engine_set_host_checksums(nullptr, 1) != 0);
   double seconds = 0;
   REQUIRE(mlf_engine_link_probe(engine, d_image, image_bytes, 1, &seconds) == 0 && seconds > 0);
 

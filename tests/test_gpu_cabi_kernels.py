@@ -675,6 +675,48 @@ def test_copy_engine_round_trip(nbytes, shm_dir, oracle_c):
     engine.destroy()
 
 
+@pytest.mark.parametrize("slot_bytes, chunk_bytes", [(1 << 20, 1 << 20), (3 << 20, 1 << 20), (1 << 20, 4 << 20),
+                                                     ((1 << 20) + 4096, 3 << 16), (32 << 20, 32 << 20)])
+@pytest.mark.parametrize("nbytes", [65536 + 1, (9 << 20) + 12345, (70 << 20) + 7])
+@pytest.mark.parametrize("misaligned", [0, 5])
+def test_checksums_taken_by_the_host_threads_equal_the_kernels_and_the_oracle(slot_bytes, chunk_bytes, nbytes, misaligned,
+                                                                             shm_dir, oracle_c):
+    """``mlf_engine_set_host_checksums``: the threads that move the pinned slots into the destination take the
+    checksums of what they move - pieces cut at chunk boundaries, three interleaved chains per piece, joined by
+    crc(A || B) = crc(A) x^(8 |B|) + crc(B).  Same bytes in the destination, same values as the kernels' and as the
+    oracle's, for slots smaller and larger than chunks, sizes that end inside a piece, destinations off the
+    32-byte grid (no streaming stores), through the mapping and through the file descriptor."""
+    from ml_flashpoint.checkpoint_object_manager.buffer_object.buffer_object_ext import BufferObject
+    from ml_flashpoint.hip import plan as P
+
+    gen = torch.Generator().manual_seed(nbytes + slot_bytes)
+    host = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=gen)
+    raw = host.numpy().tobytes()
+    dev = host.to(DEV)
+    want = np.zeros(-(-nbytes // chunk_bytes), dtype=np.uint32)
+    oracle_c.oracle_crc32c_chunks(raw, nbytes, chunk_bytes, want.ctypes.data)
+    engine = P.CopyEngine(slot_bytes=slot_bytes, n_slots=3, n_threads=5)
+    bo = BufferObject(f"{shm_dir}/hostcrc.bin", 4096 + misaligned + nbytes, True)
+    stream = torch.cuda.current_stream().cuda_stream
+    first = 4096 + misaligned
+    _, by_kernels = engine.d2h_crc(dev.data_ptr(), bo.get_data_ptr() + first, nbytes, stream, chunk_bytes)
+    assert by_kernels.tolist() == want.tolist()
+    engine.set_host_checksums(True)
+    memoryview(bo)[:] = bytes(first + nbytes)
+    stats, by_host = engine.d2h_crc(dev.data_ptr(), bo.get_data_ptr() + first, nbytes, stream, chunk_bytes)
+    assert stats.bytes == nbytes and bytes(memoryview(bo)[first:]) == raw and bytes(memoryview(bo)[:first]) == bytes(first)
+    assert by_host.tolist() == want.tolist()
+    landed = ctypes.c_uint64(0)
+    memoryview(bo)[:] = bytes(first + nbytes)
+    _, watched = engine.d2h_watched(dev.data_ptr(), bo.get_data_ptr() + first, nbytes, stream, chunk_bytes, landed)
+    assert int(landed.value) == nbytes and watched.tolist() == want.tolist() and bytes(memoryview(bo)[first:]) == raw
+    engine.set_host_checksums(False)
+    _, again = engine.d2h_crc(dev.data_ptr(), bo.get_data_ptr() + first, nbytes, stream, chunk_bytes)
+    assert again.tolist() == want.tolist()
+    bo.close()
+    engine.destroy()
+
+
 def test_watched_transfer_publishes_only_bytes_that_are_in_place(shm_dir, oracle_c):
     """While a 200 MiB image crosses the link in 1 MiB slots, a second thread follows the progress counter and copies
     whatever prefix it announces out of the mapping: the counter only grows, never runs ahead of the data, ends at the

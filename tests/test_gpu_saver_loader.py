@@ -272,12 +272,16 @@ def test_metadata_object_is_pickled_while_the_data_is_written(shm_dir, manager_f
     assert target["obj.step"] == 123
 
 
-def test_crc_sidecar_written_and_corruption_detected(shm_dir, manager_future):
+@pytest.mark.parametrize("crc_mode", ["beside", "fused", "host"])
+def test_crc_sidecar_written_and_corruption_detected(shm_dir, manager_future, crc_mode):
+    """Whoever takes the checksums of a save - a pass of kernels beside the transfer, the pack kernel itself, or the
+    host threads that move the image into the buffer - the sidecar holds the CRC-32C of the bytes in the file."""
     from ml_flashpoint.hip import integrity
 
     sd = {"a": torch.randn(300_000, device=DEV), "b": torch.randn(7, 9, device=DEV).to(torch.bfloat16)}
     ckpt = os.path.join(shm_dir, "step-2_ckpt")
-    dcp.save(sd, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(_saver(crc_chunk_bytes=1 << 18), manager_future), no_dist=True)
+    dcp.save(sd, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(
+        _saver(crc_chunk_bytes=1 << 18, crc_mode=crc_mode), manager_future), no_dist=True)
     obj = os.path.join(ckpt, "__0__0_src0.distcp")
     chunk, nbytes, crcs = integrity.read_sidecar(obj)
     raw = open(obj, "rb").read()
