@@ -67,7 +67,7 @@ _CHILD = textwrap.dedent(
     saver = HipMLFlashpointCheckpointSaver(lambda: rank, lambda: rank, dist.barrier, CheckpointObjectManager(), None,
                                            initial_buffer_size_bytes=1 << 20, crc_chunk_bytes=1 << 16)
     wrapper = _DistWrapper(None, True, 0)
-    cached, metadata, early = None, None, []
+    cached, metadata, early, respliced = None, None, [], []
     for step in (1, 2, 3):
         cid = CheckpointContainerId(os.path.join(root, f"step-{step}_ckpt"))
         writer = MemoryStorageWriter(saver, fut)
@@ -85,6 +85,7 @@ _CHILD = textwrap.dedent(
         three_calls.write_data(cid, writer, staged, replicate_after_write=False)
         three_calls.finish_write(cid, writer, metadata, wrapper)
         early.append(writer.early_metadata_used)
+        respliced.append(writer.early_metadata_respliced)
         dist.barrier()
         assert sorted(os.listdir(cid.data)) == [".metadata", "__0__0_src0.distcp", "__1__0_src1.distcp"], os.listdir(cid.data)
         written = pickle.load(open(os.path.join(cid.data, ".metadata"), "rb"))
@@ -115,6 +116,8 @@ _CHILD = textwrap.dedent(
         # the metadata object of the second and third save was pickled while their data was in flight, the other
         # rank's results predicted from the save before; the first save had nothing to go by
         assert early == [False, True, True], early
+        # and on the kept plan of the third save nothing was pickled: the second save's bytes, storage_meta exchanged
+        assert respliced == [False, False, True], respliced
         assert set(saver.last_write_locations) == set(written.storage_data)
     else:
         assert early == [False, False, False] and saver.last_write_locations is None  # never writes a metadata object
