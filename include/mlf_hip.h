@@ -259,6 +259,31 @@ void* mlf_engine_checksum_stream(mlf_engine* engine);
  * transfer.  No reference counterpart (the reference keeps no checksums). */
 int mlf_engine_set_host_checksums(mlf_engine* engine, int on);
 
+/* A device-to-host transfer of a piece of a larger data section, with the checksums of the piece cut where the
+ * section's chunks end: the piece's first `first_part_bytes` bytes (less than a chunk; 0: the piece begins on a
+ * chunk boundary) belong to a chunk that began before it and get a value of their own, then every
+ * `crc_chunk_bytes` bytes one, the last possibly short - (first_part_bytes ? 1 : 0) + ceil((nbytes -
+ * first_part_bytes) / crc_chunk_bytes) values for a piece longer than its first part, which the caller joins with
+ * its neighbours' by mlf_crc32c_combine.  Always taken by the host threads as they copy (the checksum kernels read
+ * whole chunks from their first byte).  The copies wait for `ready_event` (a hipEvent_t) if that is not NULL, else
+ * for what `producer_stream` holds at the call; `landed` as in mlf_engine_d2h_watched, or NULL.  For objects that
+ * leave the device in several transfers (an image held in pieces, windows, runs of an image around host-resident
+ * items).  No reference counterpart. */
+int mlf_engine_d2h_cut(mlf_engine* engine, const void* src_dev, void* dst_host, uint64_t nbytes, void* producer_stream,
+                       void* ready_event, uint64_t crc_chunk_bytes, uint64_t first_part_bytes, uint32_t* crc_out_host,
+                       uint64_t n_crc_out, uint64_t* landed, mlf_xfer_stats* stats);
+
+/* mlf_engine_host_copy that also yields the checksums of what it copies, cut like those of mlf_engine_d2h_cut. */
+int mlf_engine_host_copy_cut(mlf_engine* engine, void* dst_host, const void* src_host, uint64_t nbytes,
+                             uint64_t crc_chunk_bytes, uint64_t first_part_bytes, uint32_t* crc_out_host,
+                             uint64_t n_crc_out);
+
+/* File -> host memory on the engine's threads: `nbytes` from byte `file_offset` of `fd` into `dst_host`, by pread()
+ * in as many parts as the engine has threads.  For the host-resident targets of a restore (optimizer state kept in
+ * host memory): the reference copies such a record out of its mapping with one `copy_`
+ * (checkpoint_loader.py:331-336), which pays a page fault per 4 KiB of a mapping that was made for this one read. */
+int mlf_engine_read_file(mlf_engine* engine, int fd, uint64_t file_offset, void* dst_host, uint64_t nbytes);
+
 /* Host -> host on the engine's threads: `nbytes` from `src_host` to `dst_host` (ranges must not overlap).  For
  * checkpoint items that are resident in host memory - the reference copies those into the mapping with torch's
  * intra-op threads (checkpoint_saver.py:443-450,797-800); they do not visit the device here either. */

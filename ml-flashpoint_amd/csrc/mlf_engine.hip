@@ -199,6 +199,22 @@ struct CheckedPiece {
   uint32_t crc;
 };
 
+// Where the checksum chunks of a range begin: after `first` bytes (the rest of a chunk that began before the range;
+// 0: the range begins on a boundary), then every `chunk` bytes.
+struct ChunkGrid {
+  uint64_t chunk = 0, first = 0;
+  uint64_t index(uint64_t off) const { return first == 0 ? off / chunk : (off < first ? 0 : 1 + (off - first) / chunk); }
+  uint64_t next_cut(uint64_t off) const {
+    if (off < first) return first;
+    return first + ((off - first) / chunk + 1) * chunk;
+  }
+  uint64_t count(uint64_t nbytes) const {
+    if (nbytes == 0) return 0;
+    const uint64_t head = std::min(first, nbytes);
+    return (head ? 1 : 0) + (nbytes - head + chunk - 1) / chunk;
+  }
+};
+
 // The pageable end of a transfer: a plain pointer, or a byte range of an open file (pread/pwrite).  Going
 // through the file descriptor moves the same page-cache pages as a MAP_SHARED mapping would, without building
 // (and later tearing down) one page-table entry per 4 KiB of a buffer that can be 100+ GB.
@@ -231,10 +247,9 @@ int pool_host_copy(WorkerPool& pool, const HostEnd& host, uint64_t host_off, cha
 }
 
 // slot -> host end like pool_host_copy, every thread also taking the CRC-32C of what it moves.  The pieces are cut
-// where checksum chunks end (chunk k covers image bytes [k * chunk_bytes, (k + 1) * chunk_bytes)), and `out` gets
-// them in image order.
-int pool_host_copy_checked(WorkerPool& pool, const HostEnd& host, uint64_t image_off, char* slot, size_t n,
-                           uint64_t chunk_bytes, std::vector<CheckedPiece>* out) {
+// where the checksum chunks of `grid` end, and `out` gets them in image order.
+int pool_host_copy_checked(WorkerPool& pool, const HostEnd& host, uint64_t image_off, const char* slot, size_t n,
+                           const ChunkGrid& grid, std::vector<CheckedPiece>* out) {
   const unsigned parts = std::max<unsigned>(1, std::min<size_t>(pool.width(), n / ((size_t)1 << 20)));
   size_t per = (n + parts - 1) / parts;
   per = (per + 4095) & ~(size_t)4095;
@@ -246,7 +261,7 @@ int pool_host_copy_checked(WorkerPool& pool, const HostEnd& host, uint64_t image
     const size_t end = std::min(off + per, n);
     while (off < end) {
       const uint64_t at = image_off + off;
-      const size_t len = (size_t)std::min<uint64_t>(end - off, chunk_bytes - at % chunk_bytes);
+      const size_t len = (size_t)std::min<uint64_t>(end - off, grid.next_cut(at) - at);
       uint32_t crc;
       if (host.fd < 0) {
         crc = copy_crc(host.ptr + at, slot + off, len);
@@ -260,6 +275,16 @@ int pool_host_copy_checked(WorkerPool& pool, const HostEnd& host, uint64_t image
   });
   for (const auto& list : found) out->insert(out->end(), list.begin(), list.end());
   return err.load();
+}
+
+// pieces in image order -> per-chunk values: crc(A || B) = crc(A) * x^(8 |B|) + crc(B)
+void fold_pieces(const std::vector<CheckedPiece>& pieces, const ChunkGrid& grid, std::vector<uint32_t>* chunk_crc,
+                 std::vector<uint64_t>* chunk_len) {
+  for (const CheckedPiece& p : pieces) {
+    const uint64_t k = grid.index(p.image_off);
+    (*chunk_crc)[k] = (*chunk_len)[k] ? mlf_crc32c_combine((*chunk_crc)[k], p.crc, p.len) : p.crc;
+    (*chunk_len)[k] += p.len;
+  }
 }
 
 }  // namespace
@@ -406,6 +431,8 @@ struct CrcRequest {
   uint32_t* out_host = nullptr;
   uint64_t n_out = 0;
   uint64_t* landed = nullptr;  // progress counter of the caller, or null
+  uint64_t first_part = 0;     // bytes up to the first chunk boundary (a piece of a larger data section)
+  bool by_host_threads = false;  // whatever the engine's setting
 };
 
 // What a device-to-host transfer waits for before its first copy: everything enqueued so far on a stream, or an
@@ -434,9 +461,11 @@ int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t
   const char* src = static_cast<const char*>(src_dev);
   if (crc.landed) __atomic_store_n(crc.landed, (uint64_t)0, __ATOMIC_RELEASE);
   const bool want_crc = crc.chunk_bytes != 0 && nbytes != 0;
-  const uint64_t n_crc = want_crc ? (nbytes + crc.chunk_bytes - 1) / crc.chunk_bytes : 0;
+  const ChunkGrid grid{crc.chunk_bytes, crc.first_part};
+  const uint64_t n_crc = want_crc ? grid.count(nbytes) : 0;
   if (want_crc && crc.n_out < n_crc) return fail(MLF_HIP_BAD_ARG, "checksum output too small");
-  const bool on_host = want_crc && e->host_checksums.load();
+  const bool on_host = want_crc && (crc.by_host_threads || e->host_checksums.load());
+  if (want_crc && !on_host && crc.first_part) return fail(MLF_HIP_BAD_ARG, "a first part needs the host threads' checksums");
   std::vector<CheckedPiece> pieces;
   std::vector<uint32_t> chunk_crc(on_host ? n_crc : 0);
   std::vector<uint64_t> chunk_len(on_host ? n_crc : 0, 0);
@@ -477,13 +506,9 @@ int engine_d2h(mlf_engine* e, const void* src_dev, const HostEnd& host, uint64_t
     if (c == 0) wait = now_s() - w0;
     if (on_host) {
       pieces.clear();
-      if (int err = pool_host_copy_checked(*e->pool, host, off, e->slots[s], len, crc.chunk_bytes, &pieces))
+      if (int err = pool_host_copy_checked(*e->pool, host, off, e->slots[s], len, grid, &pieces))
         return fail(MLF_HIP_RUNTIME, std::string("pwrite() to the buffer file failed: ") + strerror(err));
-      for (const CheckedPiece& p : pieces) {  // in image order: crc(A || B) = crc(A) * x^(8 |B|) + crc(B)
-        const uint64_t k = p.image_off / crc.chunk_bytes;
-        chunk_crc[k] = chunk_len[k] ? mlf_crc32c_combine(chunk_crc[k], p.crc, p.len) : p.crc;
-        chunk_len[k] += p.len;
-      }
+      fold_pieces(pieces, grid, &chunk_crc, &chunk_len);
     } else if (int err = pool_host_copy(*e->pool, host, off, e->slots[s], len, true)) {
       return fail(MLF_HIP_RUNTIME, std::string("pwrite() to the buffer file failed: ") + strerror(err));
     }
@@ -705,6 +730,74 @@ int mlf_engine_link_probe(mlf_engine* e, void* dev_buf, uint64_t nbytes, int to_
   for (hipStream_t s : e->streams) HIP_TRY(hipStreamSynchronize(s));
   drain.armed = false;
   *seconds = now_s() - t0;
+  return MLF_HIP_OK;
+}
+
+int mlf_engine_d2h_cut(mlf_engine* e, const void* src_dev, void* dst_host, uint64_t nbytes, void* producer_stream,
+                       void* ready_event, uint64_t crc_chunk_bytes, uint64_t first_part_bytes, uint32_t* crc_out_host,
+                       uint64_t n_crc_out, uint64_t* landed, mlf_xfer_stats* stats) {
+  if (!crc_chunk_bytes || !crc_out_host) return fail(MLF_HIP_BAD_ARG, "chunk size and checksum output are required");
+  if (first_part_bytes >= crc_chunk_bytes) return fail(MLF_HIP_BAD_ARG, "the first part is shorter than a chunk");
+  HostEnd host;
+  host.ptr = static_cast<char*>(dst_host);
+  CrcRequest crc;
+  crc.chunk_bytes = crc_chunk_bytes;
+  crc.out_host = crc_out_host;
+  crc.n_out = n_crc_out;
+  crc.landed = landed;
+  crc.first_part = first_part_bytes;
+  crc.by_host_threads = true;
+  Gate gate;
+  if (ready_event) {
+    gate.ready = static_cast<hipEvent_t>(ready_event);
+    gate.by_event = true;
+  } else {
+    gate.producer_stream = producer_stream;
+  }
+  return engine_d2h(e, src_dev, host, nbytes, gate, stats, crc);
+}
+
+int mlf_engine_host_copy_cut(mlf_engine* e, void* dst_host, const void* src_host, uint64_t nbytes,
+                             uint64_t crc_chunk_bytes, uint64_t first_part_bytes, uint32_t* crc_out_host,
+                             uint64_t n_crc_out) {
+  if (!e) return fail(MLF_HIP_BAD_ARG, "null engine");
+  if (nbytes && (!dst_host || !src_host)) return fail(MLF_HIP_BAD_ARG, "null pointer");
+  if (!crc_chunk_bytes || !crc_out_host) return fail(MLF_HIP_BAD_ARG, "chunk size and checksum output are required");
+  if (first_part_bytes >= crc_chunk_bytes) return fail(MLF_HIP_BAD_ARG, "the first part is shorter than a chunk");
+  const ChunkGrid grid{crc_chunk_bytes, first_part_bytes};
+  const uint64_t n_crc = grid.count(nbytes);
+  if (n_crc_out < n_crc) return fail(MLF_HIP_BAD_ARG, "checksum output too small");
+  std::lock_guard<std::mutex> g(e->busy);  // the threads are the ones a transfer uses
+  std::vector<CheckedPiece> pieces;
+  std::vector<uint32_t> chunk_crc(n_crc);
+  std::vector<uint64_t> chunk_len(n_crc, 0);
+  HostEnd host;
+  host.ptr = static_cast<char*>(dst_host);
+  // a slice at a time, so that the list of pieces stays short whatever the size
+  const uint64_t slice = (uint64_t)256 << 20;
+  for (uint64_t off = 0; off < nbytes; off += slice) {
+    pieces.clear();
+    (void)pool_host_copy_checked(*e->pool, host, off, static_cast<const char*>(src_host) + off,
+                                 (size_t)std::min(slice, nbytes - off), grid, &pieces);
+    fold_pieces(pieces, grid, &chunk_crc, &chunk_len);
+  }
+  std::copy(chunk_crc.begin(), chunk_crc.end(), crc_out_host);
+  return MLF_HIP_OK;
+}
+
+int mlf_engine_read_file(mlf_engine* e, int fd, uint64_t file_offset, void* dst_host, uint64_t nbytes) {
+  if (!e) return fail(MLF_HIP_BAD_ARG, "null engine");
+  if (fd < 0) return fail(MLF_HIP_BAD_ARG, "bad file descriptor");
+  if (nbytes && !dst_host) return fail(MLF_HIP_BAD_ARG, "null pointer");
+  std::lock_guard<std::mutex> g(e->busy);  // the threads are the ones a transfer uses
+  HostEnd host;
+  host.fd = fd;
+  host.file_off = file_offset;
+  const uint64_t slice = (uint64_t)1 << 30;  // (the pool splits a call into at most one part per thread)
+  for (uint64_t off = 0; off < nbytes; off += slice)
+    if (int err = pool_host_copy(*e->pool, host, off, static_cast<char*>(dst_host) + off,
+                                 (size_t)std::min(slice, nbytes - off), false))
+      return fail(MLF_HIP_RUNTIME, std::string("pread() from the buffer file failed: ") + strerror(err));
   return MLF_HIP_OK;
 }
 

@@ -106,6 +106,9 @@ _SIGNATURES = {
     "mlf_engine_avoid_streams": (_INT, [_VP, ctypes.POINTER(_VP), _U32, ctypes.POINTER(_U32)]),
     "mlf_engine_checksum_stream": (_VP, [_VP]),
     "mlf_engine_set_host_checksums": (_INT, [_VP, _INT]),
+    "mlf_engine_d2h_cut": (_INT, [_VP, _VP, _VP, _U64, _VP, _VP, _U64, _U64, _VP, _U64, _VP, ctypes.POINTER(XferStats)]),
+    "mlf_engine_host_copy_cut": (_INT, [_VP, _VP, _VP, _U64, _U64, _U64, _VP, _U64]),
+    "mlf_engine_read_file": (_INT, [_VP, _INT, _U64, _VP, _U64]),
     "mlf_engine_host_copy": (_INT, [_VP, _VP, _VP, _U64]),
     "mlf_engine_d2h_fd": (_INT, [_VP, _VP, _INT, _U64, _U64, _VP, ctypes.POINTER(XferStats)]),
     "mlf_engine_h2d_fd": (_INT, [_VP, _INT, _U64, _VP, _U64, _VP, ctypes.POINTER(XferStats)]),

@@ -54,6 +54,8 @@ _UPLOAD_ALIGN = 4096
 # are fetched together (a range costs about 0.3 ms to set up, the time 17 MB take on the link; measured on the
 # weights of the 112 GB shard: 16 MiB 0.41 s, 128 MiB 0.47 s).
 _PARTIAL_READ_MIN_SAVING = 256 << 20
+# a host-resident target of at least this size is filled by the copy engine's threads instead of one ``copy_``
+_HOST_COPY_ON_THE_ENGINE_FROM = 8 << 20
 # neighbourhoods that share a device buffer start on this boundary in it (uploads to less aligned device addresses
 # were measured at half the link's rate)
 _SLICE_ALIGN = 2 << 20
@@ -318,16 +320,16 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
         # a read that leaves out enough of the range to be worth several smaller uploads is decided on later
         if span - sum(info.length for info in asked.values()) + 256 * len(asked) >= _PARTIAL_READ_MIN_SAVING:
             return None
-        # the device the targets live on: the first few requests say (an object all of whose first targets are
-        # host-resident is taken to be one for the host)
+        # the device the targets live on: a sample of the requests says.  An object with host-resident targets among
+        # them is left to the ordinary way, which uploads only what the device targets need.
+        wanted = [req for req in read_items if req.type != LoadItemType.BYTE_IO]
         device = None
-        for req in [req for req in read_items[:64] if req.type != LoadItemType.BYTE_IO][:8]:
+        for req in wanted[:: max(1, len(wanted) // 32)][:33]:
             resolved[id(req)] = planner.resolve_tensor(req).detach()
-            device = resolved[id(req)].device
-            if device.type != "cpu":
-                break
-        if device is None or device.type == "cpu":
-            return None
+            if device is None:
+                device = resolved[id(req)].device
+            if resolved[id(req)].device != device or device.type == "cpu":
+                return None
         with torch.cuda.device(device):
             _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
             self._keep_clear_of(device)
@@ -376,7 +378,16 @@ class HipMLFlashpointCheckpointLoader(CheckpointDiscoveryMixin, MLFlashpointChec
                 assert target.size() == tensor.size(), (
                     f"req {req.storage_index} mismatch sizes {target.size()} vs {tensor.size()}"
                 )
-                target.copy_(tensor)
+                nbytes = tensor.numel() * tensor.element_size()
+                if (nbytes >= _HOST_COPY_ON_THE_ENGINE_FROM and tensor.dtype == target.dtype and tensor.is_contiguous()
+                        and target.is_contiguous()):
+                    # a large one (optimizer state kept in host memory): read from the file by the copy engine's
+                    # threads, straight into the target - a copy out of the mapping would take a page fault per
+                    # 4 KiB of it
+                    first = tensor.data_ptr() - (stream.data_address(0) - METADATA_SIZE)  # its place in the file
+                    self._get_engine().read_file(stream.fileno(), first, target.data_ptr(), nbytes)
+                else:
+                    target.copy_(tensor)
                 planner.commit_tensor(req, target)
                 stats["host_items"] += 1
                 continue

@@ -308,8 +308,9 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         GPU and keep it beside the object), ``crc_mode`` (where those checksums are computed: ``"host"``, the default - by the
         copy engine's host threads as they move the pinned slots into the buffer, crc32 instructions beside the
         copy loop: no kernel, no second read of the image, nothing added to the blocking part, and on the hosts
-        measured no slower than the plain copy; objects that are sent in pieces or through windows are checksummed
-        as with ``"beside"``; ``"beside"`` - a pass of kernels over the finished image, on the copy engine's third
+        measured no slower than the plain copy; the same holds for objects that leave in several transfers (pieces,
+        windows, host-resident items between the runs of the image), whose parts' checksums are joined per chunk;
+        ``"beside"`` - a pass of kernels over the finished image, on the copy engine's third
         stream while the image crosses the link: nothing added to the blocking part either, but the image is read
         from device memory a second time; ``"fused"`` - inside the pack kernel, which then runs about 12 % longer),
         ``use_file_io`` (False, the default: the host threads memcpy the
@@ -696,6 +697,20 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
             kept.plan.destroy()  # releasing device memory waits for the kernels that still use it
 
     @staticmethod
+    def _blob_of_rows(rows: np.ndarray, blob: bytes) -> bytes:
+        """The part of the host blob that the blob items among ``rows`` refer to, their offsets rebased onto it: a
+        plan uploads its blob whole, and the blob of an object with host-resident tensors laid out inside its image
+        is as large as those tensors together - more than a window's plan may bring to a device that is short of
+        room.  ``rows`` is changed in place."""
+        from_blob = rows["kind"] == hip_plan.ITEM_BLOB
+        if not from_blob.any():
+            return b""
+        first = int(rows["ptr"][from_blob].min())
+        end = int((rows["ptr"][from_blob] + rows["nbytes"][from_blob]).max())
+        rows["ptr"][from_blob] -= first
+        return blob[first:end]
+
+    @staticmethod
     def _windows_of(layout: hip_plan.SaveLayout, limit: int, stop: Optional[int] = None) -> list:
         """Consecutive rows of the layout's table (the first ``stop`` of them) grouped into windows of at most
         ``limit`` image bytes (a single larger row gets a window of its own): [(first row, end row, first image
@@ -743,8 +758,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                 pad = begin % _WINDOW_PAD  # as in _stage_windowed
                 sub = layout.items[r0:r1].copy()
                 sub["image_off"] -= begin - pad
-                plan = hip_plan.Plan(sub, layout.blob, pad + end - begin, tile_bytes=self._tile_bytes,
-                                     block_threads=self._block_threads)
+                plan = hip_plan.Plan(sub, self._blob_of_rows(sub, layout.blob), pad + end - begin,
+                                     tile_bytes=self._tile_bytes, block_threads=self._block_threads)
                 plan.pack(buf, stream)
                 pieces.append((plan, buf, begin, end))
             packed = torch.cuda.Event(enable_timing=self.record_kernel_events)
@@ -814,8 +829,8 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                     pad = begin % _WINDOW_PAD
                     sub = arr[r0:r1].copy()
                     sub["image_off"] -= begin - pad
-                    plan = hip_plan.Plan(sub, layout.blob, pad + end - begin, tile_bytes=self._tile_bytes,
-                                         block_threads=self._block_threads)
+                    plan = hip_plan.Plan(sub, self._blob_of_rows(sub, layout.blob), pad + end - begin,
+                                         tile_bytes=self._tile_bytes, block_threads=self._block_threads)
                     made.append(plan)
                     if self.record_kernel_events:
                         t_begin, packed = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -837,11 +852,17 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
                     with torch.cuda.device(device):
                         _lib.check(_lib.load().mlf_hip_set_device(device.index or 0), "mlf_hip_set_device")
                         dst = writer.data_address(start + begin)
-                        st, _ = engine.d2h_gated(buf.data_ptr() + pad, dst, end - begin, packed.cuda_event, 0,
-                                                 ctypes.c_uint64(0))
+                        if sums is not None and self._crc_mode == "host":
+                            # the threads that copy the window into the file take its checksums as they go
+                            st, values = engine.d2h_cut(buf.data_ptr() + pad, dst, end - begin, begin, self._crc_chunk_bytes,
+                                                        ready_event=packed.cuda_event)
+                            sums.add(begin, end - begin, values)
+                        else:
+                            st, _ = engine.d2h_gated(buf.data_ptr() + pad, dst, end - begin, packed.cuda_event, 0,
+                                                     ctypes.c_uint64(0))
                         xfer["d2h_s"] += st.seconds
                         xfer["d2h_bytes"] += end - begin
-                        if sums is not None:
+                        if sums is not None and self._crc_mode != "host":
                             t0 = time.perf_counter()
                             sums.add(begin, end - begin, hip_plan.crc32c_device_cut(
                                 buf, pad, begin, end - begin, self._crc_chunk_bytes, dst, side))
@@ -1235,13 +1256,19 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
         for k, (plan, buf, begin, end) in enumerate(staged.pieces):
             pad = begin % _WINDOW_PAD
             dst = writer.data_address(start + begin)
-            if staged.packed_event is not None:
+            on_host = sums is not None and self._crc_mode == "host"
+            if on_host:
+                st, values = engine.d2h_cut(
+                    buf.data_ptr() + pad, dst, end - begin, begin, self._crc_chunk_bytes, producer_stream=staged.stream,
+                    ready_event=staged.packed_event.cuda_event if staged.packed_event is not None else None)
+                sums.add(begin, end - begin, values)
+            elif staged.packed_event is not None:
                 st, _ = engine.d2h_gated(buf.data_ptr() + pad, dst, end - begin, staged.packed_event.cuda_event, 0,
                                          ctypes.c_uint64(0))
             else:
                 st = engine.d2h(buf.data_ptr() + pad, dst, end - begin, staged.stream)
             self._count_transfer(xfer, st, end - begin)
-            if sums is not None:
+            if sums is not None and not on_host:
                 # the piece has left the device, so its pack is over: the side stream may read it at once
                 t0 = time.perf_counter()
                 sums.add(begin, end - begin, hip_plan.crc32c_device_cut(buf, pad, begin, end - begin,
@@ -1259,33 +1286,45 @@ class HipMLFlashpointCheckpointSaver(MLFlashpointCheckpointSaver):
     def _transfer_in_pieces(self, staged: StagedObject, writer, start: int, xfer: dict):
         """The transfer of an object some of whose tensors live in host memory: the runs of the image between them
         cross the host link, the host-resident payloads are copied from where they are into their places in the
-        buffer, in the order of the data section.  Returns the chunk checksums (taken on the host, from the pages
-        just written: the image alone is not the object) or None."""
+        buffer, in the order of the data section.  Returns the chunk checksums or None: taken by the host threads as
+        they move each piece (``crc_mode="host"``), else from the pages just written - the image alone is not the
+        object, so the kernels cannot give them."""
         layout = staged.layout
         engine = self._get_engine()
+        chunk = self._crc_chunk_bytes
+        sums = integrity.ChunkChecksums(chunk, layout.data_bytes) if chunk and self._crc_mode == "host" else None
         pieces = [(data_off, n, image_off, None) for image_off, data_off, n in layout.segments]
         pieces += [(data_off, n, None, t) for (data_off, n, _), t in zip(layout.host_spans, layout.host_tensors)]
         t_host = 0.0
         for data_off, n, image_off, tensor in sorted(pieces, key=lambda piece: piece[0]):
             dst = writer.data_address(start + data_off)
             if tensor is None:
-                st = engine.d2h(staged.image.data_ptr() + image_off, dst, n, staged.stream)
+                if sums is not None:
+                    st, values = engine.d2h_cut(staged.image.data_ptr() + image_off, dst, n, data_off, chunk,
+                                                producer_stream=staged.stream)
+                    sums.add(data_off, n, values)
+                else:
+                    st = engine.d2h(staged.image.data_ptr() + image_off, dst, n, staged.stream)
                 self._count_transfer(xfer, st, n)
             else:
                 t0 = time.perf_counter()
                 if isinstance(tensor, torch.Tensor):
                     source = tensor.detach().contiguous()  # a copy only if the tensor is a strided view
                     assert source.numel() * source.element_size() == n
-                    engine.host_copy(dst, source.data_ptr(), n)
+                    address = source.data_ptr()
                 else:  # the bytes of a large pickled object
                     source = np.frombuffer(tensor, dtype=np.uint8)
                     assert source.size == n
-                    engine.host_copy(dst, source.ctypes.data, n)
+                    address = source.ctypes.data
+                if sums is not None:
+                    sums.add(data_off, n, engine.host_copy_cut(dst, address, n, data_off, chunk))
+                else:
+                    engine.host_copy(dst, address, n)
                 t_host += time.perf_counter() - t0
                 xfer["host_copy_bytes"] = xfer.get("host_copy_bytes", 0) + n
             staged._landed.value = data_off + n
         xfer["host_copy_s"] = xfer.get("host_copy_s", 0.0) + t_host
-        return self._host_side_checksums(writer, start, layout.data_bytes)
+        return sums.result() if sums is not None else self._host_side_checksums(writer, start, layout.data_bytes)
 
     # ---- replication hand-off, metadata, finalize (host logic kept as in the reference) -------------------
     @log_execution_time(logger=_LOGGER, name="async_replicate_object")

@@ -455,6 +455,42 @@ class CopyEngine:
                                                      ctypes.byref(seconds)), "mlf_engine_link_probe")
         return seconds.value
 
+    @staticmethod
+    def _cut_count(nbytes: int, crc_chunk_bytes: int, first_part_bytes: int) -> int:
+        head = min(first_part_bytes, nbytes)
+        return (1 if head else 0) + -(-(nbytes - head) // crc_chunk_bytes)
+
+    def d2h_cut(self, src_dev_ptr: int, dst_host_ptr: int, nbytes: int, data_off: int, crc_chunk_bytes: int,
+                producer_stream: int = 0, ready_event: Optional[int] = None, landed: "Optional[ctypes.c_uint64]" = None):
+        """A piece of a data section, from byte ``data_off`` of the section on, device to host, with the checksums of
+        the piece taken by the host threads as they copy and cut where the section's chunks end: one value per part
+        of ``integrity.ChunkChecksums.cuts(data_off, nbytes, crc_chunk_bytes)``.  The copies wait for ``ready_event``
+        if given, else for what ``producer_stream`` holds now.  Returns (stats, list of values)."""
+        stats = _lib.XferStats()
+        first = -data_off % crc_chunk_bytes
+        n = self._cut_count(nbytes, crc_chunk_bytes, first)
+        crcs = np.zeros(max(n, 1), dtype=np.uint32)
+        _lib.check(
+            _lib.load().mlf_engine_d2h_cut(self._handle, src_dev_ptr, dst_host_ptr, nbytes, producer_stream, ready_event,
+                                           crc_chunk_bytes, first, crcs.ctypes.data, len(crcs),
+                                           ctypes.addressof(landed) if landed is not None else None, ctypes.byref(stats)),
+            "mlf_engine_d2h_cut",
+        )
+        return stats, [int(v) for v in crcs[:n]]
+
+    def host_copy_cut(self, dst_host_ptr: int, src_host_ptr: int, nbytes: int, data_off: int, crc_chunk_bytes: int) -> list:
+        """``host_copy`` of a piece of a data section that also yields the piece's checksums, cut like ``d2h_cut``'s."""
+        first = -data_off % crc_chunk_bytes
+        n = self._cut_count(nbytes, crc_chunk_bytes, first)
+        crcs = np.zeros(max(n, 1), dtype=np.uint32)
+        _lib.check(_lib.load().mlf_engine_host_copy_cut(self._handle, dst_host_ptr, src_host_ptr, nbytes, crc_chunk_bytes,
+                                                        first, crcs.ctypes.data, len(crcs)), "mlf_engine_host_copy_cut")
+        return [int(v) for v in crcs[:n]]
+
+    def read_file(self, fd: int, file_offset: int, dst_host_ptr: int, nbytes: int) -> None:
+        """A range of a file into host memory, by ``pread`` on the engine's threads."""
+        _lib.check(_lib.load().mlf_engine_read_file(self._handle, fd, file_offset, dst_host_ptr, nbytes), "mlf_engine_read_file")
+
     def host_copy(self, dst_host_ptr: int, src_host_ptr: int, nbytes: int) -> None:
         """Host memory to host memory on the engine's threads (checkpoint items that are resident on the host)."""
         _lib.check(_lib.load().mlf_engine_host_copy(self._handle, dst_host_ptr, src_host_ptr, nbytes), "mlf_engine_host_copy")

@@ -717,6 +717,68 @@ def test_checksums_taken_by_the_host_threads_equal_the_kernels_and_the_oracle(sl
     engine.destroy()
 
 
+@pytest.mark.parametrize("data_off, nbytes, chunk_bytes", [(0, (5 << 20) + 3, 1 << 20), (777, (5 << 20) + 3, 1 << 20),
+                                                           ((3 << 20) - 5, 4, 1 << 20), ((1 << 20) + 4096, 70 << 20, 32 << 20),
+                                                           (65536 * 3 + 1, 65536 * 9, 65536)])
+def test_pieces_of_a_data_section_are_checksummed_on_the_sections_chunk_grid(data_off, nbytes, chunk_bytes, shm_dir, oracle_c):
+    """``mlf_engine_d2h_cut`` / ``mlf_engine_host_copy_cut``: a piece that begins inside a chunk of the section it
+    belongs to gets one value for the bytes up to the next boundary, one per whole chunk and one for the rest - the
+    parts ``integrity.ChunkChecksums.cuts`` names - each equal to the oracle's CRC-32C of those bytes; joined with
+    the neighbours' parts they give the section's chunk values."""
+    from ml_flashpoint.checkpoint_object_manager.buffer_object.buffer_object_ext import BufferObject
+    from ml_flashpoint.hip import integrity
+    from ml_flashpoint.hip import plan as P
+
+    gen = torch.Generator().manual_seed(nbytes + data_off)
+    host = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=gen)
+    raw = host.numpy().tobytes()
+    dev = host.to(DEV)
+    parts = integrity.ChunkChecksums.cuts(data_off, nbytes, chunk_bytes)
+    want = []
+    for first, length in parts:
+        one = np.zeros(1, dtype=np.uint32)
+        oracle_c.oracle_crc32c_chunks(raw[first - data_off : first - data_off + length], length, 1 << 40, one.ctypes.data)
+        want.append(int(one[0]))
+    engine = P.CopyEngine(slot_bytes=1 << 20, n_slots=3, n_threads=5)
+    bo = BufferObject(f"{shm_dir}/cut.bin", 4096 + nbytes, True)
+    stream = torch.cuda.current_stream().cuda_stream
+    stats, got = engine.d2h_cut(dev.data_ptr(), bo.get_data_ptr() + 4096, nbytes, data_off, chunk_bytes, producer_stream=stream)
+    assert stats.bytes == nbytes and bytes(memoryview(bo)[4096:]) == raw and got == want
+    done = torch.cuda.Event()
+    done.record()
+    landed = ctypes.c_uint64(0)
+    memoryview(bo)[4096:] = bytes(nbytes)
+    _, got = engine.d2h_cut(dev.data_ptr(), bo.get_data_ptr() + 4096, nbytes, data_off, chunk_bytes,
+                            ready_event=done.cuda_event, landed=landed)
+    assert int(landed.value) == nbytes and bytes(memoryview(bo)[4096:]) == raw and got == want
+    memoryview(bo)[4096:] = bytes(nbytes)
+    source = host.clone()
+    assert engine.host_copy_cut(bo.get_data_ptr() + 4096, source.data_ptr(), nbytes, data_off, chunk_bytes) == want
+    assert bytes(memoryview(bo)[4096:]) == raw
+    # the section's chunk values from this piece and a neighbour on either side
+    before, after = b"\x5a" * data_off, b"\xa5" * 12345
+    whole = before + raw + after
+    sums = integrity.ChunkChecksums(chunk_bytes, len(whole))
+    for offset, data in ((0, before), (data_off, raw), (data_off + nbytes, after)):
+        if not data:
+            continue
+        values = []
+        for first, length in integrity.ChunkChecksums.cuts(offset, len(data), chunk_bytes):
+            one = np.zeros(1, dtype=np.uint32)
+            oracle_c.oracle_crc32c_chunks(data[first - offset : first - offset + length], length, 1 << 40, one.ctypes.data)
+            values.append(int(one[0]))
+        sums.add(offset, len(data), got if data is raw else values)
+    section = np.zeros(-(-len(whole) // chunk_bytes), dtype=np.uint32)
+    oracle_c.oracle_crc32c_chunks(whole, len(whole), chunk_bytes, section.ctypes.data)
+    assert sums.result().tolist() == section.tolist()
+    lib = __import__("ml_flashpoint.hip._lib", fromlist=["load"]).load()
+    out = np.zeros(4, dtype=np.uint32)
+    assert lib.mlf_engine_d2h_cut(engine._handle, dev.data_ptr(), bo.get_data_ptr() + 4096, nbytes, stream, None, chunk_bytes,
+                                  chunk_bytes, out.ctypes.data, 4, None, None) != 0  # a first part as long as a chunk
+    bo.close()
+    engine.destroy()
+
+
 def test_watched_transfer_publishes_only_bytes_that_are_in_place(shm_dir, oracle_c):
     """While a 200 MiB image crosses the link in 1 MiB slots, a second thread follows the progress counter and copies
     whatever prefix it announces out of the mapping: the counter only grows, never runs ahead of the data, ends at the

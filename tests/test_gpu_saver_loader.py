@@ -150,9 +150,9 @@ def test_dcp_save_bytes_equal_oracle_and_load_is_bit_exact(shm_dir, manager_futu
             if isinstance(v, torch.Tensor):
                 assert torch.equal(_bits(target[k]), _bits(v)), k
         assert loader.last_load_stats["device_items"] >= 8 and loader.last_load_stats["host_items"] == 1
-        # where the records lie is in the checkpoint's metadata: the range that holds them is on its way to the
-        # device before their headers are parsed
-        assert loader.last_load_stats.get("upload_began_before_parse", 0) == 1
+        # (an object with a host-resident target among the device targets is not uploaded ahead of the parse: what
+        # the device needs of it is known only once the targets are)
+        assert "upload_began_before_parse" not in loader.last_load_stats
 
     # and the oracle's CPU loader restores our file
     target = {k: (torch.zeros_like(v) if isinstance(v, torch.Tensor) else None) for k, v in sd_cpu.items()}
@@ -488,23 +488,24 @@ def test_multiple_buckets_and_overwrite_of_existing_object(shm_dir):
     assert raw == fmt.file_image([torch.ones(3)])[0]
 
 
-def test_object_larger_than_the_hbm_limit_is_saved_window_by_window(shm_dir, manager_future):
+@pytest.mark.parametrize("crc_mode", ["host", "beside"])
+def test_object_larger_than_the_hbm_limit_is_saved_window_by_window(shm_dir, manager_future, crc_mode):
     """With ``max_image_bytes`` far below the object size the saver packs and sends windows of records through
     one small device buffer; the file is the same."""
     sd_cpu = {k: v for k, v in _mixed_state_dict().items()}
     sd_cpu["big"] = torch.arange(200_000, dtype=torch.float32)  # one record larger than the limit
     sd_dev = _to_dev(sd_cpu, keep_on_host=("w.i64",))
     ckpt = os.path.join(shm_dir, "step-8_ckpt")
-    saver = _saver(max_image_bytes=64 << 10, crc_chunk_bytes=1 << 16)
+    saver = _saver(max_image_bytes=64 << 10, crc_chunk_bytes=1 << 16, crc_mode=crc_mode)
     dcp.save(sd_dev, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(saver, manager_future), no_dist=True)
     assert saver.last_save_stats["windows"] >= 4
     raw = open(os.path.join(ckpt, "__0__0_src0.distcp"), "rb").read()
     metadata = pickle.load(open(os.path.join(ckpt, ".metadata"), "rb"))
     image, spans, got_spans = _expected_file(sd_cpu, metadata, raw)
     assert raw == image and got_spans == spans
-    # windows end where records end, not where checksum chunks end: the sidecar is joined from the checksums the GPU
-    # took of the parts of each window; every value is the host's for that chunk of the file, and the GPU check of an
-    # ordinary restore accepts it
+    # windows end where records end, not where checksum chunks end: the sidecar is joined from the checksums of the
+    # parts of each window - taken by the host threads as they copy the window, or by kernels; every value is the
+    # host's for that chunk of the file, and the GPU check of an ordinary restore accepts it
     from ml_flashpoint.hip import integrity
     from ml_flashpoint.hip import plan as P
 
@@ -594,8 +595,10 @@ def test_windowed_save_reports_a_failure_of_the_part_that_follows(shm_dir, monke
     assert raw == fmt.file_image([data[r.index.fqn].cpu() for r in order])[0]
 
 
+@pytest.mark.parametrize("crc_mode", ["host", "beside"])
 @pytest.mark.parametrize("background_write", [False, True])
-def test_image_is_held_in_pieces_when_no_single_block_is_to_be_had(shm_dir, manager_future, monkeypatch, background_write):
+def test_image_is_held_in_pieces_when_no_single_block_is_to_be_had(shm_dir, manager_future, monkeypatch, background_write,
+                                                                   crc_mode):
     """Free device memory that is not in one block (the usual state of a long-running job): the image is packed into
     several smaller buffers, all resident, and sent piece by piece - same file, valid sidecar, and still an
     asynchronous save - instead of failing or falling back to the blocking window-by-window mode."""
@@ -619,7 +622,7 @@ def test_image_is_held_in_pieces_when_no_single_block_is_to_be_had(shm_dir, mana
 
     monkeypatch.setattr(P, "try_allocate", fragmented)
     monkeypatch.setattr(saver_mod, "_IMAGE_PIECE_BYTES", 1 << 18)
-    saver = _saver(crc_chunk_bytes=1 << 16, background_write=background_write)
+    saver = _saver(crc_chunk_bytes=1 << 16, background_write=background_write, crc_mode=crc_mode)
     ckpt = os.path.join(shm_dir, "step-6_ckpt")
     dcp.save(sd_dev, checkpoint_id=ckpt, storage_writer=MemoryStorageWriter(saver, manager_future), no_dist=True)
     obj = os.path.join(ckpt, "__0__0_src0.distcp")
@@ -856,8 +859,9 @@ def test_plans_are_kept_from_save_to_save_and_rebuilt_when_the_tensors_change(sh
     assert "plans_reused" not in save(9, sd_dev) and "plans_reused" not in save(10, sd_dev)
 
 
+@pytest.mark.parametrize("crc_mode", ["host", "beside"])
 @pytest.mark.parametrize("background_write", [False, True])
-def test_large_host_resident_tensors_go_from_host_memory_into_the_buffer(shm_dir, manager_future, background_write):
+def test_large_host_resident_tensors_go_from_host_memory_into_the_buffer(shm_dir, manager_future, background_write, crc_mode):
     """A state dict with part of it kept in host memory (offloaded optimizer state): the large host tensors never visit
     the device - the image holds the rest, in runs that are sent to their places around them - and the file is still
     the oracle's, byte for byte, with a valid checksum sidecar; a second save through the kept plan picks up the
@@ -879,7 +883,7 @@ def test_large_host_resident_tensors_go_from_host_memory_into_the_buffer(shm_dir
     }
     on_host = {k for k in sd_cpu if k.startswith("host.")}
     sd = {k: (v.to(DEV) if isinstance(v, torch.Tensor) and k not in on_host else v) for k, v in sd_cpu.items()}
-    saver = _saver(crc_chunk_bytes=1 << 18, background_write=background_write)
+    saver = _saver(crc_chunk_bytes=1 << 18, background_write=background_write, crc_mode=crc_mode)
     big_host_bytes = sum(sd_cpu[k].numel() * sd_cpu[k].element_size() for k in ("host.m", "host.v_view", "host.last"))
     for step in (1, 2):
         ckpt = os.path.join(shm_dir, f"step-{step}_ckpt")
@@ -905,6 +909,22 @@ def test_large_host_resident_tensors_go_from_host_memory_into_the_buffer(shm_dir
                   for k, v in sd_cpu.items()}
         dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, _loader()), no_dist=True)
         assert target["obj.step"] == 7 and target["obj.big"] == sd_cpu["obj.big"]
+        for k, v in sd_cpu.items():
+            if isinstance(v, torch.Tensor):
+                assert torch.equal(_bits(target[k]), _bits(v)), k
+        # once more with the large host-resident targets read from the file by the copy engine's threads (as
+        # targets of 8 MiB and more are), the small one by ``copy_``
+        from ml_flashpoint.hip import checkpoint_loader as loader_mod
+
+        for v in target.values():
+            if isinstance(v, torch.Tensor):
+                v.zero_()
+        threshold = loader_mod._HOST_COPY_ON_THE_ENGINE_FROM
+        loader_mod._HOST_COPY_ON_THE_ENGINE_FROM = 1 << 19
+        try:
+            dcp.load(target, checkpoint_id=ckpt, storage_reader=MemoryStorageReader(ckpt, _loader()), no_dist=True)
+        finally:
+            loader_mod._HOST_COPY_ON_THE_ENGINE_FROM = threshold
         for k, v in sd_cpu.items():
             if isinstance(v, torch.Tensor):
                 assert torch.equal(_bits(target[k]), _bits(v)), k
