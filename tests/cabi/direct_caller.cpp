@@ -175,6 +175,33 @@ int main(int argc, char** argv) {
   REQUIRE(mlf_engine_d2h_gated(engine, d_image, dst2, image_bytes, packed, chunk, chunk_got.data(), n_chunks, &landed, &stats) == 0);
   REQUIRE(landed == image_bytes && chunk_got == chunk_want && std::memcmp(dst2, want.data(), image_bytes) == 0);
   REQUIRE(mlf_engine_set_host_checksums(engine, 0) == 0 && mlf_engine_set_host_checksums(nullptr, 1) != 0);
+  // the image as two pieces of a data section, cut at an odd byte: the second begins inside a chunk, its first value
+  // covers the bytes up to the next boundary; joined, the parts give the values of the whole
+  {
+    const uint64_t cut = 3 * chunk + 4099, first_part = chunk - cut % chunk;
+    std::vector<uint32_t> head(n_chunks), tail(n_chunks + 1);
+    std::memset(dst2, 0, image_bytes);
+    REQUIRE(mlf_engine_d2h_cut(engine, d_image, dst2, cut, nullptr, packed, chunk, 0, head.data(), head.size(), nullptr, &stats) == 0);
+    REQUIRE(mlf_engine_d2h_cut(engine, static_cast<char*>(d_image) + cut, dst2 + cut, image_bytes - cut, nullptr, nullptr, chunk, first_part,
+                               tail.data(), tail.size(), &landed, &stats) == 0);
+    REQUIRE(landed == image_bytes - cut && std::memcmp(dst2, want.data(), image_bytes) == 0);
+    std::vector<uint32_t> joined(n_chunks);
+    for (uint64_t k = 0; k < 3; ++k) joined[k] = head[k];
+    joined[3] = mlf_crc32c_combine(head[3], tail[0], first_part);
+    for (uint64_t k = 4; k < n_chunks; ++k) joined[k] = tail[k - 3];
+    REQUIRE(joined == chunk_want);
+    // host memory to host memory with the same cut, and a range of the file back into host memory
+    std::vector<char> copy(image_bytes - cut);
+    std::vector<uint32_t> tail2(n_chunks + 1);
+    REQUIRE(mlf_engine_host_copy_cut(engine, copy.data(), want.data() + cut, copy.size(), chunk, first_part, tail2.data(),
+                                     tail2.size()) == 0);
+    REQUIRE(tail2 == tail && std::memcmp(copy.data(), want.data() + cut, copy.size()) == 0);
+    std::fill(copy.begin(), copy.end(), 0);
+    REQUIRE(mlf_engine_read_file(engine, mlf_buffer_fd(buf2), 4096 + cut, copy.data(), copy.size()) == 0);
+    REQUIRE(std::memcmp(copy.data(), want.data() + cut, copy.size()) == 0);
+    std::vector<char> longer(copy.size() + (1 << 20));  // more than the file holds: an error, not a hang
+    REQUIRE(mlf_engine_read_file(engine, mlf_buffer_fd(buf2), 4096 + cut, longer.data(), longer.size()) != 0);
+  }
   double seconds = 0;
   REQUIRE(mlf_engine_link_probe(engine, d_image, image_bytes, 1, &seconds) == 0 && seconds > 0);
 
