@@ -967,7 +967,8 @@ Collapsed collapse_dims(const mlf_item& it) {
 // Patches are long along the side that is written - partly written lines then meet in one L2, which matters more
 // than partly used fetched lines meeting there.  Same 667 blocks, patches of (tiles along the read side) x (along
 // the written side): 1 x 64 4.17 / 3.93 with 128 x 128-byte tiles, 64 x 1 3.13 / 4.39 (the written side is a for an
-// unpack), 8 x 8 4.10 / 4.41; with 128 x 256-byte tiles 2 x 16 4.34 / 4.49, 4 x 16 4.47 / 4.50, 8 x 8 4.36 / 4.44.
+// unpack), 8 x 8 4.10 / 4.41; with 128 x 256-byte tiles 2 x 16 4.34 / 4.49, 4 x 16 4.47 / 4.50, 8 x 8 4.36 / 4.44;
+// larger patches change nothing (8 x 16 4.43 / 4.45, 4 x 32 4.47 / 4.46, 4 x 64 4.49 / 4.43, 16 x 32 4.37 / 4.33).
 constexpr uint32_t kTransPatchRead = 4, kTransPatchWritten = 16;
 struct TransOrder {
   uint32_t patch_a = 1, patch_b = 1;
